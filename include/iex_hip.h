@@ -1,0 +1,179 @@
+/*
+ * libiex_hip.so -- C ABI of the gfx950 sparse-plus-dense GEMM path.
+ *
+ * Conventions (they replace the reference's launcher ABI, csrc/extensions.h:10-31):
+ *   - every pointer is a DEVICE pointer owned by the caller; nothing is allocated,
+ *     freed or synchronised inside the library (except the iex_graph_* host objects);
+ *   - `stream` is a hipStream_t passed as void* (NULL = the legacy default stream);
+ *   - functions return 0 (hipSuccess) on success, a positive hipError_t when the HIP
+ *     runtime refused something, or a negative IEX_ERR_* code when an argument is
+ *     rejected before any launch; iex_last_error() holds the text of the last failure
+ *     on the calling thread;
+ *   - matrices are row-major and contiguous; the batch dimension is outermost;
+ *   - a CSR matrix is (row_indices, values, row_offsets, column_indices): row_offsets
+ *     has m+1 int32 entries, column_indices are ascending inside a row, row_indices is
+ *     the scheduling swizzle (a permutation of 0..m-1, heavy rows first).  The swizzle
+ *     only orders the work: output row r is always written from CSR row r.
+ */
+#ifndef IEX_HIP_H_
+#define IEX_HIP_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define IEX_ABI_VERSION 1
+
+/* element types of values / dense operands */
+enum { IEX_F32 = 0, IEX_F16 = 1, IEX_BF16 = 2 };
+/* element types of column_indices */
+enum { IEX_I32 = 0, IEX_I16 = 1 };
+
+/* negative return codes (argument errors detected on the host) */
+enum {
+  IEX_ERR_BAD_ARGUMENT = -1,   /* null pointer, negative size, unknown enum */
+  IEX_ERR_UNSUPPORTED = -2,    /* combination the library has no kernel for */
+  IEX_ERR_TOO_LARGE = -3,      /* a dimension exceeds what the grid / index type can hold */
+  IEX_ERR_STATE = -4           /* graph object used out of order */
+};
+
+int iex_abi_version(void);
+/* Text of the most recent failure on this thread ("" when none). */
+const char* iex_last_error(void);
+/* 1 when a gfx950 device is visible to the HIP runtime, else 0. */
+int iex_device_ok(void);
+
+/* ------------------------------------------------------------------ SpMM ---- */
+/* flags for iex_spmm_ex */
+#define IEX_SPMM_PER_BATCH_VALUES 0x1 /* values is (batch, nnz) instead of (nnz)            */
+#define IEX_SPMM_ACCUMULATE 0x2       /* out += A*b (reference "atomic" store mode)         */
+#define IEX_SPMM_RELU 0x4             /* out = max(0, A*b + bias)                           */
+/* bits 8..15: force waves-per-row (1, 4 or 16); 0 = choose from nnz/m.  For tuning.       */
+#define IEX_SPMM_FORCE_WPR(w) (((w) & 0xff) << 8)
+
+/* out[z, r, :] = sum_j values[(z,) j] * dense[z, column_indices[j], :]  (+ bias[r], ReLU)
+ * dense is (batch, k, n), out is (batch, m, n), both of `dtype`; accumulation is fp32.
+ * bias (fp32, length m) may be NULL.
+ * Generalises CudaSpmmBiasRelu (sputnik_spmm_host_func.cu.inc:118-204). */
+int iex_spmm_ex(int dtype, int itype, int flags, int m, int k, int n, int nonzeros,
+                const int* row_indices, const void* values, const int* row_offsets,
+                const void* column_indices, const void* dense, const float* bias,
+                void* out, void* stream, int batch);
+
+/* Drop-ins for the three launchers the reference declares in csrc/extensions.h:28-30.
+ * CudaSpmm2: fp32, per-batch values (batch, nnz), accumulates into `out`
+ *            (spmm_sputnik_atomic, sputnik_kernels.cpp:170-172);
+ * CudaSpmm3: fp32, values shared by the batch (spmm_sputnik_reuse_weight, :173-175);
+ * CudaSpmm5: fp16 values / dense / out, int16 column indices, values shared
+ *            (spmm_sputnik_reuse_weight_half, :179-181). */
+int iex_CudaSpmm2(int m, int k, int n, int nonzeros, const int* row_indices,
+                  const float* values, const int* row_offsets, const int* column_indices,
+                  const float* dense_matrix, float* output_matrix, void* stream,
+                  int batch_size);
+int iex_CudaSpmm3(int m, int k, int n, int nonzeros, const int* row_indices,
+                  const float* values, const int* row_offsets, const int* column_indices,
+                  const float* dense_matrix, float* output_matrix, void* stream,
+                  int batch_size);
+int iex_CudaSpmm5(int m, int k, int n, int nonzeros, const int* row_indices,
+                  const uint16_t* values, const int* row_offsets,
+                  const int16_t* column_indices, const uint16_t* dense_matrix,
+                  uint16_t* output_matrix, void* stream, int batch_size);
+
+/* ----------------------------------------------------------------- SDDMM ---- */
+#define IEX_SDDMM_SUM_OVER_BATCH 0x1 /* one (nnz) output summed over the batch            */
+#define IEX_SDDMM_ACCUMULATE 0x2     /* out += ... instead of out = ...                   */
+
+/* out[(z,) j] = sum_c lhs[z, row(j), c] * rhs[z, column_indices[j], c]
+ * lhs is (batch, m, k), rhs is (batch, n, k) -- rhs rows are the sampled columns.
+ * out is (nnz) with IEX_SDDMM_SUM_OVER_BATCH, else (batch, nnz); fp32 accumulation.
+ * Generalises CudaSddmm2 (sputnik_sddmm.cu.inc:206-233) to fp16 and per-batch output. */
+int iex_sddmm_ex(int dtype, int flags, int m, int k, int n, int nonzeros,
+                 const int* row_indices, const int* row_offsets, const int* column_indices,
+                 const void* lhs_matrix, const void* rhs_matrix, void* output_values,
+                 void* stream, int batch);
+
+/* Drop-in for CudaSddmm2 (csrc/extensions.h:31; sddmm_sputnik_atomic_upd_weight,
+ * sputnik_kernels.cpp:182-184): fp32, output (nnz) = sum over the batch, written
+ * (not accumulated), so the caller need not zero it. */
+int iex_CudaSddmm2(int m, int k, int n, int nonzeros, const int* row_indices,
+                   const int* row_offsets, const int* column_indices,
+                   const float* lhs_matrix, const float* rhs_matrix, float* output_values,
+                   void* stream, int batch_size);
+
+/* In-place row-wise softmax over the stored entries of a CSR matrix:
+ * values[z, j] = exp(scale*values[z, j] - max_row) / sum_row.  values is (batch, nnz).
+ * The middle step of sparse attention between SDDMM and SpMM (no reference
+ * counterpart in tree; the reference leaves it to xformers). */
+int iex_csr_softmax(int dtype, int m, int nonzeros, const int* row_indices,
+                    const int* row_offsets, void* values, float scale, void* stream,
+                    int batch);
+
+/* ------------------------------------------------------------------ GEMM ---- */
+/* C[z] = A[z] * B[z] (trans_b == 0, B is (K,N)) or A[z] * B[z]^T (trans_b == 1, B is
+ * (N,K), the torch.nn.Linear weight layout used by MyLinear, layers_and_funcs/torch.py:17).
+ * dtype is IEX_F16 or IEX_BF16 for A, B and C; accumulation is fp32 on the matrix cores.
+ * stride_* are element strides between batch entries (0 = operand shared by the batch).
+ * Replaces the cuBLAS / CUTLASS / Triton companions of tests/test_interleaving.py:26-345. */
+int iex_gemm(int dtype, int trans_b, int M, int N, int K, const void* A, const void* B,
+             void* C, int batch, long long stride_a, long long stride_b,
+             long long stride_c, void* stream);
+
+/* ----------------------------------------------- horizontally fused launch ---- */
+/* One launch whose first `gemm_workgroups` workgroups compute tiles of the dense GEMM
+ * C = A*B (as iex_gemm, batch 1) while the remaining workgroups run the fp16 CSR SpMM
+ * (as iex_spmm_ex with dtype IEX_F16, batch 1, no flags).  Both results are identical
+ * to the separate launches.  No counterpart in the reference (the name survives only as
+ * the unused HORIZONTAL_GRAINED flag, tests/test_interleaving.py:441). */
+int iex_fused_spmm_gemm(int spmm_itype, int m, int k, int n, int nonzeros,
+                        const int* row_indices, const void* values, const int* row_offsets,
+                        const void* column_indices, const void* dense, void* spmm_out,
+                        int gemm_dtype, int trans_b, int M, int N, int K, const void* A,
+                        const void* B, void* C, int interleave, void* stream);
+
+/* ------------------------------------------------------------ graph builder ---- */
+/* Opaque builder of ONE hipGraph from per-stream captures; mirrors
+ * CUDAExperimentalGraphConstructor<cudaStream_t> + CudaGraphWrapper
+ * (common/include/helper_CUDAGraphConstructor.cu.h:106-166, 268-486) as bound by
+ * pybind.cu:337-471.  Not internally synchronised: one thread per object. */
+typedef struct iex_graph iex_graph;
+
+iex_graph* iex_graph_create(void);                 /* graph + empty root node            */
+iex_graph* iex_graph_wrap(void* hip_graph);        /* CudaGraphWrapper(long)             */
+void iex_graph_destroy(iex_graph* g);
+void* iex_graph_handle(iex_graph* g);              /* the hipGraph_t                     */
+int iex_graph_register_stream(iex_graph* g, void* stream);   /* last activity := root  */
+int iex_graph_begin_capture(iex_graph* g, void* stream);     /* notify_before_invoking_library_call */
+int iex_graph_end_capture(iex_graph* g, void* stream);       /* notify_after_invoking_library_call  */
+int iex_graph_add_event_record_node(iex_graph* g, void* event, void* stream);
+int iex_graph_add_stream_wait_event_node(iex_graph* g, void* stream, void* event);
+int iex_graph_join(iex_graph* g, void* const* streams, int num_streams, void* dst_stream);
+int iex_graph_instantiate(iex_graph* g);           /* error if already instantiated      */
+int iex_graph_launch(iex_graph* g, void* stream);
+int iex_graph_destroy_exec(iex_graph* g);
+int iex_graph_add_child_graph(iex_graph* parent, iex_graph* child);
+/* N graphs as sibling child nodes of a fresh graph (helper_cuda_graph.cu.h:34-62). */
+iex_graph* iex_graph_combine(iex_graph* const* graphs, int num_graphs);
+int iex_graph_dump_dot(iex_graph* g, const char* path);
+/* Structure queries used by tests and print_graph. */
+long long iex_graph_num_nodes(iex_graph* g);
+long long iex_graph_num_edges(iex_graph* g);
+/* Fills up to `cap` (from,to) pairs as indices into the node order of
+ * hipGraphGetNodes; returns the number of edges. */
+long long iex_graph_get_edges(iex_graph* g, long long* from, long long* to, long long cap);
+/* Node type (hipGraphNodeType) of node `index`, or negative on error. */
+int iex_graph_node_type(iex_graph* g, long long index);
+/* 1 while `stream` is being captured. */
+int iex_stream_is_capturing(void* stream);
+
+/* Handle round-trip checks (pybind.cu:17-45 print_cudastream / print_cudaevent):
+ * return the pointer value they were given after querying it with the runtime. */
+long long iex_echo_stream(void* stream);
+long long iex_echo_event(void* event);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* IEX_HIP_H_ */

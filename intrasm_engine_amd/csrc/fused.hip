@@ -1,0 +1,119 @@
+// Horizontally fused sparse + dense launch: ONE grid whose workgroups are split between
+// tiles of the dense GEMM (matrix cores) and row blocks of the fp16 CSR SpMM (vector ALU
+// + memory pipeline), so that both kinds of work are resident on the same compute units
+// at the same time without relying on the runtime to overlap two kernels.
+//
+// Workgroup roles
+//   interleave == 0 : ids [0, G) run GEMM tiles, ids [G, G+S) run SpMM blocks;
+//   interleave != 0 : the G GEMM workgroups are spread evenly through the id range
+//                     (id b is a GEMM workgroup iff floor((b+1)*G/T) > floor(b*G/T)),
+//                     so both kinds are dispatched side by side from start to end.
+// Every workgroup has 256 threads and the LDS of the larger role (the GEMM's 40 KB).
+// The device code of both roles is the code of the stand-alone kernels, so results are
+// bit-identical to separate launches.
+#include "gemm_device.cuh"
+#include "spmm_device.cuh"
+
+namespace iex {
+namespace {
+
+struct FusedParams {
+  GemmParams g;
+  SpmmParams s;
+  int gemm_blocks, spmm_blocks, spmm_by, interleave;
+};
+
+constexpr int kFusedWM = 2, kFusedWN = 2, kFusedWpr = 4;
+
+template <bool BF16, bool TRANS_B, typename IT, int VEC>
+__global__ __launch_bounds__(256) void fused_kernel(FusedParams p) {
+  extern __shared__ __align__(16) unsigned char smem[];
+  const int b = blockIdx.x;
+  const long long total = (long long)p.gemm_blocks + p.spmm_blocks;
+  bool is_gemm;
+  int idx;
+  if (p.interleave) {
+    const int before = (int)(((long long)b * p.gemm_blocks) / total);
+    const int after = (int)(((long long)(b + 1) * p.gemm_blocks) / total);
+    is_gemm = after > before;
+    idx = is_gemm ? before : b - before;
+  } else {
+    is_gemm = b < p.gemm_blocks;
+    idx = is_gemm ? b : b - p.gemm_blocks;
+  }
+  if (is_gemm) {
+    gemm_tile<BF16, TRANS_B, kFusedWM, kFusedWN>(p.g, idx / p.g.tiles_n, idx % p.g.tiles_n, 0, smem);
+  } else {
+    spmm_block<__half, IT, VEC, kFusedWpr>(p.s, idx / p.spmm_by, idx % p.spmm_by, 0, reinterpret_cast<float*>(smem));
+  }
+}
+
+template <bool BF16, bool TRANS_B, typename IT, int VEC>
+int launch(FusedParams p, hipStream_t stream) {
+  constexpr int BM = 2 * kFusedWM * 32, BN = 2 * kFusedWN * 32;
+  p.g.tiles_m = ceil_div(p.g.M, BM);
+  p.g.tiles_n = ceil_div(p.g.N, BN);
+  p.gemm_blocks = p.g.tiles_m * p.g.tiles_n;
+  const int rows_per_block = 4 / kFusedWpr;
+  p.spmm_by = ceil_div(p.s.n, kWave * VEC);
+  const long long sb = (long long)ceil_div(p.s.m, rows_per_block) * p.spmm_by;
+  IEX_REQUIRE(sb + p.gemm_blocks < (1ll << 31), IEX_ERR_TOO_LARGE, "fused: grid too large");
+  p.spmm_blocks = (int)sb;
+  constexpr int lds_gemm = gemm_lds_bytes<kFusedWM, kFusedWN>();
+  constexpr int lds_spmm = spmm_lds_floats<VEC, kFusedWpr>() * 4;
+  constexpr int lds = lds_gemm > lds_spmm ? lds_gemm : lds_spmm;
+  hipLaunchKernelGGL((fused_kernel<BF16, TRANS_B, IT, VEC>), dim3(p.gemm_blocks + p.spmm_blocks), dim3(256), lds, stream,
+                     p);
+  return check_hip(hipGetLastError(), "fused launch");
+}
+
+template <bool BF16, bool TRANS_B, typename IT>
+int launch_vec(const FusedParams& p, int vec, hipStream_t stream) {
+  switch (vec) {
+    case 8: return launch<BF16, TRANS_B, IT, 8>(p, stream);
+    case 4: return launch<BF16, TRANS_B, IT, 4>(p, stream);
+    case 2: return launch<BF16, TRANS_B, IT, 2>(p, stream);
+    default: return launch<BF16, TRANS_B, IT, 1>(p, stream);
+  }
+}
+
+template <typename IT>
+int launch_gemm_kind(const FusedParams& p, int vec, bool bf16, bool trans_b, hipStream_t stream) {
+  if (bf16 && trans_b) return launch_vec<true, true, IT>(p, vec, stream);
+  if (bf16 && !trans_b) return launch_vec<true, false, IT>(p, vec, stream);
+  if (!bf16 && trans_b) return launch_vec<false, true, IT>(p, vec, stream);
+  return launch_vec<false, false, IT>(p, vec, stream);
+}
+
+}  // namespace
+}  // namespace iex
+
+extern "C" int iex_fused_spmm_gemm(int spmm_itype, int m, int k, int n, int nonzeros, const int* row_indices,
+                                   const void* values, const int* row_offsets, const void* column_indices,
+                                   const void* dense, void* spmm_out, int gemm_dtype, int trans_b, int M, int N, int K,
+                                   const void* A, const void* B, void* C, int interleave, void* stream) {
+  using namespace iex;
+  IEX_REQUIRE(m > 0 && k > 0 && n > 0 && nonzeros >= 0, IEX_ERR_BAD_ARGUMENT, "fused: SpMM dimensions must be positive");
+  IEX_REQUIRE(M > 0 && N > 0 && K > 0, IEX_ERR_BAD_ARGUMENT, "fused: GEMM dimensions must be positive");
+  IEX_REQUIRE(row_indices && row_offsets && dense && spmm_out && A && B && C, IEX_ERR_BAD_ARGUMENT,
+              "fused: null pointer argument");
+  IEX_REQUIRE(nonzeros == 0 || (values && column_indices), IEX_ERR_BAD_ARGUMENT, "fused: null values / column_indices");
+  IEX_REQUIRE(spmm_itype == IEX_I32 || (spmm_itype == IEX_I16 && k <= 32768), IEX_ERR_BAD_ARGUMENT,
+              "fused: int16 column indices need k <= 32768");
+  IEX_REQUIRE(gemm_dtype == IEX_F16 || gemm_dtype == IEX_BF16, IEX_ERR_UNSUPPORTED, "fused: GEMM dtype must be fp16 or bf16");
+  IEX_REQUIRE(K % 8 == 0, IEX_ERR_UNSUPPORTED, "fused: K must be a multiple of 8 (K=%d)", K);
+  IEX_REQUIRE(trans_b || N % 4 == 0, IEX_ERR_UNSUPPORTED, "fused: N must be a multiple of 4 when B is (K,N)");
+  IEX_REQUIRE(aligned(A, 16) && aligned(B, trans_b ? 16 : 8), IEX_ERR_UNSUPPORTED, "fused: GEMM operands must be 16-byte aligned");
+  IEX_REQUIRE((long long)k * n < (1ll << 31) && (long long)m * n < (1ll << 31) && (long long)M * K < (1ll << 31) &&
+                  (long long)N * K < (1ll << 31) && (long long)M * N < (1ll << 31),
+              IEX_ERR_TOO_LARGE, "fused: an operand exceeds 2^31 elements");
+  FusedParams p{};
+  p.g = GemmParams{M, N, K, A, B, C, 0, 0, 0, 0, 0};
+  p.s = SpmmParams{m, k, n, nonzeros, row_indices, values, row_offsets, column_indices, dense, nullptr, spmm_out, 0, 0, 0};
+  p.interleave = interleave;
+  int vec = 8;
+  while (vec > 1 && (n % vec != 0 || kWave * vec > n || !aligned(dense, 2 * vec) || !aligned(spmm_out, 2 * vec))) vec >>= 1;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  if (spmm_itype == IEX_I16) return launch_gemm_kind<short>(p, vec, gemm_dtype == IEX_BF16, trans_b != 0, s);
+  return launch_gemm_kind<int>(p, vec, gemm_dtype == IEX_BF16, trans_b != 0, s);
+}

@@ -1,0 +1,86 @@
+// Host side of the dense companion GEMM: kernel wrapper, tile-shape choice, XCD-aware
+// tile order, argument checks and the C entry point.  Device code: gemm_device.cuh.
+#include "gemm_device.cuh"
+
+namespace iex {
+namespace {
+
+constexpr int kXcds = 8;
+
+// Workgroup ids are dealt round-robin to the 8 XCDs (each with its own L2).  Give every
+// XCD a contiguous band of C tiles (row-major over tiles) so that the A row panels a
+// band needs are fetched into one L2 instead of eight.
+__device__ __forceinline__ bool xcd_tile(int block, int tiles_m, int tiles_n, int& tile_m, int& tile_n) {
+  const int total = tiles_m * tiles_n;
+  const int per_xcd = (total + kXcds - 1) / kXcds;
+  const int linear = (block % kXcds) * per_xcd + block / kXcds;
+  if (linear >= total) return false;
+  tile_m = linear / tiles_n;
+  tile_n = linear % tiles_n;
+  return true;
+}
+
+template <bool BF16, bool TRANS_B, int WM, int WN>
+__global__ __launch_bounds__(256) void gemm_kernel(GemmParams p) {
+  extern __shared__ __align__(16) unsigned char smem[];
+  int tile_m, tile_n;
+  if (!xcd_tile(blockIdx.x, p.tiles_m, p.tiles_n, tile_m, tile_n)) return;  // uniform per block
+  gemm_tile<BF16, TRANS_B, WM, WN>(p, tile_m, tile_n, blockIdx.y, smem);
+}
+
+template <bool BF16, bool TRANS_B, int WM, int WN>
+int launch(GemmParams p, int batch, hipStream_t stream) {
+  constexpr int BM = 2 * WM * 32, BN = 2 * WN * 32;
+  p.tiles_m = ceil_div(p.M, BM);
+  p.tiles_n = ceil_div(p.N, BN);
+  const int total = p.tiles_m * p.tiles_n;
+  const int per_xcd = (total + kXcds - 1) / kXcds;
+  constexpr int lds = gemm_lds_bytes<WM, WN>();
+  auto kern = gemm_kernel<BF16, TRANS_B, WM, WN>;
+  if (lds > 64 * 1024) {
+    static thread_local bool raised = false;  // per instantiation
+    if (!raised) {
+      if (int rc = check_hip(hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
+                                                 hipFuncAttributeMaxDynamicSharedMemorySize, lds),
+                             "hipFuncSetAttribute(LDS size)"))
+        return rc;
+      raised = true;
+    }
+  }
+  hipLaunchKernelGGL(kern, dim3(per_xcd * kXcds, batch), dim3(256), lds, stream, p);
+  return check_hip(hipGetLastError(), "gemm launch");
+}
+
+template <bool BF16, bool TRANS_B>
+int launch_shape(const GemmParams& p, int batch, hipStream_t stream) {
+  // 256x128 tiles halve the LDS reads per MFMA; use them when they still give every CU a tile.
+  const long long big_tiles = (long long)ceil_div(p.M, 256) * ceil_div(p.N, 128) * batch;
+  if (big_tiles >= 256) return launch<BF16, TRANS_B, 4, 2>(p, batch, stream);
+  return launch<BF16, TRANS_B, 2, 2>(p, batch, stream);
+}
+
+}  // namespace
+}  // namespace iex
+
+extern "C" int iex_gemm(int dtype, int trans_b, int M, int N, int K, const void* A, const void* B, void* C, int batch,
+                        long long stride_a, long long stride_b, long long stride_c, void* stream) {
+  using namespace iex;
+  IEX_REQUIRE(M >= 0 && N >= 0 && K >= 0 && batch >= 0, IEX_ERR_BAD_ARGUMENT, "gemm: negative dimension");
+  if (M == 0 || N == 0 || batch == 0) return 0;
+  IEX_REQUIRE(A && B && C, IEX_ERR_BAD_ARGUMENT, "gemm: null pointer argument");
+  IEX_REQUIRE(dtype == IEX_F16 || dtype == IEX_BF16, IEX_ERR_UNSUPPORTED, "gemm: dtype must be fp16 or bf16");
+  IEX_REQUIRE(K > 0 && K % 8 == 0, IEX_ERR_UNSUPPORTED, "gemm: K must be a positive multiple of 8 (K=%d)", K);
+  IEX_REQUIRE(trans_b || N % 4 == 0, IEX_ERR_UNSUPPORTED, "gemm: N must be a multiple of 4 when B is (K,N) (N=%d)", N);
+  IEX_REQUIRE(aligned(A, 16) && aligned(B, trans_b ? 16 : 8), IEX_ERR_UNSUPPORTED, "gemm: operands must be 16-byte aligned");
+  IEX_REQUIRE(stride_a % 8 == 0 && stride_b % 8 == 0, IEX_ERR_UNSUPPORTED, "gemm: batch strides must be multiples of 8");
+  IEX_REQUIRE(batch <= 65535, IEX_ERR_TOO_LARGE, "gemm: batch %d exceeds 65535", batch);
+  IEX_REQUIRE((long long)M * K < (1ll << 31) && (long long)N * K < (1ll << 31) && (long long)M * N < (1ll << 31),
+              IEX_ERR_TOO_LARGE, "gemm: an operand exceeds 2^31 elements per batch entry");
+  GemmParams p{M, N, K, A, B, C, stride_a, stride_b, stride_c, 0, 0};
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  const bool bf = dtype == IEX_BF16;
+  if (bf && trans_b) return launch_shape<true, true>(p, batch, s);
+  if (bf && !trans_b) return launch_shape<true, false>(p, batch, s);
+  if (!bf && trans_b) return launch_shape<false, true>(p, batch, s);
+  return launch_shape<false, false>(p, batch, s);
+}

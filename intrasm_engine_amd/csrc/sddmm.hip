@@ -1,0 +1,209 @@
+// CSR SDDMM for gfx950 (wave64): out[j] = <lhs[row(j), :], rhs[col(j), :]>.
+//
+// Work decomposition
+//   * a wavefront owns one CSR row (swizzled order) or, for long rows, every WPR-th
+//     chunk of 64 nonzeros of it; outputs are independent, so no reduction crosses
+//     wavefronts and nothing is atomic;
+//   * a group of LPN adjacent lanes handles one nonzero: the LPN lanes read one rhs row
+//     as a single contiguous LPN*VEC*sizeof(T) segment (128-bit per lane when the shape
+//     allows), so G = 64/LPN nonzeros are in flight per instruction;
+//   * the lhs row fragment that a lane needs is the same for every nonzero of the row
+//     and stays in registers when k <= 2*LPN*VEC (the attention shapes); otherwise it
+//     is re-read (it hits L1: every group reads the same bytes);
+//   * the LPN partial dot products are summed with DPP row operations (quad_perm,
+//     row_half_mirror, row_mirror): no LDS, no bpermute in the reduction.
+// Accumulation is fp32; with SUM_OVER_BATCH the batch loop runs inside the kernel so
+// the (nnz) output is a deterministic sum.
+#include "iex_common.h"
+
+namespace iex {
+namespace {
+
+struct SddmmParams {
+  int m, k, n, nnz, batch;
+  const int* row_indices;
+  const int* row_offsets;
+  const int* cols;
+  const void* lhs;
+  const void* rhs;
+  void* out;
+  int sum_over_batch, accumulate;
+};
+
+typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
+
+template <typename T, int VEC>
+__device__ __forceinline__ float dot_vec(const vec_t<T, VEC>& a, const vec_t<T, VEC>& b, float acc) {
+  if constexpr (sizeof(T) == 2 && VEC >= 2 && __is_same(T, __half)) {
+#pragma unroll
+    for (int i = 0; i < VEC / 2; ++i) {
+      f16x2 x = __builtin_bit_cast(f16x2, *reinterpret_cast<const uint32_t*>(&a.v[2 * i]));
+      f16x2 y = __builtin_bit_cast(f16x2, *reinterpret_cast<const uint32_t*>(&b.v[2 * i]));
+      acc = __builtin_amdgcn_fdot2(x, y, acc, false);
+    }
+    return acc;
+  } else {
+#pragma unroll
+    for (int i = 0; i < VEC; ++i)
+      acc = fmaf(elem<T>::to_float(a.v[i]), elem<T>::to_float(b.v[i]), acc);
+    return acc;
+  }
+}
+
+// PASSES > 0: k <= PASSES*LPN*VEC and the lhs fragment is cached in registers
+//             (requires one batch entry per wave);  PASSES == 0: generic k, reload.
+template <typename T, int VEC, int LPN, int PASSES, int WPR>
+__global__ __launch_bounds__(256) void sddmm_kernel(SddmmParams p) {
+  constexpr int G = kWave / LPN;
+  constexpr int KT = LPN * VEC;
+  constexpr int kRowsPerBlock = 4 / WPR;
+  const int lane = lane_id();
+  const int wave = uniform(threadIdx.x >> 6);
+  const int sub = lane / LPN;
+  const int sl = lane % LPN;
+  const int row_slot = blockIdx.x * kRowsPerBlock + wave / WPR;
+  const int part = wave % WPR;
+  if (row_slot >= p.m) return;
+
+  const int row = uniform(p.row_indices[row_slot]);
+  const int start = uniform(p.row_offsets[row]);
+  const int end = uniform(p.row_offsets[row + 1]);
+  const int z0 = p.sum_over_batch ? 0 : (int)blockIdx.z;
+  const int zn = p.sum_over_batch ? p.batch : 1;
+  const T* __restrict__ lhs = static_cast<const T*>(p.lhs) + ((size_t)z0 * p.m + row) * p.k;
+  const T* __restrict__ rhs = static_cast<const T*>(p.rhs) + (size_t)z0 * p.n * p.k;
+  T* __restrict__ out = static_cast<T*>(p.out) + (p.sum_over_batch ? (size_t)0 : (size_t)z0 * p.nnz);
+  const size_t lhs_zstride = (size_t)p.m * p.k;
+  const size_t rhs_zstride = (size_t)p.n * p.k;
+
+  vec_t<T, VEC> lfrag[PASSES > 0 ? PASSES : 1];
+  if constexpr (PASSES > 0) {
+#pragma unroll
+    for (int ps = 0; ps < PASSES; ++ps) {
+      const int kk = ps * KT + sl * VEC;
+      if (kk < p.k) {
+        lfrag[ps] = load_vec<T, VEC>(lhs + kk);
+      } else {
+#pragma unroll
+        for (int i = 0; i < VEC; ++i) lfrag[ps].v[i] = elem<T>::from_float(0.f);
+      }
+    }
+  }
+
+  for (int base = start + part * kWave; base < end; base += kWave * WPR) {
+    const int j = base + lane;
+    const int c = (j < end) ? p.cols[j] : 0;
+    const int cnt = min(kWave, end - base);
+    const int steps = (cnt + G - 1) / G;
+    for (int s = 0; s < steps; ++s) {
+      const int t = s * G + sub;          // nonzero of this chunk handled by my lane group
+      const int cc = __shfl(c, t, kWave); // t < 64 always; slots past cnt carry column 0
+      float acc = 0.f;
+      if constexpr (PASSES > 0) {
+        const T* r = rhs + (size_t)cc * p.k;
+#pragma unroll
+        for (int ps = 0; ps < PASSES; ++ps) {
+          const int kk = ps * KT + sl * VEC;
+          if (kk < p.k) acc = dot_vec<T, VEC>(lfrag[ps], load_vec<T, VEC>(r + kk), acc);
+        }
+      } else {
+        for (int z = 0; z < zn; ++z) {
+          const T* l = lhs + (size_t)z * lhs_zstride;
+          const T* r = rhs + (size_t)z * rhs_zstride + (size_t)cc * p.k;
+          for (int kk = sl * VEC; kk < p.k; kk += KT)
+            acc = dot_vec<T, VEC>(load_vec<T, VEC>(l + kk), load_vec<T, VEC>(r + kk), acc);
+        }
+      }
+      acc = group_sum<LPN>(acc);
+      if (sl == 0 && t < cnt) {
+        const size_t o = (size_t)base + t;
+        if (p.accumulate) acc += elem<T>::to_float(out[o]);
+        out[o] = elem<T>::from_float(acc);
+      }
+    }
+  }
+}
+
+template <typename T, int VEC, int LPN, int PASSES, int WPR>
+int launch_one(const SddmmParams& p, hipStream_t stream) {
+  dim3 grid(ceil_div(p.m, 4 / WPR), 1, p.sum_over_batch ? 1 : p.batch);
+  hipLaunchKernelGGL((sddmm_kernel<T, VEC, LPN, PASSES, WPR>), grid, dim3(256), 0, stream, p);
+  return check_hip(hipGetLastError(), "sddmm launch");
+}
+
+template <typename T, int VEC, int LPN, int PASSES>
+int launch_wpr(const SddmmParams& p, int wpr, hipStream_t stream) {
+  if (wpr == 4) return launch_one<T, VEC, LPN, PASSES, 4>(p, stream);
+  return launch_one<T, VEC, LPN, PASSES, 1>(p, stream);
+}
+
+template <typename T, int VEC, int LPN>
+int launch_passes(const SddmmParams& p, int wpr, hipStream_t stream) {
+  const bool one_z = !(p.sum_over_batch && p.batch > 1);
+  const int kt = LPN * VEC;
+  if (one_z && p.k <= kt) return launch_wpr<T, VEC, LPN, 1>(p, wpr, stream);
+  if (one_z && p.k <= 2 * kt) return launch_wpr<T, VEC, LPN, 2>(p, wpr, stream);
+  return launch_wpr<T, VEC, LPN, 0>(p, wpr, stream);
+}
+
+template <typename T>
+int launch_typed(const SddmmParams& p, int wpr, hipStream_t stream) {
+  constexpr int kMax = 16 / (int)sizeof(T);
+  int vec = kMax;
+  while (vec > 1 && (p.k % vec != 0 || !aligned(p.lhs, sizeof(T) * vec) || !aligned(p.rhs, sizeof(T) * vec)))
+    vec >>= 1;
+  // lanes per nonzero: enough to cover k in one or two passes, at most 16 (one DPP row)
+  if (vec == kMax) {
+    if (p.k <= 8 * vec) return launch_passes<T, kMax, 8>(p, wpr, stream);
+    return launch_passes<T, kMax, 16>(p, wpr, stream);
+  }
+  if (vec >= 2) return launch_passes<T, 2, 16>(p, wpr, stream);
+  return launch_passes<T, 1, 16>(p, wpr, stream);
+}
+
+}  // namespace
+
+int sddmm_dispatch(int dtype, int flags, int m, int k, int n, int nonzeros, const int* row_indices,
+                   const int* row_offsets, const int* column_indices, const void* lhs, const void* rhs,
+                   void* out, void* stream, int batch) {
+  IEX_REQUIRE(m >= 0 && k >= 0 && n >= 0 && nonzeros >= 0 && batch >= 0, IEX_ERR_BAD_ARGUMENT,
+              "sddmm: negative dimension (m=%d k=%d n=%d nnz=%d batch=%d)", m, k, n, nonzeros, batch);
+  if (m == 0 || nonzeros == 0 || batch == 0) return 0;
+  IEX_REQUIRE(row_indices && row_offsets && column_indices && out, IEX_ERR_BAD_ARGUMENT,
+              "sddmm: null pointer argument");
+  IEX_REQUIRE(k == 0 || (lhs && rhs), IEX_ERR_BAD_ARGUMENT, "sddmm: null dense operand");
+  IEX_REQUIRE(batch <= 65535, IEX_ERR_TOO_LARGE, "sddmm: batch %d exceeds 65535", batch);
+  IEX_REQUIRE((long long)m * k < (1ll << 31) && (long long)n * k < (1ll << 31), IEX_ERR_TOO_LARGE,
+              "sddmm: a dense operand exceeds 2^31 elements per batch entry");
+  SddmmParams p{m, k, n, nonzeros, batch, row_indices, row_offsets, column_indices, lhs, rhs, out,
+                (flags & IEX_SDDMM_SUM_OVER_BATCH) != 0, (flags & IEX_SDDMM_ACCUMULATE) != 0};
+  const int wpr = ((double)nonzeros / m >= 128.0) ? 4 : 1;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  switch (dtype) {
+    case IEX_F32: return launch_typed<float>(p, wpr, s);
+    case IEX_F16: return launch_typed<__half>(p, wpr, s);
+    case IEX_BF16: return launch_typed<__hip_bfloat16>(p, wpr, s);
+  }
+  return fail(IEX_ERR_UNSUPPORTED, "sddmm: no kernel for dtype=%d", dtype);
+}
+
+}  // namespace iex
+
+extern "C" {
+
+int iex_sddmm_ex(int dtype, int flags, int m, int k, int n, int nonzeros, const int* row_indices,
+                 const int* row_offsets, const int* column_indices, const void* lhs_matrix,
+                 const void* rhs_matrix, void* output_values, void* stream, int batch) {
+  return iex::sddmm_dispatch(dtype, flags, m, k, n, nonzeros, row_indices, row_offsets, column_indices,
+                             lhs_matrix, rhs_matrix, output_values, stream, batch);
+}
+
+int iex_CudaSddmm2(int m, int k, int n, int nonzeros, const int* row_indices, const int* row_offsets,
+                   const int* column_indices, const float* lhs_matrix, const float* rhs_matrix,
+                   float* output_values, void* stream, int batch_size) {
+  return iex::sddmm_dispatch(IEX_F32, IEX_SDDMM_SUM_OVER_BATCH, m, k, n, nonzeros, row_indices,
+                             row_offsets, column_indices, lhs_matrix, rhs_matrix, output_values, stream,
+                             batch_size);
+}
+
+}  // extern "C"

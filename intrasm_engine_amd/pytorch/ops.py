@@ -1,0 +1,295 @@
+"""``torch.ops.iex_ops.*`` -- the operator registry of the path.
+
+Same operator names, argument order, shape rules and error texts as the reference's
+``TORCH_LIBRARY(iex_ops)`` (pytorch/csrc/extensions/sputnik_kernels.cpp:32-193); the
+body of every operator is: validate, allocate the output with ``torch.empty`` on the
+operand's device (so a surrounding graph capture routes it to the capture's pool),
+look up torch's *current* stream (never an argument, sputnik_kernels.cpp:81,151) and
+call the C ABI of ``libiex_hip.so``.  Nothing here computes on the CPU.
+
+Registered operators
+    spmm_sputnik_reuse_weight        fp32, values (nnz)                     [reference :173-175]
+    spmm_sputnik_atomic              fp32, values (batch, nnz)              [reference :170-172]
+    spmm_sputnik_reuse_weight_half   fp16, int16 or int32 column indices    [reference :179-181, unregistered there]
+    sddmm_sputnik_atomic_upd_weight  fp32, output (nnz) summed over batch   [reference :182-184]
+    sddmm_sputnik_half               fp16/bf16/fp32, output (batch, nnz)    [new: reference :185-187 is commented out]
+    spmm_sputnik_batched_values      fp16/fp32, values (batch, nnz), written (not accumulated) [new]
+    csr_softmax_                     in-place softmax over CSR rows         [new]
+    gemm_mfma                        bf16/fp16 dense companion GEMM         [replaces torch.matmul / CUTLASS / Triton companions]
+    fused_spmm_gemm                  single-launch sparse + dense           [new]
+"""
+from __future__ import annotations
+
+import torch
+
+from .. import _lib
+
+_DT = {torch.float32: _lib.F32, torch.float16: _lib.F16, torch.bfloat16: _lib.BF16}
+_IT = {torch.int32: _lib.I32, torch.int16: _lib.I16}
+
+
+def _chk(cond: bool, msg: str = "") -> None:
+    if not cond:
+        raise RuntimeError(msg or "Expected condition to be true (operator argument check failed)")
+
+
+def _stream_ptr(device) -> int:
+    return torch.cuda.current_stream(device).cuda_stream
+
+
+def _check_csr_common(first, row_indices, row_offsets, column_indices, names):
+    """The dimension / device / contiguity / layout checks shared by both launcher
+    macros (sputnik_kernels.cpp:41-79 and :109-149), same order and texts."""
+    _chk(row_indices.dim() == 1)
+    _chk(row_offsets.dim() == 1)
+    _chk(column_indices.dim() == 1)
+    tensors = list(names) + [("row_indices", row_indices), ("row_offsets", row_offsets),
+                             ("column_offsets", column_indices)]
+    for name, t in tensors:
+        _chk(t.is_cuda, f"{name} must be a CUDA tensor")
+    for name, t in tensors:
+        _chk(t.is_contiguous(), f"{name} must be a contiguous tensor")
+    for name, t in tensors:
+        _chk(not t.is_sparse and t.layout == torch.strided, f"{name} must be a dense tensor")
+
+
+def _check_index_dtypes(row_indices, row_offsets, column_indices, allow_i16=False):
+    _chk(row_indices.dtype == torch.int32, "row_indices must be int32")
+    _chk(row_offsets.dtype == torch.int32, "row_offsets must be int32")
+    ok = (torch.int32, torch.int16) if allow_i16 else (torch.int32,)
+    _chk(column_indices.dtype in ok, "column_indices must be " + " or ".join(str(d) for d in ok))
+
+
+def _spmm(b, row_indices, values, row_offsets, column_indices, m, *, per_batch_values,
+          accumulate, dtypes, allow_i16, out=None, bias=None, relu=False, force_wpr=0):
+    _chk(b.dim() == 3)
+    if per_batch_values:
+        _chk(values.dim() == 2)
+        _chk(b.size(0) == values.size(0))
+        _chk(values.size(1) == column_indices.size(0))
+    else:
+        _chk(values.dim() == 1)
+        _chk(values.size(0) == column_indices.size(0))
+    _check_csr_common(b, row_indices, row_offsets, column_indices, [("b", b), ("values", values)])
+    _chk(values.device == b.device, "values should be in the same device as b")
+    _chk(values.device == row_indices.device, "a should be in the same device as row_indices")
+    _chk(values.device == row_offsets.device, "a should be in the same device as row_offsets")
+    _chk(values.device == column_indices.device, "a should be in the same device as column_indices")
+    _chk(b.dtype in dtypes, f"b must be one of {dtypes}")
+    _chk(values.dtype == b.dtype, "values must have the dtype of b")
+    _check_index_dtypes(row_indices, row_offsets, column_indices, allow_i16)
+    batch, k, n = b.shape
+    nonzeros = column_indices.size(0)
+    m = int(m)
+    _chk(row_indices.size(0) == m, "row_indices must have m entries")
+    _chk(row_offsets.size(0) == m + 1, "row_offsets must have m + 1 entries")
+    if per_batch_values and accumulate:
+        # the one shape rule of the reference that is about data, not layout (:87-89)
+        _chk(batch == 1 or nonzeros % 4 == 0,
+             "If batch size > 1 then number of nonzeros should be a multiple of 4")
+    if out is None:
+        # "atomic" store mode adds into the output; the reference leaves it uninitialised
+        # (at::empty, :91) -- here the operator is defined as zero, then accumulate.
+        out = (torch.zeros if accumulate else torch.empty)((batch, m, n), dtype=b.dtype, device=b.device)
+    else:
+        _chk(out.shape == (batch, m, n) and out.dtype == b.dtype and out.is_contiguous()
+             and out.device == b.device, "out must be a contiguous (batch, m, n) tensor like b")
+    if bias is not None:
+        _chk(bias.dtype == torch.float32 and bias.is_contiguous() and bias.numel() == m
+             and bias.device == b.device, "bias must be a contiguous fp32 tensor with m entries")
+    flags = (_lib.SPMM_PER_BATCH_VALUES if per_batch_values else 0) | \
+            (_lib.SPMM_ACCUMULATE if accumulate else 0) | (_lib.SPMM_RELU if relu else 0) | \
+            ((int(force_wpr) & 0xff) << 8)
+    with torch.cuda.device(b.device):
+        rc = _lib.load().iex_spmm_ex(
+            _DT[b.dtype], _IT[column_indices.dtype], flags, m, k, n, nonzeros,
+            row_indices.data_ptr(), values.data_ptr(), row_offsets.data_ptr(),
+            column_indices.data_ptr(), b.data_ptr(), bias.data_ptr() if bias is not None else None,
+            out.data_ptr(), _stream_ptr(b.device), batch)
+    _lib.check(rc, "spmm")
+    return out
+
+
+def _sddmm(a, b, row_indices, row_offsets, column_indices, *, sum_over_batch, dtypes,
+           out=None, accumulate=False):
+    _chk(a.dim() == b.dim())
+    _chk(a.dim() == 3)
+    _chk(a.size(0) == b.size(0))
+    _chk(a.size(2) == b.size(2))
+    _check_csr_common(a, row_indices, row_offsets, column_indices, [("a", a), ("b", b)])
+    _chk(a.device == b.device, "a should be in the same device as b")
+    _chk(a.device == row_indices.device, "a should be in the same device as row_indices")
+    _chk(a.device == row_offsets.device, "a should be in the same device as row_offsets")
+    _chk(a.device == column_indices.device, "a should be in the same device as column_indices")
+    _chk(a.dtype in dtypes, f"a must be one of {dtypes}")
+    _chk(b.dtype == a.dtype, "b must have the dtype of a")
+    _check_index_dtypes(row_indices, row_offsets, column_indices)
+    batch, m, k = a.shape
+    n = b.size(1)
+    nonzeros = column_indices.size(0)
+    _chk(row_indices.size(0) == m, "row_indices must have m entries")
+    _chk(row_offsets.size(0) == m + 1, "row_offsets must have m + 1 entries")
+    shape = (nonzeros,) if sum_over_batch else (batch, nonzeros)
+    if out is None:
+        out = torch.empty(shape, dtype=a.dtype, device=a.device)
+    else:
+        _chk(tuple(out.shape) == shape and out.dtype == a.dtype and out.is_contiguous()
+             and out.device == a.device, "out has the wrong shape, dtype, layout or device")
+    flags = (_lib.SDDMM_SUM_OVER_BATCH if sum_over_batch else 0) | \
+            (_lib.SDDMM_ACCUMULATE if accumulate else 0)
+    with torch.cuda.device(a.device):
+        rc = _lib.load().iex_sddmm_ex(
+            _DT[a.dtype], flags, m, k, n, nonzeros, row_indices.data_ptr(), row_offsets.data_ptr(),
+            column_indices.data_ptr(), a.data_ptr(), b.data_ptr(), out.data_ptr(),
+            _stream_ptr(a.device), batch)
+    _lib.check(rc, "sddmm")
+    return out
+
+
+# ----------------------------------------------------------------- operators
+def spmm_sputnik_reuse_weight(b, row_indices, values, row_offsets, column_indices, m):
+    return _spmm(b, row_indices, values, row_offsets, column_indices, m, per_batch_values=False,
+                 accumulate=False, dtypes=(torch.float32,), allow_i16=False)
+
+
+def spmm_sputnik_atomic(b, row_indices, values, row_offsets, column_indices, m):
+    return _spmm(b, row_indices, values, row_offsets, column_indices, m, per_batch_values=True,
+                 accumulate=True, dtypes=(torch.float32,), allow_i16=False)
+
+
+def spmm_sputnik_reuse_weight_half(b, row_indices, values, row_offsets, column_indices, m):
+    return _spmm(b, row_indices, values, row_offsets, column_indices, m, per_batch_values=False,
+                 accumulate=False, dtypes=(torch.float16, torch.bfloat16), allow_i16=True)
+
+
+def spmm_sputnik_batched_values(b, row_indices, values, row_offsets, column_indices, m):
+    return _spmm(b, row_indices, values, row_offsets, column_indices, m, per_batch_values=True,
+                 accumulate=False, dtypes=(torch.float32, torch.float16, torch.bfloat16),
+                 allow_i16=True)
+
+
+def sddmm_sputnik_atomic_upd_weight(a, b, row_indices, row_offsets, column_indices):
+    return _sddmm(a, b, row_indices, row_offsets, column_indices, sum_over_batch=True,
+                  dtypes=(torch.float32,))
+
+
+def sddmm_sputnik_half(a, b, row_indices, row_offsets, column_indices):
+    return _sddmm(a, b, row_indices, row_offsets, column_indices, sum_over_batch=False,
+                  dtypes=(torch.float32, torch.float16, torch.bfloat16))
+
+
+def csr_softmax_(values, row_indices, row_offsets, scale):
+    _chk(values.dim() == 2, "values must be (batch, nnz)")
+    for name, t in (("values", values), ("row_indices", row_indices), ("row_offsets", row_offsets)):
+        _chk(t.is_cuda, f"{name} must be a CUDA tensor")
+        _chk(t.is_contiguous(), f"{name} must be a contiguous tensor")
+    _chk(values.dtype in _DT, "values must be fp32, fp16 or bf16")
+    _chk(row_indices.dtype == torch.int32 and row_offsets.dtype == torch.int32,
+         "row_indices / row_offsets must be int32")
+    m = row_indices.size(0)
+    _chk(row_offsets.size(0) == m + 1, "row_offsets must have m + 1 entries")
+    with torch.cuda.device(values.device):
+        rc = _lib.load().iex_csr_softmax(_DT[values.dtype], m, values.size(1), row_indices.data_ptr(),
+                                         row_offsets.data_ptr(), values.data_ptr(), float(scale),
+                                         _stream_ptr(values.device), values.size(0))
+    _lib.check(rc, "csr_softmax")
+    return values
+
+
+def gemm_mfma(a, b, trans_b=False, out=None):
+    """``a @ b`` (or ``a @ b.T`` with ``trans_b``) for fp16/bf16, 2-D or batched 3-D."""
+    _chk(a.is_cuda and b.is_cuda, "a and b must be CUDA tensors")
+    _chk(a.dtype in (torch.float16, torch.bfloat16), "a must be fp16 or bf16")
+    _chk(b.dtype == a.dtype, "b must have the dtype of a")
+    _chk(a.device == b.device, "a should be in the same device as b")
+    _chk(a.dim() in (2, 3) and b.dim() in (2, 3), "a and b must be 2-D or 3-D")
+    _chk(a.is_contiguous(), "a must be a contiguous tensor")
+    _chk(b.is_contiguous(), "b must be a contiguous tensor")
+    M, K = a.shape[-2], a.shape[-1]
+    N = b.shape[-2] if trans_b else b.shape[-1]
+    _chk((b.shape[-1] if trans_b else b.shape[-2]) == K, "inner dimensions of a and b differ")
+    batch = a.shape[0] if a.dim() == 3 else (b.shape[0] if b.dim() == 3 else 1)
+    if a.dim() == 3 and b.dim() == 3:
+        _chk(a.shape[0] == b.shape[0], "batch sizes of a and b differ")
+    sa = M * K if a.dim() == 3 else 0
+    sb = N * K if b.dim() == 3 else 0
+    batched = a.dim() == 3 or b.dim() == 3
+    shape = (batch, M, N) if batched else (M, N)
+    if out is None:
+        out = torch.empty(shape, dtype=a.dtype, device=a.device)
+    else:
+        _chk(tuple(out.shape) == shape and out.dtype == a.dtype and out.is_contiguous()
+             and out.device == a.device, "out has the wrong shape, dtype, layout or device")
+    with torch.cuda.device(a.device):
+        rc = _lib.load().iex_gemm(_DT[a.dtype], int(bool(trans_b)), M, N, K, a.data_ptr(), b.data_ptr(),
+                                  out.data_ptr(), batch, sa, sb, M * N, _stream_ptr(a.device))
+    _lib.check(rc, "gemm")
+    return out
+
+
+def fused_spmm_gemm(b, row_indices, values, row_offsets, column_indices, m, ga, gb, trans_b=False,
+                    interleave=0):
+    """One launch computing ``(A_csr @ b[0], ga @ gb)``; fp16 SpMM, fp16/bf16 GEMM."""
+    _chk(b.dim() == 3 and b.size(0) == 1, "fused launch takes one batch entry")
+    _chk(values.dim() == 1 and values.size(0) == column_indices.size(0))
+    _check_csr_common(b, row_indices, row_offsets, column_indices, [("b", b), ("values", values)])
+    _chk(b.dtype == torch.float16 and values.dtype == torch.float16, "fused SpMM operands must be fp16")
+    _check_index_dtypes(row_indices, row_offsets, column_indices, allow_i16=True)
+    _chk(ga.is_cuda and gb.is_cuda and ga.device == b.device and gb.device == b.device,
+         "GEMM operands must be on the device of b")
+    _chk(ga.dtype in (torch.float16, torch.bfloat16) and gb.dtype == ga.dtype, "GEMM operands must be fp16 or bf16")
+    _chk(ga.dim() == 2 and gb.dim() == 2 and ga.is_contiguous() and gb.is_contiguous(),
+         "GEMM operands must be contiguous 2-D tensors")
+    m = int(m)
+    _chk(row_indices.size(0) == m and row_offsets.size(0) == m + 1, "CSR arrays do not match m")
+    _, k, n = b.shape
+    M, K = ga.shape
+    N = gb.shape[0] if trans_b else gb.shape[1]
+    _chk((gb.shape[1] if trans_b else gb.shape[0]) == K, "inner dimensions of the GEMM differ")
+    out = torch.empty((1, m, n), dtype=b.dtype, device=b.device)
+    c = torch.empty((M, N), dtype=ga.dtype, device=b.device)
+    with torch.cuda.device(b.device):
+        rc = _lib.load().iex_fused_spmm_gemm(
+            _IT[column_indices.dtype], m, k, n, column_indices.size(0), row_indices.data_ptr(),
+            values.data_ptr(), row_offsets.data_ptr(), column_indices.data_ptr(), b.data_ptr(),
+            out.data_ptr(), _DT[ga.dtype], int(bool(trans_b)), M, N, K, ga.data_ptr(), gb.data_ptr(),
+            c.data_ptr(), int(interleave), _stream_ptr(b.device))
+    _lib.check(rc, "fused_spmm_gemm")
+    return out, c
+
+
+_SPMM_SCHEMA = "(Tensor b, Tensor row_indices, Tensor values, Tensor row_offsets, Tensor column_indices, int m) -> Tensor"
+_SDDMM_SCHEMA = "(Tensor a, Tensor b, Tensor row_indices, Tensor row_offsets, Tensor column_indices) -> Tensor"
+_registered = False
+_library = None
+
+
+def register() -> None:
+    """Define the operators under ``torch.ops.iex_ops`` (idempotent)."""
+    global _registered, _library
+    if _registered:
+        return
+    lib = torch.library.Library("iex_ops", "DEF")
+    table = [
+        ("spmm_sputnik_reuse_weight", _SPMM_SCHEMA, spmm_sputnik_reuse_weight),
+        ("spmm_sputnik_atomic", _SPMM_SCHEMA, spmm_sputnik_atomic),
+        ("spmm_sputnik_reuse_weight_half", _SPMM_SCHEMA, spmm_sputnik_reuse_weight_half),
+        ("spmm_sputnik_batched_values", _SPMM_SCHEMA, spmm_sputnik_batched_values),
+        ("sddmm_sputnik_atomic_upd_weight", _SDDMM_SCHEMA, sddmm_sputnik_atomic_upd_weight),
+        ("sddmm_sputnik_half", _SDDMM_SCHEMA, sddmm_sputnik_half),
+        ("csr_softmax_", "(Tensor(a!) values, Tensor row_indices, Tensor row_offsets, float scale) -> Tensor(a!)",
+         csr_softmax_),
+        ("gemm_mfma", "(Tensor a, Tensor b, bool trans_b=False) -> Tensor",
+         lambda a, b, trans_b=False: gemm_mfma(a, b, trans_b)),
+        ("fused_spmm_gemm",
+         "(Tensor b, Tensor row_indices, Tensor values, Tensor row_offsets, Tensor column_indices, int m, "
+         "Tensor ga, Tensor gb, bool trans_b=False, int interleave=0) -> (Tensor, Tensor)",
+         fused_spmm_gemm),
+    ]
+    for name, schema, fn in table:
+        lib.define(name + schema)
+        # one implementation for every backend: the body itself rejects non-device
+        # tensors with the reference's message ("b must be a CUDA tensor")
+        lib.impl(name, fn, "CompositeExplicitAutograd")
+    _library = lib
+    _registered = True

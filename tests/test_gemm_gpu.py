@@ -1,0 +1,91 @@
+"""GPU parity of the MFMA companion GEMM against the CPU oracle."""
+import numpy as np
+import pytest
+import torch
+
+from _util import assert_close, rounded
+
+pytestmark = pytest.mark.gpu
+ops = torch.ops.iex_ops
+
+
+def _check(oracle, dev, M, N, K, dtype, trans_b, seed=0):
+    rng = np.random.default_rng(seed)
+    a_np = rng.standard_normal((M, K)).astype(np.float32)
+    b_np = rng.standard_normal((N, K) if trans_b else (K, N)).astype(np.float32)
+    a, b = torch.from_numpy(a_np).to(dev).to(dtype), torch.from_numpy(b_np).to(dev).to(dtype)
+    out = ops.gemm_mfma(a, b, trans_b)
+    assert out.shape == (M, N) and out.dtype == dtype
+    a_r, b_r = rounded(a_np, dtype), rounded(b_np, dtype)
+    want = oracle.gemm(a_r, b_r, trans_b=trans_b)
+    scale = oracle.gemm(np.abs(a_r), np.abs(b_r), trans_b=trans_b)
+    assert_close(out.float().cpu().numpy(), want, scale, 1e-2, f"gemm {M}x{N}x{K} {dtype} trans_b={trans_b}")
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("trans_b", [False, True])
+@pytest.mark.parametrize("shape", [(128, 128, 32), (256, 128, 64), (512, 384, 256), (100, 60, 72), (33, 260, 8),
+                                   (1, 4, 8), (300, 132, 1000)])
+def test_gemm_shapes(oracle, dev, dtype, trans_b, shape):
+    _check(oracle, dev, *shape, dtype, trans_b)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_integer_inputs_are_exact(dev, dtype):
+    """randint(-3, 3) operands (the idiom of the reference's tests/test_CUDAGraphConstructor.py:88-93)
+    make the product exact: the result must equal the integer matmul, for both tile shapes."""
+    g = torch.Generator().manual_seed(2023)
+    for (M, N, K) in ((512, 512, 128), (4096, 2048, 256), (1024, 256, 512)):
+        a = torch.randint(-3, 3, (M, K), generator=g).to(dev)
+        b = torch.randint(-3, 3, (K, N), generator=g).to(dev)
+        want = (a.double() @ b.double())
+        assert want.abs().max() <= 256 * 9
+        out = ops.gemm_mfma(a.to(dtype), b.to(dtype), False)
+        # products of small integers are exact in fp32; bf16 output rounding needs |C| < 256
+        if dtype == torch.float16 or want.abs().max() < 256:
+            assert torch.equal(out.double(), want)
+        else:
+            assert torch.allclose(out.double(), want, rtol=2 ** -8)
+        out_t = ops.gemm_mfma(a.to(dtype), b.t().contiguous().to(dtype), True)
+        assert torch.equal(out_t, out)
+
+
+def test_config4_dense_branch(oracle, dev):
+    """bf16 (4096x4096)(4096x2048): a 256-row x 512-column corner is checked against the
+    oracle, the whole product against the same kernel fed the transposed-B layout."""
+    rng = np.random.default_rng(21)
+    a_np = rng.standard_normal((4096, 4096)).astype(np.float32)
+    b_np = rng.standard_normal((4096, 2048)).astype(np.float32)
+    a, b = torch.from_numpy(a_np).to(dev).bfloat16(), torch.from_numpy(b_np).to(dev).bfloat16()
+    out = ops.gemm_mfma(a, b, False)
+    a_r, b_r = rounded(a_np[:256], torch.bfloat16), rounded(b_np[:, :512], torch.bfloat16)
+    want = oracle.gemm(a_r, b_r)
+    scale = oracle.gemm(np.abs(a_r), np.abs(b_r))
+    assert_close(out[:256, :512].float().cpu().numpy(), want, scale, 1e-2, "C4 GEMM corner")
+    assert torch.equal(ops.gemm_mfma(a, b.t().contiguous(), True), out)
+
+
+def test_batched(oracle, dev):
+    rng = np.random.default_rng(5)
+    a_np = rng.standard_normal((6, 96, 64)).astype(np.float32)
+    b_np = rng.standard_normal((6, 64, 40)).astype(np.float32)
+    a, b = torch.from_numpy(a_np).to(dev).half(), torch.from_numpy(b_np).to(dev).half()
+    out = ops.gemm_mfma(a, b, False)
+    assert out.shape == (6, 96, 40)
+    for z in range(6):
+        want = oracle.gemm(rounded(a_np[z], torch.float16), rounded(b_np[z], torch.float16))
+        scale = oracle.gemm(np.abs(a_np[z]), np.abs(b_np[z]))
+        assert_close(out[z].float().cpu().numpy(), want, scale, 1e-2, f"batched z={z}")
+    # shared B
+    out2 = ops.gemm_mfma(a, b[0].contiguous(), False)
+    assert torch.equal(out2[0], out[0])
+
+
+def test_argument_checks(dev):
+    a = torch.randn(16, 12, device=dev).half()
+    with pytest.raises(RuntimeError, match="multiple of 8"):
+        ops.gemm_mfma(a, torch.randn(12, 16, device=dev).half(), False)
+    with pytest.raises(RuntimeError, match="fp16 or bf16"):
+        ops.gemm_mfma(a.float(), a.float(), True)
+    with pytest.raises(RuntimeError, match="inner dimensions"):
+        ops.gemm_mfma(torch.randn(16, 16, device=dev).half(), torch.randn(8, 16, device=dev).half(), False)

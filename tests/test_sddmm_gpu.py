@@ -1,0 +1,157 @@
+"""GPU parity of the CSR SDDMM operators and the CSR softmax against the CPU oracle."""
+import numpy as np
+import pytest
+import torch
+
+from intrasm_engine_amd import workloads as W
+from _util import RTOL, assert_close, rounded, to_dev
+
+pytestmark = pytest.mark.gpu
+ops = torch.ops.iex_ops
+
+
+def _check(oracle, csr, lhs_np, rhs_np, dev, dtype, sum_over_batch, what):
+    ri, _, ro, ci = to_dev(csr, dev)
+    lhs = torch.from_numpy(lhs_np).to(dev).to(dtype)
+    rhs = torch.from_numpy(rhs_np).to(dev).to(dtype)
+    if sum_over_batch:
+        out = ops.sddmm_sputnik_atomic_upd_weight(lhs, rhs, ri, ro, ci)
+        assert out.shape == (csr.nnz,)
+    else:
+        out = ops.sddmm_sputnik_half(lhs, rhs, ri, ro, ci)
+        assert out.shape == (lhs.shape[0], csr.nnz)
+    assert out.dtype == dtype
+    l_r, r_r = rounded(lhs_np, dtype), rounded(rhs_np, dtype)
+    want = oracle.sddmm(l_r, r_r, csr.row_indices, csr.row_offsets, csr.column_indices, sum_over_batch=sum_over_batch)
+    scale = oracle.sddmm_abs_scale(l_r, r_r, csr.row_indices, csr.row_offsets, csr.column_indices,
+                                   sum_over_batch=sum_over_batch)
+    assert_close(out.float().cpu().numpy(), want, scale, RTOL[dtype], what)
+    return out
+
+
+def test_config1_fp32(oracle, dev):
+    a, _, lhs, rhs = W.config1()
+    _check(oracle, a, lhs, rhs, dev, torch.float32, True, "C1 fp32 SDDMM")
+
+
+def test_config3_fp16_per_head_then_spmm(oracle, dev):
+    """Sparse attention of config 3: per-head SDDMM(Q, K) on the banded mask, then SpMM with
+    the per-head values against V.  4 of the 16 heads are checked against the oracle (the
+    kernel treats heads identically; all 16 run in test_full_size_config3_properties)."""
+    pattern, q, k, v = W.config3(heads=4)
+    out = _check(oracle, pattern, q, k, dev, torch.float16, False, "C3 fp16 SDDMM")
+    ri, _, ro, ci = to_dev(pattern, dev)
+    vt = torch.from_numpy(v).to(dev).half()
+    ctx = ops.spmm_sputnik_batched_values(vt, ri, out, ro, ci, pattern.m)
+    vals = out.float().cpu().numpy()
+    want = oracle.spmm(rounded(v, torch.float16), pattern.row_indices, vals, pattern.row_offsets,
+                       pattern.column_indices, pattern.m)
+    scale = oracle.spmm_abs_scale(rounded(v, torch.float16), pattern.row_indices, vals, pattern.row_offsets,
+                                  pattern.column_indices, pattern.m)
+    assert_close(ctx.float().cpu().numpy(), want, scale, 1e-2, "C3 SpMM against V")
+
+
+def test_full_size_config3_properties(dev):
+    """All 16 heads: (a) every head of the batched launch equals the same head launched alone
+    (bit-exact), (b) the diagonal entries equal the row-wise dot products <q_i, k_i>."""
+    pattern, q, k, _ = W.config3()
+    ri, _, ro, ci = to_dev(pattern, dev)
+    qt, kt = torch.from_numpy(q).to(dev).half(), torch.from_numpy(k).to(dev).half()
+    out = ops.sddmm_sputnik_half(qt, kt, ri, ro, ci)
+    for h in (0, 7, 15):
+        assert torch.equal(ops.sddmm_sputnik_half(qt[h:h + 1].contiguous(), kt[h:h + 1].contiguous(), ri, ro, ci)[0], out[h])
+    rows = torch.repeat_interleave(torch.arange(pattern.m, device=dev), torch.diff(ro.long()))
+    diag = (rows == ci.long()).nonzero().squeeze(1)
+    assert diag.numel() == pattern.m
+    want = (qt.float() * kt.float()).sum(-1)
+    got = out[:, diag].float()
+    assert torch.allclose(got, want, rtol=1e-2, atol=1e-2 * 1e-2 * 64)
+
+
+@pytest.mark.parametrize("k", [1, 3, 8, 20, 32, 64, 72, 128, 200, 1024])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16, torch.bfloat16])
+def test_ragged_shapes(oracle, dev, k, dtype):
+    rng = np.random.default_rng(k)
+    m, n = 131, 97
+    lens = rng.integers(0, 30, m)
+    lens[[0, 9, 130]] = 0
+    lens[5] = n
+    ro, ci = W.csr_from_row_lengths(rng, m, n, lens)
+    csr = W.CSR(m, n, np.ones(ci.shape[0], np.float32), W.swizzle_from_offsets(ro), ro, ci)
+    lhs = rng.standard_normal((2, m, k)).astype(np.float32)
+    rhs = rng.standard_normal((2, n, k)).astype(np.float32)
+    _check(oracle, csr, lhs, rhs, dev, dtype, False, f"ragged per-batch k={k} {dtype}")
+    if dtype == torch.float32:
+        _check(oracle, csr, lhs, rhs, dev, dtype, True, f"ragged summed k={k}")
+
+
+def test_long_rows_split_over_waves(oracle, dev):
+    rng = np.random.default_rng(77)
+    a = W.config2_matrix(0.70, m=512, k=1024)     # mean row length ~307 -> 4 wavefronts per row
+    lhs = rng.standard_normal((1, 512, 64)).astype(np.float32)
+    rhs = rng.standard_normal((1, 1024, 64)).astype(np.float32)
+    _check(oracle, a, lhs, rhs, dev, torch.float32, True, "long rows fp32")
+    _check(oracle, a, lhs, rhs, dev, torch.float16, False, "long rows fp16")
+
+
+def test_integer_inputs_are_exact_and_full_mask_is_gemm(dev):
+    rng = np.random.default_rng(3)
+    m, n, k = 64, 48, 64
+    lhs = torch.from_numpy(rng.integers(-3, 4, (1, m, k)).astype(np.float32)).to(dev)
+    rhs = torch.from_numpy(rng.integers(-3, 4, (1, n, k)).astype(np.float32)).to(dev)
+    ro = torch.arange(0, m * n + 1, n, dtype=torch.int32, device=dev)
+    ci = torch.arange(n, dtype=torch.int32, device=dev).repeat(m)
+    ri = torch.arange(m, dtype=torch.int32, device=dev)
+    want = (lhs[0].double() @ rhs[0].double().T).reshape(-1)
+    assert torch.equal(ops.sddmm_sputnik_atomic_upd_weight(lhs, rhs, ri, ro, ci).double(), want)
+    assert torch.equal(ops.sddmm_sputnik_half(lhs.half(), rhs.half(), ri, ro, ci)[0].double(), want)
+
+
+def test_reference_launcher_name_through_c_abi(oracle, dev):
+    from intrasm_engine_amd import _lib
+    a, _, lhs_np, rhs_np = W.config1()
+    ri, _, ro, ci = to_dev(a, dev)
+    lhs, rhs = torch.from_numpy(lhs_np).to(dev), torch.from_numpy(rhs_np).to(dev)
+    out = torch.full((a.nnz,), float("nan"), device=dev)   # written, not accumulated
+    rc = _lib.load().iex_CudaSddmm2(a.m, 64, a.k, a.nnz, ri.data_ptr(), ro.data_ptr(), ci.data_ptr(), lhs.data_ptr(),
+                                    rhs.data_ptr(), out.data_ptr(), torch.cuda.current_stream().cuda_stream, 1)
+    assert rc == 0, _lib.last_error()
+    want = oracle.sddmm(lhs_np, rhs_np, a.row_indices, a.row_offsets, a.column_indices)
+    scale = oracle.sddmm_abs_scale(lhs_np, rhs_np, a.row_indices, a.row_offsets, a.column_indices)
+    assert_close(out.cpu().numpy(), want, scale, 1e-5, "iex_CudaSddmm2")
+
+
+def test_empty_pattern(dev):
+    m, n, k = 9, 7, 16
+    z = torch.zeros(m + 1, dtype=torch.int32, device=dev)
+    out = ops.sddmm_sputnik_atomic_upd_weight(torch.randn(1, m, k, device=dev), torch.randn(1, n, k, device=dev),
+                                              torch.arange(m, dtype=torch.int32, device=dev), z,
+                                              torch.zeros(0, dtype=torch.int32, device=dev))
+    assert out.shape == (0,)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16])
+def test_csr_softmax(oracle, dev, dtype):
+    pattern, q, k, _ = W.config3(tokens=512, heads=2, band=64, extra=8)
+    rng = np.random.default_rng(4)
+    vals = rng.standard_normal((2, pattern.nnz)).astype(np.float32) * 3
+    ri, _, ro, _ = to_dev(pattern, dev)
+    v = torch.from_numpy(vals).to(dev).to(dtype)
+    ops.csr_softmax_(v, ri, ro, 0.125)
+    want = oracle.csr_softmax(rounded(vals, dtype).astype(np.float64) * 0.125, pattern.row_offsets)
+    tol = 2e-6 if dtype == torch.float32 else 2e-3
+    assert np.abs(v.float().cpu().numpy() - want).max() <= tol
+    sums = np.add.reduceat(v.float().cpu().numpy(), pattern.row_offsets[:-1], axis=1)
+    assert np.allclose(sums, 1.0, atol=1e-2 if dtype == torch.float16 else 1e-5)
+
+
+def test_operator_argument_checks(dev):
+    a, _, lhs_np, rhs_np = W.config1()
+    ri, _, ro, ci = to_dev(a, dev)
+    lhs, rhs = torch.from_numpy(lhs_np).to(dev), torch.from_numpy(rhs_np).to(dev)
+    with pytest.raises(RuntimeError, match="a must be a CUDA tensor"):
+        ops.sddmm_sputnik_atomic_upd_weight(lhs.cpu(), rhs, ri, ro, ci)
+    with pytest.raises(RuntimeError):
+        ops.sddmm_sputnik_atomic_upd_weight(lhs, rhs[:, :, :32].contiguous(), ri, ro, ci)   # k mismatch
+    with pytest.raises(RuntimeError, match="b must be a contiguous tensor"):
+        ops.sddmm_sputnik_atomic_upd_weight(lhs, rhs.transpose(1, 2).contiguous().transpose(1, 2), ri, ro, ci)

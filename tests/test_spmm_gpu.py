@@ -1,0 +1,276 @@
+"""GPU parity of the CSR SpMM operators against the CPU oracle (through torch.ops.iex_ops
+and, for the launcher drop-ins, straight through the C ABI)."""
+import ctypes
+
+import numpy as np
+import pytest
+import torch
+
+from intrasm_engine_amd import workloads as W
+from _util import RTOL, assert_close, rounded, to_dev
+
+pytestmark = pytest.mark.gpu
+ops = torch.ops.iex_ops
+
+
+def _check(oracle, csr, b_np, dev, dtype=torch.float32, idtype=torch.int32, op=None, what=""):
+    ri, v, ro, ci = to_dev(csr, dev, dtype, idtype)
+    b = torch.from_numpy(b_np).to(dev).to(dtype)
+    if op is None:
+        op = ops.spmm_sputnik_reuse_weight if dtype == torch.float32 else ops.spmm_sputnik_reuse_weight_half
+    out = op(b, ri, v, ro, ci, csr.m)
+    torch.cuda.synchronize()
+    assert out.shape == (b.shape[0], csr.m, b.shape[2]) and out.dtype == dtype
+    vals_r, b_r = rounded(csr.values, dtype), rounded(b_np, dtype)
+    want = oracle.spmm(b_r, csr.row_indices, vals_r, csr.row_offsets, csr.column_indices, csr.m)
+    scale = oracle.spmm_abs_scale(b_r, csr.row_indices, vals_r, csr.row_offsets, csr.column_indices, csr.m)
+    return assert_close(out.float().cpu().numpy(), want, scale, RTOL[dtype], what)
+
+
+def test_config1_fp32(oracle, dev):
+    a, b, _, _ = W.config1()
+    _check(oracle, a, b, dev, what="C1 fp32 SpMM")
+
+
+@pytest.mark.parametrize("sparsity", W.C2_SPARSITIES)
+def test_config2_sweep_fp32(oracle, dev, sparsity):
+    a = W.config2_matrix(sparsity)
+    for n in W.C2_NS:
+        _check(oracle, a, W.config2_dense(n), dev, what=f"C2 fp32 s={sparsity} n={n}")
+
+
+@pytest.mark.parametrize("sparsity", W.C2_SPARSITIES)
+def test_config2_sweep_fp16(oracle, dev, sparsity):
+    a = W.config2_matrix(sparsity, even_rows=True)
+    for n, idt in ((64, torch.int16), (128, torch.int32), (256, torch.int16)):
+        _check(oracle, a, W.config2_dense(n), dev, torch.float16, idt, what=f"C2 fp16 s={sparsity} n={n} {idt}")
+
+
+def test_bf16(oracle, dev):
+    a = W.config2_matrix(0.95, m=512, k=512)
+    _check(oracle, a, W.config2_dense(128, k=512), dev, torch.bfloat16, what="bf16 SpMM")
+
+
+@pytest.mark.parametrize("n", [1, 3, 33, 64, 70, 130, 200, 512])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16])
+def test_ragged_shapes(oracle, dev, n, dtype):
+    """m not a multiple of the rows per workgroup, empty rows, every vector width and the
+    scalar tail path."""
+    rng = np.random.default_rng(n)
+    m, k = 203, 157
+    lens = rng.integers(0, 40, m)
+    lens[[0, 5, 202]] = 0
+    lens[7] = k
+    ro, ci = W.csr_from_row_lengths(rng, m, k, lens)
+    csr = W.CSR(m, k, rng.standard_normal(ci.shape[0]).astype(np.float32), W.swizzle_from_offsets(ro), ro, ci)
+    b = rng.standard_normal((2, k, n)).astype(np.float32)
+    _check(oracle, csr, b, dev, dtype, what=f"ragged n={n} {dtype}")
+
+
+@pytest.mark.parametrize("wpr", [1, 4, 16])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16])
+def test_every_row_split_variant(oracle, dev, wpr, dtype):
+    """The three work decompositions (1, 4, 16 wavefronts per row) on one skewed matrix."""
+    from intrasm_engine_amd.pytorch import ops as pyops
+    rng = np.random.default_rng(99)
+    m, k, n = 301, 2048, 192
+    lens = np.clip(rng.geometric(1 / 150.0, m), 0, k)
+    lens[3] = k
+    lens[4] = 0
+    ro, ci = W.csr_from_row_lengths(rng, m, k, lens)
+    csr = W.CSR(m, k, rng.standard_normal(ci.shape[0]).astype(np.float32), W.swizzle_from_offsets(ro), ro, ci)
+    b_np = rng.standard_normal((1, k, n)).astype(np.float32)
+    ri, v, ro_t, ci_t = to_dev(csr, dev, dtype)
+    b = torch.from_numpy(b_np).to(dev).to(dtype)
+    out = pyops._spmm(b, ri, v, ro_t, ci_t, m, per_batch_values=False, accumulate=False,
+                      dtypes=(dtype,), allow_i16=False, force_wpr=wpr)
+    vals_r, b_r = rounded(csr.values, dtype), rounded(b_np, dtype)
+    want = oracle.spmm(b_r, csr.row_indices, vals_r, csr.row_offsets, csr.column_indices, m)
+    scale = oracle.spmm_abs_scale(b_r, csr.row_indices, vals_r, csr.row_offsets, csr.column_indices, m)
+    assert_close(out.float().cpu().numpy(), want, scale, RTOL[dtype], f"wpr={wpr}")
+
+
+def test_all_empty_matrix_and_empty_shapes(dev):
+    m, k, n = 17, 9, 64
+    z32 = lambda *s: torch.zeros(*s, dtype=torch.int32, device=dev)
+    b = torch.randn(1, k, n, device=dev)
+    out = ops.spmm_sputnik_reuse_weight(b, torch.arange(m, dtype=torch.int32, device=dev),
+                                        torch.zeros(0, device=dev), z32(m + 1), z32(0), m)
+    assert out.shape == (1, m, n) and (out == 0).all()
+    out = ops.spmm_sputnik_reuse_weight(torch.zeros(1, k, 0, device=dev), torch.arange(m, dtype=torch.int32, device=dev),
+                                        torch.zeros(0, device=dev), z32(m + 1), z32(0), m)
+    assert out.shape == (1, m, 0)
+
+
+def test_integer_inputs_are_exact(dev):
+    """Small-integer operands make every partial sum exactly representable, so the device
+    result must EQUAL the integer product (the exactness idiom of the reference's
+    tests/test_CUDAGraphConstructor.py:88-93), in fp32 and in fp16."""
+    rng = np.random.default_rng(1)
+    a = W.config2_matrix(0.95, m=1024, k=1024)
+    a.values = rng.integers(1, 4, a.nnz).astype(np.float32) * rng.choice([-1, 1], a.nnz).astype(np.float32)
+    b_np = rng.integers(-3, 4, (1, 1024, 128)).astype(np.float32)
+    dense = torch.zeros(1024, 1024, dtype=torch.float64)
+    rows = np.repeat(np.arange(1024), np.diff(a.row_offsets))
+    dense[rows, a.column_indices.astype(np.int64)] = torch.from_numpy(a.values).double()
+    want = (dense @ torch.from_numpy(b_np[0]).double()).numpy()
+    for dtype in (torch.float32, torch.float16):
+        ri, v, ro, ci = to_dev(a, dev, dtype)
+        op = ops.spmm_sputnik_reuse_weight if dtype == torch.float32 else ops.spmm_sputnik_reuse_weight_half
+        out = op(torch.from_numpy(b_np).to(dev).to(dtype), ri, v, ro, ci, 1024)
+        assert np.array_equal(out[0].double().cpu().numpy(), want), dtype
+
+
+def test_swizzle_is_scheduling_only(dev):
+    a = W.config2_matrix(0.90, m=1024, k=1024)
+    b = torch.from_numpy(W.config2_dense(64, k=1024)).to(dev)
+    ri, v, ro, ci = to_dev(a, dev)
+    base = ops.spmm_sputnik_reuse_weight(b, ri, v, ro, ci, a.m)
+    perm = torch.randperm(a.m, device=dev, generator=torch.Generator(dev).manual_seed(0)).to(torch.int32)
+    assert torch.equal(ops.spmm_sputnik_reuse_weight(b, perm, v, ro, ci, a.m), base)
+    ident = torch.arange(a.m, device=dev, dtype=torch.int32)
+    assert torch.equal(ops.spmm_sputnik_reuse_weight(b, ident, v, ro, ci, a.m), base)
+
+
+def test_batch_and_per_batch_values(oracle, dev):
+    rng = np.random.default_rng(5)
+    a = W.config2_matrix(0.875, m=256, k=512)     # nnz = 16384, a multiple of 4
+    assert a.nnz % 4 == 0
+    batch = 3
+    b_np = rng.standard_normal((batch, 512, 96)).astype(np.float32)
+    vb = rng.standard_normal((batch, a.nnz)).astype(np.float32)
+    ri, v, ro, ci = to_dev(a, dev)
+    b = torch.from_numpy(b_np).to(dev)
+    # shared values over a batch
+    out = ops.spmm_sputnik_reuse_weight(b, ri, v, ro, ci, a.m)
+    want = oracle.spmm(b_np, a.row_indices, a.values, a.row_offsets, a.column_indices, a.m)
+    scale = oracle.spmm_abs_scale(b_np, a.row_indices, a.values, a.row_offsets, a.column_indices, a.m)
+    assert_close(out.cpu().numpy(), want, scale, 1e-5, "batched reuse-weight")
+    # per-batch values: the "atomic" operator = zero, then accumulate
+    out = ops.spmm_sputnik_atomic(b, ri, torch.from_numpy(vb).to(dev), ro, ci, a.m)
+    want = oracle.spmm(b_np, a.row_indices, vb, a.row_offsets, a.column_indices, a.m)
+    scale = oracle.spmm_abs_scale(b_np, a.row_indices, vb, a.row_offsets, a.column_indices, a.m)
+    assert_close(out.cpu().numpy(), want, scale, 1e-5, "spmm_sputnik_atomic")
+    # written (not accumulated) per-batch variant in fp16
+    out = ops.spmm_sputnik_batched_values(b.half(), ri, torch.from_numpy(vb).to(dev).half(), ro, ci, a.m)
+    want = oracle.spmm(rounded(b_np, torch.float16), a.row_indices, rounded(vb, torch.float16), a.row_offsets,
+                       a.column_indices, a.m)
+    scale = oracle.spmm_abs_scale(rounded(b_np, torch.float16), a.row_indices, rounded(vb, torch.float16),
+                                  a.row_offsets, a.column_indices, a.m)
+    assert_close(out.float().cpu().numpy(), want, scale, 1e-2, "batched values fp16")
+
+
+def test_accumulate_bias_relu_through_c_abi(oracle, dev):
+    """iex_spmm_ex with the accumulate flag adds to a pre-filled output; bias + ReLU epilogue."""
+    from intrasm_engine_amd import _lib
+    rng = np.random.default_rng(6)
+    a = W.config2_matrix(0.90, m=128, k=256)
+    b_np = rng.standard_normal((1, 256, 64)).astype(np.float32)
+    init = rng.standard_normal((1, 128, 64)).astype(np.float32)
+    bias = rng.standard_normal(128).astype(np.float32)
+    ri, v, ro, ci = to_dev(a, dev)
+    b, out, bias_t = torch.from_numpy(b_np).to(dev), torch.from_numpy(init).to(dev), torch.from_numpy(bias).to(dev)
+    s = torch.cuda.current_stream().cuda_stream
+    rc = _lib.load().iex_spmm_ex(_lib.F32, _lib.I32, _lib.SPMM_ACCUMULATE, a.m, a.k, 64, a.nnz, ri.data_ptr(),
+                                 v.data_ptr(), ro.data_ptr(), ci.data_ptr(), b.data_ptr(), None, out.data_ptr(), s, 1)
+    assert rc == 0, _lib.last_error()
+    want = oracle.spmm(b_np, a.row_indices, a.values, a.row_offsets, a.column_indices, a.m, out_init=init)
+    scale = oracle.spmm_abs_scale(b_np, a.row_indices, a.values, a.row_offsets, a.column_indices, a.m) + np.abs(init)
+    assert_close(out.cpu().numpy(), want, scale, 1e-5, "accumulate")
+    out2 = torch.empty_like(out)
+    rc = _lib.load().iex_spmm_ex(_lib.F32, _lib.I32, _lib.SPMM_RELU, a.m, a.k, 64, a.nnz, ri.data_ptr(), v.data_ptr(),
+                                 ro.data_ptr(), ci.data_ptr(), b.data_ptr(), bias_t.data_ptr(), out2.data_ptr(), s, 1)
+    assert rc == 0, _lib.last_error()
+    want = oracle.spmm(b_np, a.row_indices, a.values, a.row_offsets, a.column_indices, a.m, bias=bias, relu=True)
+    assert_close(out2.cpu().numpy(), want, scale + np.abs(bias)[None, :, None], 1e-5, "bias+relu")
+
+
+def test_reference_launcher_names_through_c_abi(oracle, dev):
+    """iex_CudaSpmm3 / iex_CudaSpmm2 / iex_CudaSpmm5 called with raw pointers, the way a
+    binding of csrc/extensions.h:28-30 would."""
+    from intrasm_engine_amd import _lib
+    lib = _lib.load()
+    a, b_np, _, _ = W.config1()
+    ri, v, ro, ci = to_dev(a, dev)
+    b = torch.from_numpy(b_np).to(dev)
+    s = torch.cuda.current_stream().cuda_stream
+    want = oracle.spmm(b_np, a.row_indices, a.values, a.row_offsets, a.column_indices, a.m)
+    scale = oracle.spmm_abs_scale(b_np, a.row_indices, a.values, a.row_offsets, a.column_indices, a.m)
+    out = torch.empty(1, a.m, 256, device=dev)
+    assert lib.iex_CudaSpmm3(a.m, a.k, 256, a.nnz, ri.data_ptr(), v.data_ptr(), ro.data_ptr(), ci.data_ptr(),
+                             b.data_ptr(), out.data_ptr(), s, 1) == 0
+    assert_close(out.cpu().numpy(), want, scale, 1e-5, "iex_CudaSpmm3")
+    out.zero_()
+    assert lib.iex_CudaSpmm2(a.m, a.k, 256, a.nnz, ri.data_ptr(), v.data_ptr(), ro.data_ptr(), ci.data_ptr(),
+                             b.data_ptr(), out.data_ptr(), s, 1) == 0
+    assert_close(out.cpu().numpy(), want, scale, 1e-5, "iex_CudaSpmm2")
+    outh = torch.empty(1, a.m, 256, device=dev, dtype=torch.float16)
+    assert lib.iex_CudaSpmm5(a.m, a.k, 256, a.nnz, ri.data_ptr(), v.half().data_ptr(), ro.data_ptr(),
+                             ci.to(torch.int16).data_ptr(), b.half().data_ptr(), outh.data_ptr(), s, 1) == 0
+    wanth = oracle.spmm(rounded(b_np, torch.float16), a.row_indices, rounded(a.values, torch.float16), a.row_offsets,
+                        a.column_indices, a.m)
+    assert_close(outh.float().cpu().numpy(), wanth, scale, 1e-2, "iex_CudaSpmm5")
+
+
+def test_unreferenced_nan_rows_do_not_leak(dev):
+    """Row 0 of the dense operand holds NaN but no nonzero points at column 0: the result
+    must stay finite (padding slots never touch memory they were not asked to read)."""
+    rng = np.random.default_rng(8)
+    m, k, n = 130, 300, 64
+    lens = rng.integers(1, 70, m)
+    ro, ci = W.csr_from_row_lengths(rng, m, k - 1, lens)
+    ci = ci + 1  # shift: column 0 never used
+    csr = W.CSR(m, k, rng.standard_normal(ci.shape[0]).astype(np.float32), W.swizzle_from_offsets(ro), ro, ci)
+    b = torch.randn(1, k, n, device=dev)
+    b[0, 0] = float("nan")
+    ri, v, ro_t, ci_t = to_dev(csr, dev)
+    assert torch.isfinite(ops.spmm_sputnik_reuse_weight(b, ri, v, ro_t, ci_t, m)).all()
+    assert torch.isfinite(ops.spmm_sputnik_reuse_weight_half(b.half(), ri, v.half(), ro_t, ci_t, m)).all()
+
+
+def test_misaligned_operands_take_the_scalar_path(oracle, dev):
+    rng = np.random.default_rng(9)
+    a = W.config2_matrix(0.90, m=128, k=128)
+    n = 64
+    b_np = rng.standard_normal((1, 128, n)).astype(np.float32)
+    store = torch.empty(128 * n + 1, device=dev, dtype=torch.float16)
+    b = store[1:].view(1, 128, n)      # 2-byte aligned only
+    b.copy_(torch.from_numpy(b_np))
+    ri, v, ro, ci = to_dev(a, dev, torch.float16)
+    out = ops.spmm_sputnik_reuse_weight_half(b, ri, v, ro, ci, a.m)
+    want = oracle.spmm(rounded(b_np, torch.float16), a.row_indices, rounded(a.values, torch.float16), a.row_offsets,
+                       a.column_indices, a.m)
+    scale = oracle.spmm_abs_scale(b_np, a.row_indices, a.values, a.row_offsets, a.column_indices, a.m)
+    assert_close(out.float().cpu().numpy(), want, scale, 1e-2, "misaligned")
+
+
+def test_full_size_config4_integer_exact(dev):
+    """Config-4 shape (11008x4096 @ 90 %, 2048 tokens) with small-integer operands: the fp16
+    result must equal the exact product, computed densely in float64 on the device."""
+    rng = np.random.default_rng(20)
+    w = W.pruned_weight(20, 11008, 4096, 0.90)
+    w.values = (rng.integers(1, 3, w.nnz) * rng.choice([-1, 1], w.nnz)).astype(np.float32)
+    x = torch.from_numpy(rng.integers(-2, 3, (1, 4096, 2048)).astype(np.float32)).to(dev)
+    ri, v, ro, ci = to_dev(w, dev, torch.float16, torch.int16)
+    out = ops.spmm_sputnik_reuse_weight_half(x.half(), ri, v, ro, ci, w.m)
+    from intrasm_engine_amd.pytorch.utils import sparse_to_dense
+    dense = sparse_to_dense(w.m, w.k, v.double(), ro, ci.to(torch.int32))
+    want = dense @ x[0].double()
+    assert want.abs().max() < 2048  # exactly representable in fp16
+    assert torch.equal(out[0].double(), want)
+
+
+def test_operator_argument_checks(dev):
+    a, b_np, _, _ = W.config1()
+    ri, v, ro, ci = to_dev(a, dev)
+    b = torch.from_numpy(b_np).to(dev)
+    with pytest.raises(RuntimeError, match="b must be a CUDA tensor"):
+        ops.spmm_sputnik_reuse_weight(b.cpu(), ri, v, ro, ci, a.m)
+    with pytest.raises(RuntimeError, match="b must be a contiguous tensor"):
+        ops.spmm_sputnik_reuse_weight(b.transpose(1, 2), ri, v, ro, ci, a.m)
+    with pytest.raises(RuntimeError):
+        ops.spmm_sputnik_reuse_weight(b[0], ri, v, ro, ci, a.m)              # b.dim() != 3
+    with pytest.raises(RuntimeError):
+        ops.spmm_sputnik_reuse_weight(b, ri, v[:-1], ro, ci, a.m)            # values vs column_indices
+    with pytest.raises(RuntimeError, match="multiple of 4"):
+        ops.spmm_sputnik_atomic(b.repeat(2, 1, 1), ri, v[:-2].repeat(2, 1), ro, ci[:-2], a.m)

@@ -1,0 +1,295 @@
+#!/usr/bin/env python3
+"""Benchmark of the sparse-plus-dense GEMM path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-extras] [--no-cpu]
+
+A *step* is one pass of the hot path over the configuration the metric is quoted on:
+the fp32 CSR SpMM sweep of config 2 (4096x4096 sparse A at 70/80/90/95/98 % sparsity with
+geometric row lengths, times a dense 4096 x {64,128,256} B) = 15 SpMM launches, captured
+once into a hipGraph through the graph builder and replayed.  All operands are resident
+in HBM before the timed region; CSR construction is set-up work and is not timed.
+
+One JSON line is printed.  ``value`` = algorithmic GB of one sweep / seconds per sweep.
+``roofline`` describes the SpMM kernel instantiation that takes the most time in the
+sweep; ``cpu_baseline`` is the single-core C port of the same sweep timed on this host;
+``extras`` holds the per-cell table, the fp16 sweep, SDDMM (configs 1 and 3), the bf16
+MFMA GEMM and the sparse+dense co-run of config 4 (serialized / two-branch graph / fused).
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import statistics
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBPS = 8000.0           # MI355X HBM3E
+MFMA_PEAK_TFLOPS_16BIT = 2500.0  # dense bf16 / fp16
+VALU_PEAK_TFLOPS_FP32 = 78.6     # vector fp32 FMA without packed math (the build disables v_pk_*_f32)
+CELL_REPEATS = 20                # launches of one cell inside its timing graph
+
+
+def log(*a):
+    print(*a, file=sys.stderr, flush=True)
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--no-extras", action="store_true", help="skip fp16 / SDDMM / GEMM / co-run sections")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        log("bench.py measures one GPU: every box of this build has a single MI355X and the path has no "
+            "cross-GPU step (rows of A shard with no exchange). Run with --gpus 1.")
+        sys.exit(2)
+
+    import torch
+    if not torch.cuda.is_available():
+        log("bench.py needs a GPU (the product path has no CPU fallback).")
+        sys.exit(2)
+    import intrasm_engine_amd  # noqa: F401
+    from intrasm_engine_amd import workloads as W
+    from intrasm_engine_amd import interleaving as IL
+    from intrasm_engine_amd.pytorch.cpp_extensions.cuda_graph_constructor import TorchCUDAGraphConstructor
+
+    ops = torch.ops.iex_ops
+    dev = torch.device("cuda:0")
+    t_setup = time.time()
+
+    # ------------------------------------------------------------- inputs (config 2)
+    mats = {s: W.config2_matrix(s) for s in W.C2_SPARSITIES}
+    dens = {n: W.config2_dense(n) for n in W.C2_NS}
+
+    def csr_dev(csr, vdtype=torch.float32, idtype=torch.int32):
+        return (torch.from_numpy(csr.row_indices).to(dev), torch.from_numpy(csr.values).to(dev).to(vdtype),
+                torch.from_numpy(csr.row_offsets).to(dev), torch.from_numpy(csr.column_indices).to(dev).to(idtype))
+
+    mats32 = {s: csr_dev(m) for s, m in mats.items()}
+    dens32 = {n: torch.from_numpy(b).to(dev) for n, b in dens.items()}
+    cells = [(s, n) for s in W.C2_SPARSITIES for n in W.C2_NS]
+
+    def spmm32(s, n):
+        ri, v, ro, ci = mats32[s]
+        return lambda: ops.spmm_sputnik_reuse_weight(dens32[n], ri, v, ro, ci, mats[s].m)
+
+    def cell_bytes(s, n, sv=4, si=4):
+        c = mats[s]
+        return W.spmm_bytes(c.m, c.k, n, c.nnz, 1, sv, si)
+
+    sweep_bytes = sum(cell_bytes(s, n) for s, n in cells)
+    sweep_flops = sum(W.spmm_flops(mats[s].nnz, n) for s, n in cells)
+    log(f"[bench] set-up {time.time() - t_setup:.1f}s; sweep = {len(cells)} launches, "
+        f"{sweep_bytes / 1e6:.1f} MB algorithmic, {sweep_flops / 1e9:.2f} GFLOP")
+
+    # --------------------------------------------------------------- the timed step
+    constructor, keep = IL.capture_serialized([spmm32(s, n) for s, n in cells])
+    constructor.instantiate_graph_exec()
+    for _ in range(args.warmup):
+        constructor.execute_graph()
+    torch.cuda.synchronize()
+    start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    t0 = time.perf_counter()
+    start.record()
+    for _ in range(args.steps):
+        constructor.execute_graph()
+    end.record()
+    torch.cuda.synchronize()
+    wall_ms = (time.perf_counter() - t0) * 1e3
+    ms_per_step = start.elapsed_time(end) / args.steps
+    constructor.destroy_graph_exec()
+    del keep
+    value = sweep_bytes / 1e9 / (ms_per_step * 1e-3)
+    log(f"[bench] {ms_per_step * 1e3:.1f} us per sweep (host wall {wall_ms / args.steps * 1e3:.1f} us) -> {value:.1f} GB/s")
+
+    # ------------------------------------------- per-cell launch durations (HIP events)
+    def time_cell(fn, repeats=CELL_REPEATS, samples=5):
+        """Average duration of one launch: `repeats` launches in one graph on the current
+        stream, events around the graph launch, median of `samples`."""
+        ms = IL.time_execs([fn] * repeats, repeats=samples, warmup=1)
+        return ms / repeats * 1e3  # us
+
+    def variant_of(csr, n, sv):
+        mean = csr.nnz / csr.m
+        wpr = 16 if mean >= 768 else (4 if mean >= 96 else 1)
+        vec = 16 // sv
+        while vec > 1 and (n % vec or 64 * vec > n):
+            vec //= 2
+        return vec, wpr
+
+    table = []
+    for s, n in cells:
+        us = time_cell(spmm32(s, n))
+        by, fl = cell_bytes(s, n), W.spmm_flops(mats[s].nnz, n)
+        vec, wpr = variant_of(mats[s], n, 4)
+        table.append({"sparsity": s, "n": n, "nnz": mats[s].nnz, "us": round(us, 2), "GBps": round(by / us / 1e3, 1),
+                      "hbm_frac": round(by / us / 1e3 / HBM_PEAK_GBPS, 4), "GFLOPs": round(fl / us / 1e3, 1),
+                      "valu_frac": round(fl / us / 1e6 / VALU_PEAK_TFLOPS_FP32, 4),
+                      "kernel": f"spmm_kernel<float,int,VEC={vec},WPR={wpr}>", "bytes": by})
+        log(f"[bench] fp32 s={s} n={n}: {us:.2f} us  {by / us / 1e3:.0f} GB/s  {fl / us / 1e3:.0f} GFLOP/s")
+
+    by_kernel = {}
+    for row in table:
+        by_kernel.setdefault(row["kernel"], []).append(row)
+    dom_name, dom_rows = max(by_kernel.items(), key=lambda kv: sum(r["us"] for r in kv[1]))
+    dom_bytes = statistics.mean(r["bytes"] for r in dom_rows)
+    dom_us = statistics.mean(r["us"] for r in dom_rows)
+    roofline = {"bound": "hbm", "achieved": round(dom_bytes / dom_us / 1e3, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+                "frac": round(dom_bytes / dom_us / 1e3 / HBM_PEAK_GBPS, 4), "traffic": None,
+                "kernel": dom_name, "avg_launch_us": round(dom_us, 2),
+                "algorithmic_bytes_per_launch": int(dom_bytes),
+                "cells": [[r["sparsity"], r["n"]] for r in dom_rows],
+                "note": "gathers of B rows are served by L1/L2, not HBM: the kernel's real ceiling is the "
+                        "vector-memory pipeline (nnz*n*4 B of gathers), see extras.cells[*].valu_frac"}
+
+    result = {
+        "metric": "SpMM/SDDMM GB/s and % HBM peak; co-run makespan vs serialized (%) on 1 GPU",
+        "value": round(value, 1), "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 5), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "f32", "data": "synthetic",
+        "config": {"workload": "config 2: fp32 CSR SpMM sweep, A 4096x4096 at {70,80,90,95,98}% sparsity (geometric "
+                               "row lengths), B 4096x{64,128,256}; one step = the 15 launches in one hipGraph",
+                   "value_is": "algorithmic bytes of the sweep / time per sweep",
+                   "pct_hbm_peak": round(100 * value / HBM_PEAK_GBPS, 2), "cache": "warm (operands stay in L2 / MALL between steps)"},
+        "roofline": roofline,
+    }
+    extras = {"cells_fp32": [{k: v for k, v in r.items() if k != "bytes"} for r in table],
+              "sweep_GFLOPs": round(sweep_flops / (ms_per_step * 1e-3) / 1e9, 1)}
+
+    # ------------------------------------------------------------------ CPU baseline
+    if not args.no_cpu:
+        import oracle  # test infrastructure, used here only as the measured CPU port
+        oracle.build()
+        t0 = time.perf_counter()
+        for s, n in cells:
+            c = mats[s]
+            oracle.spmm_f32(dens[n], c.row_indices, c.values, c.row_offsets, c.column_indices, c.m)
+        cpu_s = time.perf_counter() - t0
+        result["cpu_baseline"] = {"value": round(sweep_bytes / 1e9 / cpu_s, 3), "unit": "GB/s", "cores": 1, "kind": "port",
+                                  "sample": "one full pass over the same 15 fp32 cells (single-threaded C port, "
+                                            f"gcc -O3), {cpu_s:.1f} s", "host_cpu_count": os.cpu_count()}
+        log(f"[bench] CPU port: {cpu_s:.2f} s per sweep -> {sweep_bytes / 1e9 / cpu_s:.2f} GB/s on 1 core")
+        # the library baselines the task names: torch.sparse CSR and scipy CSR on the host cores
+        try:
+            tcpu = {}
+            sample = [(s, 128) for s in W.C2_SPARSITIES]
+            nthreads = torch.get_num_threads()
+            t0 = time.perf_counter()
+            for s, n in sample:
+                c = mats[s]
+                a_t = torch.sparse_csr_tensor(torch.from_numpy(c.row_offsets), torch.from_numpy(c.column_indices),
+                                              torch.from_numpy(c.values), size=(c.m, c.k))
+                _ = a_t @ torch.from_numpy(dens[n][0])
+            tcpu["torch_sparse_csr_s"] = round(time.perf_counter() - t0, 3)
+            tcpu["torch_threads"] = nthreads
+            import scipy.sparse as sp
+            t0 = time.perf_counter()
+            for s, n in sample:
+                c = mats[s]
+                _ = sp.csr_matrix((c.values, c.column_indices, c.row_offsets), shape=(c.m, c.k)) @ dens[n][0]
+            tcpu["scipy_csr_s"] = round(time.perf_counter() - t0, 3)
+            sample_bytes = sum(cell_bytes(s, n) for s, n in sample)
+            tcpu["sample"] = "the five n=128 cells"
+            tcpu["torch_sparse_csr_GBps"] = round(sample_bytes / 1e9 / tcpu["torch_sparse_csr_s"], 3)
+            tcpu["scipy_csr_GBps"] = round(sample_bytes / 1e9 / tcpu["scipy_csr_s"], 3)
+            gpu_sample_us = sum(r["us"] for r in table if r["n"] == 128)
+            tcpu["gpu_same_sample_GBps"] = round(sample_bytes / gpu_sample_us / 1e3, 1)
+            extras["cpu_libraries"] = tcpu
+        except Exception as e:  # a library baseline must not take the bench down
+            extras["cpu_libraries"] = {"error": repr(e)}
+
+    # ------------------------------------------------------------------------ extras
+    if not args.no_extras:
+        try:
+            extras.update(run_extras(torch, ops, dev, W, IL, mats, dens, csr_dev, time_cell, variant_of, log))
+        except Exception as e:
+            import traceback
+            traceback.print_exc(file=sys.stderr)
+            extras["error"] = repr(e)
+    result["extras"] = extras
+    print(json.dumps(result), flush=True)
+
+
+def run_extras(torch, ops, dev, W, IL, mats, dens, csr_dev, time_cell, variant_of, log):
+    out = {}
+    # ---- fp16 sweep (int16 column indices, the reference's half layout)
+    rows = []
+    for s in W.C2_SPARSITIES:
+        c = mats[s]
+        ri, v, ro, ci = csr_dev(c, torch.float16, torch.int16)
+        for n in W.C2_NS:
+            b = torch.from_numpy(dens[n]).to(dev).half()
+            us = time_cell(lambda: ops.spmm_sputnik_reuse_weight_half(b, ri, v, ro, ci, c.m))
+            by = W.spmm_bytes(c.m, c.k, n, c.nnz, 1, 2, 2)
+            fl = W.spmm_flops(c.nnz, n)
+            rows.append({"sparsity": s, "n": n, "us": round(us, 2), "GBps": round(by / us / 1e3, 1),
+                         "hbm_frac": round(by / us / 1e3 / HBM_PEAK_GBPS, 4), "GFLOPs": round(fl / us / 1e3, 1)})
+    out["cells_fp16_i16"] = rows
+    log("[bench] fp16 sweep done")
+
+    # ---- SDDMM: config 1 (fp32, batch-summed) and config 3 (fp16, 16 heads, per-head output)
+    a1, _, lhs1, rhs1 = W.config1()
+    ri, _, ro, ci = csr_dev(a1)
+    l1, r1 = torch.from_numpy(lhs1).to(dev), torch.from_numpy(rhs1).to(dev)
+    us = time_cell(lambda: ops.sddmm_sputnik_atomic_upd_weight(l1, r1, ri, ro, ci))
+    by = W.sddmm_bytes(a1.m, 64, a1.k, a1.nnz, 1, 4, True)
+    out["sddmm_c1_fp32"] = {"us": round(us, 2), "GBps": round(by / us / 1e3, 1), "hbm_frac": round(by / us / 1e3 / HBM_PEAK_GBPS, 4),
+                            "GFLOPs": round(W.sddmm_flops(a1.nnz, 64) / us / 1e3, 1)}
+    pat, q, k, v = W.config3()
+    ri3, _, ro3, ci3 = csr_dev(pat)
+    qt, kt, vt = (torch.from_numpy(x).to(dev).half() for x in (q, k, v))
+    us = time_cell(lambda: ops.sddmm_sputnik_half(qt, kt, ri3, ro3, ci3), repeats=10)
+    by = W.sddmm_bytes(pat.m, 64, pat.k, pat.nnz, 16, 2, False)
+    out["sddmm_c3_fp16_16heads"] = {"nnz": pat.nnz, "sparsity": round(pat.sparsity, 4), "us": round(us, 2),
+                                    "GBps": round(by / us / 1e3, 1), "hbm_frac": round(by / us / 1e3 / HBM_PEAK_GBPS, 4),
+                                    "GFLOPs": round(W.sddmm_flops(pat.nnz, 64, 16) / us / 1e3, 1)}
+    scores = ops.sddmm_sputnik_half(qt, kt, ri3, ro3, ci3)
+    us = time_cell(lambda: ops.spmm_sputnik_batched_values(vt, ri3, scores, ro3, ci3, pat.m), repeats=10)
+    by = W.spmm_bytes(pat.m, pat.k, 64, pat.nnz, 16, 2, 4, True)
+    out["spmm_c3_fp16_16heads"] = {"us": round(us, 2), "GBps": round(by / us / 1e3, 1),
+                                   "hbm_frac": round(by / us / 1e3 / HBM_PEAK_GBPS, 4),
+                                   "GFLOPs": round(W.spmm_flops(pat.nnz, 64, 16) / us / 1e3, 1)}
+    log("[bench] SDDMM done")
+
+    # ---- config 4: fp16 SpMM 11008x4096 @90% x 4096x2048  ||  bf16 GEMM 4096x4096x2048
+    w, x, ga, gb = W.config4()
+    riw, vw, row, ciw = csr_dev(w, torch.float16, torch.int16)
+    xt = torch.from_numpy(x).to(dev).half()
+    gat, gbt = torch.from_numpy(ga).to(dev).bfloat16(), torch.from_numpy(gb).to(dev).bfloat16()
+    reps = 4
+    spmm_execs = [lambda: ops.spmm_sputnik_reuse_weight_half(xt, riw, vw, row, ciw, w.m)] * reps
+    gemm_execs = [lambda: ops.gemm_mfma(gat, gbt, False)] * reps
+    fused_execs = [lambda: ops.fused_spmm_gemm(xt, riw, vw, row, ciw, w.m, gat, gbt, False, 1)] * reps
+    t_spmm = IL.run_non_interleaving(spmm_execs) / reps
+    t_gemm = IL.run_non_interleaving(gemm_execs) / reps
+    t_serial = IL.run_non_interleaving(spmm_execs, gemm_execs) / reps
+    t_graph = IL.run_interleaving(spmm_execs, gemm_execs) / reps
+    t_fused = IL.run_non_interleaving(fused_execs) / reps
+    fl_s, fl_g = W.spmm_flops(w.nnz, 2048), W.gemm_flops(4096, 2048, 4096)
+    by_s = W.spmm_bytes(w.m, w.k, 2048, w.nnz, 1, 2, 2)
+    out["config4"] = {
+        "spmm_ms": round(t_spmm, 4), "spmm_GBps": round(by_s / t_spmm / 1e6, 1), "spmm_GFLOPs": round(fl_s / t_spmm / 1e6, 1),
+        "spmm_hbm_frac": round(by_s / t_spmm / 1e6 / HBM_PEAK_GBPS, 4),
+        "spmm_valu_frac": round(fl_s / t_spmm / 1e9 / VALU_PEAK_TFLOPS_FP32, 4),
+        "gemm_ms": round(t_gemm, 4), "gemm_TFLOPs": round(IL.gemm_tflops(4096, 2048, 4096, t_gemm), 1),
+        "gemm_mfma_frac": round(IL.gemm_tflops(4096, 2048, 4096, t_gemm) / MFMA_PEAK_TFLOPS_16BIT, 4),
+        "serialized_sum_ms": round(t_spmm + t_gemm, 4), "serialized_one_stream_ms": round(t_serial, 4),
+        "two_branch_graph_ms": round(t_graph, 4), "fused_launch_ms": round(t_fused, 4),
+        "graph_makespan_pct_of_serialized": round(100 * t_graph / (t_spmm + t_gemm), 1),
+        "fused_makespan_pct_of_serialized": round(100 * t_fused / (t_spmm + t_gemm), 1),
+        "repeats_per_graph": reps,
+    }
+    log(f"[bench] config 4: spmm {t_spmm:.3f} ms, gemm {t_gemm:.3f} ms, graph {t_graph:.3f} ms, fused {t_fused:.3f} ms")
+    return out
+
+
+if __name__ == "__main__":
+    main()

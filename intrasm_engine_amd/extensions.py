@@ -97,9 +97,17 @@ class CUDAGraphCaptureNotifier:
         return self._pool
 
     def release_pool(self):
+        """Let the allocator reclaim the capture's pool once its tensors are gone."""
         if self._pool is not None and self._device is not None:
             torch._C._cuda_releasePool(self._device, self._pool)
             self._pool = None
+
+    def __del__(self):
+        try:
+            if not self._active:
+                self.release_pool()
+        except Exception:
+            pass
 
 
 class CudaGraphWrapper:

@@ -113,11 +113,13 @@ class CUDAGraphCaptureNotifier:
 class CudaGraphWrapper:
     """Owns a graph handle and its executable graph (helper_CUDAGraphConstructor.cu.h:106-166)."""
 
-    def __init__(self, graph):
-        if isinstance(graph, int):
-            self._g = _L().iex_graph_wrap(graph)
-        else:  # an opaque builder pointer made by this module
-            self._g = graph
+    def __init__(self, graph, _builder=None):
+        """``graph``: a hipGraph_t as an integer (ownership passes to the wrapper).
+        ``_builder`` (internal): an ``iex_graph*`` this module already created."""
+        if _builder is not None:
+            self._g = _builder
+        else:
+            self._g = _L().iex_graph_wrap(int(graph))
         if not self._g:
             raise RuntimeError(_lib.last_error())
         self._added_as_child = False
@@ -182,7 +184,7 @@ class CUDAExperimentalGraphConstructor(CudaGraphWrapper):
         g = _L().iex_graph_create()
         if not g:
             raise RuntimeError(_lib.last_error())
-        super().__init__(g)
+        super().__init__(None, _builder=g)
 
     def register_stream(self, stream):
         self._check(_L().iex_graph_register_stream(self._g, int(stream) if stream else None))
@@ -217,4 +219,4 @@ class CUDAExperimentalGraphConstructor(CudaGraphWrapper):
             raise RuntimeError(_lib.last_error())
         self.notify_added_as_child_graph()
         other.notify_added_as_child_graph()
-        return CudaGraphWrapper(g)
+        return CudaGraphWrapper(None, _builder=g)

@@ -118,22 +118,30 @@ def main():
         return ms / repeats * 1e3  # us
 
     def variant_of(csr, n, sv):
+        """(VEC, LPG, WPR) the library picks for an aligned operand (spmm_pick_shape / pick_wpr)."""
         mean = csr.nnz / csr.m
-        wpr = 16 if mean >= 768 else (4 if mean >= 96 else 1)
-        vec = 16 // sv
-        while vec > 1 and (n % vec or 64 * vec > n):
+        wpr = 4 if mean >= 24 else 1
+        kmax = 16 // sv
+        vec, lpg = kmax, 64
+        while vec > 1 and n % vec:
             vec //= 2
-        return vec, wpr
+        if vec == kmax:
+            while lpg > 8 and (lpg // 2) * vec >= n:
+                lpg //= 2
+        else:
+            while vec > 1 and 64 * vec // 2 >= n:
+                vec //= 2
+        return vec, lpg, wpr
 
     table = []
     for s, n in cells:
         us = time_cell(spmm32(s, n))
         by, fl = cell_bytes(s, n), W.spmm_flops(mats[s].nnz, n)
-        vec, wpr = variant_of(mats[s], n, 4)
+        vec, lpg, wpr = variant_of(mats[s], n, 4)
         table.append({"sparsity": s, "n": n, "nnz": mats[s].nnz, "us": round(us, 2), "GBps": round(by / us / 1e3, 1),
                       "hbm_frac": round(by / us / 1e3 / HBM_PEAK_GBPS, 4), "GFLOPs": round(fl / us / 1e3, 1),
                       "valu_frac": round(fl / us / 1e6 / VALU_PEAK_TFLOPS_FP32, 4),
-                      "kernel": f"spmm_kernel<float,int,VEC={vec},WPR={wpr}>", "bytes": by})
+                      "kernel": f"spmm_kernel<float, int, {vec}, {lpg}, {wpr}>", "bytes": by})
         log(f"[bench] fp32 s={s} n={n}: {us:.2f} us  {by / us / 1e3:.0f} GB/s  {fl / us / 1e3:.0f} GFLOP/s")
 
     by_kernel = {}

@@ -51,8 +51,12 @@ int iex_device_ok(void);
 #define IEX_SPMM_PER_BATCH_VALUES 0x1 /* values is (batch, nnz) instead of (nnz)            */
 #define IEX_SPMM_ACCUMULATE 0x2       /* out += A*b (reference "atomic" store mode)         */
 #define IEX_SPMM_RELU 0x4             /* out = max(0, A*b + bias)                           */
-/* bits 8..15: force waves-per-row (1, 4 or 16); 0 = choose from nnz/m.  For tuning.       */
+/* bits 8..15: force waves-per-row (1, 4 or 8); 0 = choose from nnz/m.  For tuning.    */
 #define IEX_SPMM_FORCE_WPR(w) (((w) & 0xff) << 8)
+/* bits 16..19: force the kernel family (1 = row kernel gathering from L2, 2 = LDS-staged);
+ * bits 20..23: rows per wavefront of the LDS-staged kernel (2, 4 or 8).  0 = choose.      */
+#define IEX_SPMM_FORCE_VARIANT(v) (((v) & 0xf) << 16)
+#define IEX_SPMM_FORCE_RPW(r) (((r) & 0xf) << 20)
 
 /* out[z, r, :] = sum_j values[(z,) j] * dense[z, column_indices[j], :]  (+ bias[r], ReLU)
  * dense is (batch, k, n), out is (batch, m, n), both of `dtype`; accumulation is fp32.

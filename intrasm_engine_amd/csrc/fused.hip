@@ -10,7 +10,7 @@
 //                     so both kinds are dispatched side by side from start to end.
 // Every workgroup has 256 threads and the LDS of the larger role (the GEMM's 40 KB).
 // The device code of both roles is the code of the stand-alone kernels, so results are
-// bit-identical to separate launches.
+// bit-identical to separate launches (the SpMM with at most 4 wavefronts per row).
 #include "gemm_device.cuh"
 #include "spmm_device.cuh"
 
@@ -23,9 +23,9 @@ struct FusedParams {
   int gemm_blocks, spmm_blocks, spmm_by, interleave;
 };
 
-constexpr int kFusedWM = 2, kFusedWN = 2, kFusedWpr = 4;
+constexpr int kFusedWM = 2, kFusedWN = 2;
 
-template <bool BF16, bool TRANS_B, typename IT, int VEC>
+template <bool BF16, bool TRANS_B, typename IT, int VEC, int LPG, int WPR>
 __global__ __launch_bounds__(256) void fused_kernel(FusedParams p) {
   extern __shared__ __align__(16) unsigned char smem[];
   const int b = blockIdx.x;
@@ -44,41 +44,56 @@ __global__ __launch_bounds__(256) void fused_kernel(FusedParams p) {
   if (is_gemm) {
     gemm_tile<BF16, TRANS_B, kFusedWM, kFusedWN>(p.g, idx / p.g.tiles_n, idx % p.g.tiles_n, 0, smem);
   } else {
-    spmm_block<__half, IT, VEC, kFusedWpr>(p.s, idx / p.spmm_by, idx % p.spmm_by, 0, reinterpret_cast<float*>(smem));
+    spmm_block<__half, IT, VEC, LPG, WPR>(p.s, idx / p.spmm_by, idx % p.spmm_by, 0, reinterpret_cast<float*>(smem));
   }
 }
 
-template <bool BF16, bool TRANS_B, typename IT, int VEC>
+template <bool BF16, bool TRANS_B, typename IT, int VEC, int LPG, int WPR>
 int launch(FusedParams p, hipStream_t stream) {
   constexpr int BM = 2 * kFusedWM * 32, BN = 2 * kFusedWN * 32;
   p.g.tiles_m = ceil_div(p.g.M, BM);
   p.g.tiles_n = ceil_div(p.g.N, BN);
   p.gemm_blocks = p.g.tiles_m * p.g.tiles_n;
-  const int rows_per_block = 4 / kFusedWpr;
-  p.spmm_by = ceil_div(p.s.n, kWave * VEC);
+  const int rows_per_block = 4 / WPR;
+  p.spmm_by = ceil_div(p.s.n, LPG * VEC);
   const long long sb = (long long)ceil_div(p.s.m, rows_per_block) * p.spmm_by;
   IEX_REQUIRE(sb + p.gemm_blocks < (1ll << 31), IEX_ERR_TOO_LARGE, "fused: grid too large");
   p.spmm_blocks = (int)sb;
-  constexpr int lds_gemm = gemm_lds_bytes<kFusedWM, kFusedWN>();
-  constexpr int lds_spmm = spmm_lds_floats<VEC, kFusedWpr>() * 4;
+  constexpr int lds_gemm = gemm_lds_bytes<TRANS_B, kFusedWM, kFusedWN>();
+  constexpr int lds_spmm = spmm_lds_floats<VEC, WPR>() * 4;
   constexpr int lds = lds_gemm > lds_spmm ? lds_gemm : lds_spmm;
-  hipLaunchKernelGGL((fused_kernel<BF16, TRANS_B, IT, VEC>), dim3(p.gemm_blocks + p.spmm_blocks), dim3(256), lds, stream,
+  hipLaunchKernelGGL((fused_kernel<BF16, TRANS_B, IT, VEC, LPG, WPR>), dim3(p.gemm_blocks + p.spmm_blocks), dim3(256), lds, stream,
                      p);
   return check_hip(hipGetLastError(), "fused launch");
 }
 
+// Waves per row as the stand-alone kernel would choose, capped at the 4 wavefronts of a
+// 256-thread workgroup (so results equal the stand-alone launch with that choice).
+template <bool BF16, bool TRANS_B, typename IT, int VEC, int LPG>
+int launch_w(const FusedParams& p, hipStream_t stream) {
+  if (spmm_pick_wpr(p.s.m, p.s.nnz) >= 4) return launch<BF16, TRANS_B, IT, VEC, LPG, 4>(p, stream);
+  return launch<BF16, TRANS_B, IT, VEC, LPG, 1>(p, stream);
+}
+
 template <bool BF16, bool TRANS_B, typename IT>
-int launch_vec(const FusedParams& p, int vec, hipStream_t stream) {
-  switch (vec) {
-    case 8: return launch<BF16, TRANS_B, IT, 8>(p, stream);
-    case 4: return launch<BF16, TRANS_B, IT, 4>(p, stream);
-    case 2: return launch<BF16, TRANS_B, IT, 2>(p, stream);
-    default: return launch<BF16, TRANS_B, IT, 1>(p, stream);
+int launch_vec(const FusedParams& p, SpmmShape sh, hipStream_t stream) {
+  if (sh.vec == 8) {
+    switch (sh.lpg) {
+      case 8: return launch_w<BF16, TRANS_B, IT, 8, 8>(p, stream);
+      case 16: return launch_w<BF16, TRANS_B, IT, 8, 16>(p, stream);
+      case 32: return launch_w<BF16, TRANS_B, IT, 8, 32>(p, stream);
+      default: return launch_w<BF16, TRANS_B, IT, 8, 64>(p, stream);
+    }
+  }
+  switch (sh.vec) {
+    case 4: return launch_w<BF16, TRANS_B, IT, 4, 64>(p, stream);
+    case 2: return launch_w<BF16, TRANS_B, IT, 2, 64>(p, stream);
+    default: return launch_w<BF16, TRANS_B, IT, 1, 64>(p, stream);
   }
 }
 
 template <typename IT>
-int launch_gemm_kind(const FusedParams& p, int vec, bool bf16, bool trans_b, hipStream_t stream) {
+int launch_gemm_kind(const FusedParams& p, SpmmShape vec, bool bf16, bool trans_b, hipStream_t stream) {
   if (bf16 && trans_b) return launch_vec<true, true, IT>(p, vec, stream);
   if (bf16 && !trans_b) return launch_vec<true, false, IT>(p, vec, stream);
   if (!bf16 && trans_b) return launch_vec<false, true, IT>(p, vec, stream);
@@ -102,8 +117,8 @@ extern "C" int iex_fused_spmm_gemm(int spmm_itype, int m, int k, int n, int nonz
               "fused: int16 column indices need k <= 32768");
   IEX_REQUIRE(gemm_dtype == IEX_F16 || gemm_dtype == IEX_BF16, IEX_ERR_UNSUPPORTED, "fused: GEMM dtype must be fp16 or bf16");
   IEX_REQUIRE(K % 8 == 0, IEX_ERR_UNSUPPORTED, "fused: K must be a multiple of 8 (K=%d)", K);
-  IEX_REQUIRE(trans_b || N % 4 == 0, IEX_ERR_UNSUPPORTED, "fused: N must be a multiple of 4 when B is (K,N)");
-  IEX_REQUIRE(aligned(A, 16) && aligned(B, trans_b ? 16 : 8), IEX_ERR_UNSUPPORTED, "fused: GEMM operands must be 16-byte aligned");
+  IEX_REQUIRE(trans_b || N % 8 == 0, IEX_ERR_UNSUPPORTED, "fused: N must be a multiple of 8 when B is (K,N)");
+  IEX_REQUIRE(aligned(A, 16) && aligned(B, 16), IEX_ERR_UNSUPPORTED, "fused: GEMM operands must be 16-byte aligned");
   IEX_REQUIRE((long long)k * n < (1ll << 31) && (long long)m * n < (1ll << 31) && (long long)M * K < (1ll << 31) &&
                   (long long)N * K < (1ll << 31) && (long long)M * N < (1ll << 31),
               IEX_ERR_TOO_LARGE, "fused: an operand exceeds 2^31 elements");
@@ -111,8 +126,7 @@ extern "C" int iex_fused_spmm_gemm(int spmm_itype, int m, int k, int n, int nonz
   p.g = GemmParams{M, N, K, A, B, C, 0, 0, 0, 0, 0};
   p.s = SpmmParams{m, k, n, nonzeros, row_indices, values, row_offsets, column_indices, dense, nullptr, spmm_out, 0, 0, 0};
   p.interleave = interleave;
-  int vec = 8;
-  while (vec > 1 && (n % vec != 0 || kWave * vec > n || !aligned(dense, 2 * vec) || !aligned(spmm_out, 2 * vec))) vec >>= 1;
+  const SpmmShape vec = spmm_pick_shape<__half>(n, dense, spmm_out);
   hipStream_t s = static_cast<hipStream_t>(stream);
   if (spmm_itype == IEX_I16) return launch_gemm_kind<short>(p, vec, gemm_dtype == IEX_BF16, trans_b != 0, s);
   return launch_gemm_kind<int>(p, vec, gemm_dtype == IEX_BF16, trans_b != 0, s);

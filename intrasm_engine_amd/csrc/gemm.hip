@@ -35,7 +35,7 @@ int launch(GemmParams p, int batch, hipStream_t stream) {
   p.tiles_n = ceil_div(p.N, BN);
   const int total = p.tiles_m * p.tiles_n;
   const int per_xcd = (total + kXcds - 1) / kXcds;
-  constexpr int lds = gemm_lds_bytes<WM, WN>();
+  constexpr int lds = gemm_lds_bytes<TRANS_B, WM, WN>();
   auto kern = gemm_kernel<BF16, TRANS_B, WM, WN>;
   if (lds > 64 * 1024) {
     static thread_local bool raised = false;  // per instantiation
@@ -53,9 +53,11 @@ int launch(GemmParams p, int batch, hipStream_t stream) {
 
 template <bool BF16, bool TRANS_B>
 int launch_shape(const GemmParams& p, int batch, hipStream_t stream) {
-  // 256x128 tiles halve the LDS reads per MFMA; use them when they still give every CU a tile.
-  const long long big_tiles = (long long)ceil_div(p.M, 256) * ceil_div(p.N, 128) * batch;
-  if (big_tiles >= 256) return launch<BF16, TRANS_B, 4, 2>(p, batch, stream);
+  // 128x128 tiles keep two workgroups (two waves per SIMD) on a CU, which measured faster than
+  // 256x128 at every size tried; 256x256 tiles (128x128 per wave, half the LDS reads per MFMA)
+  // win once there are at least two of them per CU.
+  const long long huge_tiles = (long long)ceil_div(p.M, 256) * ceil_div(p.N, 256) * batch;
+  if (huge_tiles >= 512) return launch<BF16, TRANS_B, 4, 4>(p, batch, stream);
   return launch<BF16, TRANS_B, 2, 2>(p, batch, stream);
 }
 
@@ -70,8 +72,8 @@ extern "C" int iex_gemm(int dtype, int trans_b, int M, int N, int K, const void*
   IEX_REQUIRE(A && B && C, IEX_ERR_BAD_ARGUMENT, "gemm: null pointer argument");
   IEX_REQUIRE(dtype == IEX_F16 || dtype == IEX_BF16, IEX_ERR_UNSUPPORTED, "gemm: dtype must be fp16 or bf16");
   IEX_REQUIRE(K > 0 && K % 8 == 0, IEX_ERR_UNSUPPORTED, "gemm: K must be a positive multiple of 8 (K=%d)", K);
-  IEX_REQUIRE(trans_b || N % 4 == 0, IEX_ERR_UNSUPPORTED, "gemm: N must be a multiple of 4 when B is (K,N) (N=%d)", N);
-  IEX_REQUIRE(aligned(A, 16) && aligned(B, trans_b ? 16 : 8), IEX_ERR_UNSUPPORTED, "gemm: operands must be 16-byte aligned");
+  IEX_REQUIRE(trans_b || N % 8 == 0, IEX_ERR_UNSUPPORTED, "gemm: N must be a multiple of 8 when B is (K,N) (N=%d)", N);
+  IEX_REQUIRE(aligned(A, 16) && aligned(B, 16), IEX_ERR_UNSUPPORTED, "gemm: operands must be 16-byte aligned");
   IEX_REQUIRE(stride_a % 8 == 0 && stride_b % 8 == 0, IEX_ERR_UNSUPPORTED, "gemm: batch strides must be multiples of 8");
   IEX_REQUIRE(batch <= 65535, IEX_ERR_TOO_LARGE, "gemm: batch %d exceeds 65535", batch);
   IEX_REQUIRE((long long)M * K < (1ll << 31) && (long long)N * K < (1ll << 31) && (long long)M * N < (1ll << 31),

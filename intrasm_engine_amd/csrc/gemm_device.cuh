@@ -2,13 +2,19 @@
 // accumulate on the matrix cores (v_mfma_f32_32x32x16_{f16,bf16}), LDS double-buffered.
 //
 // Tiling: a workgroup of 4 wavefronts (2 x 2) owns a (2*WM*32) x (2*WN*32) tile of C;
-// a wavefront owns WM x WN MFMA tiles of 32 x 32.  The K loop advances BK = 32 per step:
-//   global -> registers (next step, 128-bit loads) | MFMA on the current LDS buffer |
-//   registers -> the other LDS buffer | one barrier.
-// Both operands sit in LDS K-contiguous ([row][k], rows padded by 8 elements so that the
-// 128-bit operand reads of 8 consecutive lanes fall in distinct banks).  When B is given
-// as (K, N) a thread transposes 4 x 4 blocks in registers (v_perm_b32) on the way in, so
-// the MFMA operand reads are identical for both layouts.
+// a wavefront owns WM x WN MFMA tiles of 32 x 32.  The K loop advances BK = 32 per step.
+// Software pipeline: global loads run kGemmSets steps ahead of the MFMAs (one register set
+// per step in flight, 128-bit loads), a set is written to the idle LDS buffer one step
+// before it is consumed, one barrier per step:
+//   step t:  MFMA on LDS[t%2] | registers(tile t+1) -> LDS[(t+1)%2] | issue loads of tile t+1+SETS
+// so a global load has kGemmSets MFMA steps to complete (L2 / MALL latency is several steps).
+// A (and B given as (N, K)) sit in LDS K-contiguous ([row][k], rows padded by 8 elements so
+// that the 128-bit operand reads of 8 consecutive lanes fall in distinct banks).  B given as
+// (K, N) is kept in LDS as it is in memory ([k][n], rows padded by 32 elements) and the MFMA
+// operand is formed by the LDS transpose read of gfx950 (ds_read_b64_tr_b16): the 16 lanes
+// of a group each point at 4 adjacent n of one k row, and lane i receives column n0+i of 4
+// consecutive k rows, so no register transposes and full 128-bit global loads for both
+// layouts.
 // The MFMA is issued with the operands swapped (B fragment as the "A" operand): a lane
 // then holds 4 adjacent columns of one row of C per accumulator quad and stores them
 // with one 64-bit store.
@@ -35,11 +41,18 @@ typedef unsigned int u32x2 __attribute__((ext_vector_type(2)));
 constexpr int kGemmBK = 32;
 constexpr int kGemmPad = 8;
 constexpr int kGemmLd = kGemmBK + kGemmPad;  // LDS row stride in elements (80 bytes)
+constexpr int kGemmSets = 3;                 // register sets = K steps of global loads in flight
 
-template <int WM, int WN>
+constexpr int kGemmLdbPad = 32;  // padding of a [k][n] row of B in LDS, elements
+
+template <bool TRANS_B, int WM, int WN>
 constexpr int gemm_lds_bytes() {
-  return 2 /*buffers*/ * (2 * WM * 32 + 2 * WN * 32) * kGemmLd * 2 /*bytes*/;
+  constexpr int a_elems = 2 * WM * 32 * kGemmLd;
+  constexpr int b_elems = TRANS_B ? 2 * WN * 32 * kGemmLd : kGemmBK * (2 * WN * 32 + kGemmLdbPad);
+  return 2 /*buffers*/ * (a_elems + b_elems) * 2 /*bytes*/;
 }
+
+typedef short s16x4 __attribute__((ext_vector_type(4)));
 
 template <bool BF16>
 __device__ __forceinline__ f32x16 mfma_32x32x16(u32x4 a, u32x4 b, f32x16 c) {
@@ -61,44 +74,22 @@ __device__ __forceinline__ unsigned short f32_to_16(float v, bool bf16) {
   return __builtin_bit_cast(unsigned short, h);
 }
 
-// One C tile.  `smem` must hold gemm_lds_bytes<WM,WN>() bytes, 16-byte aligned.
-// All 256 threads of the workgroup must call this (it contains barriers).
-template <bool BF16, bool TRANS_B, int WM, int WN>
-__device__ __forceinline__ void gemm_tile(const GemmParams& p, int tile_m, int tile_n, int z, unsigned char* smem) {
-  constexpr int BM = 2 * WM * 32;
-  constexpr int BN = 2 * WN * 32;
-  constexpr int BK = kGemmBK;
-  constexpr int LD = kGemmLd;
-  constexpr int A_CHUNKS = BM * (BK / 8) / 256;        // 128-bit chunks per thread (A, and B^T layout)
-  constexpr int B_CHUNKS = BN * (BK / 8) / 256;
-  constexpr int B_TASKS = (BK / 4) * (BN / 4) / 256;   // 4x4 blocks per thread (B as (K,N))
+// The slice of one K step that a thread carries from global memory to LDS.
+template <bool TRANS_B, int BM, int BN>
+struct GemmStage {
+  static constexpr int BK = kGemmBK;
+  static constexpr int LD = kGemmLd;
+  static constexpr int A_CHUNKS = BM * (BK / 8) / 256;       // 128-bit chunks per thread (A, and B^T layout)
+  static constexpr int B_CHUNKS = BN * (BK / 8) / 256;
+  static constexpr int LDB = BN + kGemmLdbPad;               // LDS row stride of B kept as [k][n]
+  static constexpr int B_ELEMS = TRANS_B ? BN * LD : BK * LDB;  // one LDS buffer of B, elements
   typedef unsigned short u16;
 
-  u16* sA = reinterpret_cast<u16*>(smem);               // [2][BM][LD]
-  u16* sB = sA + 2 * BM * LD;                           // [2][BN][LD]
-
-  const int tid = threadIdx.x;
-  const int lane = tid & 63;
-  const int wave = tid >> 6;
-  const int wm = wave >> 1, wn = wave & 1;
-  const int m0 = tile_m * BM, n0 = tile_n * BN;
-  const u16* __restrict__ A = static_cast<const u16*>(p.A) + (size_t)z * p.stride_a;
-  const u16* __restrict__ B = static_cast<const u16*>(p.B) + (size_t)z * p.stride_b;
-  u16* __restrict__ C = static_cast<u16*>(p.C) + (size_t)z * p.stride_c;
-
-  f32x16 acc[WM][WN];
-#pragma unroll
-  for (int i = 0; i < WM; ++i)
-#pragma unroll
-    for (int j = 0; j < WN; ++j)
-#pragma unroll
-      for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
-
   u32x4 ra[A_CHUNKS];
-  u32x4 rb[B_CHUNKS];      // trans_b layout
-  u32x2 rbt[B_TASKS][4];   // (K,N) layout: 4 k-rows x 4 n-columns per task
+  u32x4 rb[B_CHUNKS];  // (N,K): chunk = 8 k of one n row; (K,N): chunk = 8 n of one k row
 
-  auto load_global = [&](int kt) {
+  __device__ __forceinline__ void load(const GemmParams& p, const u16* __restrict__ A, const u16* __restrict__ B, int m0,
+                                       int n0, int kt, int tid) {
     const int k0 = kt * BK;
 #pragma unroll
     for (int c = 0; c < A_CHUNKS; ++c) {
@@ -121,24 +112,18 @@ __device__ __forceinline__ void gemm_tile(const GemmParams& p, int tile_m, int t
       }
     } else {
 #pragma unroll
-      for (int t = 0; t < B_TASKS; ++t) {
-        const int task = tid + t * 256;
-        const int kg = task / (BN / 4), nc = task % (BN / 4);
-        const int gn = n0 + nc * 4;
-#pragma unroll
-        for (int r = 0; r < 4; ++r) {
-          const int gk = k0 + kg * 4 + r;
-          u32x2 v = {0u, 0u};
-          if (gn < p.N && gk < p.K) v = *reinterpret_cast<const u32x2*>(B + (size_t)gk * p.N + gn);
-          rbt[t][r] = v;
-        }
+      for (int c = 0; c < B_CHUNKS; ++c) {
+        const int chunk = tid + c * 256;
+        const int kr = chunk / (BN / 8), nc = chunk % (BN / 8);
+        const int gk = k0 + kr, gn = n0 + nc * 8;
+        u32x4 v = {0u, 0u, 0u, 0u};
+        if (gk < p.K && gn < p.N) v = *reinterpret_cast<const u32x4*>(B + (size_t)gk * p.N + gn);
+        rb[c] = v;
       }
     }
-  };
+  }
 
-  auto store_lds = [&](int buf) {
-    u16* a = sA + buf * BM * LD;
-    u16* b = sB + buf * BN * LD;
+  __device__ __forceinline__ void store(u16* a, u16* b, int tid) const {
 #pragma unroll
     for (int c = 0; c < A_CHUNKS; ++c) {
       const int chunk = tid + c * 256;
@@ -154,51 +139,121 @@ __device__ __forceinline__ void gemm_tile(const GemmParams& p, int tile_m, int t
       }
     } else {
 #pragma unroll
-      for (int t = 0; t < B_TASKS; ++t) {
-        const int task = tid + t * 256;
-        const int kg = task / (BN / 4), nc = task % (BN / 4);
-        // rbt[t][r] = {B[k+r][n], B[k+r][n+1] | B[k+r][n+2], B[k+r][n+3]}; column e of the 4x4
-        // block becomes the 4 consecutive k entries of LDS row n+e.
-#pragma unroll
-        for (int e = 0; e < 4; ++e) {
-          const unsigned sel = (e & 1) ? 0x07060302u : 0x05040100u;  // high or low halves of (src1, src0)
-          u32x2 w;
-          w.x = __builtin_amdgcn_perm(rbt[t][1][e >> 1], rbt[t][0][e >> 1], sel);
-          w.y = __builtin_amdgcn_perm(rbt[t][3][e >> 1], rbt[t][2][e >> 1], sel);
-          *reinterpret_cast<u32x2*>(b + (nc * 4 + e) * LD + kg * 4) = w;
-        }
+      for (int c = 0; c < B_CHUNKS; ++c) {
+        const int chunk = tid + c * 256;
+        const int kr = chunk / (BN / 8), nc = chunk % (BN / 8);
+        *reinterpret_cast<u32x4*>(b + kr * LDB + nc * 8) = rb[c];
       }
     }
-  };
+  }
+};
+
+// One C tile.  `smem` must hold gemm_lds_bytes<WM,WN>() bytes, 16-byte aligned.
+// All 256 threads of the workgroup must call this (it contains barriers).
+template <bool BF16, bool TRANS_B, int WM, int WN>
+__device__ __forceinline__ void gemm_tile(const GemmParams& p, int tile_m, int tile_n, int z, unsigned char* smem) {
+  constexpr int BM = 2 * WM * 32;
+  constexpr int BN = 2 * WN * 32;
+  constexpr int BK = kGemmBK;
+  constexpr int LD = kGemmLd;
+  constexpr int SETS = kGemmSets;
+  typedef unsigned short u16;
+
+  typedef GemmStage<TRANS_B, BM, BN> Stage;
+  constexpr int LDB = Stage::LDB;
+  constexpr int B_ELEMS = Stage::B_ELEMS;
+  u16* sA = reinterpret_cast<u16*>(smem);  // [2][BM][LD]
+  u16* sB = sA + 2 * BM * LD;              // [2][BN][LD]  or  [2][BK][LDB]
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = tid >> 6;
+  const int wm = wave >> 1, wn = wave & 1;
+  const int m0 = tile_m * BM, n0 = tile_n * BN;
+  const u16* __restrict__ A = static_cast<const u16*>(p.A) + (size_t)z * p.stride_a;
+  const u16* __restrict__ B = static_cast<const u16*>(p.B) + (size_t)z * p.stride_b;
+  u16* __restrict__ C = static_cast<u16*>(p.C) + (size_t)z * p.stride_c;
+
+  f32x16 acc[WM][WN];
+#pragma unroll
+  for (int i = 0; i < WM; ++i)
+#pragma unroll
+    for (int j = 0; j < WN; ++j)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
+
+  Stage regs[SETS];  // regs[t % SETS] carries tile t (statically indexed below)
 
   const int KT = (p.K + BK - 1) / BK;
-  load_global(0);
-  store_lds(0);
+  // prologue: tiles 0 .. SETS-1 in flight, tile 0 into LDS[0], then tile SETS replaces it
+#pragma unroll
+  for (int s = 0; s < SETS; ++s)
+    if (s < KT) regs[s].load(p, A, B, m0, n0, s, tid);
+  regs[0].store(sA, sB, tid);
+  if (SETS < KT) regs[0].load(p, A, B, m0, n0, SETS, tid);
   __syncthreads();
 
-  const int frag_row = lane & 31;        // row of the 32-row operand block this lane feeds
-  const int frag_k = (lane >> 5) * 8;    // which 8 of the 16 k entries of a sub-step
+  const int frag_row = lane & 31;      // row of the 32-row operand block this lane feeds
+  const int frag_k = (lane >> 5) * 8;  // which 8 of the 16 k entries of a sub-step
 
-  for (int kt = 0; kt < KT; ++kt) {
-    const int buf = kt & 1;
-    if (kt + 1 < KT) load_global(kt + 1);
+  // One step; PH = t % (2*SETS) is a compile-time phase so that both the register set
+  // ((t+1) % SETS) and the LDS buffer (t % 2) are static.
+  auto step = [&](int kt, auto phase) {
+    constexpr int PH = decltype(phase)::value;
+    constexpr int buf = PH & 1;
+    constexpr int set = (PH + 1) % SETS;
     const u16* a = sA + buf * BM * LD + (wm * WM * 32 + frag_row) * LD + frag_k;
-    const u16* b = sB + buf * BN * LD + (wn * WN * 32 + frag_row) * LD + frag_k;
+    // (N,K) layout: 128-bit read of 8 k of row n.  (K,N) layout: two transpose reads; the lane
+    // group q = lane/16 covers n-half (q%2) and k-half (q/2) of the sub-step, lane r of the
+    // group points at k row r/4 and n columns 4*(r%4).., and receives column n0 + r of 4 k rows.
+    const u16* b = TRANS_B ? sB + buf * B_ELEMS + (wn * WN * 32 + frag_row) * LD + frag_k
+                           : sB + buf * B_ELEMS + ((lane >> 5) * 8 + ((lane & 15) >> 2)) * LDB + wn * WN * 32 +
+                                 ((lane >> 4) & 1) * 16 + (lane & 3) * 4;
 #pragma unroll
     for (int ks = 0; ks < BK / 16; ++ks) {
       u32x4 fa[WM], fb[WN];
 #pragma unroll
       for (int i = 0; i < WM; ++i) fa[i] = *reinterpret_cast<const u32x4*>(a + i * 32 * LD + ks * 16);
 #pragma unroll
-      for (int j = 0; j < WN; ++j) fb[j] = *reinterpret_cast<const u32x4*>(b + j * 32 * LD + ks * 16);
+      for (int j = 0; j < WN; ++j) {
+        if constexpr (TRANS_B) {
+          fb[j] = *reinterpret_cast<const u32x4*>(b + j * 32 * LD + ks * 16);
+        } else {
+          typedef __attribute__((address_space(3))) s16x4 lds_s16x4;
+          const u16* q0 = b + (ks * 16) * LDB + j * 32;
+          const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)(q0));
+          const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)(q0 + 4 * LDB));
+          const u32x2 l2 = __builtin_bit_cast(u32x2, lo), h2 = __builtin_bit_cast(u32x2, hi);
+          fb[j] = u32x4{l2.x, l2.y, h2.x, h2.y};
+        }
+      }
 #pragma unroll
       for (int i = 0; i < WM; ++i)
 #pragma unroll
         for (int j = 0; j < WN; ++j) acc[i][j] = mfma_32x32x16<BF16>(fb[j], fa[i], acc[i][j]);
     }
-    if (kt + 1 < KT) store_lds(buf ^ 1);
+    if (kt + 1 < KT) {
+      regs[set].store(sA + (buf ^ 1) * BM * LD, sB + (buf ^ 1) * B_ELEMS, tid);
+      if (kt + 1 + SETS < KT) regs[set].load(p, A, B, m0, n0, kt + 1 + SETS, tid);
+    }
     __syncthreads();
+  };
+
+  static_assert(SETS == 3, "the step loop below is unrolled for 3 register sets (period 6)");
+  int kt = 0;
+  for (; kt + 6 <= KT; kt += 6) {
+    step(kt + 0, std::integral_constant<int, 0>{});
+    step(kt + 1, std::integral_constant<int, 1>{});
+    step(kt + 2, std::integral_constant<int, 2>{});
+    step(kt + 3, std::integral_constant<int, 3>{});
+    step(kt + 4, std::integral_constant<int, 4>{});
+    step(kt + 5, std::integral_constant<int, 5>{});
   }
+  if (kt < KT) step(kt++, std::integral_constant<int, 0>{});
+  if (kt < KT) step(kt++, std::integral_constant<int, 1>{});
+  if (kt < KT) step(kt++, std::integral_constant<int, 2>{});
+  if (kt < KT) step(kt++, std::integral_constant<int, 3>{});
+  if (kt < KT) step(kt++, std::integral_constant<int, 4>{});
 
   // Swapped-operand result layout: lane holds row (lane % 32) of the 32x32 block and, in
   // accumulator quad q, columns q*8 + (lane / 32)*4 .. +3.

@@ -1,68 +1,116 @@
 // Host side of the CSR SpMM: kernel wrappers, variant selection, argument checks and
 // the C entry points.  The device code is in spmm_device.cuh.
-#include "spmm_device.cuh"
+#include "spmm_lds_device.cuh"
 
 namespace iex {
 namespace {
 
-template <typename T, typename IT, int VEC, int WPR>
-__global__ __launch_bounds__(WPR == 16 ? 1024 : 256) void spmm_kernel(SpmmParams p) {
+template <typename T, typename IT, int VEC, int LPG, int WPR>
+__global__ __launch_bounds__((WPR > 4 ? WPR : 4) * 64) void spmm_kernel(SpmmParams p) {
   __shared__ float red[spmm_lds_floats<VEC, WPR>()];
-  spmm_block<T, IT, VEC, WPR>(p, blockIdx.x, blockIdx.y, blockIdx.z, red);
+  spmm_block<T, IT, VEC, LPG, WPR>(p, blockIdx.x, blockIdx.y, blockIdx.z, red);
 }
 
-template <typename T, typename IT, int VEC, int WPR>
+template <typename T, typename IT, int VEC, int LPG, int WPR>
 int launch_one(const SpmmParams& p, int batch, hipStream_t stream) {
-  constexpr int kWavesPerBlock = (WPR == 16) ? 16 : 4;
+  constexpr int kWavesPerBlock = (WPR > 4) ? WPR : 4;
   constexpr int kRowsPerBlock = kWavesPerBlock / WPR;
-  dim3 grid(ceil_div(p.m, kRowsPerBlock), ceil_div(p.n, kWave * VEC), batch);
+  dim3 grid(ceil_div(p.m, kRowsPerBlock), ceil_div(p.n, LPG * VEC), batch);
   dim3 block(kWavesPerBlock * kWave);
-  hipLaunchKernelGGL((spmm_kernel<T, IT, VEC, WPR>), grid, block, 0, stream, p);
+  hipLaunchKernelGGL((spmm_kernel<T, IT, VEC, LPG, WPR>), grid, block, 0, stream, p);
   return check_hip(hipGetLastError(), "spmm launch");
 }
 
-template <typename T, typename IT, int VEC>
+template <typename T, typename IT, int VEC, int LPG>
 int launch_wpr(const SpmmParams& p, int batch, int wpr, hipStream_t stream) {
   switch (wpr) {
-    case 1: return launch_one<T, IT, VEC, 1>(p, batch, stream);
-    case 4: return launch_one<T, IT, VEC, 4>(p, batch, stream);
-    case 16: return launch_one<T, IT, VEC, 16>(p, batch, stream);
+    case 1: return launch_one<T, IT, VEC, LPG, 1>(p, batch, stream);
+    case 4: return launch_one<T, IT, VEC, LPG, 4>(p, batch, stream);
+    case 8: return launch_one<T, IT, VEC, LPG, 8>(p, batch, stream);
   }
-  return fail(IEX_ERR_BAD_ARGUMENT, "spmm: waves-per-row must be 1, 4 or 16 (got %d)", wpr);
+  return fail(IEX_ERR_BAD_ARGUMENT, "spmm: waves-per-row must be 1, 4 or 8 (got %d)", wpr);
 }
 
-// Widest per-lane vector such that (a) it divides n, (b) a 64-lane tile is not wider than
-// n rounded up to 64 lanes (keeps lanes busy for narrow outputs), (c) rows stay aligned.
+// ---- LDS-staged variant -----------------------------------------------------------------
+template <typename T, typename IT, int VEC, int RPW>
+__global__ __launch_bounds__(kLdsThreads, 4) void spmm_lds_kernel(SpmmParams p) {
+  extern __shared__ __align__(16) unsigned char smem[];
+  spmm_lds_block<T, IT, VEC, RPW>(p, blockIdx.x, blockIdx.y, blockIdx.z, smem);
+}
+
+template <typename T, typename IT, int VEC, int RPW>
+int launch_lds_one(const SpmmParams& p, int batch, hipStream_t stream) {
+  dim3 grid(ceil_div(p.m, kLdsWaves * RPW), ceil_div(p.n, kWave * VEC), batch);
+  hipLaunchKernelGGL((spmm_lds_kernel<T, IT, VEC, RPW>), grid, dim3(kLdsThreads), kLdsTileBytes, stream, p);
+  return check_hip(hipGetLastError(), "spmm (LDS-staged) launch");
+}
+
+template <typename T, typename IT, int VEC>
+int launch_lds_rpw(const SpmmParams& p, int batch, int rpw, hipStream_t stream) {
+  switch (rpw) {
+    case 2: return launch_lds_one<T, IT, VEC, 2>(p, batch, stream);
+    case 4: return launch_lds_one<T, IT, VEC, 4>(p, batch, stream);
+    case 8:
+      // 8 rows x 8 accumulators per lane would spill at 4 waves per SIMD: 4 rows per wave then
+      if constexpr (VEC < 8) return launch_lds_one<T, IT, VEC, 8>(p, batch, stream);
+      else return launch_lds_one<T, IT, VEC, 4>(p, batch, stream);
+  }
+  return fail(IEX_ERR_BAD_ARGUMENT, "spmm: rows-per-wave of the LDS-staged variant must be 2, 4 or 8 (got %d)", rpw);
+}
+
+struct Choice {
+  int wpr = 0;      // wavefronts per row of the row kernel
+  int variant = 0;  // 0 = choose, 1 = row kernel, 2 = LDS-staged kernel
+  int rpw = 0;      // rows per wavefront of the LDS-staged kernel (0 = choose)
+};
+
+// The LDS-staged kernel needs a full-width tile (64 lanes x VEC, VEC the full or half 128-bit
+// vector) and pays off when the rows of a workgroup share dense rows often enough:
+// gathers saved per dense row staged = density * rows per workgroup.
 template <typename T>
-int pick_vec(int n, const void* dense, const void* out) {
+bool lds_variant(const SpmmParams& p, int batch, const Choice& ch, int& vec, int& rpw) {
   constexpr int kMax = 16 / (int)sizeof(T);
-  int vec = kMax;
-  while (vec > 1 && (n % vec != 0 || kWave * vec > n || !aligned(dense, sizeof(T) * vec) ||
-                     !aligned(out, sizeof(T) * vec)))
-    vec >>= 1;
-  return vec;
+  vec = kMax;
+  auto fits = [&](int v) {
+    return p.n % v == 0 && kWave * v <= p.n && aligned(p.dense, sizeof(T) * v) && aligned(p.out, sizeof(T) * v);
+  };
+  if (!fits(vec)) vec = kMax / 2;
+  if (!fits(vec)) return false;
+  const long long tiles = (long long)ceil_div(p.n, kWave * vec) * batch;
+  rpw = ch.rpw;
+  if (rpw == 0) {
+    rpw = 8;  // largest rows-per-wave that still gives every CU two workgroups
+    while (rpw > 2 && (long long)ceil_div(p.m, kLdsWaves * rpw) * tiles < 512) rpw >>= 1;
+  }
+  // Measured on MI355X (config-2 and config-4 shapes) the row kernel is faster: with 16 rows
+  // per CU there are too few wavefronts to keep the LDS pipeline busy and the per-stage
+  // barriers expose row-length imbalance.  The staged kernel therefore runs only on request.
+  return ch.variant == 2;
 }
 
 template <typename T, typename IT>
-int launch_typed(const SpmmParams& p, int batch, int wpr, hipStream_t stream) {
-  const int vec = pick_vec<T>(p.n, p.dense, p.out);
-  if constexpr (sizeof(T) == 2) {
-    if (vec == 8) return launch_wpr<T, IT, 8>(p, batch, wpr, stream);
+int launch_typed(const SpmmParams& p, int batch, const Choice& ch, hipStream_t stream) {
+  constexpr int kMax = 16 / (int)sizeof(T);
+  int lvec = 0, rpw = 0;
+  if (lds_variant<T>(p, batch, ch, lvec, rpw)) {
+    if (lvec == kMax) return launch_lds_rpw<T, IT, kMax>(p, batch, rpw, stream);
+    return launch_lds_rpw<T, IT, kMax / 2>(p, batch, rpw, stream);
   }
-  switch (vec) {
-    case 4: return launch_wpr<T, IT, 4>(p, batch, wpr, stream);
-    case 2: return launch_wpr<T, IT, 2>(p, batch, wpr, stream);
-    default: return launch_wpr<T, IT, 1>(p, batch, wpr, stream);
+  const int wpr = ch.wpr;
+  const SpmmShape sh = spmm_pick_shape<T>(p.n, p.dense, p.out);
+  if (sh.vec == kMax) {
+    switch (sh.lpg) {
+      case 8: return launch_wpr<T, IT, kMax, 8>(p, batch, wpr, stream);
+      case 16: return launch_wpr<T, IT, kMax, 16>(p, batch, wpr, stream);
+      case 32: return launch_wpr<T, IT, kMax, 32>(p, batch, wpr, stream);
+      default: return launch_wpr<T, IT, kMax, 64>(p, batch, wpr, stream);
+    }
   }
-}
-
-// Waves per row from the mean row length: short rows get a wave each, long rows a
-// workgroup, so that the heaviest row of a skewed matrix never runs on a single wave.
-int pick_wpr(int m, int nnz) {
-  const double mean = m > 0 ? (double)nnz / m : 0.0;
-  if (mean >= 768.0) return 16;
-  if (mean >= 96.0) return 4;
-  return 1;
+  if constexpr (kMax == 8) {
+    if (sh.vec == 4) return launch_wpr<T, IT, 4, 64>(p, batch, wpr, stream);
+  }
+  if (sh.vec == 2) return launch_wpr<T, IT, 2, 64>(p, batch, wpr, stream);
+  return launch_wpr<T, IT, 1, 64>(p, batch, wpr, stream);
 }
 
 }  // namespace
@@ -83,16 +131,19 @@ int spmm_dispatch(int dtype, int itype, int flags, int m, int k, int n, int nonz
               "spmm: a dense operand exceeds 2^31 elements per batch entry");
   IEX_REQUIRE(itype == IEX_I32 || (itype == IEX_I16 && k <= 32768), IEX_ERR_BAD_ARGUMENT,
               "spmm: int16 column indices need k <= 32768 (k=%d)", k);
-  int wpr = (flags >> 8) & 0xff;
-  if (wpr == 0) wpr = pick_wpr(m, nonzeros);
+  Choice ch;
+  ch.wpr = (flags >> 8) & 0xff;
+  if (ch.wpr == 0) ch.wpr = spmm_pick_wpr(m, nonzeros);
+  ch.variant = (flags >> 16) & 0xf;
+  ch.rpw = (flags >> 20) & 0xf;
   SpmmParams p{m, k, n, nonzeros, row_indices, values, row_offsets, column_indices, dense, bias, out,
                (flags & IEX_SPMM_PER_BATCH_VALUES) != 0, (flags & IEX_SPMM_ACCUMULATE) != 0,
                (flags & IEX_SPMM_RELU) != 0};
   hipStream_t s = static_cast<hipStream_t>(stream);
-  if (dtype == IEX_F32 && itype == IEX_I32) return launch_typed<float, int>(p, batch, wpr, s);
-  if (dtype == IEX_F16 && itype == IEX_I32) return launch_typed<__half, int>(p, batch, wpr, s);
-  if (dtype == IEX_F16 && itype == IEX_I16) return launch_typed<__half, short>(p, batch, wpr, s);
-  if (dtype == IEX_BF16 && itype == IEX_I32) return launch_typed<__hip_bfloat16, int>(p, batch, wpr, s);
+  if (dtype == IEX_F32 && itype == IEX_I32) return launch_typed<float, int>(p, batch, ch, s);
+  if (dtype == IEX_F16 && itype == IEX_I32) return launch_typed<__half, int>(p, batch, ch, s);
+  if (dtype == IEX_F16 && itype == IEX_I16) return launch_typed<__half, short>(p, batch, ch, s);
+  if (dtype == IEX_BF16 && itype == IEX_I32) return launch_typed<__hip_bfloat16, int>(p, batch, ch, s);
   return fail(IEX_ERR_UNSUPPORTED, "spmm: no kernel for dtype=%d itype=%d", dtype, itype);
 }
 

@@ -61,7 +61,7 @@ def _check_index_dtypes(row_indices, row_offsets, column_indices, allow_i16=Fals
 
 
 def _spmm(b, row_indices, values, row_offsets, column_indices, m, *, per_batch_values,
-          accumulate, dtypes, allow_i16, out=None, bias=None, relu=False, force_wpr=0):
+          accumulate, dtypes, allow_i16, out=None, bias=None, relu=False, force_wpr=0, force_variant=0, force_rpw=0):
     _chk(b.dim() == 3)
     if per_batch_values:
         _chk(values.dim() == 2)
@@ -99,7 +99,7 @@ def _spmm(b, row_indices, values, row_offsets, column_indices, m, *, per_batch_v
              and bias.device == b.device, "bias must be a contiguous fp32 tensor with m entries")
     flags = (_lib.SPMM_PER_BATCH_VALUES if per_batch_values else 0) | \
             (_lib.SPMM_ACCUMULATE if accumulate else 0) | (_lib.SPMM_RELU if relu else 0) | \
-            ((int(force_wpr) & 0xff) << 8)
+            ((int(force_wpr) & 0xff) << 8) | ((int(force_variant) & 0xf) << 16) | ((int(force_rpw) & 0xf) << 20)
     with torch.cuda.device(b.device):
         rc = _lib.load().iex_spmm_ex(
             _DT[b.dtype], _IT[column_indices.dtype], flags, m, k, n, nonzeros,

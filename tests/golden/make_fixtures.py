@@ -66,7 +66,7 @@ def main():
     rng = np.random.default_rng(104)
     import torch
     ga = torch.from_numpy(rng.standard_normal((40, 24)).astype(np.float32)).bfloat16().float().numpy()
-    gb = torch.from_numpy(rng.standard_normal((24, 36)).astype(np.float32)).bfloat16().float().numpy()
+    gb = torch.from_numpy(rng.standard_normal((24, 40)).astype(np.float32)).bfloat16().float().numpy()
     c = oracle.gemm(ga, gb)
     assert np.allclose(c, ga.astype(np.float64) @ gb.astype(np.float64), rtol=1e-13, atol=1e-13)
     np.savez(os.path.join(HERE, "gemm_bf16_inputs.npz"), a=ga, b=gb, expected=c)

@@ -1,0 +1,48 @@
+"""Horizontally fused sparse + dense launch: both results must be bit-identical to the
+separate launches, for both workgroup-role layouts."""
+import numpy as np
+import pytest
+import torch
+
+from intrasm_engine_amd import workloads as W
+from _util import to_dev
+
+pytestmark = pytest.mark.gpu
+ops = torch.ops.iex_ops
+
+
+@pytest.mark.parametrize("interleave", [0, 1])
+@pytest.mark.parametrize("gdtype,trans_b", [(torch.bfloat16, False), (torch.float16, True)])
+@pytest.mark.parametrize("n,idtype", [(512, torch.int16), (64, torch.int32), (200, torch.int32)])
+def test_fused_equals_separate_launches(dev, interleave, gdtype, trans_b, n, idtype):
+    rng = np.random.default_rng(n)
+    a = W.config2_matrix(0.90, m=700, k=512)
+    ri, v, ro, ci = to_dev(a, dev, torch.float16, idtype)
+    x = torch.from_numpy(rng.standard_normal((1, 512, n)).astype(np.float32)).to(dev).half()
+    M, N, K = 300, 264, 136
+    ga = torch.from_numpy(rng.standard_normal((M, K)).astype(np.float32)).to(dev).to(gdtype)
+    gb = torch.from_numpy(rng.standard_normal((N, K) if trans_b else (K, N)).astype(np.float32)).to(dev).to(gdtype)
+    out, c = ops.fused_spmm_gemm(x, ri, v, ro, ci, a.m, ga, gb, trans_b, interleave)
+    assert torch.equal(out, ops.spmm_sputnik_reuse_weight_half(x, ri, v, ro, ci, a.m))
+    assert torch.equal(c, ops.gemm_mfma(ga, gb, trans_b))
+
+
+def test_fused_config4_shape(dev):
+    w, x, ga, gb = W.config4()
+    ri, v, ro, ci = to_dev(w, dev, torch.float16, torch.int16)
+    xt = torch.from_numpy(x).to(dev).half()
+    gat, gbt = torch.from_numpy(ga).to(dev).bfloat16(), torch.from_numpy(gb).to(dev).bfloat16()
+    out, c = ops.fused_spmm_gemm(xt, ri, v, ro, ci, w.m, gat, gbt, False, 1)
+    assert torch.equal(out, ops.spmm_sputnik_reuse_weight_half(xt, ri, v, ro, ci, w.m))
+    assert torch.equal(c, ops.gemm_mfma(gat, gbt, False))
+
+
+def test_argument_checks(dev):
+    a = W.config2_matrix(0.90, m=64, k=64)
+    ri, v, ro, ci = to_dev(a, dev, torch.float16)
+    x = torch.randn(1, 64, 64, device=dev).half()
+    g = torch.randn(64, 64, device=dev).half()
+    with pytest.raises(RuntimeError, match="fp16"):
+        ops.fused_spmm_gemm(x.float(), ri, v.float(), ro, ci, a.m, g, g, False, 0)
+    with pytest.raises(RuntimeError, match="one batch entry"):
+        ops.fused_spmm_gemm(x.repeat(2, 1, 1), ri, v, ro, ci, a.m, g, g, False, 0)

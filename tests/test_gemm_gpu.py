@@ -24,10 +24,33 @@ def _check(oracle, dev, M, N, K, dtype, trans_b, seed=0):
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
 @pytest.mark.parametrize("trans_b", [False, True])
-@pytest.mark.parametrize("shape", [(128, 128, 32), (256, 128, 64), (512, 384, 256), (100, 60, 72), (33, 260, 8),
-                                   (1, 4, 8), (300, 132, 1000)])
+@pytest.mark.parametrize("shape", [(128, 128, 32), (256, 128, 64), (512, 384, 256), (100, 64, 72), (33, 264, 8),
+                                   (1, 8, 8), (300, 136, 1000), (257, 520, 200)])
 def test_gemm_shapes(oracle, dev, dtype, trans_b, shape):
     _check(oracle, dev, *shape, dtype, trans_b)
+
+
+@pytest.mark.parametrize("shape", [(100, 60, 72), (33, 260, 8), (1, 4, 8), (300, 131, 1000)])
+def test_gemm_ragged_n_with_transposed_b(oracle, dev, shape):
+    """B given as (N, K) has no constraint on N (B as (K, N) needs N % 8 == 0)."""
+    _check(oracle, dev, *shape, torch.bfloat16, True)
+    with pytest.raises(RuntimeError, match="multiple of 8"):
+        ops.gemm_mfma(torch.zeros(8, 8, device=dev).half(), torch.zeros(8, shape[1] | 1, device=dev).half(), False)
+
+
+def test_large_tiles(oracle, dev):
+    """Enough 256x256 tiles to select the large-tile kernel; a corner is checked against the
+    oracle and the whole result against the transposed-B layout of the same kernel."""
+    rng = np.random.default_rng(3)
+    M, N, K = 4096, 8192, 64
+    a_np = rng.standard_normal((M, K)).astype(np.float32)
+    b_np = rng.standard_normal((K, N)).astype(np.float32)
+    a, b = torch.from_numpy(a_np).to(dev).half(), torch.from_numpy(b_np).to(dev).half()
+    out = ops.gemm_mfma(a, b, False)
+    want = oracle.gemm(rounded(a_np[-300:], torch.float16), rounded(b_np[:, -520:], torch.float16))
+    scale = oracle.gemm(np.abs(a_np[-300:]), np.abs(b_np[:, -520:]))
+    assert_close(out[-300:, -520:].float().cpu().numpy(), want, scale, 1e-2, "large tiles corner")
+    assert torch.equal(ops.gemm_mfma(a, b.t().contiguous(), True), out)
 
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])

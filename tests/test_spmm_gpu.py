@@ -67,10 +67,10 @@ def test_ragged_shapes(oracle, dev, n, dtype):
     _check(oracle, csr, b, dev, dtype, what=f"ragged n={n} {dtype}")
 
 
-@pytest.mark.parametrize("wpr", [1, 4, 16])
+@pytest.mark.parametrize("wpr", [1, 4, 8])
 @pytest.mark.parametrize("dtype", [torch.float32, torch.float16])
 def test_every_row_split_variant(oracle, dev, wpr, dtype):
-    """The three work decompositions (1, 4, 16 wavefronts per row) on one skewed matrix."""
+    """The three work decompositions (1, 4, 8 wavefronts per row) on one skewed matrix."""
     from intrasm_engine_amd.pytorch import ops as pyops
     rng = np.random.default_rng(99)
     m, k, n = 301, 2048, 192
@@ -274,3 +274,36 @@ def test_operator_argument_checks(dev):
         ops.spmm_sputnik_reuse_weight(b, ri, v[:-1], ro, ci, a.m)            # values vs column_indices
     with pytest.raises(RuntimeError, match="multiple of 4"):
         ops.spmm_sputnik_atomic(b.repeat(2, 1, 1), ri, v[:-2].repeat(2, 1), ro, ci[:-2], a.m)
+
+
+@pytest.mark.parametrize("rpw", [2, 4, 8])
+@pytest.mark.parametrize("dtype,n", [(torch.float32, 256), (torch.float32, 384), (torch.float32, 128),
+                                     (torch.float16, 512), (torch.float16, 256), (torch.bfloat16, 512)])
+def test_lds_staged_variant(oracle, dev, rpw, dtype, n):
+    """The LDS-staged kernel (forced) on a skewed matrix with empty rows, a dense row, a
+    k that is not a multiple of the stage height and an m that leaves idle row slots."""
+    from intrasm_engine_amd.pytorch import ops as pyops
+    rng = np.random.default_rng(7 * rpw + n)
+    m, k = 333, 1000
+    lens = np.clip(rng.geometric(1 / 120.0, m), 0, k)
+    lens[[0, 17, 332]] = 0
+    lens[5] = k
+    lens[6] = 1
+    ro, ci = W.csr_from_row_lengths(rng, m, k, lens)
+    csr = W.CSR(m, k, rng.standard_normal(ci.shape[0]).astype(np.float32), W.swizzle_from_offsets(ro), ro, ci)
+    b_np = rng.standard_normal((2, k, n)).astype(np.float32)
+    ri, v, ro_t, ci_t = to_dev(csr, dev, dtype)
+    b = torch.from_numpy(b_np).to(dev).to(dtype)
+    out = pyops._spmm(b, ri, v, ro_t, ci_t, m, per_batch_values=False, accumulate=False, dtypes=(dtype,),
+                      allow_i16=False, force_variant=2, force_rpw=rpw)
+    vals_r, b_r = rounded(csr.values, dtype), rounded(b_np, dtype)
+    want = oracle.spmm(b_r, csr.row_indices, vals_r, csr.row_offsets, csr.column_indices, m)
+    scale = oracle.spmm_abs_scale(b_r, csr.row_indices, vals_r, csr.row_offsets, csr.column_indices, m)
+    assert_close(out.float().cpu().numpy(), want, scale, RTOL[dtype], f"lds rpw={rpw} {dtype} n={n}")
+    # both kernel families agree on integer-valued data exactly
+    csr.values = rng.integers(-2, 3, csr.nnz).astype(np.float32)
+    bi = torch.from_numpy(rng.integers(-2, 3, (1, k, n)).astype(np.float32)).to(dev).to(dtype)
+    ri, v, ro_t, ci_t = to_dev(csr, dev, dtype)
+    kw = dict(per_batch_values=False, accumulate=False, dtypes=(dtype,), allow_i16=False)
+    assert torch.equal(pyops._spmm(bi, ri, v, ro_t, ci_t, m, force_variant=2, force_rpw=rpw, **kw),
+                       pyops._spmm(bi, ri, v, ro_t, ci_t, m, force_variant=1, **kw))

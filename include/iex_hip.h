@@ -46,6 +46,11 @@ const char* iex_last_error(void);
 /* 1 when a gfx950 device is visible to the HIP runtime, else 0. */
 int iex_device_ok(void);
 
+/* dst[0:nbytes] = src[0:nbytes] with a plain 128-bit-per-lane streaming kernel (nbytes and both
+ * pointers multiples of 16).  Measurement aid with no counterpart in the reference: hardware
+ * traffic counters are scaled by what they read for this copy of known size. */
+int iex_copy_bytes(void* dst, const void* src, size_t nbytes, void* stream);
+
 /* ------------------------------------------------------------------ SpMM ---- */
 /* flags for iex_spmm_ex */
 #define IEX_SPMM_PER_BATCH_VALUES 0x1 /* values is (batch, nnz) instead of (nnz)            */

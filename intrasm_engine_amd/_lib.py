@@ -29,6 +29,7 @@ SIGNATURES = {
     "iex_abi_version": (_i, []),
     "iex_last_error": (_c.c_char_p, []),
     "iex_device_ok": (_i, []),
+    "iex_copy_bytes": (_i, [_vp, _vp, _c.c_size_t, _vp]),
     "iex_spmm_ex": (_i, [_i, _i, _i, _i, _i, _i, _i, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i]),
     "iex_CudaSpmm2": (_i, [_i, _i, _i, _i, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i]),
     "iex_CudaSpmm3": (_i, [_i, _i, _i, _i, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i]),
@@ -69,8 +70,8 @@ _lib = None
 
 def load() -> ctypes.CDLL:
     """Load the library and bind every entry point.  Raises ImportError when the
-    shared object has not been built (``python -c 'import __graft_entry__ as g; g.build()'``
-    or ``make -C intrasm_engine_amd/csrc``)."""
+    shared object has not been built (``python -c 'import __graft_entry__ as g; g.build()'``,
+    ``python intrasm_engine_amd/csrc/build.py`` or ``make -C intrasm_engine_amd/csrc``)."""
     global _lib
     if _lib is not None:
         return _lib

@@ -1,4 +1,5 @@
-"""Compile ``libiex_hip.so`` for gfx950.  ``python -m intrasm_engine_amd.csrc.build``."""
+"""Compile ``libiex_hip.so`` for gfx950:  ``python intrasm_engine_amd/csrc/build.py``
+(run it as a script: importing the package needs the library to exist already)."""
 import os
 import subprocess
 import sys

@@ -26,7 +26,26 @@ int check_hip(hipError_t err, const char* what) {
 
 }  // namespace iex
 
+namespace {
+// Plain streaming copy, 128 bits per lane per step, grid-stride.
+__global__ __launch_bounds__(256) void copy_kernel(uint4* __restrict__ dst, const uint4* __restrict__ src, size_t n16) {
+  for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < n16; i += (size_t)gridDim.x * 256) dst[i] = src[i];
+}
+}  // namespace
+
 extern "C" {
+
+int iex_copy_bytes(void* dst, const void* src, size_t nbytes, void* stream) {
+  IEX_REQUIRE(dst && src, IEX_ERR_BAD_ARGUMENT, "copy: null pointer argument");
+  IEX_REQUIRE(nbytes % 16 == 0 && iex::aligned(dst, 16) && iex::aligned(src, 16), IEX_ERR_UNSUPPORTED,
+              "copy: size and pointers must be multiples of 16 bytes");
+  if (nbytes == 0) return 0;
+  const size_t n16 = nbytes / 16;
+  const int blocks = (int)((n16 + 255) / 256 < 256 * 64 ? (n16 + 255) / 256 : 256 * 64);
+  hipLaunchKernelGGL(copy_kernel, dim3(blocks), dim3(256), 0, static_cast<hipStream_t>(stream), static_cast<uint4*>(dst),
+                     static_cast<const uint4*>(src), n16);
+  return iex::check_hip(hipGetLastError(), "copy launch");
+}
 
 int iex_abi_version(void) { return IEX_ABI_VERSION; }
 

@@ -24,6 +24,9 @@ struct FusedParams {
 };
 
 constexpr int kFusedWM = 2, kFusedWN = 2;
+// The GEMM role's registers and LDS leave two waves per SIMD; the SpMM role makes up for the
+// missing waves by keeping four times as many gathers in flight per wave.
+constexpr int kFusedWin = 32;
 
 template <bool BF16, bool TRANS_B, typename IT, int VEC, int LPG, int WPR>
 __global__ __launch_bounds__(256) void fused_kernel(FusedParams p) {
@@ -32,11 +35,17 @@ __global__ __launch_bounds__(256) void fused_kernel(FusedParams p) {
   const long long total = (long long)p.gemm_blocks + p.spmm_blocks;
   bool is_gemm;
   int idx;
-  if (p.interleave) {
-    const int before = (int)(((long long)b * p.gemm_blocks) / total);
-    const int after = (int)(((long long)(b + 1) * p.gemm_blocks) / total);
-    is_gemm = after > before;
-    idx = is_gemm ? before : b - before;
+  if (p.interleave > 0) {
+    // GEMM tiles in groups of `interleave` consecutive ids; group q starts at id q*total/groups
+    const int gsz = p.interleave;
+    const long long groups = (p.gemm_blocks + gsz - 1) / gsz;
+    long long q = ((long long)b * groups) / total;
+    if ((q + 1) * total / groups <= b) ++q;
+    const long long start = q * total / groups;
+    const int in_group = min(gsz, p.gemm_blocks - (int)q * gsz);
+    const int off = b - (int)start;
+    is_gemm = off < in_group;
+    idx = is_gemm ? (int)q * gsz + off : b - ((int)q * gsz + in_group);
   } else {
     is_gemm = b < p.gemm_blocks;
     idx = is_gemm ? b : b - p.gemm_blocks;
@@ -44,7 +53,7 @@ __global__ __launch_bounds__(256) void fused_kernel(FusedParams p) {
   if (is_gemm) {
     gemm_tile<BF16, TRANS_B, kFusedWM, kFusedWN>(p.g, idx / p.g.tiles_n, idx % p.g.tiles_n, 0, smem);
   } else {
-    spmm_block<__half, IT, VEC, LPG, WPR>(p.s, idx / p.spmm_by, idx % p.spmm_by, 0, reinterpret_cast<float*>(smem));
+    spmm_block<__half, IT, VEC, LPG, WPR, kFusedWin>(p.s, idx / p.spmm_by, idx % p.spmm_by, 0, reinterpret_cast<float*>(smem));
   }
 }
 

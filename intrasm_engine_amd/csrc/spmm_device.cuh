@@ -50,7 +50,8 @@ __device__ __forceinline__ void fma_vec(float (&acc)[VEC], float a, const vec_t<
 //   (ceil(m / rows_per_block), ceil(n / (LPG*VEC)), batch).
 // `red` must hold spmm_lds_floats<VEC,WPR>() floats.  Every thread of the workgroup
 // must call this when WPR > 1 (it contains a barrier).
-template <typename T, typename IT, int VEC, int LPG, int WPR>
+// WIN = gathers a wave keeps in flight (rolling window); raise it where few waves fit a CU.
+template <typename T, typename IT, int VEC, int LPG, int WPR, int WIN = kSpmmUnroll>
 __device__ __forceinline__ void spmm_block(const SpmmParams& p, int bx, int by, int bz, float* red) {
   constexpr int kWavesPerBlock = (WPR > 4) ? WPR : 4;
   constexpr int kRowsPerBlock = kWavesPerBlock / WPR;
@@ -102,30 +103,30 @@ __device__ __forceinline__ void spmm_block(const SpmmParams& p, int bx, int by, 
       if constexpr (G == 1) {
         auto gather = [&](int t) { return load_vec<T, VEC>(dense + (size_t)bcast_i(c, t) * p.n); };
         if (cnt == kWave) {
-          // full chunk: rolling window of kSpmmUnroll gathers in flight, refilled after every FMA
-          vec_t<T, VEC> bv[kSpmmUnroll];
+          // full chunk: rolling window of WIN gathers in flight, refilled after every FMA
+          vec_t<T, VEC> bv[WIN];
 #pragma unroll
-          for (int u = 0; u < kSpmmUnroll; ++u) bv[u] = gather(u);
+          for (int u = 0; u < WIN; ++u) bv[u] = gather(u);
 #pragma unroll
           for (int t = 0; t < kWave; ++t) {
-            fma_vec<T, VEC>(acc, bcast_f(v, t), bv[t % kSpmmUnroll]);
-            if (t + kSpmmUnroll < kWave) bv[t % kSpmmUnroll] = gather(t + kSpmmUnroll);
+            fma_vec<T, VEC>(acc, bcast_f(v, t), bv[t % WIN]);
+            if (t + WIN < kWave) bv[t % WIN] = gather(t + WIN);
           }
         } else {
           int t = 0;
-          for (; t + kSpmmUnroll <= cnt; t += kSpmmUnroll) {
-            vec_t<T, VEC> bv[kSpmmUnroll];
+          for (; t + WIN <= cnt; t += WIN) {
+            vec_t<T, VEC> bv[WIN];
 #pragma unroll
-            for (int u = 0; u < kSpmmUnroll; ++u) bv[u] = gather(t + u);
+            for (int u = 0; u < WIN; ++u) bv[u] = gather(t + u);
 #pragma unroll
-            for (int u = 0; u < kSpmmUnroll; ++u) fma_vec<T, VEC>(acc, bcast_f(v, t + u), bv[u]);
+            for (int u = 0; u < WIN; ++u) fma_vec<T, VEC>(acc, bcast_f(v, t + u), bv[u]);
           }
           for (; t < cnt; ++t) fma_vec<T, VEC>(acc, bcast_f(v, t), gather(t));
         }
       } else {
         // step s: group g works on nonzero s*G + g of this chunk
         constexpr int kSteps = kWave / G;
-        constexpr int kWin = kSteps < kSpmmUnroll ? kSteps : kSpmmUnroll;
+        constexpr int kWin = kSteps < WIN ? kSteps : WIN;
         auto fetch = [&](int s, float& vs) {
           const int src = ((s * G + grp) & (kWave - 1)) << 2;
           vs = __int_as_float(__builtin_amdgcn_ds_bpermute(src, __float_as_int(v)));

@@ -33,6 +33,15 @@ HBM_PEAK_GBPS = 8000.0           # MI355X HBM3E
 MFMA_PEAK_TFLOPS_16BIT = 2500.0  # dense bf16 / fp16
 VALU_PEAK_TFLOPS_FP32 = 78.6     # vector fp32 FMA without packed math (the build disables v_pk_*_f32)
 CELL_REPEATS = 20                # launches of one cell inside its timing graph
+# HBM-side bytes per launch (L2 misses + write-backs), mean over the five sparsities a kernel serves in
+# the sweep, from two `rocprofv3 --pmc` runs (FETCH_SIZE, WRITE_SIZE) of `bench.py --pmc-probe`, each
+# scaled by the counter's reading for a plain 256 MiB copy (x2.000 and x1.000): see
+# profiles/spmm_fp32_config2_hbm_traffic_pmc.txt.  Counters cannot be read inside a timing run.
+MEASURED_TRAFFIC_BYTES = {
+    "spmm_kernel<float, int, 4, 64, 4>": 100.7e6,   # n = 256
+    "spmm_kernel<float, int, 4, 32, 4>": 38.6e6,    # n = 128
+    "spmm_kernel<float, int, 4, 16, 4>": 28.9e6,    # n = 64
+}
 
 
 def log(*a):
@@ -97,13 +106,13 @@ def main():
             _lib.check(_lib.load().iex_copy_bytes(dst.data_ptr(), src.data_ptr(), nbytes,
                                                   torch.cuda.current_stream().cuda_stream), "copy")
         torch.cuda.synchronize()
-        for s_, n_ in ((0.7, 256), (0.8, 256)):
+        for s_, n_ in cells:       # dispatch order = cell order, 3 launches each
             fn = spmm32(s_, n_)
             for _ in range(3):
                 fn()
             torch.cuda.synchronize()
-        log(f"[bench] pmc probe done: copy of {nbytes} bytes x3 (copy_kernel), cells (0.7,256) and (0.8,256) x3; "
-            f"algorithmic bytes {cell_bytes(0.7, 256)} and {cell_bytes(0.8, 256)}")
+        log(f"[bench] pmc probe done: copy of {nbytes} bytes x3 (copy_kernel), then every fp32 cell x3 in the order "
+            + " ".join(f"({s_},{n_}):{cell_bytes(s_, n_)}B" for s_, n_ in cells))
         return
 
     sweep_bytes = sum(cell_bytes(s, n) for s, n in cells)
@@ -172,12 +181,16 @@ def main():
     dom_bytes = statistics.mean(r["bytes"] for r in dom_rows)
     dom_us = statistics.mean(r["us"] for r in dom_rows)
     roofline = {"bound": "hbm", "achieved": round(dom_bytes / dom_us / 1e3, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
-                "frac": round(dom_bytes / dom_us / 1e3 / HBM_PEAK_GBPS, 4), "traffic": None,
+                "frac": round(dom_bytes / dom_us / 1e3 / HBM_PEAK_GBPS, 4),
+                "traffic": MEASURED_TRAFFIC_BYTES.get(dom_name),
                 "kernel": dom_name, "avg_launch_us": round(dom_us, 2),
                 "algorithmic_bytes_per_launch": int(dom_bytes),
                 "cells": [[r["sparsity"], r["n"]] for r in dom_rows],
-                "note": "gathers of B rows are served by L1/L2, not HBM: the kernel's real ceiling is the "
-                        "vector-memory pipeline (nnz*n*4 B of gathers), see extras.cells[*].valu_frac"}
+                "gather_bytes_per_launch": int(statistics.mean(r["nnz"] * r["n"] * 4 for r in dom_rows)),
+                "gather_TBps": round(statistics.mean(r["nnz"] * r["n"] * 4 for r in dom_rows) / dom_us / 1e6, 2),
+                "note": "every nonzero gathers n*4 bytes of the dense operand from L2 (gather_bytes_per_launch); the "
+                        "kernel is bound by that L2->CU bandwidth (gather_TBps), not by HBM, so frac stays small; "
+                        "traffic = HBM-side bytes per launch from rocprofv3 --pmc FETCH_SIZE + WRITE_SIZE"}
 
     result = {
         "metric": "SpMM/SDDMM GB/s and % HBM peak; co-run makespan vs serialized (%) on 1 GPU",

@@ -313,12 +313,14 @@ def run_extras(torch, ops, dev, W, IL, mats, dens, csr_dev, time_cell, variant_o
     reps = 4
     spmm_execs = [lambda: ops.spmm_sputnik_reuse_weight_half(xt, riw, vw, row, ciw, w.m)] * reps
     gemm_execs = [lambda: ops.gemm_mfma(gat, gbt, False)] * reps
-    fused_execs = [lambda: ops.fused_spmm_gemm(xt, riw, vw, row, ciw, w.m, gat, gbt, False, 1)] * reps
+    fused_execs = [lambda: ops.fused_spmm_gemm(xt, riw, vw, row, ciw, w.m, gat, gbt, False, 0)] * reps
+    fused_g_execs = [lambda: ops.fused_spmm_gemm(xt, riw, vw, row, ciw, w.m, gat, gbt, False, 64)] * reps
     t_spmm = IL.run_non_interleaving(spmm_execs) / reps
     t_gemm = IL.run_non_interleaving(gemm_execs) / reps
     t_serial = IL.run_non_interleaving(spmm_execs, gemm_execs) / reps
     t_graph = IL.run_interleaving(spmm_execs, gemm_execs) / reps
     t_fused = IL.run_non_interleaving(fused_execs) / reps
+    t_fused_g = IL.run_non_interleaving(fused_g_execs) / reps
     fl_s, fl_g = W.spmm_flops(w.nnz, 2048), W.gemm_flops(4096, 2048, 4096)
     by_s = W.spmm_bytes(w.m, w.k, 2048, w.nnz, 1, 2, 2)
     out["config4"] = {
@@ -329,11 +331,45 @@ def run_extras(torch, ops, dev, W, IL, mats, dens, csr_dev, time_cell, variant_o
         "gemm_mfma_frac": round(IL.gemm_tflops(4096, 2048, 4096, t_gemm) / MFMA_PEAK_TFLOPS_16BIT, 4),
         "serialized_sum_ms": round(t_spmm + t_gemm, 4), "serialized_one_stream_ms": round(t_serial, 4),
         "two_branch_graph_ms": round(t_graph, 4), "fused_launch_ms": round(t_fused, 4),
+        "fused_launch_gemm_in_groups_of_64_ms": round(t_fused_g, 4),
         "graph_makespan_pct_of_serialized": round(100 * t_graph / (t_spmm + t_gemm), 1),
         "fused_makespan_pct_of_serialized": round(100 * t_fused / (t_spmm + t_gemm), 1),
         "repeats_per_graph": reps,
     }
     log(f"[bench] config 4: spmm {t_spmm:.3f} ms, gemm {t_gemm:.3f} ms, graph {t_graph:.3f} ms, fused {t_fused:.3f} ms")
+    del w, x, ga, gb, riw, vw, row, ciw, xt, gat, gbt, spmm_execs, gemm_execs, fused_execs, fused_g_execs
+
+    # ---- config 5: LLaMA-7B-shaped sparse decoder layer, 16 sequences x 512 tokens, three variants
+    from intrasm_engine_amd.decoder_layer import SparseDecoderLayer
+    hidden, heads, mlp, seqs, L = 4096, 32, 11008, 16, 512
+    weights = W.config5_weights()
+    layer = SparseDecoderLayer(weights, hidden, heads, mlp, dev)
+    x5 = torch.from_numpy(W.config5_activation(hidden=hidden, tokens=seqs * L)[0]).to(dev).half()
+    half = seqs * L // 2
+    xa, xb = x5[:, :half].contiguous(), x5[:, half:].contiguous()
+
+    def time_capture(make, samples=3):
+        constructor, keep = make()
+        ms = statistics.median(IL._time_graph(constructor, samples, 1))
+        del keep
+        return ms
+
+    t_ser = time_capture(lambda: layer.capture_serialized(x5, seqs))
+    t_ser_halves = time_capture(lambda: IL.capture_serialized([lambda: (layer.forward(xa, seqs // 2), layer.forward(xb, seqs // 2))]))
+    t_ms = time_capture(lambda: layer.capture_multistream(xa, xb, seqs // 2))
+    t_fu = time_capture(lambda: layer.capture_fused(xa, xb, seqs // 2, 0))
+    spmm_flops5 = sum(2 * weights[n_].nnz * seqs * L for n_ in weights)
+    attn_flops5 = 2 * 2 * seqs * heads * L * L * (hidden // heads)
+    out["config5"] = {
+        "shape": "hidden 4096, 32 heads, MLP 11008, 16 x 512 tokens, fp16; q/k/v/o 2:4, gate/up/down 80% unstructured",
+        "elementwise_ops_included": "softmax(QK^T/sqrt(d)), SiLU(gate)*up, two residual adds (PyTorch kernels); no RoPE / norm / mask",
+        "serialized_ms": round(t_ser, 3), "serialized_two_halves_ms": round(t_ser_halves, 3),
+        "multistream_graph_ms": round(t_ms, 3), "fused_ms": round(t_fu, 3),
+        "multistream_pct_of_serialized": round(100 * t_ms / t_ser, 1), "fused_pct_of_serialized": round(100 * t_fu / t_ser, 1),
+        "spmm_GFLOP": round(spmm_flops5 / 1e9, 1), "attention_GFLOP": round(attn_flops5 / 1e9, 1),
+        "layer_TFLOPs_serialized": round((spmm_flops5 + attn_flops5) / t_ser / 1e9, 1),
+    }
+    log(f"[bench] config 5: serialized {t_ser:.2f} ms, two-stream graph {t_ms:.2f} ms, fused {t_fu:.2f} ms")
     return out
 
 

@@ -62,6 +62,10 @@ int iex_copy_bytes(void* dst, const void* src, size_t nbytes, void* stream);
  * bits 20..23: rows per wavefront of the LDS-staged kernel (2, 4 or 8).  0 = choose.      */
 #define IEX_SPMM_FORCE_VARIANT(v) (((v) & 0xf) << 16)
 #define IEX_SPMM_FORCE_RPW(r) (((r) & 0xf) << 20)
+/* bits 24..27: adjacent 64-lane column tiles per wavefront of the row kernel (1 or 2).    */
+#define IEX_SPMM_FORCE_NT(t) (((t) & 0xf) << 24)
+/* bits 28..30: lanes per nonzero of the row kernel, coded 1..4 = 8, 16, 32, 64 lanes.      */
+#define IEX_SPMM_FORCE_LPG_CODE(c) (((c) & 0x7) << 28)
 
 /* out[z, r, :] = sum_j values[(z,) j] * dense[z, column_indices[j], :]  (+ bias[r], ReLU)
  * dense is (batch, k, n), out is (batch, m, n), both of `dtype`; accumulation is fp32.
@@ -131,16 +135,18 @@ int iex_gemm(int dtype, int trans_b, int M, int N, int K, const void* A, const v
              long long stride_c, void* stream);
 
 /* ----------------------------------------------- horizontally fused launch ---- */
-/* One launch whose first `gemm_workgroups` workgroups compute tiles of the dense GEMM
- * C = A*B (as iex_gemm, batch 1) while the remaining workgroups run the fp16 CSR SpMM
- * (as iex_spmm_ex with dtype IEX_F16, batch 1, no flags).  Both results are identical
- * to the separate launches.  No counterpart in the reference (the name survives only as
- * the unused HORIZONTAL_GRAINED flag, tests/test_interleaving.py:441). */
+/* One launch whose workgroups are split between tiles of the dense GEMM C[z] = A[z]*B[z]
+ * (as iex_gemm: gemm_batch entries, element strides stride_*) and row blocks of the fp16 CSR
+ * SpMM (as iex_spmm_ex with dtype IEX_F16, batch 1, no flags).  interleave == 0: the GEMM
+ * workgroups come first; interleave == g > 0: they are spread through the grid in groups of
+ * g.  Both results are identical to the separate launches.  No counterpart in the reference
+ * (the name survives only as the unused HORIZONTAL_GRAINED flag, tests/test_interleaving.py:441). */
 int iex_fused_spmm_gemm(int spmm_itype, int m, int k, int n, int nonzeros,
                         const int* row_indices, const void* values, const int* row_offsets,
                         const void* column_indices, const void* dense, void* spmm_out,
                         int gemm_dtype, int trans_b, int M, int N, int K, const void* A,
-                        const void* B, void* C, int interleave, void* stream);
+                        const void* B, void* C, int gemm_batch, long long stride_a,
+                        long long stride_b, long long stride_c, int interleave, void* stream);
 
 /* ------------------------------------------------------------ graph builder ---- */
 /* Opaque builder of ONE hipGraph from per-stream captures; mirrors

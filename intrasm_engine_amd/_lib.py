@@ -39,7 +39,7 @@ SIGNATURES = {
     "iex_csr_softmax": (_i, [_i, _i, _i, _vp, _vp, _vp, _f, _vp, _i]),
     "iex_gemm": (_i, [_i, _i, _i, _i, _i, _vp, _vp, _vp, _i, _ll, _ll, _ll, _vp]),
     "iex_fused_spmm_gemm": (_i, [_i, _i, _i, _i, _i, _vp, _vp, _vp, _vp, _vp, _vp,
-                                 _i, _i, _i, _i, _i, _vp, _vp, _vp, _i, _vp]),
+                                 _i, _i, _i, _i, _i, _vp, _vp, _vp, _i, _ll, _ll, _ll, _i, _vp]),
     "iex_graph_create": (_vp, []),
     "iex_graph_wrap": (_vp, [_vp]),
     "iex_graph_destroy": (None, [_vp]),

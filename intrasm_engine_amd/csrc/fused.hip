@@ -5,9 +5,11 @@
 //
 // Workgroup roles
 //   interleave == 0 : ids [0, G) run GEMM tiles, ids [G, G+S) run SpMM blocks;
-//   interleave != 0 : the G GEMM workgroups are spread evenly through the id range
-//                     (id b is a GEMM workgroup iff floor((b+1)*G/T) > floor(b*G/T)),
-//                     so both kinds are dispatched side by side from start to end.
+//   interleave == g : the G GEMM workgroups are spread through the id range in groups of g
+//                     consecutive ids (group q starts at id q*T/ceil(G/g)), so both kinds are
+//                     dispatched side by side from start to end while the tiles of a group
+//                     still share their operand panels in L2.
+// The GEMM may be batched (tiles of all batch entries are enumerated).
 // Every workgroup has 256 threads and the LDS of the larger role (the GEMM's 40 KB).
 // The device code of both roles is the code of the stand-alone kernels, so results are
 // bit-identical to separate launches (the SpMM with at most 4 wavefronts per row).
@@ -20,7 +22,7 @@ namespace {
 struct FusedParams {
   GemmParams g;
   SpmmParams s;
-  int gemm_blocks, spmm_blocks, spmm_by, interleave;
+  int gemm_batch, gemm_blocks, spmm_blocks, spmm_by, interleave;
 };
 
 constexpr int kFusedWM = 2, kFusedWN = 2;
@@ -51,7 +53,9 @@ __global__ __launch_bounds__(256) void fused_kernel(FusedParams p) {
     idx = is_gemm ? b : b - p.gemm_blocks;
   }
   if (is_gemm) {
-    gemm_tile<BF16, TRANS_B, kFusedWM, kFusedWN>(p.g, idx / p.g.tiles_n, idx % p.g.tiles_n, 0, smem);
+    const int per_batch = p.g.tiles_m * p.g.tiles_n;
+    const int z = idx / per_batch, t = idx % per_batch;
+    gemm_tile<BF16, TRANS_B, kFusedWM, kFusedWN>(p.g, t / p.g.tiles_n, t % p.g.tiles_n, z, smem);
   } else {
     spmm_block<__half, IT, VEC, LPG, WPR, kFusedWin>(p.s, idx / p.spmm_by, idx % p.spmm_by, 0, reinterpret_cast<float*>(smem));
   }
@@ -62,7 +66,8 @@ int launch(FusedParams p, hipStream_t stream) {
   constexpr int BM = 2 * kFusedWM * 32, BN = 2 * kFusedWN * 32;
   p.g.tiles_m = ceil_div(p.g.M, BM);
   p.g.tiles_n = ceil_div(p.g.N, BN);
-  p.gemm_blocks = p.g.tiles_m * p.g.tiles_n;
+  IEX_REQUIRE((long long)p.g.tiles_m * p.g.tiles_n * p.gemm_batch < (1ll << 30), IEX_ERR_TOO_LARGE, "fused: too many GEMM tiles");
+  p.gemm_blocks = p.g.tiles_m * p.g.tiles_n * p.gemm_batch;
   const int rows_per_block = 4 / WPR;
   p.spmm_by = ceil_div(p.s.n, LPG * VEC);
   const long long sb = (long long)ceil_div(p.s.m, rows_per_block) * p.spmm_by;
@@ -115,10 +120,12 @@ int launch_gemm_kind(const FusedParams& p, SpmmShape vec, bool bf16, bool trans_
 extern "C" int iex_fused_spmm_gemm(int spmm_itype, int m, int k, int n, int nonzeros, const int* row_indices,
                                    const void* values, const int* row_offsets, const void* column_indices,
                                    const void* dense, void* spmm_out, int gemm_dtype, int trans_b, int M, int N, int K,
-                                   const void* A, const void* B, void* C, int interleave, void* stream) {
+                                   const void* A, const void* B, void* C, int gemm_batch, long long stride_a,
+                                   long long stride_b, long long stride_c, int interleave, void* stream) {
   using namespace iex;
   IEX_REQUIRE(m > 0 && k > 0 && n > 0 && nonzeros >= 0, IEX_ERR_BAD_ARGUMENT, "fused: SpMM dimensions must be positive");
-  IEX_REQUIRE(M > 0 && N > 0 && K > 0, IEX_ERR_BAD_ARGUMENT, "fused: GEMM dimensions must be positive");
+  IEX_REQUIRE(M > 0 && N > 0 && K > 0 && gemm_batch > 0, IEX_ERR_BAD_ARGUMENT, "fused: GEMM dimensions must be positive");
+  IEX_REQUIRE(stride_a % 8 == 0 && stride_b % 8 == 0, IEX_ERR_UNSUPPORTED, "fused: GEMM batch strides must be multiples of 8");
   IEX_REQUIRE(row_indices && row_offsets && dense && spmm_out && A && B && C, IEX_ERR_BAD_ARGUMENT,
               "fused: null pointer argument");
   IEX_REQUIRE(nonzeros == 0 || (values && column_indices), IEX_ERR_BAD_ARGUMENT, "fused: null values / column_indices");
@@ -132,7 +139,8 @@ extern "C" int iex_fused_spmm_gemm(int spmm_itype, int m, int k, int n, int nonz
                   (long long)N * K < (1ll << 31) && (long long)M * N < (1ll << 31),
               IEX_ERR_TOO_LARGE, "fused: an operand exceeds 2^31 elements");
   FusedParams p{};
-  p.g = GemmParams{M, N, K, A, B, C, 0, 0, 0, 0, 0};
+  p.g = GemmParams{M, N, K, A, B, C, stride_a, stride_b, stride_c, 0, 0};
+  p.gemm_batch = gemm_batch;
   p.s = SpmmParams{m, k, n, nonzeros, row_indices, values, row_offsets, column_indices, dense, nullptr, spmm_out, 0, 0, 0};
   p.interleave = interleave;
   const SpmmShape vec = spmm_pick_shape<__half>(n, dense, spmm_out);

@@ -5,24 +5,28 @@
 namespace iex {
 namespace {
 
-template <typename T, typename IT, int VEC, int LPG, int WPR>
+template <typename T, typename IT, int VEC, int LPG, int WPR, int NT>
 __global__ __launch_bounds__((WPR > 4 ? WPR : 4) * 64) void spmm_kernel(SpmmParams p) {
-  __shared__ float red[spmm_lds_floats<VEC, WPR>()];
-  spmm_block<T, IT, VEC, LPG, WPR>(p, blockIdx.x, blockIdx.y, blockIdx.z, red);
+  __shared__ float red[spmm_lds_floats<VEC, WPR, NT>()];
+  spmm_block<T, IT, VEC, LPG, WPR, (NT > 1 ? kSpmmUnroll / 2 : kSpmmUnroll), NT>(p, blockIdx.x, blockIdx.y, blockIdx.z, red);
 }
 
-template <typename T, typename IT, int VEC, int LPG, int WPR>
+template <typename T, typename IT, int VEC, int LPG, int WPR, int NT = 1>
 int launch_one(const SpmmParams& p, int batch, hipStream_t stream) {
   constexpr int kWavesPerBlock = (WPR > 4) ? WPR : 4;
   constexpr int kRowsPerBlock = kWavesPerBlock / WPR;
-  dim3 grid(ceil_div(p.m, kRowsPerBlock), ceil_div(p.n, LPG * VEC), batch);
+  dim3 grid(ceil_div(p.m, kRowsPerBlock), ceil_div(p.n, NT * LPG * VEC), batch);
   dim3 block(kWavesPerBlock * kWave);
-  hipLaunchKernelGGL((spmm_kernel<T, IT, VEC, LPG, WPR>), grid, block, 0, stream, p);
+  hipLaunchKernelGGL((spmm_kernel<T, IT, VEC, LPG, WPR, NT>), grid, block, 0, stream, p);
   return check_hip(hipGetLastError(), "spmm launch");
 }
 
 template <typename T, typename IT, int VEC, int LPG>
-int launch_wpr(const SpmmParams& p, int batch, int wpr, hipStream_t stream) {
+int launch_wpr(const SpmmParams& p, int batch, int wpr, int nt, hipStream_t stream) {
+  if constexpr (LPG == kWave && VEC * sizeof(T) == 16) {
+    // full-width tiles: a wave may cover 2 adjacent tiles (4 waves per row only)
+    if (nt == 2 && wpr == 4) return launch_one<T, IT, VEC, LPG, 4, 2>(p, batch, stream);
+  }
   switch (wpr) {
     case 1: return launch_one<T, IT, VEC, LPG, 1>(p, batch, stream);
     case 4: return launch_one<T, IT, VEC, LPG, 4>(p, batch, stream);
@@ -62,6 +66,8 @@ struct Choice {
   int wpr = 0;      // wavefronts per row of the row kernel
   int variant = 0;  // 0 = choose, 1 = row kernel, 2 = LDS-staged kernel
   int rpw = 0;      // rows per wavefront of the LDS-staged kernel (0 = choose)
+  int nt = 0;       // adjacent column tiles per wavefront of the row kernel (0 = choose)
+  int lpg = 0;      // lanes per nonzero of the row kernel: 8, 16, 32 or 64 (0 = choose)
 };
 
 // The LDS-staged kernel needs a full-width tile (64 lanes x VEC, VEC the full or half 128-bit
@@ -97,20 +103,24 @@ int launch_typed(const SpmmParams& p, int batch, const Choice& ch, hipStream_t s
     return launch_lds_rpw<T, IT, kMax / 2>(p, batch, rpw, stream);
   }
   const int wpr = ch.wpr;
-  const SpmmShape sh = spmm_pick_shape<T>(p.n, p.dense, p.out);
+  SpmmShape sh = spmm_pick_shape<T>(p.n, p.dense, p.out);
+  if (ch.lpg && sh.vec == kMax && ch.lpg <= sh.lpg) sh.lpg = ch.lpg;  // narrower tiles on request
+  // Two tiles per wave double the slice of the dense operand that the waves of an XCD share in
+  // its L2 and measured slower (2x at k = 4096, n = 8192): only on request.
+  const int nt = ch.nt ? ch.nt : 1;
   if (sh.vec == kMax) {
     switch (sh.lpg) {
-      case 8: return launch_wpr<T, IT, kMax, 8>(p, batch, wpr, stream);
-      case 16: return launch_wpr<T, IT, kMax, 16>(p, batch, wpr, stream);
-      case 32: return launch_wpr<T, IT, kMax, 32>(p, batch, wpr, stream);
-      default: return launch_wpr<T, IT, kMax, 64>(p, batch, wpr, stream);
+      case 8: return launch_wpr<T, IT, kMax, 8>(p, batch, wpr, nt, stream);
+      case 16: return launch_wpr<T, IT, kMax, 16>(p, batch, wpr, nt, stream);
+      case 32: return launch_wpr<T, IT, kMax, 32>(p, batch, wpr, nt, stream);
+      default: return launch_wpr<T, IT, kMax, 64>(p, batch, wpr, nt, stream);
     }
   }
   if constexpr (kMax == 8) {
-    if (sh.vec == 4) return launch_wpr<T, IT, 4, 64>(p, batch, wpr, stream);
+    if (sh.vec == 4) return launch_wpr<T, IT, 4, 64>(p, batch, wpr, nt, stream);
   }
-  if (sh.vec == 2) return launch_wpr<T, IT, 2, 64>(p, batch, wpr, stream);
-  return launch_wpr<T, IT, 1, 64>(p, batch, wpr, stream);
+  if (sh.vec == 2) return launch_wpr<T, IT, 2, 64>(p, batch, wpr, nt, stream);
+  return launch_wpr<T, IT, 1, 64>(p, batch, wpr, nt, stream);
 }
 
 }  // namespace
@@ -136,6 +146,8 @@ int spmm_dispatch(int dtype, int itype, int flags, int m, int k, int n, int nonz
   if (ch.wpr == 0) ch.wpr = spmm_pick_wpr(m, nonzeros);
   ch.variant = (flags >> 16) & 0xf;
   ch.rpw = (flags >> 20) & 0xf;
+  ch.nt = (flags >> 24) & 0xf;
+  ch.lpg = ((flags >> 28) & 0x7) ? (4 << ((flags >> 28) & 0x7)) : 0;
   SpmmParams p{m, k, n, nonzeros, row_indices, values, row_offsets, column_indices, dense, bias, out,
                (flags & IEX_SPMM_PER_BATCH_VALUES) != 0, (flags & IEX_SPMM_ACCUMULATE) != 0,
                (flags & IEX_SPMM_RELU) != 0};

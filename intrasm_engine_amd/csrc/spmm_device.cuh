@@ -37,8 +37,8 @@ struct SpmmParams {
 
 constexpr int kSpmmUnroll = 8;
 
-template <int VEC, int WPR>
-constexpr int spmm_lds_floats() { return (WPR > 1) ? WPR * kWave * VEC : 1; }
+template <int VEC, int WPR, int NT = 1>
+constexpr int spmm_lds_floats() { return (WPR > 1) ? WPR * kWave * VEC * NT : 1; }
 
 template <typename T, int VEC>
 __device__ __forceinline__ void fma_vec(float (&acc)[VEC], float a, const vec_t<T, VEC>& b) {
@@ -46,16 +46,28 @@ __device__ __forceinline__ void fma_vec(float (&acc)[VEC], float a, const vec_t<
   for (int i = 0; i < VEC; ++i) acc[i] = fmaf(a, elem<T>::to_float(b.v[i]), acc[i]);
 }
 
+// NT adjacent column tiles of one dense row (NT * LPG*VEC contiguous elements).
+template <typename T, int VEC, int NT>
+struct row_slab {
+  vec_t<T, VEC> t[NT];
+};
+
 // One workgroup's share: block (bx, by, bz) of the grid
-//   (ceil(m / rows_per_block), ceil(n / (LPG*VEC)), batch).
-// `red` must hold spmm_lds_floats<VEC,WPR>() floats.  Every thread of the workgroup
+//   (ceil(m / rows_per_block), ceil(n / (NT*LPG*VEC)), batch).
+// `red` must hold spmm_lds_floats<VEC,WPR,NT>() floats.  Every thread of the workgroup
 // must call this when WPR > 1 (it contains a barrier).
 // WIN = gathers a wave keeps in flight (rolling window); raise it where few waves fit a CU.
-template <typename T, typename IT, int VEC, int LPG, int WPR, int WIN = kSpmmUnroll>
+// NT  = adjacent 64*VEC-column tiles a wave covers (G == 1 only): per nonzero the wave then
+//       reads NT*64*VEC contiguous elements of one dense row, which amortises the broadcast
+//       of (column, value) and keeps very wide dense operands on fewer pages.
+template <typename T, typename IT, int VEC, int LPG, int WPR, int WIN = kSpmmUnroll, int NT = 1>
 __device__ __forceinline__ void spmm_block(const SpmmParams& p, int bx, int by, int bz, float* red) {
   constexpr int kWavesPerBlock = (WPR > 4) ? WPR : 4;
   constexpr int kRowsPerBlock = kWavesPerBlock / WPR;
   constexpr int G = kWave / LPG;
+  constexpr int TW = LPG * VEC;  // columns of one tile
+  static_assert(NT == 1 || G == 1, "several tiles per wave need the whole wave on one nonzero");
+  typedef row_slab<T, VEC, NT> Slab;
   const int lane = lane_id();
   const int wave = uniform(threadIdx.x >> 6);
   const int z = bz;
@@ -63,13 +75,16 @@ __device__ __forceinline__ void spmm_block(const SpmmParams& p, int bx, int by, 
   const int part = wave % WPR;  // which share of the row this wave sums
   const int grp = lane / LPG;   // which nonzero of a step this lane works on (0 when G == 1)
 
-  const int col0 = by * (LPG * VEC) + (lane % LPG) * VEC;
-  const bool lane_live = col0 < p.n;
-  const int col_ld = lane_live ? col0 : 0;  // idle lanes gather a valid address, result unused
-
-  float acc[VEC];
+  const int col0 = by * (NT * TW) + (lane % LPG) * VEC;  // first tile; tile t starts TW*t further
+  int col_ld[NT];                                         // idle lanes gather a valid address, result unused
 #pragma unroll
-  for (int i = 0; i < VEC; ++i) acc[i] = 0.f;
+  for (int t = 0; t < NT; ++t) col_ld[t] = (col0 + t * TW < p.n) ? col0 + t * TW : 0;
+
+  float acc[NT][VEC];
+#pragma unroll
+  for (int t = 0; t < NT; ++t)
+#pragma unroll
+    for (int i = 0; i < VEC; ++i) acc[t][i] = 0.f;
 
   const bool row_live = row_slot < p.m;  // wave-uniform
   int row = 0;
@@ -80,7 +95,19 @@ __device__ __forceinline__ void spmm_block(const SpmmParams& p, int bx, int by, 
     const T* __restrict__ values =
         static_cast<const T*>(p.values) + (p.per_batch_values ? (size_t)z * p.nnz : (size_t)0);
     const IT* __restrict__ cols = static_cast<const IT*>(p.cols);
-    const T* __restrict__ dense = static_cast<const T*>(p.dense) + (size_t)z * p.k * p.n + col_ld;
+    const T* __restrict__ dense = static_cast<const T*>(p.dense) + (size_t)z * p.k * p.n;
+
+    auto load_row = [&](int column) {
+      Slab s;
+      const T* r = dense + (size_t)column * p.n;
+#pragma unroll
+      for (int t = 0; t < NT; ++t) s.t[t] = load_vec<T, VEC>(r + col_ld[t]);
+      return s;
+    };
+    auto fma_row = [&](float a, const Slab& s) {
+#pragma unroll
+      for (int t = 0; t < NT; ++t) fma_vec<T, VEC>(acc[t], a, s.t[t]);
+    };
 
     // (value, column) of nonzero base+lane; the next chunk is fetched while the current
     // one is being processed, so its latency hides behind the gathers.
@@ -101,27 +128,27 @@ __device__ __forceinline__ void spmm_block(const SpmmParams& p, int bx, int by, 
       }
       const int cnt = min(kWave, end - base);  // wave-uniform
       if constexpr (G == 1) {
-        auto gather = [&](int t) { return load_vec<T, VEC>(dense + (size_t)bcast_i(c, t) * p.n); };
+        auto gather = [&](int t) { return load_row(bcast_i(c, t)); };
         if (cnt == kWave) {
           // full chunk: rolling window of WIN gathers in flight, refilled after every FMA
-          vec_t<T, VEC> bv[WIN];
+          Slab bv[WIN];
 #pragma unroll
           for (int u = 0; u < WIN; ++u) bv[u] = gather(u);
 #pragma unroll
           for (int t = 0; t < kWave; ++t) {
-            fma_vec<T, VEC>(acc, bcast_f(v, t), bv[t % WIN]);
+            fma_row(bcast_f(v, t), bv[t % WIN]);
             if (t + WIN < kWave) bv[t % WIN] = gather(t + WIN);
           }
         } else {
           int t = 0;
           for (; t + WIN <= cnt; t += WIN) {
-            vec_t<T, VEC> bv[WIN];
+            Slab bv[WIN];
 #pragma unroll
             for (int u = 0; u < WIN; ++u) bv[u] = gather(t + u);
 #pragma unroll
-            for (int u = 0; u < WIN; ++u) fma_vec<T, VEC>(acc, bcast_f(v, t + u), bv[u]);
+            for (int u = 0; u < WIN; ++u) fma_row(bcast_f(v, t + u), bv[u]);
           }
-          for (; t < cnt; ++t) fma_vec<T, VEC>(acc, bcast_f(v, t), gather(t));
+          for (; t < cnt; ++t) fma_row(bcast_f(v, t), gather(t));
         }
       } else {
         // step s: group g works on nonzero s*G + g of this chunk
@@ -133,30 +160,30 @@ __device__ __forceinline__ void spmm_block(const SpmmParams& p, int bx, int by, 
           return __builtin_amdgcn_ds_bpermute(src, c);
         };
         if (cnt == kWave) {
-          vec_t<T, VEC> bv[kWin];
+          Slab bv[kWin];
           float vv[kWin];
 #pragma unroll
-          for (int u = 0; u < kWin; ++u) bv[u] = load_vec<T, VEC>(dense + (size_t)fetch(u, vv[u]) * p.n);
+          for (int u = 0; u < kWin; ++u) bv[u] = load_row(fetch(u, vv[u]));
 #pragma unroll
           for (int s = 0; s < kSteps; ++s) {
-            fma_vec<T, VEC>(acc, vv[s % kWin], bv[s % kWin]);
-            if (s + kWin < kSteps) bv[s % kWin] = load_vec<T, VEC>(dense + (size_t)fetch(s + kWin, vv[s % kWin]) * p.n);
+            fma_row(vv[s % kWin], bv[s % kWin]);
+            if (s + kWin < kSteps) bv[s % kWin] = load_row(fetch(s + kWin, vv[s % kWin]));
           }
         } else {
           const int steps = cnt / G;  // full steps: every group has a real nonzero
           int s = 0;
           for (; s + kWin <= steps; s += kWin) {
-            vec_t<T, VEC> bv[kWin];
+            Slab bv[kWin];
             float vv[kWin];
 #pragma unroll
-            for (int u = 0; u < kWin; ++u) bv[u] = load_vec<T, VEC>(dense + (size_t)fetch(s + u, vv[u]) * p.n);
+            for (int u = 0; u < kWin; ++u) bv[u] = load_row(fetch(s + u, vv[u]));
 #pragma unroll
-            for (int u = 0; u < kWin; ++u) fma_vec<T, VEC>(acc, vv[u], bv[u]);
+            for (int u = 0; u < kWin; ++u) fma_row(vv[u], bv[u]);
           }
           for (; s * G < cnt; ++s) {
             float vu;
             const int cu = fetch(s, vu);
-            if (s * G + grp < cnt) fma_vec<T, VEC>(acc, vu, load_vec<T, VEC>(dense + (size_t)cu * p.n));
+            if (s * G + grp < cnt) fma_row(vu, load_row(cu));
           }
         }
       }
@@ -171,7 +198,7 @@ __device__ __forceinline__ void spmm_block(const SpmmParams& p, int bx, int by, 
 #pragma unroll
     for (int off = LPG; off < kWave; off <<= 1) {
 #pragma unroll
-      for (int i = 0; i < VEC; ++i) acc[i] += __shfl_xor(acc[i], off, kWave);
+      for (int i = 0; i < VEC; ++i) acc[0][i] += __shfl_xor(acc[0][i], off, kWave);
     }
   }
 
@@ -180,33 +207,42 @@ __device__ __forceinline__ void spmm_block(const SpmmParams& p, int bx, int by, 
     // WPR > 1, so row_live is uniform over the block and idle blocks fall through with
     // zero partials.
 #pragma unroll
-    for (int i = 0; i < VEC; ++i) red[(wave * VEC + i) * kWave + lane] = acc[i];
+    for (int t = 0; t < NT; ++t)
+#pragma unroll
+      for (int i = 0; i < VEC; ++i) red[((wave * NT + t) * VEC + i) * kWave + lane] = acc[t][i];
     __syncthreads();
     if (part != 0) return;
 #pragma unroll
-    for (int i = 0; i < VEC; ++i) {
-      float s = acc[i];
-      for (int w = 1; w < WPR; ++w) s += red[((wave + w) * VEC + i) * kWave + lane];
-      acc[i] = s;
-    }
+    for (int t = 0; t < NT; ++t)
+#pragma unroll
+      for (int i = 0; i < VEC; ++i) {
+        float s = acc[t][i];
+        for (int w = 1; w < WPR; ++w) s += red[(((wave + w) * NT + t) * VEC + i) * kWave + lane];
+        acc[t][i] = s;
+      }
   }
 
-  if (!row_live || !lane_live || grp != 0) return;
+  if (!row_live || grp != 0) return;
   const float bias = p.bias ? p.bias[row] : 0.f;
-  T* __restrict__ out = static_cast<T*>(p.out) + ((size_t)z * p.m + row) * p.n + col0;
-  vec_t<T, VEC> o;
-  if (p.accumulate) {
-    const vec_t<T, VEC> prev = load_vec<T, VEC>(out);
 #pragma unroll
-    for (int i = 0; i < VEC; ++i) acc[i] += elem<T>::to_float(prev.v[i]);
-  }
+  for (int t = 0; t < NT; ++t) {
+    const int col = col0 + t * TW;
+    if (col >= p.n) continue;
+    T* __restrict__ out = static_cast<T*>(p.out) + ((size_t)z * p.m + row) * p.n + col;
+    vec_t<T, VEC> o;
+    if (p.accumulate) {
+      const vec_t<T, VEC> prev = load_vec<T, VEC>(out);
 #pragma unroll
-  for (int i = 0; i < VEC; ++i) {
-    float r = acc[i] + bias;
-    if (p.relu) r = fmaxf(r, 0.f);
-    o.v[i] = elem<T>::from_float(r);
+      for (int i = 0; i < VEC; ++i) acc[t][i] += elem<T>::to_float(prev.v[i]);
+    }
+#pragma unroll
+    for (int i = 0; i < VEC; ++i) {
+      float r = acc[t][i] + bias;
+      if (p.relu) r = fmaxf(r, 0.f);
+      o.v[i] = elem<T>::from_float(r);
+    }
+    store_vec<T, VEC>(out, o);
   }
-  store_vec<T, VEC>(out, o);
 }
 
 // Host-side shape choice shared by the stand-alone and the fused launcher.

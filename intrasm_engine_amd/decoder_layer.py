@@ -1,0 +1,136 @@
+"""One sparse transformer decoder layer of LLaMA-7B shape, built only from the operators of
+this package -- the workload of benchmark configuration 5.
+
+Every projection is ``W_csr @ X`` (SpMM) with activations stored feature-major
+``(features, tokens)``; attention scores and context are batched MFMA GEMMs.  Included
+element-wise steps, done by PyTorch between the launches: softmax(QK^T / sqrt(d)) over
+keys, SiLU(gate) * up, and the two residual additions.  Not included (the configuration
+names none of them): RoPE, normalisation layers, causal masking, KV cache.
+
+Three ways to run the same arithmetic, mirroring how the reference's harness compares
+"serialized" with "interleaved" (tests/test_interleaving.py:348-369, 434-476):
+
+  serialized   everything captured on one stream of a ``TorchCUDAGraphConstructor``;
+  multistream  the batch is split into two halves that are captured on two streams of one
+               graph (two branches joined at the end), so the sparse projections of one half
+               can overlap the dense attention of the other;
+  fused        the same two halves on one stream, with each dense attention GEMM of one half
+               launched together with a sparse projection of the other half through the
+               horizontally fused kernel.
+"""
+from __future__ import annotations
+
+import math
+
+import torch
+
+from . import interleaving as IL
+from .pytorch.cpp_extensions.cuda_graph_constructor import TorchCUDAGraphConstructor
+
+ops = torch.ops.iex_ops
+
+
+class SparseDecoderLayer:
+    def __init__(self, weights: dict, hidden: int, heads: int, mlp: int, device, index_dtype=torch.int16):
+        """``weights``: name -> workloads.CSR for q, k, v, o (hidden x hidden), gate, up
+        (mlp x hidden), down (hidden x mlp); values are cast to fp16."""
+        self.hidden, self.heads, self.mlp = hidden, heads, mlp
+        self.head_dim = hidden // heads
+        self.device = device
+        self.w = {}
+        for name, csr in weights.items():
+            idt = index_dtype if csr.k <= 32768 else torch.int32
+            self.w[name] = (torch.from_numpy(csr.row_indices).to(device),
+                            torch.from_numpy(csr.values).to(device).half(),
+                            torch.from_numpy(csr.row_offsets).to(device),
+                            torch.from_numpy(csr.column_indices).to(device).to(idt), csr.m)
+
+    # ---- building blocks ---------------------------------------------------------------
+    def proj(self, name: str, x: torch.Tensor) -> torch.Tensor:
+        """(k, tokens) -> (m, tokens)."""
+        ri, v, ro, ci, m = self.w[name]
+        return ops.spmm_sputnik_reuse_weight_half(x.unsqueeze(0), ri, v, ro, ci, m)[0]
+
+    def _split_heads(self, t: torch.Tensor, seqs: int) -> torch.Tensor:
+        """(hidden, seqs*L) feature-major -> (seqs*heads, L, head_dim)."""
+        L = t.shape[1] // seqs
+        return t.view(self.heads, self.head_dim, seqs, L).permute(2, 0, 3, 1).contiguous().view(
+            seqs * self.heads, L, self.head_dim)
+
+    def _merge_heads(self, o: torch.Tensor, seqs: int) -> torch.Tensor:
+        """(seqs*heads, L, head_dim) -> (hidden, seqs*L)."""
+        L = o.shape[1]
+        return o.view(seqs, self.heads, L, self.head_dim).permute(1, 3, 0, 2).contiguous().view(
+            self.hidden, seqs * L)
+
+    def _softmax(self, s: torch.Tensor) -> torch.Tensor:
+        return torch.softmax(s.float() * (1.0 / math.sqrt(self.head_dim)), dim=-1).half()
+
+    def attention(self, q, k, v, seqs: int) -> torch.Tensor:
+        Q, K, V = (self._split_heads(t, seqs) for t in (q, k, v))
+        P = self._softmax(ops.gemm_mfma(Q, K, True))      # (B, L, L)
+        return self._merge_heads(ops.gemm_mfma(P, V, False), seqs)
+
+    def mlp_block(self, h: torch.Tensor) -> torch.Tensor:
+        act = torch.nn.functional.silu(self.proj("gate", h)) * self.proj("up", h)
+        return h + self.proj("down", act)
+
+    def forward(self, x: torch.Tensor, seqs: int) -> torch.Tensor:
+        """x: (hidden, seqs*L) fp16, contiguous -> same shape."""
+        q, k, v = self.proj("q", x), self.proj("k", x), self.proj("v", x)
+        h = x + self.proj("o", self.attention(q, k, v, seqs))
+        return self.mlp_block(h)
+
+    # ---- fused schedule over two half-batches ----------------------------------------------
+    def _fused(self, name: str, x: torch.Tensor, ga: torch.Tensor, gb: torch.Tensor, trans_b: bool, group: int):
+        ri, v, ro, ci, m = self.w[name]
+        out, c = ops.fused_spmm_gemm(x.unsqueeze(0), ri, v, ro, ci, m, ga, gb, trans_b, group)
+        return out[0], c
+
+    def forward_fused(self, xa: torch.Tensor, xb: torch.Tensor, seqs_half: int, group: int = 0):
+        """Halves a and b of the batch; the dense GEMMs of one half ride along with sparse
+        projections of the other half."""
+        qa, ka, va = self.proj("q", xa), self.proj("k", xa), self.proj("v", xa)
+        Qa, Ka, Va = (self._split_heads(t, seqs_half) for t in (qa, ka, va))
+        qb, Sa = self._fused("q", xb, Qa, Ka, True, group)              # b.q  ||  a.QK^T
+        Pa = self._softmax(Sa)
+        kb, Oa = self._fused("k", xb, Pa, Va, False, group)             # b.k  ||  a.PV
+        vb = self.proj("v", xb)
+        Qb, Kb, Vb = (self._split_heads(t, seqs_half) for t in (qb, kb, vb))
+        oa, Sb = self._fused("o", self._merge_heads(Oa, seqs_half), Qb, Kb, True, group)   # a.o  ||  b.QK^T
+        ha = xa + oa
+        Pb = self._softmax(Sb)
+        ga, Ob = self._fused("gate", ha, Pb, Vb, False, group)          # a.gate  ||  b.PV
+        acta = torch.nn.functional.silu(ga) * self.proj("up", ha)
+        ya = ha + self.proj("down", acta)
+        hb = xb + self.proj("o", self._merge_heads(Ob, seqs_half))
+        return ya, self.mlp_block(hb)
+
+    # ---- the three timed variants --------------------------------------------------------
+    def capture_serialized(self, x: torch.Tensor, seqs: int):
+        return IL.capture_serialized([lambda: self.forward(x, seqs)])
+
+    def capture_multistream(self, xa: torch.Tensor, xb: torch.Tensor, seqs_half: int):
+        return IL.capture_interleaved([lambda: self.forward(xa, seqs_half)], [lambda: self.forward(xb, seqs_half)])
+
+    def capture_fused(self, xa: torch.Tensor, xb: torch.Tensor, seqs_half: int, group: int = 0):
+        return IL.capture_serialized([lambda: self.forward_fused(xa, xb, seqs_half, group)])
+
+
+def reference_forward(weights_dense: dict, x: torch.Tensor, heads: int, seqs: int) -> torch.Tensor:
+    """The same layer with dense fp32 matrices and plain PyTorch (for tests at small sizes).
+    weights_dense: name -> (m, k) fp32 tensor; x: (hidden, tokens) fp32."""
+    hidden = x.shape[0]
+    hd = hidden // heads
+    L = x.shape[1] // seqs
+
+    def split(t):
+        return t.view(heads, hd, seqs, L).permute(2, 0, 3, 1).reshape(seqs * heads, L, hd)
+
+    q, k, v = (weights_dense[n] @ x for n in ("q", "k", "v"))
+    Q, K, V = split(q), split(k), split(v)
+    P = torch.softmax((Q @ K.transpose(1, 2)) / math.sqrt(hd), dim=-1)
+    O = (P @ V).view(seqs, heads, L, hd).permute(1, 3, 0, 2).reshape(hidden, seqs * L)
+    h = x + weights_dense["o"] @ O
+    act = torch.nn.functional.silu(weights_dense["gate"] @ h) * (weights_dense["up"] @ h)
+    return h + weights_dense["down"] @ act

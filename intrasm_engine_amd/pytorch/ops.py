@@ -61,7 +61,8 @@ def _check_index_dtypes(row_indices, row_offsets, column_indices, allow_i16=Fals
 
 
 def _spmm(b, row_indices, values, row_offsets, column_indices, m, *, per_batch_values,
-          accumulate, dtypes, allow_i16, out=None, bias=None, relu=False, force_wpr=0, force_variant=0, force_rpw=0):
+          accumulate, dtypes, allow_i16, out=None, bias=None, relu=False, force_wpr=0, force_variant=0, force_rpw=0,
+          force_nt=0, force_lpg=0):
     _chk(b.dim() == 3)
     if per_batch_values:
         _chk(values.dim() == 2)
@@ -99,7 +100,8 @@ def _spmm(b, row_indices, values, row_offsets, column_indices, m, *, per_batch_v
              and bias.device == b.device, "bias must be a contiguous fp32 tensor with m entries")
     flags = (_lib.SPMM_PER_BATCH_VALUES if per_batch_values else 0) | \
             (_lib.SPMM_ACCUMULATE if accumulate else 0) | (_lib.SPMM_RELU if relu else 0) | \
-            ((int(force_wpr) & 0xff) << 8) | ((int(force_variant) & 0xf) << 16) | ((int(force_rpw) & 0xf) << 20)
+            ((int(force_wpr) & 0xff) << 8) | ((int(force_variant) & 0xf) << 16) | ((int(force_rpw) & 0xf) << 20) | \
+            ((int(force_nt) & 0xf) << 24) | ({0: 0, 8: 1, 16: 2, 32: 3, 64: 4}[int(force_lpg)] << 28)
     with torch.cuda.device(b.device):
         rc = _lib.load().iex_spmm_ex(
             _DT[b.dtype], _IT[column_indices.dtype], flags, m, k, n, nonzeros,
@@ -229,7 +231,8 @@ def gemm_mfma(a, b, trans_b=False, out=None):
 
 def fused_spmm_gemm(b, row_indices, values, row_offsets, column_indices, m, ga, gb, trans_b=False,
                     interleave=0):
-    """One launch computing ``(A_csr @ b[0], ga @ gb)``; fp16 SpMM, fp16/bf16 GEMM."""
+    """One launch computing ``(A_csr @ b[0], ga @ gb)``; fp16 SpMM, fp16/bf16 GEMM (2-D, or
+    3-D batched with equal batch sizes)."""
     _chk(b.dim() == 3 and b.size(0) == 1, "fused launch takes one batch entry")
     _chk(values.dim() == 1 and values.size(0) == column_indices.size(0))
     _check_csr_common(b, row_indices, row_offsets, column_indices, [("b", b), ("values", values)])
@@ -238,22 +241,24 @@ def fused_spmm_gemm(b, row_indices, values, row_offsets, column_indices, m, ga, 
     _chk(ga.is_cuda and gb.is_cuda and ga.device == b.device and gb.device == b.device,
          "GEMM operands must be on the device of b")
     _chk(ga.dtype in (torch.float16, torch.bfloat16) and gb.dtype == ga.dtype, "GEMM operands must be fp16 or bf16")
-    _chk(ga.dim() == 2 and gb.dim() == 2 and ga.is_contiguous() and gb.is_contiguous(),
-         "GEMM operands must be contiguous 2-D tensors")
+    _chk(ga.dim() == gb.dim() and ga.dim() in (2, 3) and ga.is_contiguous() and gb.is_contiguous(),
+         "GEMM operands must be contiguous, both 2-D or both 3-D")
     m = int(m)
     _chk(row_indices.size(0) == m and row_offsets.size(0) == m + 1, "CSR arrays do not match m")
     _, k, n = b.shape
-    M, K = ga.shape
-    N = gb.shape[0] if trans_b else gb.shape[1]
-    _chk((gb.shape[1] if trans_b else gb.shape[0]) == K, "inner dimensions of the GEMM differ")
+    M, K = ga.shape[-2], ga.shape[-1]
+    N = gb.shape[-2] if trans_b else gb.shape[-1]
+    _chk((gb.shape[-1] if trans_b else gb.shape[-2]) == K, "inner dimensions of the GEMM differ")
+    gbatch = ga.shape[0] if ga.dim() == 3 else 1
+    _chk(ga.dim() == 2 or gb.shape[0] == gbatch, "batch sizes of the GEMM operands differ")
     out = torch.empty((1, m, n), dtype=b.dtype, device=b.device)
-    c = torch.empty((M, N), dtype=ga.dtype, device=b.device)
+    c = torch.empty((gbatch, M, N) if ga.dim() == 3 else (M, N), dtype=ga.dtype, device=b.device)
     with torch.cuda.device(b.device):
         rc = _lib.load().iex_fused_spmm_gemm(
             _IT[column_indices.dtype], m, k, n, column_indices.size(0), row_indices.data_ptr(),
             values.data_ptr(), row_offsets.data_ptr(), column_indices.data_ptr(), b.data_ptr(),
             out.data_ptr(), _DT[ga.dtype], int(bool(trans_b)), M, N, K, ga.data_ptr(), gb.data_ptr(),
-            c.data_ptr(), int(interleave), _stream_ptr(b.device))
+            c.data_ptr(), gbatch, M * K, N * K, M * N, int(interleave), _stream_ptr(b.device))
     _lib.check(rc, "fused_spmm_gemm")
     return out, c
 

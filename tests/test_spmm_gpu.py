@@ -307,3 +307,30 @@ def test_lds_staged_variant(oracle, dev, rpw, dtype, n):
     kw = dict(per_batch_values=False, accumulate=False, dtypes=(dtype,), allow_i16=False)
     assert torch.equal(pyops._spmm(bi, ri, v, ro_t, ci_t, m, force_variant=2, force_rpw=rpw, **kw),
                        pyops._spmm(bi, ri, v, ro_t, ci_t, m, force_variant=1, **kw))
+
+
+@pytest.mark.parametrize("dtype,n", [(torch.float32, 1024), (torch.float32, 1280), (torch.float16, 2048),
+                                     (torch.float16, 2560), (torch.bfloat16, 2048)])
+def test_two_tiles_per_wave(oracle, dev, dtype, n):
+    """Wide outputs: a wave covers two adjacent 64-lane tiles (chosen automatically from four
+    tiles upwards); n = 1280 / 2560 leave the second tile of the last block empty."""
+    from intrasm_engine_amd.pytorch import ops as pyops
+    rng = np.random.default_rng(n)
+    m, k = 150, 600
+    lens = np.clip(rng.geometric(1 / 90.0, m), 0, k)
+    lens[[0, 149]] = 0
+    lens[3] = k
+    ro, ci = W.csr_from_row_lengths(rng, m, k, lens)
+    csr = W.CSR(m, k, rng.standard_normal(ci.shape[0]).astype(np.float32), W.swizzle_from_offsets(ro), ro, ci)
+    b_np = rng.standard_normal((1, k, n)).astype(np.float32)
+    ri, v, ro_t, ci_t = to_dev(csr, dev, dtype)
+    b = torch.from_numpy(b_np).to(dev).to(dtype)
+    kw = dict(per_batch_values=False, accumulate=False, dtypes=(dtype,), allow_i16=False)
+    out = pyops._spmm(b, ri, v, ro_t, ci_t, m, **kw)
+    vals_r, b_r = rounded(csr.values, dtype), rounded(b_np, dtype)
+    want = oracle.spmm(b_r, csr.row_indices, vals_r, csr.row_offsets, csr.column_indices, m)
+    scale = oracle.spmm_abs_scale(b_r, csr.row_indices, vals_r, csr.row_offsets, csr.column_indices, m)
+    assert_close(out.float().cpu().numpy(), want, scale, RTOL[dtype], f"nt auto {dtype} n={n}")
+    # one and two tiles per wave sum a row in the same order: bit-equal
+    assert torch.equal(out, pyops._spmm(b, ri, v, ro_t, ci_t, m, force_nt=1, force_wpr=4, **kw))
+    assert torch.equal(out, pyops._spmm(b, ri, v, ro_t, ci_t, m, force_nt=2, force_wpr=4, **kw))

@@ -98,6 +98,8 @@ int iex_CudaSpmm5(int m, int k, int n, int nonzeros, const int* row_indices,
 /* ----------------------------------------------------------------- SDDMM ---- */
 #define IEX_SDDMM_SUM_OVER_BATCH 0x1 /* one (nnz) output summed over the batch            */
 #define IEX_SDDMM_ACCUMULATE 0x2     /* out += ... instead of out = ...                   */
+/* bits 8..15: force wavefronts per row (1 or 4); 0 = choose from nnz/m.  For tuning.     */
+#define IEX_SDDMM_FORCE_WPR(w) (((w) & 0xff) << 8)
 
 /* out[(z,) j] = sum_c lhs[z, row(j), c] * rhs[z, column_indices[j], c]
  * lhs is (batch, m, k), rhs is (batch, n, k) -- rhs rows are the sampled columns.

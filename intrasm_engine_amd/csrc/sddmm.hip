@@ -8,8 +8,10 @@
 //     as a single contiguous LPN*VEC*sizeof(T) segment (128-bit per lane when the shape
 //     allows), so G = 64/LPN nonzeros are in flight per instruction;
 //   * the lhs row fragment that a lane needs is the same for every nonzero of the row
-//     and stays in registers when k <= 2*LPN*VEC (the attention shapes); otherwise it
+//     and is held in registers when k <= 2*LPN*VEC (the attention shapes); otherwise it
 //     is re-read (it hits L1: every group reads the same bytes);
+//   * column indices are read 64 at a time (one per lane, the next 64 prefetched) and a
+//     full chunk issues all its gathers before the first reduction;
 //   * the LPN partial dot products are summed with DPP row operations (quad_perm,
 //     row_half_mirror, row_mirror): no LDS, no bpermute in the reduction.
 // Accumulation is fp32; with SUM_OVER_BATCH the batch loop runs inside the kernel so
@@ -50,9 +52,19 @@ __device__ __forceinline__ float dot_vec(const vec_t<T, VEC>& a, const vec_t<T, 
   }
 }
 
-// PASSES > 0: k <= PASSES*LPN*VEC and the lhs fragment is cached in registers
-//             (requires one batch entry per wave);  PASSES == 0: generic k, reload.
-template <typename T, int VEC, int LPN, int PASSES, int WPR>
+// PASSES > 0: k <= PASSES*LPN*VEC (EXACT: k equals it, so no load needs a predicate): the lhs
+//             fragment of a (row, batch entry) is one register load per pass; a chunk of 64
+//             nonzeros takes LPN steps of G nonzeros: all column indices are shuffled out and
+//             all gathers issued first, then step s reduces and leaves its result in lane s of
+//             every group, so each lane ends up with exactly one output (nonzero lane%LPN*G +
+//             lane/LPN) and the chunk is written with ONE store instruction that covers 64
+//             consecutive outputs.  Plain stores only (no accumulate mode).
+// PASSES == 0: generic k and accumulate mode, operands streamed in LPN*VEC slices.
+// A block serves kSddmmZb batch entries (grid.z = ceil(batch / kSddmmZb)) in per-entry output
+// mode, so the row's column indices are fetched once and reused.
+constexpr int kSddmmZb = 4;
+
+template <typename T, int VEC, int LPN, int PASSES, int WPR, bool EXACT>
 __global__ __launch_bounds__(256) void sddmm_kernel(SddmmParams p) {
   constexpr int G = kWave / LPN;
   constexpr int KT = LPN * VEC;
@@ -68,82 +80,114 @@ __global__ __launch_bounds__(256) void sddmm_kernel(SddmmParams p) {
   const int row = uniform(p.row_indices[row_slot]);
   const int start = uniform(p.row_offsets[row]);
   const int end = uniform(p.row_offsets[row + 1]);
-  const int z0 = p.sum_over_batch ? 0 : (int)blockIdx.z;
+  // per-entry output: this block's slice of the batch; batch-summed output: one pass that
+  // loops over the whole batch inside the dot product
+  const int zbeg = p.sum_over_batch ? 0 : (int)blockIdx.z * kSddmmZb;
+  const int zend = p.sum_over_batch ? 1 : min(p.batch, zbeg + kSddmmZb);
   const int zn = p.sum_over_batch ? p.batch : 1;
-  const T* __restrict__ lhs = static_cast<const T*>(p.lhs) + ((size_t)z0 * p.m + row) * p.k;
-  const T* __restrict__ rhs = static_cast<const T*>(p.rhs) + (size_t)z0 * p.n * p.k;
-  T* __restrict__ out = static_cast<T*>(p.out) + (p.sum_over_batch ? (size_t)0 : (size_t)z0 * p.nnz);
   const size_t lhs_zstride = (size_t)p.m * p.k;
   const size_t rhs_zstride = (size_t)p.n * p.k;
+  const T* __restrict__ lhs_row = static_cast<const T*>(p.lhs) + (size_t)row * p.k;
+  const T* __restrict__ rhs_all = static_cast<const T*>(p.rhs);
+  T* __restrict__ out_all = static_cast<T*>(p.out);
 
-  vec_t<T, VEC> lfrag[PASSES > 0 ? PASSES : 1];
-  if constexpr (PASSES > 0) {
-#pragma unroll
-    for (int ps = 0; ps < PASSES; ++ps) {
-      const int kk = ps * KT + sl * VEC;
-      if (kk < p.k) {
-        lfrag[ps] = load_vec<T, VEC>(lhs + kk);
-      } else {
-#pragma unroll
-        for (int i = 0; i < VEC; ++i) lfrag[ps].v[i] = elem<T>::from_float(0.f);
-      }
-    }
-  }
-
-  for (int base = start + part * kWave; base < end; base += kWave * WPR) {
-    const int j = base + lane;
-    const int c = (j < end) ? p.cols[j] : 0;
+  // column index of nonzero base+lane; the next chunk's indices are fetched while the
+  // current chunk is processed
+  int base = start + part * kWave;
+  int c = (base + lane < end) ? p.cols[base + lane] : 0;
+  for (; base < end; base += kWave * WPR) {
+    const int next = base + kWave * WPR;
+    const int c_next = (next + lane < end) ? p.cols[next + lane] : 0;
     const int cnt = min(kWave, end - base);
-    const int steps = (cnt + G - 1) / G;
-    for (int s = 0; s < steps; ++s) {
-      const int t = s * G + sub;          // nonzero of this chunk handled by my lane group
-      const int cc = __shfl(c, t, kWave); // t < 64 always; slots past cnt carry column 0
-      float acc = 0.f;
-      if constexpr (PASSES > 0) {
-        const T* r = rhs + (size_t)cc * p.k;
+    if constexpr (PASSES > 0) {
+      // slots past cnt carry column 0: they gather a valid row and their result is dropped
+      int cc[LPN];
+#pragma unroll
+      for (int st = 0; st < LPN; ++st) cc[st] = __shfl(c, st * G + sub, kWave);
+      const int my_t = sl * G + sub;  // the nonzero whose result this lane will hold
+      for (int z = zbeg; z < zend; ++z) {
+        const T* __restrict__ lhs = lhs_row + (size_t)z * lhs_zstride;
+        const T* __restrict__ rhs = rhs_all + (size_t)z * rhs_zstride;
+        vec_t<T, VEC> lfrag[PASSES];
+        vec_t<T, VEC> rv[LPN][PASSES];
 #pragma unroll
         for (int ps = 0; ps < PASSES; ++ps) {
           const int kk = ps * KT + sl * VEC;
-          if (kk < p.k) acc = dot_vec<T, VEC>(lfrag[ps], load_vec<T, VEC>(r + kk), acc);
+          if (EXACT || kk < p.k) lfrag[ps] = load_vec<T, VEC>(lhs + kk);
         }
-      } else {
-        for (int z = 0; z < zn; ++z) {
-          const T* l = lhs + (size_t)z * lhs_zstride;
-          const T* r = rhs + (size_t)z * rhs_zstride + (size_t)cc * p.k;
-          for (int kk = sl * VEC; kk < p.k; kk += KT)
-            acc = dot_vec<T, VEC>(load_vec<T, VEC>(l + kk), load_vec<T, VEC>(r + kk), acc);
+#pragma unroll
+        for (int st = 0; st < LPN; ++st) {
+          const T* r = rhs + (size_t)cc[st] * p.k;
+#pragma unroll
+          for (int ps = 0; ps < PASSES; ++ps) {
+            const int kk = ps * KT + sl * VEC;
+            if (EXACT || kk < p.k) rv[st][ps] = load_vec<T, VEC>(r + kk);
+          }
         }
+        float res = 0.f;
+#pragma unroll
+        for (int st = 0; st < LPN; ++st) {
+          float acc = 0.f;
+#pragma unroll
+          for (int ps = 0; ps < PASSES; ++ps)
+            if (EXACT || ps * KT + sl * VEC < p.k) acc = dot_vec<T, VEC>(lfrag[ps], rv[st][ps], acc);
+          acc = group_sum<LPN>(acc);
+          res = (sl == st) ? acc : res;
+        }
+        if (my_t < cnt) out_all[(p.sum_over_batch ? (size_t)0 : (size_t)z * p.nnz) + base + my_t] = elem<T>::from_float(res);
       }
-      acc = group_sum<LPN>(acc);
-      if (sl == 0 && t < cnt) {
-        const size_t o = (size_t)base + t;
-        if (p.accumulate) acc += elem<T>::to_float(out[o]);
-        out[o] = elem<T>::from_float(acc);
+    } else {
+      for (int z = zbeg; z < zend; ++z) {
+        const T* __restrict__ lhs = lhs_row + (size_t)z * lhs_zstride;
+        const T* __restrict__ rhs = rhs_all + (size_t)z * rhs_zstride;
+        T* __restrict__ out = out_all + (p.sum_over_batch ? (size_t)0 : (size_t)z * p.nnz);
+        const int steps = (cnt + G - 1) / G;
+        for (int st = 0; st < steps; ++st) {
+          const int t = st * G + sub;           // nonzero of this chunk handled by my lane group
+          const int col = __shfl(c, t, kWave);  // t < 64 always; slots past cnt carry column 0
+          float acc = 0.f;
+          for (int zz = 0; zz < zn; ++zz) {
+            const T* l = lhs + (size_t)zz * lhs_zstride;
+            const T* r = rhs + (size_t)zz * rhs_zstride + (size_t)col * p.k;
+            for (int kk = sl * VEC; kk < p.k; kk += KT)
+              acc = dot_vec<T, VEC>(load_vec<T, VEC>(l + kk), load_vec<T, VEC>(r + kk), acc);
+          }
+          acc = group_sum<LPN>(acc);
+          if (sl == 0 && t < cnt) {
+            const size_t o = (size_t)base + t;
+            if (p.accumulate) acc += elem<T>::to_float(out[o]);
+            out[o] = elem<T>::from_float(acc);
+          }
+        }
       }
     }
+    c = c_next;
   }
 }
 
-template <typename T, int VEC, int LPN, int PASSES, int WPR>
+template <typename T, int VEC, int LPN, int PASSES, int WPR, bool EXACT>
 int launch_one(const SddmmParams& p, hipStream_t stream) {
-  dim3 grid(ceil_div(p.m, 4 / WPR), 1, p.sum_over_batch ? 1 : p.batch);
-  hipLaunchKernelGGL((sddmm_kernel<T, VEC, LPN, PASSES, WPR>), grid, dim3(256), 0, stream, p);
+  dim3 grid(ceil_div(p.m, 4 / WPR), 1, p.sum_over_batch ? 1 : ceil_div(p.batch, kSddmmZb));
+  hipLaunchKernelGGL((sddmm_kernel<T, VEC, LPN, PASSES, WPR, EXACT>), grid, dim3(256), 0, stream, p);
   return check_hip(hipGetLastError(), "sddmm launch");
 }
 
-template <typename T, int VEC, int LPN, int PASSES>
+template <typename T, int VEC, int LPN, int PASSES, bool EXACT>
 int launch_wpr(const SddmmParams& p, int wpr, hipStream_t stream) {
-  if (wpr == 4) return launch_one<T, VEC, LPN, PASSES, 4>(p, stream);
-  return launch_one<T, VEC, LPN, PASSES, 1>(p, stream);
+  if (wpr == 4) return launch_one<T, VEC, LPN, PASSES, 4, EXACT>(p, stream);
+  return launch_one<T, VEC, LPN, PASSES, 1, EXACT>(p, stream);
 }
 
 template <typename T, int VEC, int LPN>
 int launch_passes(const SddmmParams& p, int wpr, hipStream_t stream) {
-  const bool one_z = !(p.sum_over_batch && p.batch > 1);
-  const int kt = LPN * VEC;
-  if (one_z && p.k <= kt) return launch_wpr<T, VEC, LPN, 1>(p, wpr, stream);
-  if (one_z && p.k <= 2 * kt) return launch_wpr<T, VEC, LPN, 2>(p, wpr, stream);
-  return launch_wpr<T, VEC, LPN, 0>(p, wpr, stream);
+  // register-resident lhs needs one batch entry per dot product and plain stores
+  const bool fast = !(p.sum_over_batch && p.batch > 1) && !p.accumulate;
+  constexpr int kt = LPN * VEC;
+  if (fast && p.k == kt) return launch_wpr<T, VEC, LPN, 1, true>(p, wpr, stream);
+  if (fast && p.k == 2 * kt) return launch_wpr<T, VEC, LPN, 2, true>(p, wpr, stream);
+  if (fast && p.k < kt) return launch_wpr<T, VEC, LPN, 1, false>(p, wpr, stream);
+  if (fast && p.k < 2 * kt) return launch_wpr<T, VEC, LPN, 2, false>(p, wpr, stream);
+  return launch_wpr<T, VEC, LPN, 0, false>(p, wpr, stream);
 }
 
 template <typename T>
@@ -177,7 +221,8 @@ int sddmm_dispatch(int dtype, int flags, int m, int k, int n, int nonzeros, cons
               "sddmm: a dense operand exceeds 2^31 elements per batch entry");
   SddmmParams p{m, k, n, nonzeros, batch, row_indices, row_offsets, column_indices, lhs, rhs, out,
                 (flags & IEX_SDDMM_SUM_OVER_BATCH) != 0, (flags & IEX_SDDMM_ACCUMULATE) != 0};
-  const int wpr = ((double)nonzeros / m >= 128.0) ? 4 : 1;
+  int wpr = (flags >> 8) & 0xff;  // forced (1 or 4), else from the mean row length
+  if (wpr != 1 && wpr != 4) wpr = ((double)nonzeros / m >= 64.0) ? 4 : 1;
   hipStream_t s = static_cast<hipStream_t>(stream);
   switch (dtype) {
     case IEX_F32: return launch_typed<float>(p, wpr, s);

@@ -88,10 +88,21 @@ bool lds_variant(const SpmmParams& p, int batch, const Choice& ch, int& vec, int
     rpw = 8;  // largest rows-per-wave that still gives every CU two workgroups
     while (rpw > 2 && (long long)ceil_div(p.m, kLdsWaves * rpw) * tiles < 512) rpw >>= 1;
   }
-  // Measured on MI355X (config-2 and config-4 shapes) the row kernel is faster: with 16 rows
-  // per CU there are too few wavefronts to keep the LDS pipeline busy and the per-stage
-  // barriers expose row-length imbalance.  The staged kernel therefore runs only on request.
-  return ch.variant == 2;
+  if (ch.variant == 2) return true;
+  if (ch.variant == 1) return false;
+  // Measured on MI355X: the staged kernel wins when the rows of a workgroup reuse a staged
+  // dense row a dozen times or more (2:4 weights: 4.5 -> 3.6 ms at 4096x4096, n = 8192), and
+  // from a reuse of 4 when the slice of the dense operand one column tile touches (k rows of
+  // a 64-lane tile) outgrows an XCD's 4 MB L2 (k = 11008: 10.8 -> 4.9 ms).  It loses on small
+  // problems (fewer than two workgroups per CU: per-stage barriers expose row-length imbalance)
+  // and at low reuse (90 % sparsity: 0.67 -> 0.90 ms).
+  const double density = (p.m > 0 && p.k > 0) ? (double)p.nnz / ((double)p.m * p.k) : 0.0;
+  const int eff_rpw = (vec * (int)sizeof(T) == 16 && sizeof(T) == 2 && rpw == 8) ? 4 : rpw;
+  const double reuse = density * kLdsWaves * eff_rpw;
+  const long long groups = (long long)ceil_div(p.m, kLdsWaves * eff_rpw) * tiles;
+  const double slice_bytes = (double)p.k * kWave * vec * sizeof(T);
+  if (groups < 512) return false;
+  return reuse >= 12.0 || (slice_bytes > 6.0 * 1024 * 1024 && reuse >= 4.0);
 }
 
 template <typename T, typename IT>

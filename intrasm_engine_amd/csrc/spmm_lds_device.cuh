@@ -2,9 +2,12 @@
 //
 // The row kernel of spmm_device.cuh gathers every dense row it needs from L2: nnz * tile
 // bytes of L2 -> CU traffic, which is what bounds it.  When a block of rows shares a dense
-// row often enough (density * rows-per-workgroup >= ~2), it is cheaper to stream the dense
-// operand through LDS once per workgroup and gather from LDS, whose gather bandwidth is
-// about three times that of L2 on this part.
+// row often enough (density * rows-per-workgroup of a dozen or more), or when the slice of
+// the dense operand that the row kernel keeps re-reading no longer fits an XCD's L2 (large
+// k), it is cheaper to stream the dense operand through LDS once per workgroup and gather
+// from LDS, whose gather bandwidth is about three times that of L2 on this part.  The kernel
+// is then bound by vector-ALU issue (8 FMAs + 3 bookkeeping instructions per nonzero and
+// 128-bit column vector).
 //
 // Workgroup = 8 wavefronts, owns RB = 8 * RPW consecutive CSR rows (swizzled order, so rows
 // of similar length share a workgroup) and one tile of 64*VEC output columns.
@@ -118,7 +121,7 @@ __device__ __forceinline__ void spmm_lds_block(const SpmmParams& p, int bx, int 
         const int num = __popcll(inb);
         int t = pos[r];
         const int te = t + num;
-        for (; t + 4 <= te; t += 4) {
+        for (; t + 4 <= te; t += 4) {  // (8 in flight measured no faster and costs registers)
           V bv[4];
 #pragma unroll
           for (int u = 0; u < 4; ++u) bv[u] = tile[(bcast_i(c[r], t + u) - kb0) * kWave + lane];

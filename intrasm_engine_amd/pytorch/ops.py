@@ -113,7 +113,7 @@ def _spmm(b, row_indices, values, row_offsets, column_indices, m, *, per_batch_v
 
 
 def _sddmm(a, b, row_indices, row_offsets, column_indices, *, sum_over_batch, dtypes,
-           out=None, accumulate=False):
+           out=None, accumulate=False, force_wpr=0):
     _chk(a.dim() == b.dim())
     _chk(a.dim() == 3)
     _chk(a.size(0) == b.size(0))
@@ -138,7 +138,7 @@ def _sddmm(a, b, row_indices, row_offsets, column_indices, *, sum_over_batch, dt
         _chk(tuple(out.shape) == shape and out.dtype == a.dtype and out.is_contiguous()
              and out.device == a.device, "out has the wrong shape, dtype, layout or device")
     flags = (_lib.SDDMM_SUM_OVER_BATCH if sum_over_batch else 0) | \
-            (_lib.SDDMM_ACCUMULATE if accumulate else 0)
+            (_lib.SDDMM_ACCUMULATE if accumulate else 0) | ((int(force_wpr) & 0xff) << 8)
     with torch.cuda.device(a.device):
         rc = _lib.load().iex_sddmm_ex(
             _DT[a.dtype], flags, m, k, n, nonzeros, row_indices.data_ptr(), row_offsets.data_ptr(),

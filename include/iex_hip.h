@@ -58,13 +58,21 @@ int iex_copy_bytes(void* dst, const void* src, size_t nbytes, void* stream);
 #define IEX_SPMM_RELU 0x4             /* out = max(0, A*b + bias)                           */
 /* bits 8..15: force waves-per-row (1, 4 or 8); 0 = choose from nnz/m.  For tuning.    */
 #define IEX_SPMM_FORCE_WPR(w) (((w) & 0xff) << 8)
-/* bits 16..19: force the kernel family (1 = row kernel gathering from L2, 2 = LDS-staged);
- * bits 20..23: rows per wavefront of the LDS-staged kernel (2, 4 or 8).  0 = choose.      */
+/* bits 16..19: force the kernel family: 1 = row kernel gathering from L2, 2 = LDS-staged
+ * gather, 3 / 4 = matrix-core kernels (fp16 / bf16: A expanded to dense tiles in LDS; 4 waves
+ * and 128 x 256 tiles / 8 waves and 128 x 512 tiles).  0 = choose.
+ * Families 2-4 rely on strictly ascending column indices inside a row (canonical CSR, what
+ * dense_to_sparse produces); family 1 accepts any order and duplicates -- force it for such
+ * input.  Families 3-4 multiply explicit zeros with the dense operand, so a non-finite entry
+ * in a row of `dense` that no nonzero references still reaches the output (0 * inf = NaN).
+ * bits 20..23: rows per wavefront of family 2 (2, 4 or 8), windows of 16 nonzeros held in
+ * registers per row of family 4 (1, 2 or 4).  0 = choose.                                 */
 #define IEX_SPMM_FORCE_VARIANT(v) (((v) & 0xf) << 16)
 #define IEX_SPMM_FORCE_RPW(r) (((r) & 0xf) << 20)
 /* bits 24..27: adjacent 64-lane column tiles per wavefront of the row kernel (1 or 2).    */
 #define IEX_SPMM_FORCE_NT(t) (((t) & 0xf) << 24)
-/* bits 28..30: lanes per nonzero of the row kernel, coded 1..4 = 8, 16, 32, 64 lanes.      */
+/* bits 28..30: lanes per nonzero of the row kernel, coded 1..4 = 8, 16, 32, 64 lanes; for
+ * family 3 the lanes that share a row during expansion (8 or 16).                          */
 #define IEX_SPMM_FORCE_LPG_CODE(c) (((c) & 0x7) << 28)
 
 /* out[z, r, :] = sum_j values[(z,) j] * dense[z, column_indices[j], :]  (+ bias[r], ReLU)

@@ -1,6 +1,7 @@
 // Host side of the CSR SpMM: kernel wrappers, variant selection, argument checks and
 // the C entry points.  The device code is in spmm_device.cuh.
 #include "spmm_lds_device.cuh"
+#include "spmm_mfma2_device.cuh"
 
 namespace iex {
 namespace {
@@ -62,9 +63,84 @@ int launch_lds_rpw(const SpmmParams& p, int batch, int rpw, hipStream_t stream) 
   return fail(IEX_ERR_BAD_ARGUMENT, "spmm: rows-per-wave of the LDS-staged variant must be 2, 4 or 8 (got %d)", rpw);
 }
 
+// ---- matrix-core variant (fp16 / bf16) ----------------------------------------------------
+template <bool BF16, typename IT, int LPR>
+__global__ __launch_bounds__(kMfmaThreads, 2) void spmm_mfma_kernel(SpmmParams p, int tiles_m) {
+  extern __shared__ __align__(16) unsigned char smem[];
+  // consecutive workgroups walk the row blocks of one column panel of the dense operand
+  spmm_mfma_block<BF16, IT, LPR>(p, blockIdx.x % tiles_m, blockIdx.x / tiles_m, blockIdx.y, smem);
+}
+
+template <typename T, typename IT, int LPR>
+int launch_mfma_one(const SpmmParams& p, int batch, hipStream_t stream) {
+  constexpr bool kBf16 = std::is_same<T, __hip_bfloat16>::value;
+  const int tiles_m = ceil_div(p.m, kMfmaBM), tiles_n = ceil_div(p.n, kMfmaBN);
+  auto kernel = spmm_mfma_kernel<kBf16, IT, LPR>;
+  static thread_local bool raised = false;  // more than 64 KB of dynamic LDS needs the attribute (per instantiation)
+  if (!raised) {
+    if (int rc = check_hip(hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
+                                               hipFuncAttributeMaxDynamicSharedMemorySize, kMfmaLdsBytes),
+                           "hipFuncSetAttribute(LDS size)"))
+      return rc;
+    raised = true;
+  }
+  hipLaunchKernelGGL(kernel, dim3(tiles_m * tiles_n, batch), dim3(kMfmaThreads), kMfmaLdsBytes, stream, p, tiles_m);
+  return check_hip(hipGetLastError(), "spmm (matrix-core) launch");
+}
+
+template <typename T, typename IT>
+int launch_mfma(const SpmmParams& p, int batch, int lpr, hipStream_t stream) {
+  if constexpr (sizeof(T) == 2) {
+    switch (lpr) {
+      case 8: return launch_mfma_one<T, IT, 8>(p, batch, stream);
+      case 16: return launch_mfma_one<T, IT, 16>(p, batch, stream);
+    }
+    return fail(IEX_ERR_BAD_ARGUMENT, "spmm: lanes-per-row of the matrix-core variant must be 8 or 16 (got %d)", lpr);
+  } else {
+    return fail(IEX_ERR_UNSUPPORTED, "spmm: the matrix-core variant handles fp16 and bf16 only");
+  }
+}
+
+template <bool BF16, typename IT, int W>
+__global__ __launch_bounds__(kMfma2Threads, 2) void spmm_mfma2_kernel(SpmmParams p, int tiles_m) {
+  extern __shared__ __align__(16) unsigned char smem[];
+  spmm_mfma2_block<BF16, IT, W>(p, blockIdx.x % tiles_m, blockIdx.x / tiles_m, blockIdx.y, smem);
+}
+
+template <typename T, typename IT, int W>
+int launch_mfma2_one(const SpmmParams& p, int batch, hipStream_t stream) {
+  constexpr bool kBf16 = std::is_same<T, __hip_bfloat16>::value;
+  const int tiles_m = ceil_div(p.m, kMfmaBM), tiles_n = ceil_div(p.n, kMfma2BN);
+  auto kernel = spmm_mfma2_kernel<kBf16, IT, W>;
+  static thread_local bool raised = false;
+  if (!raised) {
+    if (int rc = check_hip(hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
+                                               hipFuncAttributeMaxDynamicSharedMemorySize, kMfma2LdsBytes),
+                           "hipFuncSetAttribute(LDS size)"))
+      return rc;
+    raised = true;
+  }
+  hipLaunchKernelGGL(kernel, dim3(tiles_m * tiles_n, batch), dim3(kMfma2Threads), kMfma2LdsBytes, stream, p, tiles_m);
+  return check_hip(hipGetLastError(), "spmm (matrix-core, 8 waves) launch");
+}
+
+template <typename T, typename IT>
+int launch_mfma2(const SpmmParams& p, int batch, int windows, hipStream_t stream) {
+  if constexpr (sizeof(T) == 2) {
+    switch (windows) {
+      case 1: return launch_mfma2_one<T, IT, 1>(p, batch, stream);
+      case 2: return launch_mfma2_one<T, IT, 2>(p, batch, stream);
+      case 4: return launch_mfma2_one<T, IT, 4>(p, batch, stream);
+    }
+    return fail(IEX_ERR_BAD_ARGUMENT, "spmm: windows of the matrix-core variant must be 1, 2 or 4 (got %d)", windows);
+  } else {
+    return fail(IEX_ERR_UNSUPPORTED, "spmm: the matrix-core variant handles fp16 and bf16 only");
+  }
+}
+
 struct Choice {
   int wpr = 0;      // wavefronts per row of the row kernel
-  int variant = 0;  // 0 = choose, 1 = row kernel, 2 = LDS-staged kernel
+  int variant = 0;  // 0 = choose, 1 = row kernel, 2 = LDS-staged kernel, 3 = matrix-core kernel
   int rpw = 0;      // rows per wavefront of the LDS-staged kernel (0 = choose)
   int nt = 0;       // adjacent column tiles per wavefront of the row kernel (0 = choose)
   int lpg = 0;      // lanes per nonzero of the row kernel: 8, 16, 32 or 64 (0 = choose)
@@ -105,9 +181,49 @@ bool lds_variant(const SpmmParams& p, int batch, const Choice& ch, int& vec, int
   return reuse >= 12.0 || (slice_bytes > 6.0 * 1024 * 1024 && reuse >= 4.0);
 }
 
+// The matrix-core kernels: 16-bit types, n a multiple of 8, 16-byte aligned dense operands,
+// k < 65535 for the 8-wave arrangement (packed columns).  Sets kind = 3 (4 waves, 128 x 256
+// tiles; param = lanes per row) or 4 (8 waves, 128 x 512 tiles; param = windows per row);
+// kind 0 = use a gather kernel.
+struct MfmaChoice {
+  int kind = 0, param = 0;
+};
+
+template <typename T>
+MfmaChoice mfma_variant(const SpmmParams& p, int batch, const Choice& ch) {
+  MfmaChoice mc;
+  if (sizeof(T) != 2 || (ch.variant != 0 && ch.variant != 3 && ch.variant != 4)) return mc;
+  if (!(p.n % 8 == 0 && aligned(p.dense, 16) && aligned(p.out, 16))) return mc;  // (also when forced)
+  const double density = (p.m > 0 && p.k > 0) ? (double)p.nnz / ((double)p.m * p.k) : 0.0;
+  const double run = density * kMfmaBKA;  // nonzeros of a row per 128-column chunk
+  const bool wide_ok = p.k < 65535;
+  const long long tiles_m = ceil_div(p.m, kMfmaBM);
+  const long long wgs_wide = tiles_m * ceil_div(p.n, kMfma2BN) * batch;
+  const long long wgs_narrow = tiles_m * ceil_div(p.n, kMfmaBN) * batch;
+  int kind = ch.variant;
+  if (kind == 0) {
+    // Measured on MI355X (fp16, m x k = 11008 x 4096, n = 2048): the gather kernels and the
+    // matrix-core kernels meet at about 5 % density (0.34 vs 0.32 ms); at 10 % the matrix cores
+    // are 1.7x faster, at 50 % (4096 x 4096, n = 8192) 7x; at 2 % the gather kernel is 2x faster.
+    // Small outputs (a handful of tiles) leave most CUs idle and stay with the gather kernels.
+    if (density < 0.05) return mc;
+    if (wide_ok && wgs_wide >= 128) kind = 4;
+    else if (wgs_narrow >= 128) kind = 3;
+    else return mc;
+  }
+  if (kind == 4 && !wide_ok) kind = 3;
+  mc.kind = kind;
+  if (kind == 3) mc.param = ch.lpg ? ch.lpg : (run > 24.0 ? 16 : 8);
+  else mc.param = ch.rpw ? ch.rpw : (run >= 48.0 ? 4 : 1);
+  return mc;
+}
+
 template <typename T, typename IT>
 int launch_typed(const SpmmParams& p, int batch, const Choice& ch, hipStream_t stream) {
   constexpr int kMax = 16 / (int)sizeof(T);
+  const MfmaChoice mc = mfma_variant<T>(p, batch, ch);
+  if (mc.kind == 4) return launch_mfma2<T, IT>(p, batch, mc.param, stream);
+  if (mc.kind == 3) return launch_mfma<T, IT>(p, batch, mc.param, stream);
   int lvec = 0, rpw = 0;
   if (lds_variant<T>(p, batch, ch, lvec, rpw)) {
     if (lvec == kMax) return launch_lds_rpw<T, IT, kMax>(p, batch, rpw, stream);

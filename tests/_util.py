@@ -12,16 +12,19 @@ import torch
 RTOL = {torch.float32: 1e-5, torch.float16: 1e-2, torch.bfloat16: 1e-2,
         np.dtype("float32"): 1e-5, np.dtype("float16"): 1e-2}
 FLOOR = 0.1
+# An fp16 output below 6.1e-5 is a subnormal with an absolute spacing of 2^-24: half of that
+# is the rounding error of storing the result, whatever its relative size.
+FP16_SUBNORMAL_HALF_STEP = 2.0 ** -25
 
 
-def assert_close(got, want, scale, rtol, what=""):
+def assert_close(got, want, scale, rtol, what="", atol=0.0):
     got = np.asarray(got, dtype=np.float64)
     want = np.asarray(want, dtype=np.float64)
     scale = np.asarray(scale, dtype=np.float64)
     assert got.shape == want.shape, f"{what}: shape {got.shape} != {want.shape}"
     assert np.isfinite(got).all(), f"{what}: non-finite output"
     err = np.abs(got - want)
-    bound = rtol * np.abs(want) + rtol * FLOOR * scale
+    bound = rtol * np.abs(want) + rtol * FLOOR * scale + atol
     bad = err > bound
     if bad.any():
         idx = np.unravel_index(np.argmax(err - bound), err.shape)

@@ -7,7 +7,7 @@ import pytest
 import torch
 
 from intrasm_engine_amd import workloads as W
-from _util import RTOL, assert_close, rounded, to_dev
+from _util import FP16_SUBNORMAL_HALF_STEP, RTOL, assert_close, rounded, to_dev
 
 pytestmark = pytest.mark.gpu
 ops = torch.ops.iex_ops
@@ -307,6 +307,111 @@ def test_lds_staged_variant(oracle, dev, rpw, dtype, n):
     kw = dict(per_batch_values=False, accumulate=False, dtypes=(dtype,), allow_i16=False)
     assert torch.equal(pyops._spmm(bi, ri, v, ro_t, ci_t, m, force_variant=2, force_rpw=rpw, **kw),
                        pyops._spmm(bi, ri, v, ro_t, ci_t, m, force_variant=1, **kw))
+
+
+@pytest.mark.parametrize("family,knob", [(3, 8), (3, 16), (4, 1), (4, 2), (4, 4)])
+@pytest.mark.parametrize("dtype,n,itype", [(torch.float16, 264, torch.int16), (torch.float16, 512, torch.int32),
+                                           (torch.bfloat16, 776, torch.int32), (torch.float16, 8, torch.int16)])
+def test_matrix_core_variants(oracle, dev, family, knob, dtype, n, itype):
+    """The kernels that expand A to dense tiles in LDS and multiply on the matrix cores
+    (forced): skewed matrix with empty rows, a completely dense row (runs longer than the
+    register windows), k not a multiple of the 32- and 128-column steps, m that leaves idle
+    row slots, n that leaves a partial column tile."""
+    from intrasm_engine_amd.pytorch import ops as pyops
+    rng = np.random.default_rng(11 * family + knob + n)
+    m, k = 333, 1000
+    lens = np.clip(rng.geometric(1 / 120.0, m), 0, k)
+    lens[[0, 17, 332]] = 0
+    lens[5] = k
+    lens[6] = 1
+    lens[7] = 700
+    ro, ci = W.csr_from_row_lengths(rng, m, k, lens)
+    csr = W.CSR(m, k, rng.standard_normal(ci.shape[0]).astype(np.float32), W.swizzle_from_offsets(ro), ro, ci)
+    b_np = rng.standard_normal((2, k, n)).astype(np.float32)
+    ri, v, ro_t, ci_t = to_dev(csr, dev, dtype)
+    ci_t = ci_t.to(itype)
+    b = torch.from_numpy(b_np).to(dev).to(dtype)
+    force = dict(force_variant=family, force_lpg=knob) if family == 3 else dict(force_variant=family, force_rpw=knob)
+    kw = dict(per_batch_values=False, accumulate=False, dtypes=(dtype,), allow_i16=True)
+    out = pyops._spmm(b, ri, v, ro_t, ci_t, m, **force, **kw)
+    vals_r, b_r = rounded(csr.values, dtype), rounded(b_np, dtype)
+    want = oracle.spmm(b_r, csr.row_indices, vals_r, csr.row_offsets, csr.column_indices, m)
+    scale = oracle.spmm_abs_scale(b_r, csr.row_indices, vals_r, csr.row_offsets, csr.column_indices, m)
+    assert_close(out.float().cpu().numpy(), want, scale, RTOL[dtype], f"matrix-core family {family}/{knob} {dtype} n={n}",
+                 atol=FP16_SUBNORMAL_HALF_STEP if dtype == torch.float16 else 0.0)
+    # integer-valued data: every family is exact, so they agree bit for bit
+    csr.values = rng.integers(-2, 3, csr.nnz).astype(np.float32)
+    bi = torch.from_numpy(rng.integers(-2, 3, (1, k, n)).astype(np.float32)).to(dev).to(dtype)
+    ri, v, ro_t, ci_t = to_dev(csr, dev, dtype)
+    ci_t = ci_t.to(itype)
+    assert torch.equal(pyops._spmm(bi, ri, v, ro_t, ci_t, m, **force, **kw),
+                       pyops._spmm(bi, ri, v, ro_t, ci_t, m, force_variant=1, **kw))
+
+
+@pytest.mark.parametrize("family", [3, 4])
+def test_matrix_core_epilogue_options(oracle, dev, family):
+    """bias + ReLU, accumulation into the output and per-batch values on the matrix-core kernels."""
+    from intrasm_engine_amd.pytorch import ops as pyops
+    rng = np.random.default_rng(family)
+    m, k, n, batch = 200, 300, 128, 3
+    csr = W.pruned_weight(40 + family, m, k, 0.8)
+    ri, v, ro_t, ci_t = to_dev(csr, dev, torch.float16)
+    b_np = rng.standard_normal((batch, k, n)).astype(np.float32)
+    b = torch.from_numpy(b_np).to(dev).half()
+    b_r, vals_r = rounded(b_np, torch.float16), rounded(csr.values, torch.float16)
+    base = oracle.spmm(b_r, csr.row_indices, vals_r, csr.row_offsets, csr.column_indices, m)
+    scale = oracle.spmm_abs_scale(b_r, csr.row_indices, vals_r, csr.row_offsets, csr.column_indices, m)
+    kw = dict(dtypes=(torch.float16,), allow_i16=True, force_variant=family)
+    # bias + ReLU
+    bias_np = rng.standard_normal(m).astype(np.float32)
+    out = pyops._spmm(b, ri, v, ro_t, ci_t, m, per_batch_values=False, accumulate=False,
+                      bias=torch.from_numpy(bias_np).to(dev), relu=True, **kw)
+    assert_close(out.float().cpu().numpy(), np.maximum(base + bias_np[None, :, None], 0.0), scale + np.abs(bias_np)[None, :, None],
+                 RTOL[torch.float16], "bias+relu")
+    # accumulate
+    prev_np = rounded(rng.standard_normal((batch, m, n)).astype(np.float32), torch.float16)
+    prev = torch.from_numpy(prev_np).to(dev).half()
+    out = pyops._spmm(b, ri, v, ro_t, ci_t, m, per_batch_values=False, accumulate=True, out=prev, **kw)
+    assert out.data_ptr() == prev.data_ptr()
+    assert_close(out.float().cpu().numpy(), base + prev_np, scale + np.abs(prev_np), RTOL[torch.float16], "accumulate")
+    # per-batch values
+    vb_np = rng.standard_normal((batch, csr.nnz)).astype(np.float32)
+    vb = torch.from_numpy(vb_np).to(dev).half()
+    out = pyops._spmm(b, ri, vb, ro_t, ci_t, m, per_batch_values=True, accumulate=False, **kw)
+    vb_r = rounded(vb_np, torch.float16)
+    for z in range(batch):
+        want = oracle.spmm(b_r[z:z + 1], csr.row_indices, vb_r[z], csr.row_offsets, csr.column_indices, m)
+        sc = oracle.spmm_abs_scale(b_r[z:z + 1], csr.row_indices, vb_r[z], csr.row_offsets, csr.column_indices, m)
+        assert_close(out[z:z + 1].float().cpu().numpy(), want, sc, RTOL[torch.float16], f"per-batch values z={z}")
+
+
+@pytest.mark.parametrize("dtype,n,density,family", [(torch.float16, 2048, 0.5, 4), (torch.float16, 1024, 0.5, 3),
+                                                    (torch.float32, 1024, 0.5, 2)])
+def test_automatic_choice_of_kernel_family(oracle, dev, dtype, n, density, family):
+    """Shapes on which the library leaves the row kernel by itself: 16-bit operands of moderate
+    density go to the matrix-core kernels (8 waves when that still fills the chip, else 4),
+    fp32 with many row blocks and high reuse of a staged dense row to the LDS-staged gather.
+    Checked against the oracle, and bit-equal to the forced family, which shows which one ran."""
+    from intrasm_engine_amd.pytorch import ops as pyops
+    rng = np.random.default_rng(n)
+    m, k = 4096, 320
+    lens = np.full(m, int(density * k))
+    lens[::97] = 0
+    ro, ci = W.csr_from_row_lengths(rng, m, k, lens)
+    csr = W.CSR(m, k, rng.standard_normal(ci.shape[0]).astype(np.float32), W.swizzle_from_offsets(ro), ro, ci)
+    b_np = rng.standard_normal((1, k, n)).astype(np.float32)
+    ri, v, ro_t, ci_t = to_dev(csr, dev, dtype)
+    b = torch.from_numpy(b_np).to(dev).to(dtype)
+    kw = dict(per_batch_values=False, accumulate=False, dtypes=(dtype,), allow_i16=False)
+    out = pyops._spmm(b, ri, v, ro_t, ci_t, m, **kw)
+    vals_r, b_r = rounded(csr.values, dtype), rounded(b_np, dtype)
+    want = oracle.spmm(b_r, csr.row_indices, vals_r, csr.row_offsets, csr.column_indices, m)
+    scale = oracle.spmm_abs_scale(b_r, csr.row_indices, vals_r, csr.row_offsets, csr.column_indices, m)
+    assert_close(out.float().cpu().numpy(), want, scale, RTOL[dtype], f"auto staged {dtype} n={n}")
+    assert torch.equal(out, pyops._spmm(b, ri, v, ro_t, ci_t, m, force_variant=family, **kw))
+    row = pyops._spmm(b, ri, v, ro_t, ci_t, m, force_variant=1, **kw)
+    assert not torch.equal(out, row)   # different summation order
+    assert torch.allclose(out.float(), row.float(), rtol=1e-2, atol=1e-2 * float(scale.max()))
 
 
 @pytest.mark.parametrize("dtype,n", [(torch.float32, 1024), (torch.float32, 1280), (torch.float16, 2048),

@@ -2,6 +2,7 @@
 // the C entry points.  The device code is in spmm_device.cuh.
 #include "spmm_lds_device.cuh"
 #include "spmm_mfma2_device.cuh"
+#include "spmm_mfma_f32_device.cuh"
 
 namespace iex {
 namespace {
@@ -138,9 +139,47 @@ int launch_mfma2(const SpmmParams& p, int batch, int windows, hipStream_t stream
   }
 }
 
+// ---- matrix-core variant, fp32 ---------------------------------------------------------------
+// arrangement code: 1 = 32 x 64 tile (4 k slices), 2 = 32 x 128 tile as 2 x 64 columns (2 k
+// slices), 4 = 32 x 128 tile, 128 columns per wave (4 k slices)
+template <int NJ, int WAVES_N, int W>
+__global__ __launch_bounds__(kF32Threads, 2) void spmm_mfma_f32_kernel(SpmmParams p, int tiles_m) {
+  extern __shared__ __align__(16) unsigned char smem[];
+  spmm_mfma_f32_block<NJ, WAVES_N, W>(p, blockIdx.x % tiles_m, blockIdx.x / tiles_m, blockIdx.y, smem);
+}
+
+template <int NJ, int WAVES_N, int W>
+int launch_mfma_f32_one(const SpmmParams& p, int batch, hipStream_t stream) {
+  constexpr int kBN = 32 * NJ * WAVES_N;
+  const int tiles_m = ceil_div(p.m, kF32BM), tiles_n = ceil_div(p.n, kBN);
+  constexpr int kLds = spmm_mfma_f32_lds_bytes<NJ, WAVES_N>();
+  hipLaunchKernelGGL((spmm_mfma_f32_kernel<NJ, WAVES_N, W>), dim3(tiles_m * tiles_n, batch), dim3(kF32Threads), kLds,
+                     stream, p, tiles_m);
+  return check_hip(hipGetLastError(), "spmm (matrix-core, fp32) launch");
+}
+
+template <int NJ, int WAVES_N>
+int launch_mfma_f32_w(const SpmmParams& p, int batch, int windows, hipStream_t stream) {
+  switch (windows) {
+    case 2: return launch_mfma_f32_one<NJ, WAVES_N, 2>(p, batch, stream);
+    case 4: return launch_mfma_f32_one<NJ, WAVES_N, 4>(p, batch, stream);
+    case 8: return launch_mfma_f32_one<NJ, WAVES_N, 8>(p, batch, stream);
+  }
+  return fail(IEX_ERR_BAD_ARGUMENT, "spmm: windows of the fp32 matrix-core variant must be 2, 4 or 8 (got %d)", windows);
+}
+
+inline int launch_mfma_f32(const SpmmParams& p, int batch, int arrangement, int windows, hipStream_t stream) {
+  switch (arrangement) {
+    case 1: return launch_mfma_f32_w<2, 1>(p, batch, windows, stream);
+    case 2: return launch_mfma_f32_w<2, 2>(p, batch, windows, stream);
+    case 4: return launch_mfma_f32_w<4, 1>(p, batch, windows, stream);
+  }
+  return fail(IEX_ERR_BAD_ARGUMENT, "spmm: arrangement of the fp32 matrix-core variant must be 1, 2 or 4 (got %d)", arrangement);
+}
+
 struct Choice {
   int wpr = 0;      // wavefronts per row of the row kernel
-  int variant = 0;  // 0 = choose, 1 = row kernel, 2 = LDS-staged kernel, 3 = matrix-core kernel
+  int variant = 0;  // 0 = choose, 1 = row kernel, 2 = LDS-staged kernel, 3 / 4 = matrix-core kernels (16-bit), 5 = (fp32)
   int rpw = 0;      // rows per wavefront of the LDS-staged kernel (0 = choose)
   int nt = 0;       // adjacent column tiles per wavefront of the row kernel (0 = choose)
   int lpg = 0;      // lanes per nonzero of the row kernel: 8, 16, 32 or 64 (0 = choose)
@@ -193,7 +232,7 @@ template <typename T>
 MfmaChoice mfma_variant(const SpmmParams& p, int batch, const Choice& ch) {
   MfmaChoice mc;
   if (sizeof(T) != 2 || (ch.variant != 0 && ch.variant != 3 && ch.variant != 4)) return mc;
-  if (!(p.n % 8 == 0 && aligned(p.dense, 16) && aligned(p.out, 16))) return mc;  // (also when forced)
+  if (!(p.nnz > 0 && p.n % 8 == 0 && aligned(p.dense, 16) && aligned(p.out, 16))) return mc;  // (also when forced)
   const double density = (p.m > 0 && p.k > 0) ? (double)p.nnz / ((double)p.m * p.k) : 0.0;
   const double run = density * kMfmaBKA;  // nonzeros of a row per 128-column chunk
   const bool wide_ok = p.k < 65535;
@@ -214,13 +253,41 @@ MfmaChoice mfma_variant(const SpmmParams& p, int batch, const Choice& ch) {
   if (kind == 4 && !wide_ok) kind = 3;
   mc.kind = kind;
   if (kind == 3) mc.param = ch.lpg ? ch.lpg : (run > 24.0 ? 16 : 8);
-  else mc.param = ch.rpw ? ch.rpw : (run >= 48.0 ? 4 : 1);
+  else mc.param = ch.rpw ? ch.rpw : (run > 20.0 ? 4 : run > 8.0 ? 2 : 1);
   return mc;
+}
+
+// fp32 on the matrix cores: int32 indices, n a multiple of 4, 16-byte aligned dense operands.
+// Returns the arrangement code (0 = use a gather kernel) and sets the number of register windows.
+template <typename T, typename IT>
+int mfma_f32_variant(const SpmmParams& p, int batch, const Choice& ch, int& windows) {
+  if (!std::is_same<T, float>::value || !std::is_same<IT, int>::value) return 0;
+  if (ch.variant != 0 && ch.variant != 5) return 0;
+  if (!(p.nnz > 0 && p.n % 4 == 0 && aligned(p.dense, 16) && aligned(p.out, 16))) return 0;  // (also when forced)
+  const double density = (p.m > 0 && p.k > 0) ? (double)p.nnz / ((double)p.m * p.k) : 0.0;
+  const double run = density * kF32BKA;
+  windows = ch.rpw ? ch.rpw : (run <= 12.0 ? 2 : run <= 40.0 ? 4 : 8);
+  // 128 columns per wave when that still gives most CUs a workgroup, else 64 per wave
+  const long long tiles_m = ceil_div(p.m, kF32BM);
+  int arrangement = p.n <= 64 ? 1 : (tiles_m * ceil_div(p.n, 128) * batch >= 200 ? 4 : 2);
+  if (ch.nt) arrangement = ch.nt;
+  if (ch.variant == 5) return arrangement;
+  // Measured on MI355X: 85-105 dense-equivalent TFLOP/s (the fp32 MFMA rate is 153), which
+  // beats the gather kernels from 25-30 % density on large outputs (4096 x 4096 at 50 %,
+  // n = 8192: 5.0 -> 2.9 ms; at 30 %, n = 1024: 0.69 -> 0.38 ms) and loses below 20 %
+  // (11008 x 4096 at 20 %: 6.6 vs 7.3 ms).  With one workgroup per CU (4096 x 4096, n = 256:
+  // 256 tiles) the expansion is not hidden and the gather kernel stays ahead (0.19 vs 0.22 ms).
+  if (p.nnz > 0 && density >= 0.25 && arrangement == 4 && tiles_m * ceil_div(p.n, 128) * batch >= 512) return arrangement;
+  return 0;
 }
 
 template <typename T, typename IT>
 int launch_typed(const SpmmParams& p, int batch, const Choice& ch, hipStream_t stream) {
   constexpr int kMax = 16 / (int)sizeof(T);
+  if constexpr (std::is_same<T, float>::value && std::is_same<IT, int>::value) {
+    int windows = 0;
+    if (const int arr = mfma_f32_variant<T, IT>(p, batch, ch, windows)) return launch_mfma_f32(p, batch, arr, windows, stream);
+  }
   const MfmaChoice mc = mfma_variant<T>(p, batch, ch);
   if (mc.kind == 4) return launch_mfma2<T, IT>(p, batch, mc.param, stream);
   if (mc.kind == 3) return launch_mfma<T, IT>(p, batch, mc.param, stream);

@@ -73,14 +73,19 @@ __device__ __forceinline__ void spmm_mfma2_block(const SpmmParams& p, int tile_m
   const int group = tid / LPR;
   const int gshift = lane & ~(LPR - 1);
   int pos[R], end[R];
-  unsigned win[R][W];
+  // A window entry is the pair (value, column) as two 16-bit halves of one register, filled by
+  // two 16-bit loads with a clamped index and no arithmetic on the result: nothing here waits
+  // for the loads, so they overlap the MFMAs.  Whether the entry belongs to the row (index
+  // below the row end) is decided when it is used.  The host guarantees nnz > 0.
+  u16 wval[R][W];
+  IT wcol[R][W];
+  const int last_nz = p.nnz - 1;
   auto load_windows = [&](int j) {
 #pragma unroll
     for (int w = 0; w < W; ++w) {
-      const int idx = pos[j] + w * LPR + sub;
-      unsigned e = kNone;
-      if (idx < end[j]) e = ((unsigned)(u16)cols[idx] << 16) | (unsigned)values[idx];
-      win[j][w] = e;
+      const int safe = min(pos[j] + w * LPR + sub, last_nz);
+      wval[j][w] = values[safe];
+      wcol[j][w] = cols[safe];
     }
   };
 #pragma unroll
@@ -100,18 +105,22 @@ __device__ __forceinline__ void spmm_mfma2_block(const SpmmParams& p, int tile_m
   auto expand_row = [&](int j, int ka0, u16* abuf) {
     u16* rowp = abuf + (group + j * GROUPS) * LDA;
     *reinterpret_cast<u32x4*>(rowp + sub * 8) = u32x4{0u, 0u, 0u, 0u};
-    const unsigned lim = (unsigned)(ka0 + BKA) << 16;
+    const int kend = ka0 + BKA;
+    const unsigned lim = (unsigned)kend << 16;
     int consumed = 0;
 #pragma unroll
     for (int w = 0; w < W; ++w) {
-      const unsigned e = win[j][w];
-      const bool in = e < lim;
-      if (in) rowp[(int)(e >> 16) - ka0] = (u16)e;
+      const int c = (int)wcol[j][w];
+      const bool in = pos[j] + w * LPR + sub < end[j] && c < kend;
+      if (in) rowp[c - ka0] = wval[j][w];
       consumed += __popcll((__ballot(in) >> gshift) & 0xffffull);
     }
     pos[j] += consumed;
     bool more = consumed == W * LPR;
-    while (__any(more)) {  // a run longer than the windows held in registers: loads are exposed here
+    // A run longer than the windows held in registers: the loads of these passes are exposed.
+    // (Unrolling this loop into forward branches, so that the compiler could keep counting the
+    // loads in flight across it, was measured: the extra register pressure costs far more.)
+    while (__any(more)) {
       unsigned e = kNone;
       const int idx = pos[j] + sub;
       if (more && idx < end[j]) e = ((unsigned)(u16)cols[idx] << 16) | (unsigned)values[idx];

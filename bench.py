@@ -321,6 +321,13 @@ def run_extras(torch, ops, dev, W, IL, mats, dens, csr_dev, time_cell, variant_o
     t_graph = IL.run_interleaving(spmm_execs, gemm_execs) / reps
     t_fused = IL.run_non_interleaving(fused_execs) / reps
     t_fused_g = IL.run_non_interleaving(fused_g_execs) / reps
+    # the same pair with the SpMM forced onto the gather (row) kernel: vector ALU + L2 beside the matrix cores,
+    # the resource split the reference's co-run experiment is about
+    from intrasm_engine_amd.pytorch import ops as pyops
+    gather_execs = [lambda: pyops._spmm(xt, riw, vw, row, ciw, w.m, per_batch_values=False, accumulate=False,
+                                        dtypes=(torch.float16,), allow_i16=True, force_variant=1)] * reps
+    t_gather = IL.run_non_interleaving(gather_execs) / reps
+    t_graph_gather = IL.run_interleaving(gather_execs, gemm_execs) / reps
     fl_s, fl_g = W.spmm_flops(w.nnz, 2048), W.gemm_flops(4096, 2048, 4096)
     by_s = W.spmm_bytes(w.m, w.k, 2048, w.nnz, 1, 2, 2)
     out["config4"] = {
@@ -334,10 +341,13 @@ def run_extras(torch, ops, dev, W, IL, mats, dens, csr_dev, time_cell, variant_o
         "fused_launch_gemm_in_groups_of_64_ms": round(t_fused_g, 4),
         "graph_makespan_pct_of_serialized": round(100 * t_graph / (t_spmm + t_gemm), 1),
         "fused_makespan_pct_of_serialized": round(100 * t_fused / (t_spmm + t_gemm), 1),
+        "spmm_row_kernel_ms": round(t_gather, 4), "two_branch_graph_row_kernel_ms": round(t_graph_gather, 4),
+        "row_kernel_graph_makespan_pct_of_serialized": round(100 * t_graph_gather / (t_gather + t_gemm), 1),
+        "spmm_dense_equivalent_TFLOPs": round(2.0 * w.m * w.k * 2048 / t_spmm / 1e9, 1),
         "repeats_per_graph": reps,
     }
     log(f"[bench] config 4: spmm {t_spmm:.3f} ms, gemm {t_gemm:.3f} ms, graph {t_graph:.3f} ms, fused {t_fused:.3f} ms")
-    del w, x, ga, gb, riw, vw, row, ciw, xt, gat, gbt, spmm_execs, gemm_execs, fused_execs, fused_g_execs
+    del w, x, ga, gb, riw, vw, row, ciw, xt, gat, gbt, spmm_execs, gemm_execs, fused_execs, fused_g_execs, gather_execs
 
     # ---- config 5: LLaMA-7B-shaped sparse decoder layer, 16 sequences x 512 tokens, three variants
     from intrasm_engine_amd.decoder_layer import SparseDecoderLayer
@@ -370,6 +380,33 @@ def run_extras(torch, ops, dev, W, IL, mats, dens, csr_dev, time_cell, variant_o
         "layer_TFLOPs_serialized": round((spmm_flops5 + attn_flops5) / t_ser / 1e9, 1),
     }
     log(f"[bench] config 5: serialized {t_ser:.2f} ms, two-stream graph {t_ms:.2f} ms, fused {t_fu:.2f} ms")
+    del layer
+
+    # ---- the SpMM kernel families side by side on three projections of that layer (n = 8192 tokens, fp16,
+    # int16 indices) and on the config-4 operand: row kernel (gathers from L2), LDS-staged gather, matrix cores
+    from intrasm_engine_amd.pytorch import ops as pyops
+    fam = {}
+    w4 = W.config4()[0]
+    for name, c, n_ in (("q_2to4_4096x4096_n8192", weights["q"], seqs * L), ("gate_80pct_11008x4096_n8192", weights["gate"], seqs * L),
+                        ("down_80pct_4096x11008_n8192", weights["down"], seqs * L), ("config4_90pct_11008x4096_n2048", w4, 2048)):
+        ri, v, ro, ci = csr_dev(c, torch.float16, torch.int16)
+        xin = torch.randn(1, c.k, n_, device=dev, generator=torch.Generator(dev).manual_seed(1)).half()
+        kw = dict(per_batch_values=False, accumulate=False, dtypes=(torch.float16,), allow_i16=True)
+        row = {}
+        for label, force in (("row_kernel_ms", dict(force_variant=1)), ("lds_staged_ms", dict(force_variant=2)),
+                             ("matrix_core_4waves_ms", dict(force_variant=3)), ("matrix_core_8waves_ms", dict(force_variant=4)),
+                             ("library_choice_ms", {})):
+            row[label] = round(IL.time_execs([lambda: pyops._spmm(xin, ri, v, ro, ci, c.m, **force, **kw)] * 2, repeats=3) / 2, 4)
+        dense_flops = 2.0 * c.m * c.k * n_
+        row["density"] = round(c.nnz / (c.m * c.k), 4)
+        row["library_choice_dense_equivalent_TFLOPs"] = round(dense_flops / row["library_choice_ms"] / 1e9, 1)
+        row["library_choice_nonzero_TFLOPs"] = round(2.0 * c.nnz * n_ / row["library_choice_ms"] / 1e9, 1)
+        row["library_choice_mfma_frac_dense_equivalent"] = round(dense_flops / row["library_choice_ms"] / 1e9 / MFMA_PEAK_TFLOPS_16BIT, 4)
+        fam[name] = row
+        del ri, v, ro, ci, xin
+    out["spmm_kernel_families_fp16"] = fam
+    log("[bench] kernel families: " + ", ".join(f"{k_}: row {r_['row_kernel_ms']} / lds {r_['lds_staged_ms']} / mfma {r_['matrix_core_8waves_ms']} ms"
+                                               for k_, r_ in fam.items()))
     return out
 
 

@@ -245,9 +245,14 @@ MfmaChoice mfma_variant(const SpmmParams& p, int batch, const Choice& ch) {
     // matrix-core kernels meet at about 5 % density (0.34 vs 0.32 ms); at 10 % the matrix cores
     // are 1.7x faster, at 50 % (4096 x 4096, n = 8192) 7x; at 2 % the gather kernel is 2x faster.
     // Small outputs (a handful of tiles) leave most CUs idle and stay with the gather kernels.
+    // A tile computes all of its 256 / 512 columns: an n that fills less than three quarters of
+    // its tiles wastes the difference (n = 64 on 512-column tiles measured 3.5x slower than the
+    // gather kernel).
     if (density < 0.05) return mc;
-    if (wide_ok && wgs_wide >= 128) kind = 4;
-    else if (wgs_narrow >= 128) kind = 3;
+    const double fill_wide = (double)p.n / ((double)ceil_div(p.n, kMfma2BN) * kMfma2BN);
+    const double fill_narrow = (double)p.n / ((double)ceil_div(p.n, kMfmaBN) * kMfmaBN);
+    if (wide_ok && wgs_wide >= 128 && fill_wide >= 0.75) kind = 4;
+    else if (wgs_narrow >= 128 && fill_narrow >= 0.75) kind = 3;
     else return mc;
   }
   if (kind == 4 && !wide_ok) kind = 3;
@@ -277,7 +282,8 @@ int mfma_f32_variant(const SpmmParams& p, int batch, const Choice& ch, int& wind
   // n = 8192: 5.0 -> 2.9 ms; at 30 %, n = 1024: 0.69 -> 0.38 ms) and loses below 20 %
   // (11008 x 4096 at 20 %: 6.6 vs 7.3 ms).  With one workgroup per CU (4096 x 4096, n = 256:
   // 256 tiles) the expansion is not hidden and the gather kernel stays ahead (0.19 vs 0.22 ms).
-  if (p.nnz > 0 && density >= 0.25 && arrangement == 4 && tiles_m * ceil_div(p.n, 128) * batch >= 512) return arrangement;
+  const double fill = (double)p.n / ((double)ceil_div(p.n, 128) * 128);  // share of the computed columns that exist
+  if (density >= 0.25 && arrangement == 4 && fill >= 0.75 && tiles_m * ceil_div(p.n, 128) * batch >= 512) return arrangement;
   return 0;
 }
 

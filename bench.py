@@ -37,10 +37,10 @@ CELL_REPEATS = 20                # launches of one cell inside its timing graph
 # the sweep, from two `rocprofv3 --pmc` runs (FETCH_SIZE, WRITE_SIZE) of `bench.py --pmc-probe`, each
 # scaled by the counter's reading for a plain 256 MiB copy (x2.000 and x1.000): see
 # profiles/spmm_fp32_config2_hbm_traffic_pmc.txt.  Counters cannot be read inside a timing run.
-MEASURED_TRAFFIC_BYTES = {
-    "spmm_kernel<float, int, 4, 64, 4>": 100.7e6,   # n = 256
-    "spmm_kernel<float, int, 4, 32, 4>": 38.6e6,    # n = 128
-    "spmm_kernel<float, int, 4, 16, 4>": 28.9e6,    # n = 64
+MEASURED_TRAFFIC_MB = {   # (sparsity, n) -> MB per launch of the row kernel
+    (0.7, 64): 51.30, (0.7, 128): 61.56, (0.7, 256): 174.86, (0.8, 64): 37.78, (0.8, 128): 47.37, (0.8, 256): 134.22,
+    (0.9, 64): 24.31, (0.9, 128): 33.78, (0.9, 256): 83.51, (0.95, 64): 17.59, (0.95, 128): 27.04, (0.95, 256): 61.88,
+    (0.98, 64): 13.56, (0.98, 128): 23.01, (0.98, 256): 49.03,
 }
 
 
@@ -148,7 +148,7 @@ def main():
         return ms / repeats * 1e3  # us
 
     def variant_of(csr, n, sv):
-        """(VEC, LPG, WPR) the library picks for an aligned operand (spmm_pick_shape / pick_wpr)."""
+        """(VEC, LPG, WPR) of the row kernel for an aligned operand (spmm_pick_shape / pick_wpr)."""
         mean = csr.nnz / csr.m
         wpr = 4 if mean >= 24 else 1
         kmax = 16 // sv
@@ -168,10 +168,15 @@ def main():
         us = time_cell(spmm32(s, n))
         by, fl = cell_bytes(s, n), W.spmm_flops(mats[s].nnz, n)
         vec, lpg, wpr = variant_of(mats[s], n, 4)
+        kernel = f"spmm_kernel<float, int, {vec}, {lpg}, {wpr}>"
+        c = mats[s]
+        # the dispatcher's rule for the fp32 matrix-core kernel (spmm.hip, mfma_f32_variant)
+        if c.nnz / (c.m * c.k) >= 0.27 and n % 4 == 0 and -(-c.m // 32) * -(-n // 128) >= 200 and n / (-(-n // 128) * 128) >= 0.75:
+            kernel = "spmm_mfma_f32_kernel<32, 4, 1, 16, true>"
         table.append({"sparsity": s, "n": n, "nnz": mats[s].nnz, "us": round(us, 2), "GBps": round(by / us / 1e3, 1),
                       "hbm_frac": round(by / us / 1e3 / HBM_PEAK_GBPS, 4), "GFLOPs": round(fl / us / 1e3, 1),
                       "valu_frac": round(fl / us / 1e6 / VALU_PEAK_TFLOPS_FP32, 4),
-                      "kernel": f"spmm_kernel<float, int, {vec}, {lpg}, {wpr}>", "bytes": by})
+                      "kernel": kernel, "bytes": by})
         log(f"[bench] fp32 s={s} n={n}: {us:.2f} us  {by / us / 1e3:.0f} GB/s  {fl / us / 1e3:.0f} GFLOP/s")
 
     by_kernel = {}
@@ -182,7 +187,9 @@ def main():
     dom_us = statistics.mean(r["us"] for r in dom_rows)
     roofline = {"bound": "hbm", "achieved": round(dom_bytes / dom_us / 1e3, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                 "frac": round(dom_bytes / dom_us / 1e3 / HBM_PEAK_GBPS, 4),
-                "traffic": MEASURED_TRAFFIC_BYTES.get(dom_name),
+                "traffic": (round(statistics.mean(MEASURED_TRAFFIC_MB[(r["sparsity"], r["n"])] for r in dom_rows) * 1e6)
+                            if dom_name.startswith("spmm_kernel<float") and all((r["sparsity"], r["n"]) in MEASURED_TRAFFIC_MB for r in dom_rows)
+                            else None),
                 "kernel": dom_name, "avg_launch_us": round(dom_us, 2),
                 "algorithmic_bytes_per_launch": int(dom_bytes),
                 "cells": [[r["sparsity"], r["n"]] for r in dom_rows],

@@ -140,41 +140,47 @@ int launch_mfma2(const SpmmParams& p, int batch, int windows, hipStream_t stream
 }
 
 // ---- matrix-core variant, fp32 ---------------------------------------------------------------
-// arrangement code: 1 = 32 x 64 tile (4 k slices), 2 = 32 x 128 tile as 2 x 64 columns (2 k
-// slices), 4 = 32 x 128 tile, 128 columns per wave (4 k slices)
-template <int NJ, int WAVES_N, int W>
-__global__ __launch_bounds__(kF32Threads, 2) void spmm_mfma_f32_kernel(SpmmParams p, int tiles_m) {
+// arrangement code = MFMA tile height and how the 4 multiplying waves split the C tile:
+//   1 = 32 x 64 (4 k slices)    2 = 32 x 128 as 2 x 64 columns (2 k slices)    4 = 32 x 128 (4 k slices)
+//   5 = 16 x 64 (4 k slices)    6 = 16 x 128 as 2 x 64 columns (2 k slices)
+template <int MT, int NJ, int WAVES_N, int W, bool SPLIT>
+__global__ __launch_bounds__(kF32Threads + (SPLIT ? MT * 8 : 0), 2) void spmm_mfma_f32_kernel(SpmmParams p, int tiles_m) {
   extern __shared__ __align__(16) unsigned char smem[];
-  spmm_mfma_f32_block<NJ, WAVES_N, W>(p, blockIdx.x % tiles_m, blockIdx.x / tiles_m, blockIdx.y, smem);
+  spmm_mfma_f32_block<MT, NJ, WAVES_N, W, SPLIT>(p, blockIdx.x % tiles_m, blockIdx.x / tiles_m, blockIdx.y, smem);
 }
 
-template <int NJ, int WAVES_N, int W>
+template <int MT, int NJ, int WAVES_N, int W, bool SPLIT>
 int launch_mfma_f32_one(const SpmmParams& p, int batch, hipStream_t stream) {
-  constexpr int kBN = 32 * NJ * WAVES_N;
-  const int tiles_m = ceil_div(p.m, kF32BM), tiles_n = ceil_div(p.n, kBN);
-  constexpr int kLds = spmm_mfma_f32_lds_bytes<NJ, WAVES_N>();
-  hipLaunchKernelGGL((spmm_mfma_f32_kernel<NJ, WAVES_N, W>), dim3(tiles_m * tiles_n, batch), dim3(kF32Threads), kLds,
-                     stream, p, tiles_m);
+  constexpr int kBN = MT * NJ * WAVES_N;
+  const int tiles_m = ceil_div(p.m, MT), tiles_n = ceil_div(p.n, kBN);
+  constexpr int kLds = spmm_mfma_f32_lds_bytes<MT, NJ, WAVES_N>();
+  hipLaunchKernelGGL((spmm_mfma_f32_kernel<MT, NJ, WAVES_N, W, SPLIT>), dim3(tiles_m * tiles_n, batch),
+                     dim3(kF32Threads + (SPLIT ? MT * 8 : 0)), kLds, stream, p, tiles_m);
   return check_hip(hipGetLastError(), "spmm (matrix-core, fp32) launch");
 }
 
-template <int NJ, int WAVES_N>
-int launch_mfma_f32_w(const SpmmParams& p, int batch, int windows, hipStream_t stream) {
+template <int MT, int NJ, int WAVES_N>
+int launch_mfma_f32_w(const SpmmParams& p, int batch, int windows, bool split, hipStream_t stream) {
+  // with separate expanding waves there are registers for 16 windows (the kernel uses as many
+  // of them as the rows of a wave need); waves that do both hold 2, 4 or 8
+  if (split) return launch_mfma_f32_one<MT, NJ, WAVES_N, 16, true>(p, batch, stream);
   switch (windows) {
-    case 2: return launch_mfma_f32_one<NJ, WAVES_N, 2>(p, batch, stream);
-    case 4: return launch_mfma_f32_one<NJ, WAVES_N, 4>(p, batch, stream);
-    case 8: return launch_mfma_f32_one<NJ, WAVES_N, 8>(p, batch, stream);
+    case 2: return launch_mfma_f32_one<MT, NJ, WAVES_N, 2, false>(p, batch, stream);
+    case 4: return launch_mfma_f32_one<MT, NJ, WAVES_N, 4, false>(p, batch, stream);
+    case 8: return launch_mfma_f32_one<MT, NJ, WAVES_N, 8, false>(p, batch, stream);
   }
   return fail(IEX_ERR_BAD_ARGUMENT, "spmm: windows of the fp32 matrix-core variant must be 2, 4 or 8 (got %d)", windows);
 }
 
-inline int launch_mfma_f32(const SpmmParams& p, int batch, int arrangement, int windows, hipStream_t stream) {
+inline int launch_mfma_f32(const SpmmParams& p, int batch, int arrangement, int windows, bool split, hipStream_t stream) {
   switch (arrangement) {
-    case 1: return launch_mfma_f32_w<2, 1>(p, batch, windows, stream);
-    case 2: return launch_mfma_f32_w<2, 2>(p, batch, windows, stream);
-    case 4: return launch_mfma_f32_w<4, 1>(p, batch, windows, stream);
+    case 1: return launch_mfma_f32_w<32, 2, 1>(p, batch, windows, split, stream);
+    case 2: return launch_mfma_f32_w<32, 2, 2>(p, batch, windows, split, stream);
+    case 4: return launch_mfma_f32_w<32, 4, 1>(p, batch, windows, split, stream);
+    case 5: return launch_mfma_f32_w<16, 4, 1>(p, batch, windows, split, stream);
+    case 6: return launch_mfma_f32_w<16, 4, 2>(p, batch, windows, split, stream);
   }
-  return fail(IEX_ERR_BAD_ARGUMENT, "spmm: arrangement of the fp32 matrix-core variant must be 1, 2 or 4 (got %d)", arrangement);
+  return fail(IEX_ERR_BAD_ARGUMENT, "spmm: arrangement of the fp32 matrix-core variant must be 1, 2, 4, 5 or 6 (got %d)", arrangement);
 }
 
 struct Choice {
@@ -270,20 +276,22 @@ int mfma_f32_variant(const SpmmParams& p, int batch, const Choice& ch, int& wind
   if (ch.variant != 0 && ch.variant != 5) return 0;
   if (!(p.nnz > 0 && p.n % 4 == 0 && aligned(p.dense, 16) && aligned(p.out, 16))) return 0;  // (also when forced)
   const double density = (p.m > 0 && p.k > 0) ? (double)p.nnz / ((double)p.m * p.k) : 0.0;
-  const double run = density * kF32BKA;
-  windows = ch.rpw ? ch.rpw : (run <= 12.0 ? 2 : run <= 40.0 ? 4 : 8);
-  // 128 columns per wave when that still gives most CUs a workgroup, else 64 per wave
-  const long long tiles_m = ceil_div(p.m, kF32BM);
-  int arrangement = p.n <= 64 ? 1 : (tiles_m * ceil_div(p.n, 128) * batch >= 200 ? 4 : 2);
+  // 32-row tiles with 128 columns per wave when that still gives most CUs a workgroup; else
+  // 16-row tiles (twice the workgroups, twice the reads of the dense operand)
+  const long long tiles_m = ceil_div(p.m, 32);
+  int arrangement = tiles_m * ceil_div(p.n, 128) * batch >= 200 ? 4 : (p.n <= 64 ? 5 : 6);
   if (ch.nt) arrangement = ch.nt;
+  const double run = density * 128;  // nonzeros of a row per chunk
+  windows = ch.rpw ? ch.rpw : (run <= 12.0 ? 2 : run <= 40.0 ? 4 : 8);
   if (ch.variant == 5) return arrangement;
-  // Measured on MI355X: 85-105 dense-equivalent TFLOP/s (the fp32 MFMA rate is 153), which
-  // beats the gather kernels from 25-30 % density on large outputs (4096 x 4096 at 50 %,
-  // n = 8192: 5.0 -> 2.9 ms; at 30 %, n = 1024: 0.69 -> 0.38 ms) and loses below 20 %
-  // (11008 x 4096 at 20 %: 6.6 vs 7.3 ms).  With one workgroup per CU (4096 x 4096, n = 256:
-  // 256 tiles) the expansion is not hidden and the gather kernel stays ahead (0.19 vs 0.22 ms).
+  // Measured on MI355X: 70-105 dense-equivalent TFLOP/s (the fp32 MFMA rate is 153; fp32 MFMAs
+  // run on the vector ALUs, so the expansion's instructions add to their time instead of hiding
+  // behind them).  That beats the gather kernels from 25-30 % density (4096 x 4096 at 50 %,
+  // n = 8192: 5.0 -> 2.9 ms; at 30 %, n = 1024: 0.69 -> 0.38 ms; at 30 %, n = 256: 0.19 -> 0.13 ms),
+  // ties at 20 % and loses below (11008 x 4096 at 20 %: 6.6 vs 7.3 ms).  The 16-row arrangements
+  // for small outputs stay on request: at 30 % and n = 128 they only tie (0.096 vs 0.100 ms).
   const double fill = (double)p.n / ((double)ceil_div(p.n, 128) * 128);  // share of the computed columns that exist
-  if (density >= 0.25 && arrangement == 4 && fill >= 0.75 && tiles_m * ceil_div(p.n, 128) * batch >= 512) return arrangement;
+  if (density >= 0.27 && arrangement == 4 && fill >= 0.75) return arrangement;
   return 0;
 }
 
@@ -292,7 +300,7 @@ int launch_typed(const SpmmParams& p, int batch, const Choice& ch, hipStream_t s
   constexpr int kMax = 16 / (int)sizeof(T);
   if constexpr (std::is_same<T, float>::value && std::is_same<IT, int>::value) {
     int windows = 0;
-    if (const int arr = mfma_f32_variant<T, IT>(p, batch, ch, windows)) return launch_mfma_f32(p, batch, arr, windows, stream);
+    if (const int arr = mfma_f32_variant<T, IT>(p, batch, ch, windows)) return launch_mfma_f32(p, batch, arr, windows, ch.lpg != 8, stream);  // (lanes-per-group code 8 = no role split, for tuning)
   }
   const MfmaChoice mc = mfma_variant<T>(p, batch, ch);
   if (mc.kind == 4) return launch_mfma2<T, IT>(p, batch, mc.param, stream);

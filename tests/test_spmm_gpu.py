@@ -348,12 +348,13 @@ def test_matrix_core_variants(oracle, dev, family, knob, dtype, n, itype):
                        pyops._spmm(bi, ri, v, ro_t, ci_t, m, force_variant=1, **kw))
 
 
-@pytest.mark.parametrize("arrangement", [1, 2, 4])
-@pytest.mark.parametrize("windows", [2, 4, 8])
+@pytest.mark.parametrize("arrangement", [1, 2, 4, 5, 6])
+@pytest.mark.parametrize("windows", [0, 2, 4, 8])
 @pytest.mark.parametrize("n", [260, 128, 64, 4])
 def test_matrix_core_fp32(oracle, dev, arrangement, windows, n):
-    """The fp32 kernel on v_mfma_f32_32x32x2 (forced), every tile arrangement and window count,
-    on the same skewed matrix: empty rows, a completely dense row, ragged m, k and n."""
+    """The fp32 kernel on v_mfma_f32_32x32x2 / 16x16x4 (forced), every tile arrangement, with
+    separate expanding waves (windows = 0) and with waves that do both and hold 2, 4 or 8
+    windows, on the same skewed matrix: empty rows, a completely dense row, ragged m, k and n."""
     from intrasm_engine_amd.pytorch import ops as pyops
     rng = np.random.default_rng(100 * arrangement + windows + n)
     m, k = 333, 1000
@@ -368,7 +369,9 @@ def test_matrix_core_fp32(oracle, dev, arrangement, windows, n):
     ri, v, ro_t, ci_t = to_dev(csr, dev)
     b = torch.from_numpy(b_np).to(dev)
     kw = dict(per_batch_values=False, accumulate=False, dtypes=(torch.float32,), allow_i16=False)
-    force = dict(force_variant=5, force_nt=arrangement, force_rpw=windows)
+    force = dict(force_variant=5, force_nt=arrangement)
+    if windows:
+        force.update(force_rpw=windows, force_lpg=8)   # lanes-per-group code 8 = no separate expanding waves
     out = pyops._spmm(b, ri, v, ro_t, ci_t, m, **force, **kw)
     want = oracle.spmm(b_np, csr.row_indices, csr.values, csr.row_offsets, csr.column_indices, m)
     scale = oracle.spmm_abs_scale(b_np, csr.row_indices, csr.values, csr.row_offsets, csr.column_indices, m)

@@ -21,11 +21,12 @@ __device__ __forceinline__ bool xcd_tile(int block, int tiles_m, int tiles_n, in
 }
 
 template <bool BF16, bool TRANS_B, int WM, int WN>
-__global__ __launch_bounds__(256) void gemm_kernel(GemmParams p) {
+__global__ __launch_bounds__(256, (WM * WN <= 8 ? 2 : 1)) void gemm_kernel(GemmParams p) {
   extern __shared__ __align__(16) unsigned char smem[];
   int tile_m, tile_n;
   if (!xcd_tile(blockIdx.x, p.tiles_m, p.tiles_n, tile_m, tile_n)) return;  // uniform per block
-  gemm_tile<BF16, TRANS_B, WM, WN>(p, tile_m, tile_n, blockIdx.y, smem);
+  // 128 x 256 tiles: 128 accumulators per lane leave room for two register sets in flight, not three
+  gemm_tile<BF16, TRANS_B, WM, WN, (WM * WN == 8 ? 2 : kGemmSets)>(p, tile_m, tile_n, blockIdx.y, smem);
 }
 
 template <bool BF16, bool TRANS_B, int WM, int WN>
@@ -52,21 +53,29 @@ int launch(GemmParams p, int batch, hipStream_t stream) {
 }
 
 template <bool BF16, bool TRANS_B>
-int launch_shape(const GemmParams& p, int batch, hipStream_t stream) {
-  // 128x128 tiles keep two workgroups (two waves per SIMD) on a CU, which measured faster than
-  // 256x128 at every size tried; 256x256 tiles (128x128 per wave, half the LDS reads per MFMA)
-  // win once there are at least two of them per CU.
-  const long long huge_tiles = (long long)ceil_div(p.M, 256) * ceil_div(p.N, 256) * batch;
-  if (huge_tiles >= 512) return launch<BF16, TRANS_B, 4, 4>(p, batch, stream);
+int launch_shape(const GemmParams& p, int batch, int force, hipStream_t stream) {
+  if (force == 1) return launch<BF16, TRANS_B, 2, 2>(p, batch, stream);
+  if (force == 2) return launch<BF16, TRANS_B, 2, 4>(p, batch, stream);
+  if (force == 3) return launch<BF16, TRANS_B, 4, 4>(p, batch, stream);
+  // 128x256 tiles (64x128 per wave: a third fewer LDS bytes per MFMA than 64x64) once there are
+  // two of them per CU: 865-912 TFLOP/s against 710-736 with 128x128 tiles at 4096..11008 x 8192
+  // x 4096..8192; below that 128x128 keeps more workgroups in flight (config 4's 4096 x 2048:
+  // 643 vs 575).  256x256 tiles (one wave per SIMD, 504 registers) never beat 128x256 by more
+  // than noise and stay on request.
+  const long long wide_tiles = (long long)ceil_div(p.M, 128) * ceil_div(p.N, 256) * batch;
+  if (wide_tiles >= 512 && p.K >= 256) return launch<BF16, TRANS_B, 2, 4>(p, batch, stream);
   return launch<BF16, TRANS_B, 2, 2>(p, batch, stream);
 }
 
 }  // namespace
 }  // namespace iex
 
-extern "C" int iex_gemm(int dtype, int trans_b, int M, int N, int K, const void* A, const void* B, void* C, int batch,
+// trans_b: bit 0 = B is (N, K); bits 4..7 force the tile shape for tuning (1 = 128x128, 2 = 128x256,
+// 3 = 256x256; 0 = choose).
+extern "C" int iex_gemm(int dtype, int trans_b_and_shape, int M, int N, int K, const void* A, const void* B, void* C, int batch,
                         long long stride_a, long long stride_b, long long stride_c, void* stream) {
   using namespace iex;
+  const int trans_b = trans_b_and_shape & 1, force = (trans_b_and_shape >> 4) & 0xf;
   IEX_REQUIRE(M >= 0 && N >= 0 && K >= 0 && batch >= 0, IEX_ERR_BAD_ARGUMENT, "gemm: negative dimension");
   if (M == 0 || N == 0 || batch == 0) return 0;
   IEX_REQUIRE(A && B && C, IEX_ERR_BAD_ARGUMENT, "gemm: null pointer argument");
@@ -81,8 +90,8 @@ extern "C" int iex_gemm(int dtype, int trans_b, int M, int N, int K, const void*
   GemmParams p{M, N, K, A, B, C, stride_a, stride_b, stride_c, 0, 0};
   hipStream_t s = static_cast<hipStream_t>(stream);
   const bool bf = dtype == IEX_BF16;
-  if (bf && trans_b) return launch_shape<true, true>(p, batch, s);
-  if (bf && !trans_b) return launch_shape<true, false>(p, batch, s);
-  if (!bf && trans_b) return launch_shape<false, true>(p, batch, s);
-  return launch_shape<false, false>(p, batch, s);
+  if (bf && trans_b) return launch_shape<true, true>(p, batch, force, s);
+  if (bf && !trans_b) return launch_shape<true, false>(p, batch, force, s);
+  if (!bf && trans_b) return launch_shape<false, true>(p, batch, force, s);
+  return launch_shape<false, false>(p, batch, force, s);
 }

@@ -150,13 +150,14 @@ struct GemmStage {
 
 // One C tile.  `smem` must hold gemm_lds_bytes<WM,WN>() bytes, 16-byte aligned.
 // All 256 threads of the workgroup must call this (it contains barriers).
-template <bool BF16, bool TRANS_B, int WM, int WN>
+template <bool BF16, bool TRANS_B, int WM, int WN, int SETS = kGemmSets>
 __device__ __forceinline__ void gemm_tile(const GemmParams& p, int tile_m, int tile_n, int z, unsigned char* smem) {
   constexpr int BM = 2 * WM * 32;
   constexpr int BN = 2 * WN * 32;
   constexpr int BK = kGemmBK;
   constexpr int LD = kGemmLd;
-  constexpr int SETS = kGemmSets;
+  static_assert(SETS == 2 || SETS == 3, "register sets in flight");
+  constexpr int PERIOD = SETS == 2 ? 2 : 6;  // steps after which LDS buffer and register set repeat
   typedef unsigned short u16;
 
   typedef GemmStage<TRANS_B, BM, BN> Stage;
@@ -239,21 +240,28 @@ __device__ __forceinline__ void gemm_tile(const GemmParams& p, int tile_m, int t
     __syncthreads();
   };
 
-  static_assert(SETS == 3, "the step loop below is unrolled for 3 register sets (period 6)");
   int kt = 0;
-  for (; kt + 6 <= KT; kt += 6) {
-    step(kt + 0, std::integral_constant<int, 0>{});
-    step(kt + 1, std::integral_constant<int, 1>{});
-    step(kt + 2, std::integral_constant<int, 2>{});
-    step(kt + 3, std::integral_constant<int, 3>{});
-    step(kt + 4, std::integral_constant<int, 4>{});
-    step(kt + 5, std::integral_constant<int, 5>{});
+  if constexpr (PERIOD == 6) {
+    for (; kt + 6 <= KT; kt += 6) {
+      step(kt + 0, std::integral_constant<int, 0>{});
+      step(kt + 1, std::integral_constant<int, 1>{});
+      step(kt + 2, std::integral_constant<int, 2>{});
+      step(kt + 3, std::integral_constant<int, 3>{});
+      step(kt + 4, std::integral_constant<int, 4>{});
+      step(kt + 5, std::integral_constant<int, 5>{});
+    }
+    if (kt < KT) step(kt++, std::integral_constant<int, 0>{});
+    if (kt < KT) step(kt++, std::integral_constant<int, 1>{});
+    if (kt < KT) step(kt++, std::integral_constant<int, 2>{});
+    if (kt < KT) step(kt++, std::integral_constant<int, 3>{});
+    if (kt < KT) step(kt++, std::integral_constant<int, 4>{});
+  } else {
+    for (; kt + 2 <= KT; kt += 2) {
+      step(kt + 0, std::integral_constant<int, 0>{});
+      step(kt + 1, std::integral_constant<int, 1>{});
+    }
+    if (kt < KT) step(kt++, std::integral_constant<int, 0>{});
   }
-  if (kt < KT) step(kt++, std::integral_constant<int, 0>{});
-  if (kt < KT) step(kt++, std::integral_constant<int, 1>{});
-  if (kt < KT) step(kt++, std::integral_constant<int, 2>{});
-  if (kt < KT) step(kt++, std::integral_constant<int, 3>{});
-  if (kt < KT) step(kt++, std::integral_constant<int, 4>{});
 
   // Swapped-operand result layout: lane holds row (lane % 32) of the 32x32 block and, in
   // accumulator quad q, columns q*8 + (lane / 32)*4 .. +3.

@@ -38,11 +38,34 @@ def test_gemm_ragged_n_with_transposed_b(oracle, dev, shape):
         ops.gemm_mfma(torch.zeros(8, 8, device=dev).half(), torch.zeros(8, shape[1] | 1, device=dev).half(), False)
 
 
+@pytest.mark.parametrize("shape_code", [1, 2, 3])
+@pytest.mark.parametrize("trans_b", [False, True])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_every_tile_shape(oracle, dev, shape_code, trans_b, dtype):
+    """128x128, 128x256 and 256x256 tiles forced through the C ABI on a ragged problem
+    (m, n and k leave partial tiles and a partial last K step)."""
+    from intrasm_engine_amd import _lib
+    rng = np.random.default_rng(shape_code)
+    M, N, K = 300, 520, 200
+    a_np = rng.standard_normal((M, K)).astype(np.float32)
+    b_np = rng.standard_normal((N, K) if trans_b else (K, N)).astype(np.float32)
+    a, b = torch.from_numpy(a_np).to(dev).to(dtype), torch.from_numpy(b_np).to(dev).to(dtype)
+    out = torch.empty(M, N, device=dev, dtype=dtype)
+    rc = _lib.load().iex_gemm(2 if dtype == torch.bfloat16 else 1, int(trans_b) | (shape_code << 4), M, N, K,
+                              a.data_ptr(), b.data_ptr(), out.data_ptr(), 1, 0, 0, 0, torch.cuda.current_stream().cuda_stream)
+    assert rc == 0, _lib.load().iex_last_error()
+    a_r, b_r = rounded(a_np, dtype), rounded(b_np, dtype)
+    want = oracle.gemm(a_r, b_r, trans_b=trans_b)
+    scale = oracle.gemm(np.abs(a_r), np.abs(b_r), trans_b=trans_b)
+    assert_close(out.float().cpu().numpy(), want, scale, 1e-2, f"tile shape {shape_code} {dtype} trans_b={trans_b}")
+
+
 def test_large_tiles(oracle, dev):
-    """Enough 256x256 tiles to select the large-tile kernel; a corner is checked against the
-    oracle and the whole result against the transposed-B layout of the same kernel."""
+    """Enough 128x256 tiles (and a long enough K) to select the wide-tile kernel; a corner is
+    checked against the oracle and the whole result against the transposed-B layout of the
+    same kernel."""
     rng = np.random.default_rng(3)
-    M, N, K = 4096, 8192, 64
+    M, N, K = 4096, 8192, 256
     a_np = rng.standard_normal((M, K)).astype(np.float32)
     b_np = rng.standard_normal((K, N)).astype(np.float32)
     a, b = torch.from_numpy(a_np).to(dev).half(), torch.from_numpy(b_np).to(dev).half()

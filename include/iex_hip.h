@@ -67,15 +67,17 @@ int iex_copy_bytes(void* dst, const void* src, size_t nbytes, void* stream);
  * input.  Families 3-5 multiply explicit zeros with the dense operand, so a non-finite entry
  * in a row of `dense` that no nonzero references still reaches the output (0 * inf = NaN).
  * bits 20..23: rows per wavefront of family 2 (2, 4 or 8); windows of nonzeros held in
- * registers per row of family 4 (1, 2 or 4 windows of 16) and 5 (2, 4 or 8 windows of 8).
+ * registers per row of family 4 (1, 2, 4 or 5 windows of 16) and 5 (2, 4 or 8 windows of 8).
  * 0 = choose.                                                                            */
 #define IEX_SPMM_FORCE_VARIANT(v) (((v) & 0xf) << 16)
 #define IEX_SPMM_FORCE_RPW(r) (((r) & 0xf) << 20)
 /* bits 24..27: adjacent 64-lane column tiles per wavefront of the row kernel (1 or 2); tile
- * arrangement of family 5 (1 = 32 x 64, 2 = 32 x 128 as two 64-column waves, 4 = 32 x 128). */
+ * arrangement of family 5 (1 = 32 x 64, 2 = 32 x 128 as two 64-column waves, 4 = 32 x 128,
+ * 5 = 16 x 64, 6 = 16 x 128 as two 64-column waves).                                        */
 #define IEX_SPMM_FORCE_NT(t) (((t) & 0xf) << 24)
 /* bits 28..30: lanes per nonzero of the row kernel, coded 1..4 = 8, 16, 32, 64 lanes; for
- * family 3 the lanes that share a row during expansion (8 or 16).                          */
+ * family 3 the lanes that share a row during expansion (8 or 16); for family 5 code 1 turns
+ * the separate expanding wavefronts off (every wave then expands and multiplies in turn).  */
 #define IEX_SPMM_FORCE_LPG_CODE(c) (((c) & 0x7) << 28)
 
 /* out[z, r, :] = sum_j values[(z,) j] * dense[z, column_indices[j], :]  (+ bias[r], ReLU)

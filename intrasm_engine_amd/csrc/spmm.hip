@@ -102,17 +102,18 @@ int launch_mfma(const SpmmParams& p, int batch, int lpr, hipStream_t stream) {
   }
 }
 
-template <bool BF16, typename IT, int W>
+template <bool BF16, typename IT, int W, int BKA>
 __global__ __launch_bounds__(kMfma2Threads, 2) void spmm_mfma2_kernel(SpmmParams p, int tiles_m) {
   extern __shared__ __align__(16) unsigned char smem[];
-  spmm_mfma2_block<BF16, IT, W>(p, blockIdx.x % tiles_m, blockIdx.x / tiles_m, blockIdx.y, smem);
+  spmm_mfma2_block<BF16, IT, W, BKA>(p, blockIdx.x % tiles_m, blockIdx.x / tiles_m, blockIdx.y, smem);
 }
 
-template <typename T, typename IT, int W>
+template <typename T, typename IT, int W, int BKA = 128>
 int launch_mfma2_one(const SpmmParams& p, int batch, hipStream_t stream) {
   constexpr bool kBf16 = std::is_same<T, __hip_bfloat16>::value;
+  constexpr int kMfma2LdsBytes = spmm_mfma2_lds_bytes<BKA>();
   const int tiles_m = ceil_div(p.m, kMfmaBM), tiles_n = ceil_div(p.n, kMfma2BN);
-  auto kernel = spmm_mfma2_kernel<kBf16, IT, W>;
+  auto kernel = spmm_mfma2_kernel<kBf16, IT, W, BKA>;
   static thread_local bool raised = false;
   if (!raised) {
     if (int rc = check_hip(hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
@@ -132,8 +133,9 @@ int launch_mfma2(const SpmmParams& p, int batch, int windows, hipStream_t stream
       case 1: return launch_mfma2_one<T, IT, 1>(p, batch, stream);
       case 2: return launch_mfma2_one<T, IT, 2>(p, batch, stream);
       case 4: return launch_mfma2_one<T, IT, 4>(p, batch, stream);
+      case 5: return launch_mfma2_one<T, IT, 5>(p, batch, stream);
     }
-    return fail(IEX_ERR_BAD_ARGUMENT, "spmm: windows of the matrix-core variant must be 1, 2 or 4 (got %d)", windows);
+    return fail(IEX_ERR_BAD_ARGUMENT, "spmm: windows of the matrix-core variant must be 1, 2, 4 or 5 (got %d)", windows);
   } else {
     return fail(IEX_ERR_UNSUPPORTED, "spmm: the matrix-core variant handles fp16 and bf16 only");
   }
@@ -264,7 +266,9 @@ MfmaChoice mfma_variant(const SpmmParams& p, int batch, const Choice& ch) {
   if (kind == 4 && !wide_ok) kind = 3;
   mc.kind = kind;
   if (kind == 3) mc.param = ch.lpg ? ch.lpg : (run > 24.0 ? 16 : 8);
-  else mc.param = ch.rpw ? ch.rpw : (run > 20.0 ? 4 : run > 8.0 ? 2 : 1);
+  // windows of 16 nonzeros per row: enough for the run of a chunk (2:4 rows have exactly 64 per
+  // chunk and need the fifth, or every row-visit would make one exposed pass to find nothing)
+  else mc.param = ch.rpw ? ch.rpw : (run > 56.0 ? 5 : run > 20.0 ? 4 : run > 8.0 ? 2 : 1);
   return mc;
 }
 

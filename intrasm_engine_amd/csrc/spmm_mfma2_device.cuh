@@ -7,6 +7,11 @@
 // nonzeros each, packed (column << 16 | 16-bit value) so that one unsigned compare against
 // (chunk end << 16) tells whether a nonzero belongs to the chunk.  After a row-visit the
 // windows are reloaded at the new cursor; they land during the next four steps.
+// BKA = columns of A per chunk.  With 128 (what the library launches) a row-visit happens once
+// per four steps and W windows may not hold a dense row's run: a loop with exposed loads picks up
+// the rest, and because of that loop the compiler drains every load in flight at each wait.
+// 64 with W = 4 always holds the whole run and needs no loop, but doubles the row-visits and
+// spills 150 bytes: measured 2-2.6x slower, so it is not instantiated.
 // Requirements (checked by the host): n % 8 == 0, 16-byte aligned dense operand and output,
 // k < 65535 (packed columns), ascending column indices without duplicates inside a row.
 #pragma once
@@ -17,7 +22,8 @@ namespace iex {
 constexpr int kMfma2BN = 512;
 constexpr int kMfma2LDB = kMfma2BN + kGemmLdbPad;
 constexpr int kMfma2Threads = 512;
-constexpr int kMfma2LdsBytes = (2 * kMfmaBM * kMfmaLDA + 2 * kGemmBK * kMfma2LDB) * 2;
+template <int BKA>
+constexpr int spmm_mfma2_lds_bytes() { return (2 * kMfmaBM * (BKA + 8) + 2 * kGemmBK * kMfma2LDB) * 2; }
 
 struct SpmmMfma2BStage {
   static constexpr int CHUNKS = kMfma2BN * kGemmBK / 8 / kMfma2Threads;  // 128-bit chunks per thread
@@ -45,14 +51,17 @@ struct SpmmMfma2BStage {
   }
 };
 
-template <bool BF16, typename IT, int W>
+template <bool BF16, typename IT, int W, int BKA>
 __device__ __forceinline__ void spmm_mfma2_block(const SpmmParams& p, int tile_m, int tile_n, int z, unsigned char* smem) {
-  constexpr int BM = kMfmaBM, BN = kMfma2BN, BK = kGemmBK, BKA = kMfmaBKA, LDA = kMfmaLDA, LDB = kMfma2LDB;
+  constexpr int BM = kMfmaBM, BN = kMfma2BN, BK = kGemmBK, LDA = BKA + 8, LDB = kMfma2LDB;
   constexpr int WM = 2, WN = 4;
   constexpr int LPR = 16;
   constexpr int GROUPS = kMfma2Threads / LPR;  // 32 lane groups
-  constexpr int R = BM / GROUPS;               // 4 rows per group = steps per chunk
-  static_assert(R == BKA / BK, "one row of a lane group per MFMA step of a chunk");
+  constexpr int R = BM / GROUPS;               // 4 rows per group
+  constexpr int SPC = BKA / BK;                // steps per chunk (4 or 2)
+  constexpr int RPS = R / SPC;                 // rows a lane group expands per step (1 or 2)
+  static_assert(BKA == 128 || BKA == 64, "chunk width");
+  static_assert(BK / 16 >= RPS, "one row-visit per 16-wide MFMA sub-step at most");
   constexpr unsigned kNone = 0xffffffffu;
   typedef unsigned short u16;
 
@@ -104,7 +113,8 @@ __device__ __forceinline__ void spmm_mfma2_block(const SpmmParams& p, int tile_m
   // come from the same wavefront, and LDS keeps the order of a wavefront's accesses.
   auto expand_row = [&](int j, int ka0, u16* abuf) {
     u16* rowp = abuf + (group + j * GROUPS) * LDA;
-    *reinterpret_cast<u32x4*>(rowp + sub * 8) = u32x4{0u, 0u, 0u, 0u};
+    if constexpr (BKA == 128) *reinterpret_cast<u32x4*>(rowp + sub * 8) = u32x4{0u, 0u, 0u, 0u};
+    else *reinterpret_cast<u32x2*>(rowp + sub * 4) = u32x2{0u, 0u};
     const int kend = ka0 + BKA;
     const unsigned lim = (unsigned)kend << 16;
     int consumed = 0;
@@ -116,19 +126,21 @@ __device__ __forceinline__ void spmm_mfma2_block(const SpmmParams& p, int tile_m
       consumed += __popcll((__ballot(in) >> gshift) & 0xffffull);
     }
     pos[j] += consumed;
-    bool more = consumed == W * LPR;
-    // A run longer than the windows held in registers: the loads of these passes are exposed.
-    // (Unrolling this loop into forward branches, so that the compiler could keep counting the
-    // loads in flight across it, was measured: the extra register pressure costs far more.)
-    while (__any(more)) {
-      unsigned e = kNone;
-      const int idx = pos[j] + sub;
-      if (more && idx < end[j]) e = ((unsigned)(u16)cols[idx] << 16) | (unsigned)values[idx];
-      const bool in = e < lim;
-      if (in) rowp[(int)(e >> 16) - ka0] = (u16)e;
-      const int cnt = __popcll((__ballot(in) >> gshift) & 0xffffull);
-      pos[j] += cnt;
-      more = cnt == LPR;
+    if constexpr (W * LPR < BKA) {
+      bool more = consumed == W * LPR;
+      // A run longer than the windows held in registers: the loads of these passes are exposed.
+      // (Unrolling this loop into forward branches, so that the compiler could keep counting the
+      // loads in flight across it, was measured: the extra register pressure costs far more.)
+      while (__any(more)) {
+        unsigned e = kNone;
+        const int idx = pos[j] + sub;
+        if (more && idx < end[j]) e = ((unsigned)(u16)cols[idx] << 16) | (unsigned)values[idx];
+        const bool in = e < lim;
+        if (in) rowp[(int)(e >> 16) - ka0] = (u16)e;
+        const int cnt = __popcll((__ballot(in) >> gshift) & 0xffffull);
+        pos[j] += cnt;
+        more = cnt == LPR;
+      }
     }
     load_windows(j);
   };
@@ -160,8 +172,8 @@ __device__ __forceinline__ void spmm_mfma2_block(const SpmmParams& p, int tile_m
     constexpr int J = decltype(jc)::value;
     constexpr int buf = J & 1;
     constexpr int set = (J + 1) & 1;
-    const int chunk = kt >> 2;
-    const u16* a = sA + (chunk & 1) * BM * LDA + (wm * WM * 32 + frag_row) * LDA + J * BK + frag_k;
+    const int chunk = kt / SPC;
+    const u16* a = sA + (chunk & 1) * BM * LDA + (wm * WM * 32 + frag_row) * LDA + (J % SPC) * BK + frag_k;
     const u16* b = sB + buf * BK * LDB + ((lane >> 5) * 8 + ((lane & 15) >> 2)) * LDB + wn * WN * 32 +
                    ((lane >> 4) & 1) * 16 + (lane & 3) * 4;
     const bool next_chunk = (chunk + 1) * BKA < p.k;
@@ -183,7 +195,7 @@ __device__ __forceinline__ void spmm_mfma2_block(const SpmmParams& p, int tile_m
       for (int i = 0; i < WM; ++i)
 #pragma unroll
         for (int j = 0; j < WN; ++j) acc[i][j] = mfma_32x32x16<BF16>(fb[j], fa[i], acc[i][j]);
-      if (ks == 0 && next_chunk) expand_row(J, (chunk + 1) * BKA, sA + ((chunk + 1) & 1) * BM * LDA);
+      if (ks < RPS && next_chunk) expand_row((J % SPC) * RPS + ks, (chunk + 1) * BKA, sA + ((chunk + 1) & 1) * BM * LDA);
     }
     if (kt + 1 < KT) {
       regs[set].store(sB + (buf ^ 1) * BK * LDB, tid);

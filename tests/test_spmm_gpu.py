@@ -309,7 +309,7 @@ def test_lds_staged_variant(oracle, dev, rpw, dtype, n):
                        pyops._spmm(bi, ri, v, ro_t, ci_t, m, force_variant=1, **kw))
 
 
-@pytest.mark.parametrize("family,knob", [(3, 8), (3, 16), (4, 1), (4, 2), (4, 4)])
+@pytest.mark.parametrize("family,knob", [(3, 8), (3, 16), (4, 1), (4, 2), (4, 4), (4, 5)])
 @pytest.mark.parametrize("dtype,n,itype", [(torch.float16, 264, torch.int16), (torch.float16, 512, torch.int32),
                                            (torch.bfloat16, 776, torch.int32), (torch.float16, 8, torch.int16)])
 def test_matrix_core_variants(oracle, dev, family, knob, dtype, n, itype):

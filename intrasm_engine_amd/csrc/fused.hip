@@ -10,11 +10,17 @@
 //                     dispatched side by side from start to end while the tiles of a group
 //                     still share their operand panels in L2.
 // The GEMM may be batched (tiles of all batch entries are enumerated).
-// Every workgroup has 256 threads and the LDS of the larger role (the GEMM's 40 KB).
+// Two kernels, picked by what the stand-alone SpMM of the same shape would run on:
+//   gather     256 threads; GEMM tiles of 128 x 128 beside row blocks of the row kernel (at most 4
+//              wavefronts per row); LDS of the larger role (the GEMM's 40 KB);
+//   matrix     512 threads; GEMM tiles of 128 x 256 (2 x 4 wavefronts) beside 128 x 512 tiles of
+//   cores      the 8-wave matrix-core SpMM.  Both roles then want the matrix cores: the launch is
+//              a grouped GEMM whose sparse member is expanded in LDS, and what fusing buys is
+//              one launch and full tails, not complementary units.
 // The device code of both roles is the code of the stand-alone kernels, so results are
-// bit-identical to separate launches (the SpMM with at most 4 wavefronts per row).
+// bit-identical to separate launches.
 #include "gemm_device.cuh"
-#include "spmm_device.cuh"
+#include "spmm_mfma2_device.cuh"
 
 namespace iex {
 namespace {
@@ -30,13 +36,9 @@ constexpr int kFusedWM = 2, kFusedWN = 2;
 // missing waves by keeping four times as many gathers in flight per wave.
 constexpr int kFusedWin = 32;
 
-template <bool BF16, bool TRANS_B, typename IT, int VEC, int LPG, int WPR>
-__global__ __launch_bounds__(256) void fused_kernel(FusedParams p) {
-  extern __shared__ __align__(16) unsigned char smem[];
-  const int b = blockIdx.x;
+// Role of workgroup b: GEMM tile `idx` or SpMM block `idx`.
+__device__ __forceinline__ void fused_role(const FusedParams& p, int b, bool& is_gemm, int& idx) {
   const long long total = (long long)p.gemm_blocks + p.spmm_blocks;
-  bool is_gemm;
-  int idx;
   if (p.interleave > 0) {
     // GEMM tiles in groups of `interleave` consecutive ids; group q starts at id q*total/groups
     const int gsz = p.interleave;
@@ -52,6 +54,14 @@ __global__ __launch_bounds__(256) void fused_kernel(FusedParams p) {
     is_gemm = b < p.gemm_blocks;
     idx = is_gemm ? b : b - p.gemm_blocks;
   }
+}
+
+template <bool BF16, bool TRANS_B, typename IT, int VEC, int LPG, int WPR>
+__global__ __launch_bounds__(256) void fused_kernel(FusedParams p) {
+  extern __shared__ __align__(16) unsigned char smem[];
+  bool is_gemm;
+  int idx;
+  fused_role(p, blockIdx.x, is_gemm, idx);
   if (is_gemm) {
     const int per_batch = p.g.tiles_m * p.g.tiles_n;
     const int z = idx / per_batch, t = idx % per_batch;
@@ -59,6 +69,69 @@ __global__ __launch_bounds__(256) void fused_kernel(FusedParams p) {
   } else {
     spmm_block<__half, IT, VEC, LPG, WPR, kFusedWin>(p.s, idx / p.spmm_by, idx % p.spmm_by, 0, reinterpret_cast<float*>(smem));
   }
+}
+
+// ---- both roles on the matrix cores -------------------------------------------------------------
+constexpr int kFusedMcWM = 2, kFusedMcWN = 2, kFusedMcWCN = 4;  // GEMM tile 128 x 256 by 2 x 4 wavefronts
+
+template <bool BF16, bool TRANS_B, typename IT, int W>
+__global__ __launch_bounds__(kMfma2Threads, 2) void fused_mc_kernel(FusedParams p) {
+  extern __shared__ __align__(16) unsigned char smem[];
+  bool is_gemm;
+  int idx;
+  fused_role(p, blockIdx.x, is_gemm, idx);
+  if (is_gemm) {
+    const int per_batch = p.g.tiles_m * p.g.tiles_n;
+    const int z = idx / per_batch, t = idx % per_batch;
+    gemm_tile<BF16, TRANS_B, kFusedMcWM, kFusedMcWN, kGemmSets, kFusedMcWCN>(p.g, t / p.g.tiles_n, t % p.g.tiles_n, z, smem);
+  } else {
+    // p.spmm_by = row tiles here: consecutive ids walk the row blocks of one column panel
+    spmm_mfma2_block<false, IT, W, 128>(p.s, idx % p.spmm_by, idx / p.spmm_by, 0, smem);
+  }
+}
+
+template <bool BF16, bool TRANS_B, typename IT, int W>
+int launch_mc(FusedParams p, hipStream_t stream) {
+  constexpr int BM = 2 * kFusedMcWM * 32, BN = kFusedMcWCN * kFusedMcWN * 32;
+  p.g.tiles_m = ceil_div(p.g.M, BM);
+  p.g.tiles_n = ceil_div(p.g.N, BN);
+  IEX_REQUIRE((long long)p.g.tiles_m * p.g.tiles_n * p.gemm_batch < (1ll << 30), IEX_ERR_TOO_LARGE, "fused: too many GEMM tiles");
+  p.gemm_blocks = p.g.tiles_m * p.g.tiles_n * p.gemm_batch;
+  p.spmm_by = ceil_div(p.s.m, kMfmaBM);
+  p.spmm_blocks = p.spmm_by * ceil_div(p.s.n, kMfma2BN);
+  constexpr int lds_gemm = gemm_lds_bytes<TRANS_B, kFusedMcWM, kFusedMcWN, kFusedMcWCN>();
+  constexpr int lds_spmm = spmm_mfma2_lds_bytes<128>();
+  constexpr int lds = lds_gemm > lds_spmm ? lds_gemm : lds_spmm;
+  auto kernel = fused_mc_kernel<BF16, TRANS_B, IT, W>;
+  static thread_local bool raised = false;  // per instantiation: more than 64 KB of dynamic LDS
+  if (!raised) {
+    if (int rc = check_hip(hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
+                                               hipFuncAttributeMaxDynamicSharedMemorySize, lds),
+                           "hipFuncSetAttribute(LDS size)"))
+      return rc;
+    raised = true;
+  }
+  hipLaunchKernelGGL(kernel, dim3(p.gemm_blocks + p.spmm_blocks), dim3(kMfma2Threads), lds, stream, p);
+  return check_hip(hipGetLastError(), "fused (matrix-core) launch");
+}
+
+template <bool BF16, bool TRANS_B, typename IT>
+int launch_mc_w(const FusedParams& p, int windows, hipStream_t stream) {
+  switch (windows) {
+    case 1: return launch_mc<BF16, TRANS_B, IT, 1>(p, stream);
+    case 2: return launch_mc<BF16, TRANS_B, IT, 2>(p, stream);
+    case 4: return launch_mc<BF16, TRANS_B, IT, 4>(p, stream);
+    case 5: return launch_mc<BF16, TRANS_B, IT, 5>(p, stream);
+  }
+  return fail(IEX_ERR_BAD_ARGUMENT, "fused: unexpected window count %d", windows);
+}
+
+template <typename IT>
+int launch_mc_kind(const FusedParams& p, int windows, bool bf16, bool trans_b, hipStream_t stream) {
+  if (bf16 && trans_b) return launch_mc_w<true, true, IT>(p, windows, stream);
+  if (bf16 && !trans_b) return launch_mc_w<true, false, IT>(p, windows, stream);
+  if (!bf16 && trans_b) return launch_mc_w<false, true, IT>(p, windows, stream);
+  return launch_mc_w<false, false, IT>(p, windows, stream);
 }
 
 template <bool BF16, bool TRANS_B, typename IT, int VEC, int LPG, int WPR>
@@ -143,8 +216,12 @@ extern "C" int iex_fused_spmm_gemm(int spmm_itype, int m, int k, int n, int nonz
   p.gemm_batch = gemm_batch;
   p.s = SpmmParams{m, k, n, nonzeros, row_indices, values, row_offsets, column_indices, dense, nullptr, spmm_out, 0, 0, 0};
   p.interleave = interleave;
-  const SpmmShape vec = spmm_pick_shape<__half>(n, dense, spmm_out);
   hipStream_t s = static_cast<hipStream_t>(stream);
+  if (const int windows = spmm_matrix_core_windows(p.s)) {  // what the stand-alone SpMM of this shape runs on
+    if (spmm_itype == IEX_I16) return launch_mc_kind<short>(p, windows, gemm_dtype == IEX_BF16, trans_b != 0, s);
+    return launch_mc_kind<int>(p, windows, gemm_dtype == IEX_BF16, trans_b != 0, s);
+  }
+  const SpmmShape vec = spmm_pick_shape<__half>(n, dense, spmm_out);
   if (spmm_itype == IEX_I16) return launch_gemm_kind<short>(p, vec, gemm_dtype == IEX_BF16, trans_b != 0, s);
   return launch_gemm_kind<int>(p, vec, gemm_dtype == IEX_BF16, trans_b != 0, s);
 }

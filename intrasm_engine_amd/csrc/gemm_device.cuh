@@ -1,8 +1,9 @@
 // Dense companion GEMM for gfx950: C = A * B (or A * B^T), fp16 / bf16 in, fp32
 // accumulate on the matrix cores (v_mfma_f32_32x32x16_{f16,bf16}), LDS double-buffered.
 //
-// Tiling: a workgroup of 4 wavefronts (2 x 2) owns a (2*WM*32) x (2*WN*32) tile of C;
-// a wavefront owns WM x WN MFMA tiles of 32 x 32.  The K loop advances BK = 32 per step.
+// Tiling: a workgroup of 2 x WCN wavefronts (WCN = 2, or 4 for the 512-thread workgroups of
+// the fused launch) owns a (2*WM*32) x (WCN*WN*32) tile of C; a wavefront owns WM x WN MFMA
+// tiles of 32 x 32.  The K loop advances BK = 32 per step.
 // Software pipeline: global loads run kGemmSets steps ahead of the MFMAs (one register set
 // per step in flight, 128-bit loads), a set is written to the idle LDS buffer one step
 // before it is consumed, one barrier per step:
@@ -45,10 +46,10 @@ constexpr int kGemmSets = 3;                 // register sets = K steps of globa
 
 constexpr int kGemmLdbPad = 32;  // padding of a [k][n] row of B in LDS, elements
 
-template <bool TRANS_B, int WM, int WN>
+template <bool TRANS_B, int WM, int WN, int WCN = 2>
 constexpr int gemm_lds_bytes() {
   constexpr int a_elems = 2 * WM * 32 * kGemmLd;
-  constexpr int b_elems = TRANS_B ? 2 * WN * 32 * kGemmLd : kGemmBK * (2 * WN * 32 + kGemmLdbPad);
+  constexpr int b_elems = TRANS_B ? WCN * WN * 32 * kGemmLd : kGemmBK * (WCN * WN * 32 + kGemmLdbPad);
   return 2 /*buffers*/ * (a_elems + b_elems) * 2 /*bytes*/;
 }
 
@@ -75,12 +76,13 @@ __device__ __forceinline__ unsigned short f32_to_16(float v, bool bf16) {
 }
 
 // The slice of one K step that a thread carries from global memory to LDS.
-template <bool TRANS_B, int BM, int BN>
+template <bool TRANS_B, int BM, int BN, int THREADS = 256>
 struct GemmStage {
   static constexpr int BK = kGemmBK;
   static constexpr int LD = kGemmLd;
-  static constexpr int A_CHUNKS = BM * (BK / 8) / 256;       // 128-bit chunks per thread (A, and B^T layout)
-  static constexpr int B_CHUNKS = BN * (BK / 8) / 256;
+  static constexpr int A_CHUNKS = BM * (BK / 8) / THREADS;   // 128-bit chunks per thread (A, and B^T layout)
+  static constexpr int B_CHUNKS = BN * (BK / 8) / THREADS;
+  static_assert(A_CHUNKS >= 1 && B_CHUNKS >= 1, "a stage must give every thread a chunk of A and of B");
   static constexpr int LDB = BN + kGemmLdbPad;               // LDS row stride of B kept as [k][n]
   static constexpr int B_ELEMS = TRANS_B ? BN * LD : BK * LDB;  // one LDS buffer of B, elements
   typedef unsigned short u16;
@@ -93,7 +95,7 @@ struct GemmStage {
     const int k0 = kt * BK;
 #pragma unroll
     for (int c = 0; c < A_CHUNKS; ++c) {
-      const int chunk = tid + c * 256;
+      const int chunk = tid + c * THREADS;
       const int row = chunk / (BK / 8), kc = chunk % (BK / 8);
       const int gm = m0 + row, gk = k0 + kc * 8;
       u32x4 v = {0u, 0u, 0u, 0u};
@@ -103,7 +105,7 @@ struct GemmStage {
     if constexpr (TRANS_B) {
 #pragma unroll
       for (int c = 0; c < B_CHUNKS; ++c) {
-        const int chunk = tid + c * 256;
+        const int chunk = tid + c * THREADS;
         const int row = chunk / (BK / 8), kc = chunk % (BK / 8);
         const int gn = n0 + row, gk = k0 + kc * 8;
         u32x4 v = {0u, 0u, 0u, 0u};
@@ -113,7 +115,7 @@ struct GemmStage {
     } else {
 #pragma unroll
       for (int c = 0; c < B_CHUNKS; ++c) {
-        const int chunk = tid + c * 256;
+        const int chunk = tid + c * THREADS;
         const int kr = chunk / (BN / 8), nc = chunk % (BN / 8);
         const int gk = k0 + kr, gn = n0 + nc * 8;
         u32x4 v = {0u, 0u, 0u, 0u};
@@ -126,21 +128,21 @@ struct GemmStage {
   __device__ __forceinline__ void store(u16* a, u16* b, int tid) const {
 #pragma unroll
     for (int c = 0; c < A_CHUNKS; ++c) {
-      const int chunk = tid + c * 256;
+      const int chunk = tid + c * THREADS;
       const int row = chunk / (BK / 8), kc = chunk % (BK / 8);
       *reinterpret_cast<u32x4*>(a + row * LD + kc * 8) = ra[c];
     }
     if constexpr (TRANS_B) {
 #pragma unroll
       for (int c = 0; c < B_CHUNKS; ++c) {
-        const int chunk = tid + c * 256;
+        const int chunk = tid + c * THREADS;
         const int row = chunk / (BK / 8), kc = chunk % (BK / 8);
         *reinterpret_cast<u32x4*>(b + row * LD + kc * 8) = rb[c];
       }
     } else {
 #pragma unroll
       for (int c = 0; c < B_CHUNKS; ++c) {
-        const int chunk = tid + c * 256;
+        const int chunk = tid + c * THREADS;
         const int kr = chunk / (BN / 8), nc = chunk % (BN / 8);
         *reinterpret_cast<u32x4*>(b + kr * LDB + nc * 8) = rb[c];
       }
@@ -149,18 +151,18 @@ struct GemmStage {
 };
 
 // One C tile.  `smem` must hold gemm_lds_bytes<WM,WN>() bytes, 16-byte aligned.
-// All 256 threads of the workgroup must call this (it contains barriers).
-template <bool BF16, bool TRANS_B, int WM, int WN, int SETS = kGemmSets>
+// All 2 * WCN * 64 threads of the workgroup must call this (it contains barriers).
+template <bool BF16, bool TRANS_B, int WM, int WN, int SETS = kGemmSets, int WCN = 2>
 __device__ __forceinline__ void gemm_tile(const GemmParams& p, int tile_m, int tile_n, int z, unsigned char* smem) {
   constexpr int BM = 2 * WM * 32;
-  constexpr int BN = 2 * WN * 32;
+  constexpr int BN = WCN * WN * 32;
   constexpr int BK = kGemmBK;
   constexpr int LD = kGemmLd;
   static_assert(SETS == 2 || SETS == 3, "register sets in flight");
   constexpr int PERIOD = SETS == 2 ? 2 : 6;  // steps after which LDS buffer and register set repeat
   typedef unsigned short u16;
 
-  typedef GemmStage<TRANS_B, BM, BN> Stage;
+  typedef GemmStage<TRANS_B, BM, BN, 2 * WCN * 64> Stage;
   constexpr int LDB = Stage::LDB;
   constexpr int B_ELEMS = Stage::B_ELEMS;
   u16* sA = reinterpret_cast<u16*>(smem);  // [2][BM][LD]
@@ -169,7 +171,7 @@ __device__ __forceinline__ void gemm_tile(const GemmParams& p, int tile_m, int t
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int wave = tid >> 6;
-  const int wm = wave >> 1, wn = wave & 1;
+  const int wm = wave / WCN, wn = wave % WCN;
   const int m0 = tile_m * BM, n0 = tile_n * BN;
   const u16* __restrict__ A = static_cast<const u16*>(p.A) + (size_t)z * p.stride_a;
   const u16* __restrict__ B = static_cast<const u16*>(p.B) + (size_t)z * p.stride_b;

@@ -337,6 +337,13 @@ int launch_typed(const SpmmParams& p, int batch, const Choice& ch, hipStream_t s
 
 }  // namespace
 
+// For the fused launcher: the number of register windows if the dispatcher would run this
+// fp16 SpMM (one batch entry, nothing forced) on the 8-wave matrix-core kernel, else 0.
+int spmm_matrix_core_windows(const SpmmParams& p) {
+  const MfmaChoice mc = mfma_variant<__half>(p, 1, Choice{});
+  return mc.kind == 4 ? mc.param : 0;
+}
+
 int spmm_dispatch(int dtype, int itype, int flags, int m, int k, int n, int nonzeros,
                   const int* row_indices, const void* values, const int* row_offsets,
                   const void* column_indices, const void* dense, const float* bias, void* out,

@@ -275,4 +275,8 @@ inline int spmm_pick_wpr(int m, int nnz) {
   return mean >= 24.0 ? 4 : 1;
 }
 
+// Defined with the dispatcher (spmm.hip): register windows of the 8-wave matrix-core kernel if
+// that is what an fp16 SpMM of this shape runs on, else 0.
+int spmm_matrix_core_windows(const SpmmParams& p);
+
 }  // namespace iex

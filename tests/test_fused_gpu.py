@@ -35,15 +35,37 @@ def test_fused_equals_separate_launches(dev, interleave, gdtype, trans_b, n, idt
 
 
 def test_fused_config4_shape(dev):
+    """At this shape the stand-alone SpMM runs on the 8-wave matrix-core kernel, and so does the
+    sparse role of the fused launch (512-thread workgroups beside 128 x 256 GEMM tiles): both
+    outputs stay bit-identical to the separate launches, for both layouts of B and both
+    workgroup-role layouts."""
     w, x, ga, gb = W.config4()
     ri, v, ro, ci = to_dev(w, dev, torch.float16, torch.int16)
     xt = torch.from_numpy(x).to(dev).half()
     gat, gbt = torch.from_numpy(ga).to(dev).bfloat16(), torch.from_numpy(gb).to(dev).bfloat16()
-    out, c = ops.fused_spmm_gemm(xt, ri, v, ro, ci, w.m, gat, gbt, False, 1)
-    assert torch.equal(out, _row_kernel_spmm(xt, ri, v, ro, ci, w.m))
-    auto = ops.spmm_sputnik_reuse_weight_half(xt, ri, v, ro, ci, w.m)   # picks a matrix-core kernel at this shape
-    assert torch.allclose(out.float(), auto.float(), rtol=1e-2, atol=1e-2)
-    assert torch.equal(c, ops.gemm_mfma(gat, gbt, False))
+    alone = ops.spmm_sputnik_reuse_weight_half(xt, ri, v, ro, ci, w.m)
+    assert not torch.equal(alone, _row_kernel_spmm(xt, ri, v, ro, ci, w.m))     # i.e. not the row kernel
+    c_alone = ops.gemm_mfma(gat, gbt, False)
+    for interleave in (1, 0, 16):
+        out, c = ops.fused_spmm_gemm(xt, ri, v, ro, ci, w.m, gat, gbt, False, interleave)
+        assert torch.equal(out, alone) and torch.equal(c, c_alone), interleave
+    gbt_t = gbt.t().contiguous()
+    out, c = ops.fused_spmm_gemm(xt, ri, v, ro, ci, w.m, gat, gbt_t, True, 0)
+    assert torch.equal(out, alone) and torch.equal(c, ops.gemm_mfma(gat, gbt_t, True))
+
+
+def test_fused_matrix_core_batched_gemm(dev):
+    """Matrix-core fused launch with a batched, ragged GEMM (the attention products of the
+    decoder layer ride along like this) and int32 column indices."""
+    rng = np.random.default_rng(9)
+    a = W.pruned_weight(77, 2048, 640, 0.8)
+    ri, v, ro, ci = to_dev(a, dev, torch.float16, torch.int32)
+    x = torch.from_numpy(rng.standard_normal((1, 640, 4096)).astype(np.float32)).to(dev).half()
+    q = torch.from_numpy(rng.standard_normal((6, 200, 72)).astype(np.float32)).to(dev).half()
+    kmat = torch.from_numpy(rng.standard_normal((6, 136, 72)).astype(np.float32)).to(dev).half()
+    out, c = ops.fused_spmm_gemm(x, ri, v, ro, ci, a.m, q, kmat, True, 0)
+    assert torch.equal(out, ops.spmm_sputnik_reuse_weight_half(x, ri, v, ro, ci, a.m))
+    assert torch.equal(c, ops.gemm_mfma(q, kmat, True))
 
 
 def test_argument_checks(dev):

@@ -212,29 +212,33 @@ __device__ __forceinline__ void gemm_tile(const GemmParams& p, int tile_m, int t
     const u16* b = TRANS_B ? sB + buf * B_ELEMS + (wn * WN * 32 + frag_row) * LD + frag_k
                            : sB + buf * B_ELEMS + ((lane >> 5) * 8 + ((lane & 15) >> 2)) * LDB + wn * WN * 32 +
                                  ((lane >> 4) & 1) * 16 + (lane & 3) * 4;
+    // all operand fragments of the step are requested before the first MFMA: the reads of the
+    // second 16-wide sub-step land while the MFMAs of the first one run
+    u32x4 fa[BK / 16][WM], fb[BK / 16][WN];
 #pragma unroll
     for (int ks = 0; ks < BK / 16; ++ks) {
-      u32x4 fa[WM], fb[WN];
 #pragma unroll
-      for (int i = 0; i < WM; ++i) fa[i] = *reinterpret_cast<const u32x4*>(a + i * 32 * LD + ks * 16);
+      for (int i = 0; i < WM; ++i) fa[ks][i] = *reinterpret_cast<const u32x4*>(a + i * 32 * LD + ks * 16);
 #pragma unroll
       for (int j = 0; j < WN; ++j) {
         if constexpr (TRANS_B) {
-          fb[j] = *reinterpret_cast<const u32x4*>(b + j * 32 * LD + ks * 16);
+          fb[ks][j] = *reinterpret_cast<const u32x4*>(b + j * 32 * LD + ks * 16);
         } else {
           typedef __attribute__((address_space(3))) s16x4 lds_s16x4;
           const u16* q0 = b + (ks * 16) * LDB + j * 32;
           const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)(q0));
           const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)(q0 + 4 * LDB));
           const u32x2 l2 = __builtin_bit_cast(u32x2, lo), h2 = __builtin_bit_cast(u32x2, hi);
-          fb[j] = u32x4{l2.x, l2.y, h2.x, h2.y};
+          fb[ks][j] = u32x4{l2.x, l2.y, h2.x, h2.y};
         }
       }
+    }
+#pragma unroll
+    for (int ks = 0; ks < BK / 16; ++ks)
 #pragma unroll
       for (int i = 0; i < WM; ++i)
 #pragma unroll
-        for (int j = 0; j < WN; ++j) acc[i][j] = mfma_32x32x16<BF16>(fb[j], fa[i], acc[i][j]);
-    }
+        for (int j = 0; j < WN; ++j) acc[i][j] = mfma_32x32x16<BF16>(fb[ks][j], fa[ks][i], acc[i][j]);
     if (kt + 1 < KT) {
       regs[set].store(sA + (buf ^ 1) * BM * LD, sB + (buf ^ 1) * B_ELEMS, tid);
       if (kt + 1 + SETS < KT) regs[set].load(p, A, B, m0, n0, kt + 1 + SETS, tid);

@@ -20,24 +20,24 @@ __device__ __forceinline__ bool xcd_tile(int block, int tiles_m, int tiles_n, in
   return true;
 }
 
-template <bool BF16, bool TRANS_B, int WM, int WN>
+template <bool BF16, bool TRANS_B, int WM, int WN, int BK>
 __global__ __launch_bounds__(256, (WM * WN <= 8 ? 2 : 1)) void gemm_kernel(GemmParams p) {
   extern __shared__ __align__(16) unsigned char smem[];
   int tile_m, tile_n;
   if (!xcd_tile(blockIdx.x, p.tiles_m, p.tiles_n, tile_m, tile_n)) return;  // uniform per block
   // 128 x 256 tiles: 128 accumulators per lane leave room for two register sets in flight, not three
-  gemm_tile<BF16, TRANS_B, WM, WN, (WM * WN == 8 ? 2 : kGemmSets)>(p, tile_m, tile_n, blockIdx.y, smem);
+  gemm_tile<BF16, TRANS_B, WM, WN, (WM * WN == 8 || (BK == 64 && !TRANS_B) ? 2 : kGemmSets), 2, BK>(p, tile_m, tile_n, blockIdx.y, smem);
 }
 
-template <bool BF16, bool TRANS_B, int WM, int WN>
+template <bool BF16, bool TRANS_B, int WM, int WN, int BK = kGemmBK>
 int launch(GemmParams p, int batch, hipStream_t stream) {
   constexpr int BM = 2 * WM * 32, BN = 2 * WN * 32;
   p.tiles_m = ceil_div(p.M, BM);
   p.tiles_n = ceil_div(p.N, BN);
   const int total = p.tiles_m * p.tiles_n;
   const int per_xcd = (total + kXcds - 1) / kXcds;
-  constexpr int lds = gemm_lds_bytes<TRANS_B, WM, WN>();
-  auto kern = gemm_kernel<BF16, TRANS_B, WM, WN>;
+  constexpr int lds = gemm_lds_bytes<TRANS_B, WM, WN, 2, BK>();
+  auto kern = gemm_kernel<BF16, TRANS_B, WM, WN, BK>;
   if (lds > 64 * 1024) {
     static thread_local bool raised = false;  // per instantiation
     if (!raised) {
@@ -57,6 +57,7 @@ int launch_shape(const GemmParams& p, int batch, int force, hipStream_t stream) 
   if (force == 1) return launch<BF16, TRANS_B, 2, 2>(p, batch, stream);
   if (force == 2) return launch<BF16, TRANS_B, 2, 4>(p, batch, stream);
   if (force == 3) return launch<BF16, TRANS_B, 4, 4>(p, batch, stream);
+  if (force == 4) return launch<BF16, TRANS_B, 2, 2, 64>(p, batch, stream);
   // 128x256 tiles (64x128 per wave: a third fewer LDS bytes per MFMA than 64x64) once there are
   // two of them per CU: 865-912 TFLOP/s against 710-736 with 128x128 tiles at 4096..11008 x 8192
   // x 4096..8192; below that 128x128 keeps more workgroups in flight (config 4's 4096 x 2048:
@@ -64,6 +65,9 @@ int launch_shape(const GemmParams& p, int batch, int force, hipStream_t stream) 
   // than noise and stay on request.
   const long long wide_tiles = (long long)ceil_div(p.M, 128) * ceil_div(p.N, 256) * batch;
   if (wide_tiles >= 512 && p.K >= 256) return launch<BF16, TRANS_B, 2, 4>(p, batch, stream);
+  // 128x128 tiles: K steps of 64 halve the barriers and double the distance between a global load
+  // and its use (670-830 TFLOP/s against 640-740 with steps of 32 on the same shapes)
+  if (p.K >= 128) return launch<BF16, TRANS_B, 2, 2, 64>(p, batch, stream);
   return launch<BF16, TRANS_B, 2, 2>(p, batch, stream);
 }
 
@@ -71,7 +75,7 @@ int launch_shape(const GemmParams& p, int batch, int force, hipStream_t stream) 
 }  // namespace iex
 
 // trans_b: bit 0 = B is (N, K); bits 4..7 force the tile shape for tuning (1 = 128x128, 2 = 128x256,
-// 3 = 256x256; 0 = choose).
+// 3 = 256x256, 4 = 128x128 with K steps of 64; 0 = choose).
 extern "C" int iex_gemm(int dtype, int trans_b_and_shape, int M, int N, int K, const void* A, const void* B, void* C, int batch,
                         long long stride_a, long long stride_b, long long stride_c, void* stream) {
   using namespace iex;

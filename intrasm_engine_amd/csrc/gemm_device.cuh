@@ -46,10 +46,10 @@ constexpr int kGemmSets = 3;                 // register sets = K steps of globa
 
 constexpr int kGemmLdbPad = 32;  // padding of a [k][n] row of B in LDS, elements
 
-template <bool TRANS_B, int WM, int WN, int WCN = 2>
+template <bool TRANS_B, int WM, int WN, int WCN = 2, int BK = kGemmBK>
 constexpr int gemm_lds_bytes() {
-  constexpr int a_elems = 2 * WM * 32 * kGemmLd;
-  constexpr int b_elems = TRANS_B ? WCN * WN * 32 * kGemmLd : kGemmBK * (WCN * WN * 32 + kGemmLdbPad);
+  constexpr int a_elems = 2 * WM * 32 * (BK + kGemmPad);
+  constexpr int b_elems = TRANS_B ? WCN * WN * 32 * (BK + kGemmPad) : BK * (WCN * WN * 32 + kGemmLdbPad);
   return 2 /*buffers*/ * (a_elems + b_elems) * 2 /*bytes*/;
 }
 
@@ -76,10 +76,10 @@ __device__ __forceinline__ unsigned short f32_to_16(float v, bool bf16) {
 }
 
 // The slice of one K step that a thread carries from global memory to LDS.
-template <bool TRANS_B, int BM, int BN, int THREADS = 256>
+template <bool TRANS_B, int BM, int BN, int THREADS = 256, int BK_ = kGemmBK>
 struct GemmStage {
-  static constexpr int BK = kGemmBK;
-  static constexpr int LD = kGemmLd;
+  static constexpr int BK = BK_;
+  static constexpr int LD = BK_ + kGemmPad;
   static constexpr int A_CHUNKS = BM * (BK / 8) / THREADS;   // 128-bit chunks per thread (A, and B^T layout)
   static constexpr int B_CHUNKS = BN * (BK / 8) / THREADS;
   static_assert(A_CHUNKS >= 1 && B_CHUNKS >= 1, "a stage must give every thread a chunk of A and of B");
@@ -152,17 +152,16 @@ struct GemmStage {
 
 // One C tile.  `smem` must hold gemm_lds_bytes<WM,WN>() bytes, 16-byte aligned.
 // All 2 * WCN * 64 threads of the workgroup must call this (it contains barriers).
-template <bool BF16, bool TRANS_B, int WM, int WN, int SETS = kGemmSets, int WCN = 2>
+template <bool BF16, bool TRANS_B, int WM, int WN, int SETS = kGemmSets, int WCN = 2, int BK = kGemmBK>
 __device__ __forceinline__ void gemm_tile(const GemmParams& p, int tile_m, int tile_n, int z, unsigned char* smem) {
   constexpr int BM = 2 * WM * 32;
   constexpr int BN = WCN * WN * 32;
-  constexpr int BK = kGemmBK;
-  constexpr int LD = kGemmLd;
+  constexpr int LD = BK + kGemmPad;
   static_assert(SETS == 2 || SETS == 3, "register sets in flight");
   constexpr int PERIOD = SETS == 2 ? 2 : 6;  // steps after which LDS buffer and register set repeat
   typedef unsigned short u16;
 
-  typedef GemmStage<TRANS_B, BM, BN, 2 * WCN * 64> Stage;
+  typedef GemmStage<TRANS_B, BM, BN, 2 * WCN * 64, BK> Stage;
   constexpr int LDB = Stage::LDB;
   constexpr int B_ELEMS = Stage::B_ELEMS;
   u16* sA = reinterpret_cast<u16*>(smem);  // [2][BM][LD]
@@ -212,33 +211,37 @@ __device__ __forceinline__ void gemm_tile(const GemmParams& p, int tile_m, int t
     const u16* b = TRANS_B ? sB + buf * B_ELEMS + (wn * WN * 32 + frag_row) * LD + frag_k
                            : sB + buf * B_ELEMS + ((lane >> 5) * 8 + ((lane & 15) >> 2)) * LDB + wn * WN * 32 +
                                  ((lane >> 4) & 1) * 16 + (lane & 3) * 4;
-    // all operand fragments of the step are requested before the first MFMA: the reads of the
-    // second 16-wide sub-step land while the MFMAs of the first one run
-    u32x4 fa[BK / 16][WM], fb[BK / 16][WN];
+    // the operand fragments of two 16-wide sub-steps are requested before their MFMAs: the reads
+    // of the second land while the MFMAs of the first run
 #pragma unroll
-    for (int ks = 0; ks < BK / 16; ++ks) {
+    for (int kp = 0; kp < BK / 32; ++kp) {
+      u32x4 fa[2][WM], fb[2][WN];
 #pragma unroll
-      for (int i = 0; i < WM; ++i) fa[ks][i] = *reinterpret_cast<const u32x4*>(a + i * 32 * LD + ks * 16);
+      for (int h = 0; h < 2; ++h) {
+        const int ks = kp * 2 + h;
 #pragma unroll
-      for (int j = 0; j < WN; ++j) {
-        if constexpr (TRANS_B) {
-          fb[ks][j] = *reinterpret_cast<const u32x4*>(b + j * 32 * LD + ks * 16);
-        } else {
-          typedef __attribute__((address_space(3))) s16x4 lds_s16x4;
-          const u16* q0 = b + (ks * 16) * LDB + j * 32;
-          const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)(q0));
-          const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)(q0 + 4 * LDB));
-          const u32x2 l2 = __builtin_bit_cast(u32x2, lo), h2 = __builtin_bit_cast(u32x2, hi);
-          fb[ks][j] = u32x4{l2.x, l2.y, h2.x, h2.y};
+        for (int i = 0; i < WM; ++i) fa[h][i] = *reinterpret_cast<const u32x4*>(a + i * 32 * LD + ks * 16);
+#pragma unroll
+        for (int j = 0; j < WN; ++j) {
+          if constexpr (TRANS_B) {
+            fb[h][j] = *reinterpret_cast<const u32x4*>(b + j * 32 * LD + ks * 16);
+          } else {
+            typedef __attribute__((address_space(3))) s16x4 lds_s16x4;
+            const u16* q0 = b + (ks * 16) * LDB + j * 32;
+            const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)(q0));
+            const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)(q0 + 4 * LDB));
+            const u32x2 l2 = __builtin_bit_cast(u32x2, lo), h2 = __builtin_bit_cast(u32x2, hi);
+            fb[h][j] = u32x4{l2.x, l2.y, h2.x, h2.y};
+          }
         }
       }
+#pragma unroll
+      for (int h = 0; h < 2; ++h)
+#pragma unroll
+        for (int i = 0; i < WM; ++i)
+#pragma unroll
+          for (int j = 0; j < WN; ++j) acc[i][j] = mfma_32x32x16<BF16>(fb[h][j], fa[h][i], acc[i][j]);
     }
-#pragma unroll
-    for (int ks = 0; ks < BK / 16; ++ks)
-#pragma unroll
-      for (int i = 0; i < WM; ++i)
-#pragma unroll
-        for (int j = 0; j < WN; ++j) acc[i][j] = mfma_32x32x16<BF16>(fb[ks][j], fa[ks][i], acc[i][j]);
     if (kt + 1 < KT) {
       regs[set].store(sA + (buf ^ 1) * BM * LD, sB + (buf ^ 1) * B_ELEMS, tid);
       if (kt + 1 + SETS < KT) regs[set].load(p, A, B, m0, n0, kt + 1 + SETS, tid);

@@ -38,11 +38,11 @@ def test_gemm_ragged_n_with_transposed_b(oracle, dev, shape):
         ops.gemm_mfma(torch.zeros(8, 8, device=dev).half(), torch.zeros(8, shape[1] | 1, device=dev).half(), False)
 
 
-@pytest.mark.parametrize("shape_code", [1, 2, 3])
+@pytest.mark.parametrize("shape_code", [1, 2, 3, 4])
 @pytest.mark.parametrize("trans_b", [False, True])
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
 def test_every_tile_shape(oracle, dev, shape_code, trans_b, dtype):
-    """128x128, 128x256 and 256x256 tiles forced through the C ABI on a ragged problem
+    """128x128, 128x256, 256x256 tiles and 128x128 with K steps of 64 forced through the C ABI on a ragged problem
     (m, n and k leave partial tiles and a partial last K step)."""
     from intrasm_engine_amd import _lib
     rng = np.random.default_rng(shape_code)

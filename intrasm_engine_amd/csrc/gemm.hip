@@ -58,15 +58,18 @@ int launch_shape(const GemmParams& p, int batch, int force, hipStream_t stream) 
   if (force == 2) return launch<BF16, TRANS_B, 2, 4>(p, batch, stream);
   if (force == 3) return launch<BF16, TRANS_B, 4, 4>(p, batch, stream);
   if (force == 4) return launch<BF16, TRANS_B, 2, 2, 64>(p, batch, stream);
-  // 128x256 tiles (64x128 per wave: a third fewer LDS bytes per MFMA than 64x64) once there are
-  // two of them per CU: 865-912 TFLOP/s against 710-736 with 128x128 tiles at 4096..11008 x 8192
-  // x 4096..8192; below that 128x128 keeps more workgroups in flight (config 4's 4096 x 2048:
-  // 643 vs 575).  256x256 tiles (one wave per SIMD, 504 registers) never beat 128x256 by more
-  // than noise and stay on request.
+  // The larger the tile of a wave, the fewer LDS bytes each MFMA needs (128x128 per wave: half of
+  // what 64x64 needs), and LDS bandwidth is what the main loop runs against; the smaller the tile,
+  // the more workgroups there are to fill 256 CUs.  Measured at 4096..11008 x 8192 x 4096..8192:
+  // 256x256 tiles (one wave per SIMD, 504 registers) 830-960 TFLOP/s, 128x256 770-890, 128x128
+  // 715-770; at config 4's 4096 x 2048 x 4096 the order reverses (450-470, 620-690, 720-750).
+  // Two tiles per CU is where the larger shape starts to win.
+  const long long huge_tiles = (long long)ceil_div(p.M, 256) * ceil_div(p.N, 256) * batch;
+  if (huge_tiles >= 512 && p.K >= 256) return launch<BF16, TRANS_B, 4, 4>(p, batch, stream);
   const long long wide_tiles = (long long)ceil_div(p.M, 128) * ceil_div(p.N, 256) * batch;
   if (wide_tiles >= 512 && p.K >= 256) return launch<BF16, TRANS_B, 2, 4>(p, batch, stream);
   // 128x128 tiles: K steps of 64 halve the barriers and double the distance between a global load
-  // and its use (670-830 TFLOP/s against 640-740 with steps of 32 on the same shapes)
+  // and its use (720-830 TFLOP/s against 660-770 with steps of 32 on the same shapes)
   if (p.K >= 128) return launch<BF16, TRANS_B, 2, 2, 64>(p, batch, stream);
   return launch<BF16, TRANS_B, 2, 2>(p, batch, stream);
 }

@@ -90,61 +90,66 @@ struct GemmStage {
   u32x4 ra[A_CHUNKS];
   u32x4 rb[B_CHUNKS];  // (N,K): chunk = 8 k of one n row; (K,N): chunk = 8 n of one k row
 
+  // Loads are unconditional, from addresses clamped into the matrices, and nothing is computed
+  // on their results here: guarded loads are branches, and behind a branch the compiler can no
+  // longer count the loads in flight and waits for all of them wherever one is needed.  Rows of A
+  // (columns of B) beyond the matrix only feed rows (columns) of C that are never stored; the K
+  // tail is zeroed when the set is written to LDS.
   __device__ __forceinline__ void load(const GemmParams& p, const u16* __restrict__ A, const u16* __restrict__ B, int m0,
                                        int n0, int kt, int tid) {
     const int k0 = kt * BK;
+    const int last_k8 = p.K - 8;  // K % 8 == 0: the last whole chunk of a row
 #pragma unroll
     for (int c = 0; c < A_CHUNKS; ++c) {
       const int chunk = tid + c * THREADS;
       const int row = chunk / (BK / 8), kc = chunk % (BK / 8);
-      const int gm = m0 + row, gk = k0 + kc * 8;
-      u32x4 v = {0u, 0u, 0u, 0u};
-      if (gm < p.M && gk < p.K) v = *reinterpret_cast<const u32x4*>(A + (size_t)gm * p.K + gk);
-      ra[c] = v;
+      const int gm = min(m0 + row, p.M - 1), gk = min(k0 + kc * 8, last_k8);
+      ra[c] = *reinterpret_cast<const u32x4*>(A + (size_t)gm * p.K + gk);
     }
     if constexpr (TRANS_B) {
 #pragma unroll
       for (int c = 0; c < B_CHUNKS; ++c) {
         const int chunk = tid + c * THREADS;
         const int row = chunk / (BK / 8), kc = chunk % (BK / 8);
-        const int gn = n0 + row, gk = k0 + kc * 8;
-        u32x4 v = {0u, 0u, 0u, 0u};
-        if (gn < p.N && gk < p.K) v = *reinterpret_cast<const u32x4*>(B + (size_t)gn * p.K + gk);
-        rb[c] = v;
+        const int gn = min(n0 + row, p.N - 1), gk = min(k0 + kc * 8, last_k8);
+        rb[c] = *reinterpret_cast<const u32x4*>(B + (size_t)gn * p.K + gk);
       }
     } else {
+      const int last_n8 = p.N - 8;  // N % 8 == 0 in this layout
 #pragma unroll
       for (int c = 0; c < B_CHUNKS; ++c) {
         const int chunk = tid + c * THREADS;
         const int kr = chunk / (BN / 8), nc = chunk % (BN / 8);
-        const int gk = k0 + kr, gn = n0 + nc * 8;
-        u32x4 v = {0u, 0u, 0u, 0u};
-        if (gk < p.K && gn < p.N) v = *reinterpret_cast<const u32x4*>(B + (size_t)gk * p.N + gn);
-        rb[c] = v;
+        const int gk = min(k0 + kr, p.K - 1), gn = min(n0 + nc * 8, last_n8);
+        rb[c] = *reinterpret_cast<const u32x4*>(B + (size_t)gk * p.N + gn);
       }
     }
   }
 
-  __device__ __forceinline__ void store(u16* a, u16* b, int tid) const {
+  // kt = the K step the set carries (for the K tail: entries at k >= K are written as zeros)
+  __device__ __forceinline__ void store(const GemmParams& p, u16* a, u16* b, int kt, int tid) const {
+    const int k0 = kt * BK;
+    const bool tail = k0 + BK > p.K;  // uniform
+    const u32x4 zero = {0u, 0u, 0u, 0u};
 #pragma unroll
     for (int c = 0; c < A_CHUNKS; ++c) {
       const int chunk = tid + c * THREADS;
       const int row = chunk / (BK / 8), kc = chunk % (BK / 8);
-      *reinterpret_cast<u32x4*>(a + row * LD + kc * 8) = ra[c];
+      *reinterpret_cast<u32x4*>(a + row * LD + kc * 8) = (tail && k0 + kc * 8 >= p.K) ? zero : ra[c];
     }
     if constexpr (TRANS_B) {
 #pragma unroll
       for (int c = 0; c < B_CHUNKS; ++c) {
         const int chunk = tid + c * THREADS;
         const int row = chunk / (BK / 8), kc = chunk % (BK / 8);
-        *reinterpret_cast<u32x4*>(b + row * LD + kc * 8) = rb[c];
+        *reinterpret_cast<u32x4*>(b + row * LD + kc * 8) = (tail && k0 + kc * 8 >= p.K) ? zero : rb[c];
       }
     } else {
 #pragma unroll
       for (int c = 0; c < B_CHUNKS; ++c) {
         const int chunk = tid + c * THREADS;
         const int kr = chunk / (BN / 8), nc = chunk % (BN / 8);
-        *reinterpret_cast<u32x4*>(b + kr * LDB + nc * 8) = rb[c];
+        *reinterpret_cast<u32x4*>(b + kr * LDB + nc * 8) = (tail && k0 + kr >= p.K) ? zero : rb[c];
       }
     }
   }
@@ -190,9 +195,9 @@ __device__ __forceinline__ void gemm_tile(const GemmParams& p, int tile_m, int t
   // prologue: tiles 0 .. SETS-1 in flight, tile 0 into LDS[0], then tile SETS replaces it
 #pragma unroll
   for (int s = 0; s < SETS; ++s)
-    if (s < KT) regs[s].load(p, A, B, m0, n0, s, tid);
-  regs[0].store(sA, sB, tid);
-  if (SETS < KT) regs[0].load(p, A, B, m0, n0, SETS, tid);
+    regs[s].load(p, A, B, m0, n0, s, tid);  // (a tile beyond the last one loads clamped addresses and is never used)
+  regs[0].store(p, sA, sB, 0, tid);
+  regs[0].load(p, A, B, m0, n0, SETS, tid);
   __syncthreads();
 
   const int frag_row = lane & 31;      // row of the 32-row operand block this lane feeds
@@ -242,10 +247,10 @@ __device__ __forceinline__ void gemm_tile(const GemmParams& p, int tile_m, int t
 #pragma unroll
           for (int j = 0; j < WN; ++j) acc[i][j] = mfma_32x32x16<BF16>(fb[h][j], fa[h][i], acc[i][j]);
     }
-    if (kt + 1 < KT) {
-      regs[set].store(sA + (buf ^ 1) * BM * LD, sB + (buf ^ 1) * B_ELEMS, tid);
-      if (kt + 1 + SETS < KT) regs[set].load(p, A, B, m0, n0, kt + 1 + SETS, tid);
-    }
+    // unconditional on purpose (see GemmStage::load): past the last tile this writes zeros to the
+    // idle buffer and fetches clamped addresses
+    regs[set].store(p, sA + (buf ^ 1) * BM * LD, sB + (buf ^ 1) * B_ELEMS, kt + 1, tid);
+    regs[set].load(p, A, B, m0, n0, kt + 1 + SETS, tid);
     __syncthreads();
   };
 

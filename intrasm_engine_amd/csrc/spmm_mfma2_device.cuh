@@ -4,14 +4,15 @@
 // shadow of the matrix cores.  See spmm_mfma_device.cuh for the idea.
 //
 // Expansion state per lane group (16 lanes own 4 rows): cursor, row end and W windows of 16
-// nonzeros each, packed (column << 16 | 16-bit value) so that one unsigned compare against
-// (chunk end << 16) tells whether a nonzero belongs to the chunk.  After a row-visit the
-// windows are reloaded at the new cursor; they land during the next four steps.
-// BKA = columns of A per chunk.  With 128 (what the library launches) a row-visit happens once
-// per four steps and W windows may not hold a dense row's run: a loop with exposed loads picks up
-// the rest, and because of that loop the compiler drains every load in flight at each wait.
-// 64 with W = 4 always holds the whole run and needs no loop, but doubles the row-visits and
-// spills 150 bytes: measured 2-2.6x slower, so it is not instantiated.
+// nonzeros each (value and column, as loaded).  After a row-visit the windows are reloaded at
+// the new cursor; they land during the next four steps.
+// BKA = columns of A per chunk (128: a row-visit once per four steps).  W windows may not hold a
+// dense row's run inside a chunk.  Then the workgroup multiplies the same chunk once more with
+// what the windows left behind (the products add up to the same sum), instead of a loop over
+// exposed loads inside the row-visit: every load of the main loop is unconditional and outside
+// any inner loop, so the compiler counts the loads in flight and each wait names exactly the
+// ones it needs.  The host picks W so that such a second pass is rare (W * 16 above the mean
+// run by a margin); a matrix with a few much denser rows pays one extra pass per chunk they touch.
 // Requirements (checked by the host): n % 8 == 0, 16-byte aligned dense operand and output,
 // k < 65535 (packed columns), ascending column indices without duplicates inside a row.
 #pragma once
@@ -23,7 +24,7 @@ constexpr int kMfma2BN = 512;
 constexpr int kMfma2LDB = kMfma2BN + kGemmLdbPad;
 constexpr int kMfma2Threads = 512;
 template <int BKA>
-constexpr int spmm_mfma2_lds_bytes() { return (2 * kMfmaBM * (BKA + 8) + 2 * kGemmBK * kMfma2LDB) * 2; }
+constexpr int spmm_mfma2_lds_bytes() { return (2 * kMfmaBM * (BKA + 8) + 2 * kGemmBK * kMfma2LDB) * 2 + 16; }
 
 struct SpmmMfma2BStage {
   static constexpr int CHUNKS = kMfma2BN * kGemmBK / 8 / kMfma2Threads;  // 128-bit chunks per thread
@@ -35,10 +36,11 @@ struct SpmmMfma2BStage {
     for (int c = 0; c < CHUNKS; ++c) {
       const int chunk = tid + c * kMfma2Threads;
       const int kr = chunk / (kMfma2BN / 8), nc = chunk % (kMfma2BN / 8);
-      const int gk = k0 + kr, gn = n0 + nc * 8;
-      u32x4 v = {0u, 0u, 0u, 0u};
-      if (gk < k && gn < n) v = *reinterpret_cast<const u32x4*>(B + (size_t)gk * n + gn);
-      rb[c] = v;
+      // unconditional, clamped into the matrix: a guarded load is a branch, and behind a branch the
+      // compiler waits for every load in flight wherever one is needed.  A k row beyond the matrix
+      // meets zeros of A, a column beyond n feeds columns of C that are never stored.
+      const int gk = min(k0 + kr, k - 1), gn = min(n0 + nc * 8, n - 8);
+      rb[c] = *reinterpret_cast<const u32x4*>(B + (size_t)gk * n + gn);
     }
   }
   __device__ __forceinline__ void store(u16* b, int tid) const {
@@ -59,14 +61,12 @@ __device__ __forceinline__ void spmm_mfma2_block(const SpmmParams& p, int tile_m
   constexpr int GROUPS = kMfma2Threads / LPR;  // 32 lane groups
   constexpr int R = BM / GROUPS;               // 4 rows per group
   constexpr int SPC = BKA / BK;                // steps per chunk (4 or 2)
-  constexpr int RPS = R / SPC;                 // rows a lane group expands per step (1 or 2)
-  static_assert(BKA == 128 || BKA == 64, "chunk width");
-  static_assert(BK / 16 >= RPS, "one row-visit per 16-wide MFMA sub-step at most");
-  constexpr unsigned kNone = 0xffffffffu;
+  static_assert(BKA == 128 && R == SPC, "one row of every lane group is expanded per step");
   typedef unsigned short u16;
 
   u16* sA = reinterpret_cast<u16*>(smem);  // [2][BM][LDA]
   u16* sB = sA + 2 * BM * LDA;             // [2][BK][LDB]
+  int* again = reinterpret_cast<int*>(sB + 2 * BK * LDB);  // [2], one per A buffer
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
@@ -110,13 +110,14 @@ __device__ __forceinline__ void spmm_mfma2_block(const SpmmParams& p, int tile_m
   }
 
   // Row j of this lane group, columns [ka0, ka0 + BKA) -> abuf.  The zero fill and the scatter
-  // come from the same wavefront, and LDS keeps the order of a wavefront's accesses.
-  auto expand_row = [&](int j, int ka0, u16* abuf) {
+  // come from the same wavefront, and LDS keeps the order of a wavefront's accesses.  A run that
+  // fills every window may continue beyond them: the row raises *again, and the workgroup gives
+  // the same chunk another pass with what is left (no loop over loads here: inside one, the
+  // compiler could no longer count the loads in flight and would drain them all at every wait).
+  auto expand_row = [&](int j, int ka0, u16* abuf, int* again) {
     u16* rowp = abuf + (group + j * GROUPS) * LDA;
-    if constexpr (BKA == 128) *reinterpret_cast<u32x4*>(rowp + sub * 8) = u32x4{0u, 0u, 0u, 0u};
-    else *reinterpret_cast<u32x2*>(rowp + sub * 4) = u32x2{0u, 0u};
+    *reinterpret_cast<u32x4*>(rowp + sub * 8) = u32x4{0u, 0u, 0u, 0u};
     const int kend = ka0 + BKA;
-    const unsigned lim = (unsigned)kend << 16;
     int consumed = 0;
 #pragma unroll
     for (int w = 0; w < W; ++w) {
@@ -126,22 +127,7 @@ __device__ __forceinline__ void spmm_mfma2_block(const SpmmParams& p, int tile_m
       consumed += __popcll((__ballot(in) >> gshift) & 0xffffull);
     }
     pos[j] += consumed;
-    if constexpr (W * LPR < BKA) {
-      bool more = consumed == W * LPR;
-      // A run longer than the windows held in registers: the loads of these passes are exposed.
-      // (Unrolling this loop into forward branches, so that the compiler could keep counting the
-      // loads in flight across it, was measured: the extra register pressure costs far more.)
-      while (__any(more)) {
-        unsigned e = kNone;
-        const int idx = pos[j] + sub;
-        if (more && idx < end[j]) e = ((unsigned)(u16)cols[idx] << 16) | (unsigned)values[idx];
-        const bool in = e < lim;
-        if (in) rowp[(int)(e >> 16) - ka0] = (u16)e;
-        const int cnt = __popcll((__ballot(in) >> gshift) & 0xffffull);
-        pos[j] += cnt;
-        more = cnt == LPR;
-      }
-    }
+    if (consumed == W * LPR) *again = 1;
     load_windows(j);
   };
 
@@ -153,30 +139,32 @@ __device__ __forceinline__ void spmm_mfma2_block(const SpmmParams& p, int tile_m
 #pragma unroll
       for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
 
-  SpmmMfma2BStage regs[2];  // regs[t % 2] carries B tile t
-  const int KT = (p.k + BK - 1) / BK;
+  if (tid < 2) again[tid] = 0;
+  __syncthreads();
+  SpmmMfma2BStage regs[2];  // regs[s % 2] carries the B tile of step s
+  const int chunks = (p.k + BKA - 1) / BKA;
   regs[0].load(B, p.k, p.n, n0, 0, tid);
-  if (1 < KT) regs[1].load(B, p.k, p.n, n0, 1, tid);
+  regs[1].load(B, p.k, p.n, n0, 1, tid);
 #pragma unroll
-  for (int j = 0; j < R; ++j) expand_row(j, 0, sA);
+  for (int j = 0; j < R; ++j) expand_row(j, 0, sA, again);
   regs[0].store(sB, tid);
-  if (2 < KT) regs[0].load(B, p.k, p.n, n0, 2, tid);
+  regs[0].load(B, p.k, p.n, n0, 2, tid);
   __syncthreads();
 
   const int frag_row = lane & 31;
   const int frag_k = (lane >> 5) * 8;
 
-  // One BK step; J = kt % 4 is static (row of the lane groups to expand, LDS buffer and
-  // register set of B alternate with its parity).
-  auto step = [&](int kt, auto jc) {
+  // Step J of a pass: multiply B tile J of chunk `cur` (LDS buffer J % 2) with columns
+  // [J * BK, J * BK + BK) of the expanded chunk in A buffer `ab`; expand row J of every lane group
+  // for chunk `nxt` into the other A buffer; hand the B tile of the next step to LDS and request
+  // the one three steps ahead (`ahead`; beyond the matrix it is clamped and meets zeros of A).
+  auto step = [&](int ab, int nxt, int ahead, auto jc) {
     constexpr int J = decltype(jc)::value;
     constexpr int buf = J & 1;
     constexpr int set = (J + 1) & 1;
-    const int chunk = kt / SPC;
-    const u16* a = sA + (chunk & 1) * BM * LDA + (wm * WM * 32 + frag_row) * LDA + (J % SPC) * BK + frag_k;
+    const u16* a = sA + ab * BM * LDA + (wm * WM * 32 + frag_row) * LDA + J * BK + frag_k;
     const u16* b = sB + buf * BK * LDB + ((lane >> 5) * 8 + ((lane & 15) >> 2)) * LDB + wn * WN * 32 +
                    ((lane >> 4) & 1) * 16 + (lane & 3) * 4;
-    const bool next_chunk = (chunk + 1) * BKA < p.k;
 #pragma unroll
     for (int ks = 0; ks < BK / 16; ++ks) {
       u32x4 fa[WM], fb[WN];
@@ -195,25 +183,26 @@ __device__ __forceinline__ void spmm_mfma2_block(const SpmmParams& p, int tile_m
       for (int i = 0; i < WM; ++i)
 #pragma unroll
         for (int j = 0; j < WN; ++j) acc[i][j] = mfma_32x32x16<BF16>(fb[j], fa[i], acc[i][j]);
-      if (ks < RPS && next_chunk) expand_row((J % SPC) * RPS + ks, (chunk + 1) * BKA, sA + ((chunk + 1) & 1) * BM * LDA);
+      if (ks == 0) expand_row(J, nxt * BKA, sA + (ab ^ 1) * BM * LDA, again + (ab ^ 1));
     }
-    if (kt + 1 < KT) {
-      regs[set].store(sB + (buf ^ 1) * BK * LDB, tid);
-      if (kt + 3 < KT) regs[set].load(B, p.k, p.n, n0, kt + 3, tid);
-    }
+    if (J == 1 && tid == 0) again[ab] = 0;  // read before this pass, raised again in the next one
+    regs[set].store(sB + (buf ^ 1) * BK * LDB, tid);
+    regs[set].load(B, p.k, p.n, n0, ahead, tid);
     __syncthreads();
   };
 
-  int kt = 0;
-  for (; kt + 4 <= KT; kt += 4) {
-    step(kt + 0, std::integral_constant<int, 0>{});
-    step(kt + 1, std::integral_constant<int, 1>{});
-    step(kt + 2, std::integral_constant<int, 2>{});
-    step(kt + 3, std::integral_constant<int, 3>{});
+  int cur = 0, ab = 0;
+  bool repeat = __builtin_amdgcn_readfirstlane(again[0]) != 0;
+  while (cur < chunks) {
+    const int nxt = repeat ? cur : cur + 1;
+    step(ab, nxt, cur * SPC + 3, std::integral_constant<int, 0>{});
+    step(ab, nxt, nxt * SPC + 0, std::integral_constant<int, 1>{});
+    step(ab, nxt, nxt * SPC + 1, std::integral_constant<int, 2>{});
+    step(ab, nxt, nxt * SPC + 2, std::integral_constant<int, 3>{});
+    ab ^= 1;
+    repeat = __builtin_amdgcn_readfirstlane(again[ab]) != 0;
+    cur = nxt;
   }
-  if (kt < KT) step(kt++, std::integral_constant<int, 0>{});
-  if (kt < KT) step(kt++, std::integral_constant<int, 1>{});
-  if (kt < KT) step(kt++, std::integral_constant<int, 2>{});
 
   spmm_mfma_epilogue<BF16, WM, WN>(p, acc, C, m0, n0, wm, wn, lane);
 }

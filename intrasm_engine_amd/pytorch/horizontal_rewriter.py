@@ -91,6 +91,67 @@ def make_kernel_pair_or_triple_autograd_function(
                 raise TypeError(f"unknown forward options: {sorted(unknown)} (expected {sorted(known)})")
             return [normalise_kwargs((fwd_kwargs or {}).get(f"fwd_kwargs_{i + 1}")) for i in range(len(funcs))]
 
+        # ---- tuning hooks: the group's search space is the product of its parts' (reference :109-205)
+        @classmethod
+        def _split(cls, items: Optional[Sequence], counts: Sequence[int]) -> list:
+            if items is None:
+                return [None] * len(counts)
+            out, beg = [], 0
+            for n in counts:
+                out.append(list(items[beg:beg + n]))
+                beg += n
+            return out
+
+        @classmethod
+        def get_search_space(cls, sample_inputs, sample_grads=None):
+            ins = cls._split(sample_inputs, [f.num_inputs() for f in funcs])
+            grads = cls._split(sample_grads, [1] * len(funcs))
+            return simple_combine_search_space(*(f.get_search_space(i, g) for f, i, g in zip(funcs, ins, grads)))
+
+        @classmethod
+        def _unpack(cls, params: dict) -> list[dict]:
+            parts = list(simple_unpack_params(params))
+            if len(parts) > len(funcs):
+                raise ValueError("parameters for a third operator given to a pair")
+            return parts + [{}] * (len(funcs) - len(parts))
+
+        @classmethod
+        def check_params_sanity(cls, params: dict) -> None:
+            for f, part in zip(funcs, cls._unpack(params)):
+                f.check_params_sanity(part)
+
+        @classmethod
+        def get_test_fwd_kwargs(cls, params: dict, constructor=None, backward_constructor=None,
+                                stream_beg: int = 0) -> dict[str, Any]:
+            """Part i at its share of ``params`` on stream ``stream_beg + i`` (reference :168-189)."""
+            return {f"fwd_kwargs_{i + 1}": f.get_test_fwd_kwargs(part, constructor, backward_constructor,
+                                                                   stream_beg + i)["fwd_kwargs_1"]
+                    for i, (f, part) in enumerate(zip(funcs, cls._unpack(params)))}
+
+        @classmethod
+        def build_and_test(cls, sample_inputs, sample_grads, params: dict, repeats: int = 5) -> float:
+            """Both passes of every part recorded on parallel branches of one forward and one backward
+            graph; returns the sum of the two median launch times in milliseconds (the reference
+            leaves this open, :207-236)."""
+            from .cpp_extensions.layers_and_funcs.utils import time_constructor
+
+            fwd, bwd = TorchCUDAGraphConstructor(), TorchCUDAGraphConstructor()
+            fwd.register_new_streams(len(funcs) - 1)
+            bwd.register_new_streams(len(funcs) - 1)
+            kwargs = cls.check_fwd_kwargs_sanity(cls.get_test_fwd_kwargs(params, fwd, bwd))
+            ins = cls._split(sample_inputs, [f.num_inputs() for f in funcs])
+            grads = cls._split(sample_grads, [1] * len(funcs))
+            keep = []
+            with torch.no_grad():
+                for f, kw, i, g in zip(funcs, kwargs, ins, grads):
+                    outputs, ctx_dict, to_save = f._forward(*i, **kw)
+                    g = g if g is not None else [torch.randn_like(o) for o in outputs]
+                    keep.append((outputs, f._backward(*g, *to_save, needs_input_grad=f.differentiable_inputs(i),
+                                                      **ctx_dict)))
+            latency = time_constructor(fwd, repeats) + time_constructor(bwd, repeats)
+            del keep
+            return latency
+
         @classmethod
         def forward(cls, ctx, fwd_kwargs, *inputs):
             kwargs = cls.check_fwd_kwargs_sanity(fwd_kwargs)

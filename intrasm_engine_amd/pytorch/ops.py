@@ -20,12 +20,41 @@ Registered operators
 """
 from __future__ import annotations
 
+import contextlib
+import threading
+
 import torch
 
 from .. import _lib
 
 _DT = {torch.float32: _lib.F32, torch.float16: _lib.F16, torch.bfloat16: _lib.BF16}
 _IT = {torch.int32: _lib.I32, torch.int16: _lib.I16}
+
+
+_TUNING = threading.local()
+_SPMM_KEYS = ("force_wpr", "force_variant", "force_rpw", "force_nt", "force_lpg")
+
+
+@contextlib.contextmanager
+def kernel_params(*, spmm: dict | None = None, sddmm: dict | None = None, gemm: dict | None = None):
+    """Kernel choices for the operators called inside the block (this thread only), for tuning:
+    ``spmm`` = any of force_variant / force_rpw / force_nt / force_lpg / force_wpr (the tuning
+    bits of ``iex_spmm_ex``), ``sddmm`` = force_wpr, ``gemm`` = tile (the shape code of
+    ``iex_gemm``: 1 = 128x128, 2 = 128x256, 3 = 256x256, 4 = 128x128 with K steps of 64).
+    Without a block, or for a key left out, the library chooses.  A kernel family that cannot
+    take the operands at hand (a matrix-core family for an n that is not a multiple of 8, say)
+    falls back to a gather kernel, as the C entry points document: results stay correct, the
+    timing is then that of the fallback."""
+    for name, given, known in (("spmm", spmm, _SPMM_KEYS), ("sddmm", sddmm, ("force_wpr",)), ("gemm", gemm, ("tile",))):
+        unknown = set(given or {}) - set(known)
+        if unknown:
+            raise TypeError(f"unknown {name} kernel parameters: {sorted(unknown)}")
+    before = {k: getattr(_TUNING, k, None) for k in ("spmm", "sddmm", "gemm")}
+    _TUNING.spmm, _TUNING.sddmm, _TUNING.gemm = spmm or None, sddmm or None, gemm or None
+    try:
+        yield
+    finally:
+        _TUNING.spmm, _TUNING.sddmm, _TUNING.gemm = before["spmm"], before["sddmm"], before["gemm"]
 
 
 def _chk(cond: bool, msg: str = "") -> None:
@@ -63,6 +92,9 @@ def _check_index_dtypes(row_indices, row_offsets, column_indices, allow_i16=Fals
 def _spmm(b, row_indices, values, row_offsets, column_indices, m, *, per_batch_values,
           accumulate, dtypes, allow_i16, out=None, bias=None, relu=False, force_wpr=0, force_variant=0, force_rpw=0,
           force_nt=0, force_lpg=0):
+    tuned = getattr(_TUNING, "spmm", None)
+    if tuned and not (force_wpr or force_variant or force_rpw or force_nt or force_lpg):
+        force_wpr, force_variant, force_rpw, force_nt, force_lpg = (tuned.get(key, 0) for key in _SPMM_KEYS)
     _chk(b.dim() == 3)
     if per_batch_values:
         _chk(values.dim() == 2)
@@ -114,6 +146,9 @@ def _spmm(b, row_indices, values, row_offsets, column_indices, m, *, per_batch_v
 
 def _sddmm(a, b, row_indices, row_offsets, column_indices, *, sum_over_batch, dtypes,
            out=None, accumulate=False, force_wpr=0):
+    tuned = getattr(_TUNING, "sddmm", None)
+    if tuned and not force_wpr:
+        force_wpr = tuned.get("force_wpr", 0)
     _chk(a.dim() == b.dim())
     _chk(a.dim() == 3)
     _chk(a.size(0) == b.size(0))
@@ -223,7 +258,8 @@ def gemm_mfma(a, b, trans_b=False, out=None):
         _chk(tuple(out.shape) == shape and out.dtype == a.dtype and out.is_contiguous()
              and out.device == a.device, "out has the wrong shape, dtype, layout or device")
     with torch.cuda.device(a.device):
-        rc = _lib.load().iex_gemm(_DT[a.dtype], int(bool(trans_b)), M, N, K, a.data_ptr(), b.data_ptr(),
+        tile = (getattr(_TUNING, "gemm", None) or {}).get("tile", 0)
+        rc = _lib.load().iex_gemm(_DT[a.dtype], int(bool(trans_b)) | ((int(tile) & 0xf) << 4), M, N, K, a.data_ptr(), b.data_ptr(),
                                   out.data_ptr(), batch, sa, sb, M * N, _stream_ptr(a.device))
     _lib.check(rc, "gemm")
     return out

@@ -310,6 +310,13 @@ def run_extras(torch, ops, dev, W, IL, mats, dens, csr_dev, time_cell, variant_o
     out["spmm_c3_fp16_16heads"] = {"us": round(us, 2), "GBps": round(by / us / 1e3, 1),
                                    "hbm_frac": round(by / us / 1e3 / HBM_PEAK_GBPS, 4),
                                    "GFLOPs": round(W.spmm_flops(pat.nnz, 64, 16) / us / 1e3, 1)}
+    from intrasm_engine_amd.pytorch.sparse_attention import sparse_attention
+    us_block = time_cell(lambda: sparse_attention(qt, kt, vt, ri3, ro3, ci3), repeats=10)
+    us_softmax = time_cell(lambda: ops.csr_softmax_(scores, ri3, ro3, 0.125), repeats=10)
+    out["attention_block_c3_fp16_16heads"] = {
+        "us": round(us_block, 2), "softmax_us": round(us_softmax, 2),
+        "what": "SDDMM -> softmax over CSR rows -> SpMM, three launches; 16 heads x 4096 tokens x 64",
+        "GFLOPs": round((W.sddmm_flops(pat.nnz, 64, 16) + W.spmm_flops(pat.nnz, 64, 16)) / us_block / 1e3, 1)}
     log("[bench] SDDMM done")
 
     # ---- config 4: fp16 SpMM 11008x4096 @90% x 4096x2048  ||  bf16 GEMM 4096x4096x2048

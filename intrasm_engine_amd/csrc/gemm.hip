@@ -1,11 +1,12 @@
 // Host side of the dense companion GEMM: kernel wrapper, tile-shape choice, XCD-aware
 // tile order, argument checks and the C entry point.  Device code: gemm_device.cuh.
-#include "gemm_device.cuh"
+#include "gemm_dma_device.cuh"
 
 namespace iex {
 namespace {
 
 constexpr int kXcds = 8;
+constexpr int kGroupM = 4;
 
 // Workgroup ids are dealt round-robin to the 8 XCDs (each with its own L2).  Give every
 // XCD a contiguous band of C tiles (row-major over tiles) so that the A row panels a
@@ -15,8 +16,14 @@ __device__ __forceinline__ bool xcd_tile(int block, int tiles_m, int tiles_n, in
   const int per_xcd = (total + kXcds - 1) / kXcds;
   const int linear = (block % kXcds) * per_xcd + block / kXcds;
   if (linear >= total) return false;
-  tile_m = linear / tiles_n;
-  tile_n = linear % tiles_n;
+  // inside the band, walk kGroupM tile rows column by column: the 32 tiles an XCD works on at one
+  // time then share kGroupM row panels of A and 32 / kGroupM column panels of B in its L2
+  const int per_group = kGroupM * tiles_n;
+  const int first_row = (linear / per_group) * kGroupM;
+  const int rows = min(tiles_m - first_row, kGroupM);
+  const int in_group = linear % per_group;
+  tile_m = first_row + in_group % rows;
+  tile_n = in_group / rows;
   return true;
 }
 
@@ -52,33 +59,67 @@ int launch(GemmParams p, int batch, hipStream_t stream) {
   return check_hip(hipGetLastError(), "gemm launch");
 }
 
+template <bool BF16, bool TRANS_B, int WM, int WN, int BK, int STAGES, int WCN>
+__global__ __launch_bounds__(WCN * 128, (WCN == 2 && WM * WN <= 8 && gemm_dma_lds_bytes<WM, WN, WCN, BK, STAGES>() <= 80 * 1024 ? 2 : 1)) void gemm_dma_kernel(GemmParams p) {
+  extern __shared__ __align__(16) unsigned char smem[];
+  int tile_m, tile_n;
+  if (!xcd_tile(blockIdx.x, p.tiles_m, p.tiles_n, tile_m, tile_n)) return;  // uniform per block
+  gemm_tile_dma<BF16, TRANS_B, WM, WN, WCN, BK, STAGES>(p, tile_m, tile_n, blockIdx.y, smem);
+}
+
+template <bool BF16, bool TRANS_B, int WM, int WN, int BK, int STAGES, int WCN = 2>
+int launch_dma(GemmParams p, int batch, hipStream_t stream) {
+  constexpr int BM = 2 * WM * 32, BN = WCN * WN * 32;
+  p.tiles_m = ceil_div(p.M, BM);
+  p.tiles_n = ceil_div(p.N, BN);
+  const int total = p.tiles_m * p.tiles_n;
+  const int per_xcd = (total + kXcds - 1) / kXcds;
+  constexpr int lds = gemm_dma_lds_bytes<WM, WN, WCN, BK, STAGES>();
+  auto kern = gemm_dma_kernel<BF16, TRANS_B, WM, WN, BK, STAGES, WCN>;
+  if (lds > 64 * 1024) {
+    static thread_local bool raised = false;  // per instantiation
+    if (!raised) {
+      if (int rc = check_hip(hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
+                                                 hipFuncAttributeMaxDynamicSharedMemorySize, lds),
+                             "hipFuncSetAttribute(LDS size)"))
+        return rc;
+      raised = true;
+    }
+  }
+  hipLaunchKernelGGL(kern, dim3(per_xcd * kXcds, batch), dim3(WCN * 128), lds, stream, p);
+  return check_hip(hipGetLastError(), "gemm launch");
+}
+
 template <bool BF16, bool TRANS_B>
 int launch_shape(const GemmParams& p, int batch, int force, hipStream_t stream) {
   if (force == 1) return launch<BF16, TRANS_B, 2, 2>(p, batch, stream);
   if (force == 2) return launch<BF16, TRANS_B, 2, 4>(p, batch, stream);
   if (force == 3) return launch<BF16, TRANS_B, 4, 4>(p, batch, stream);
   if (force == 4) return launch<BF16, TRANS_B, 2, 2, 64>(p, batch, stream);
-  // The larger the tile of a wave, the fewer LDS bytes each MFMA needs (128x128 per wave: half of
-  // what 64x64 needs), and LDS bandwidth is what the main loop runs against; the smaller the tile,
-  // the more workgroups there are to fill 256 CUs.  Measured at 4096..11008 x 8192 x 4096..8192:
-  // 256x256 tiles (one wave per SIMD, 504 registers) 830-960 TFLOP/s, 128x256 770-890, 128x128
-  // 715-770; at config 4's 4096 x 2048 x 4096 the order reverses (450-470, 620-690, 720-750).
-  // Two tiles per CU is where the larger shape starts to win.
+  if (force == 5) return launch_dma<BF16, TRANS_B, 2, 2, 32, 4>(p, batch, stream);
+  if (force == 6) return launch_dma<BF16, TRANS_B, 2, 4, 32, 4>(p, batch, stream);
+  if (force == 7) return launch_dma<BF16, TRANS_B, 4, 4, 32, 4>(p, batch, stream);
+  // Default: operands straight from global memory into LDS (gemm_dma_device.cuh).  The larger the
+  // tile of a wave, the fewer LDS bytes each MFMA needs, and LDS time is what the main loop runs
+  // against; the smaller the tile, the more workgroups there are to fill 256 CUs, and a tile wider
+  // than what is left of the matrix computes columns nobody stores.  Measured (bf16, TFLOP/s):
+  //   8192^3: 256x256 1200, 128x256 1040, register-staged 256x256 980;   4096 x 8192 x 4096: 1140 / 1000 / 920
+  //   config 4's 4096 x 2048 x 4096 (128 tiles of 256x256): 620 / 860 / 470, 128x128 750
+  //   2048^3: 290 / 420 / 220, 128x128 550
+  auto fill = [](int n, int tile) { return (double)n / ((double)ceil_div(n, tile) * tile); };
   const long long huge_tiles = (long long)ceil_div(p.M, 256) * ceil_div(p.N, 256) * batch;
-  if (huge_tiles >= 512 && p.K >= 256) return launch<BF16, TRANS_B, 4, 4>(p, batch, stream);
+  if (huge_tiles >= 512 && fill(p.M, 256) * fill(p.N, 256) >= 0.8) return launch_dma<BF16, TRANS_B, 4, 4, 32, 4>(p, batch, stream);
   const long long wide_tiles = (long long)ceil_div(p.M, 128) * ceil_div(p.N, 256) * batch;
-  if (wide_tiles >= 512 && p.K >= 256) return launch<BF16, TRANS_B, 2, 4>(p, batch, stream);
-  // 128x128 tiles: K steps of 64 halve the barriers and double the distance between a global load
-  // and its use (720-830 TFLOP/s against 660-770 with steps of 32 on the same shapes)
-  if (p.K >= 128) return launch<BF16, TRANS_B, 2, 2, 64>(p, batch, stream);
-  return launch<BF16, TRANS_B, 2, 2>(p, batch, stream);
+  if (wide_tiles >= 256 && fill(p.N, 256) >= 0.8) return launch_dma<BF16, TRANS_B, 2, 4, 32, 4>(p, batch, stream);
+  return launch_dma<BF16, TRANS_B, 2, 2, 32, 4>(p, batch, stream);
 }
 
 }  // namespace
 }  // namespace iex
 
-// trans_b: bit 0 = B is (N, K); bits 4..7 force the tile shape for tuning (1 = 128x128, 2 = 128x256,
-// 3 = 256x256, 4 = 128x128 with K steps of 64; 0 = choose).
+// trans_b: bit 0 = B is (N, K); bits 4..7 force the kernel for tuning.  Register-staged operands:
+// 1 = 128x128 tiles, 2 = 128x256, 3 = 256x256, 4 = 128x128 with K steps of 64.  Operands loaded
+// straight into LDS: 5 = 128x128, 6 = 128x256, 7 = 256x256.  0 = choose (one of 5..7).
 extern "C" int iex_gemm(int dtype, int trans_b_and_shape, int M, int N, int K, const void* A, const void* B, void* C, int batch,
                         long long stride_a, long long stride_b, long long stride_c, void* stream) {
   using namespace iex;

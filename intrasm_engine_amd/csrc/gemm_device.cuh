@@ -155,6 +155,43 @@ struct GemmStage {
   }
 };
 
+// Writes the WM x WN accumulator blocks of one wavefront to C (rounded to the 16-bit type).
+template <bool BF16, int WM, int WN>
+__device__ __forceinline__ void gemm_store_tile(const GemmParams& p, const f32x16 (&acc)[WM][WN], unsigned short* __restrict__ C,
+                                                int m0, int n0, int wm, int wn, int lane) {
+  typedef unsigned short u16;
+  // Swapped-operand result layout: lane holds row (lane % 32) of the 32x32 block and, in
+  // accumulator quad q, columns q*8 + (lane / 32)*4 .. +3.
+  const bool vec_ok = (p.N % 4 == 0) && ((reinterpret_cast<uintptr_t>(C) & 7) == 0);
+#pragma unroll
+  for (int i = 0; i < WM; ++i) {
+    const int gm = m0 + (wm * WM + i) * 32 + (lane & 31);
+    if (gm >= p.M) continue;
+#pragma unroll
+    for (int j = 0; j < WN; ++j) {
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        const int gn = n0 + (wn * WN + j) * 32 + q * 8 + (lane >> 5) * 4;
+        if (gn >= p.N) continue;
+        u16 h[4];
+#pragma unroll
+        for (int e = 0; e < 4; ++e) h[e] = f32_to_16(acc[i][j][q * 4 + e], BF16);
+        u16* dst = C + (size_t)gm * p.N + gn;
+        if (vec_ok) {
+          u32x2 w;
+          w.x = (unsigned)h[0] | ((unsigned)h[1] << 16);
+          w.y = (unsigned)h[2] | ((unsigned)h[3] << 16);
+          *reinterpret_cast<u32x2*>(dst) = w;
+        } else {
+#pragma unroll
+          for (int e = 0; e < 4; ++e)
+            if (gn + e < p.N) dst[e] = h[e];
+        }
+      }
+    }
+  }
+}
+
 // One C tile.  `smem` must hold gemm_lds_bytes<WM,WN>() bytes, 16-byte aligned.
 // All 2 * WCN * 64 threads of the workgroup must call this (it contains barriers).
 template <bool BF16, bool TRANS_B, int WM, int WN, int SETS = kGemmSets, int WCN = 2, int BK = kGemmBK>
@@ -277,36 +314,7 @@ __device__ __forceinline__ void gemm_tile(const GemmParams& p, int tile_m, int t
     if (kt < KT) step(kt++, std::integral_constant<int, 0>{});
   }
 
-  // Swapped-operand result layout: lane holds row (lane % 32) of the 32x32 block and, in
-  // accumulator quad q, columns q*8 + (lane / 32)*4 .. +3.
-  const bool vec_ok = (p.N % 4 == 0) && ((reinterpret_cast<uintptr_t>(C) & 7) == 0);
-#pragma unroll
-  for (int i = 0; i < WM; ++i) {
-    const int gm = m0 + (wm * WM + i) * 32 + (lane & 31);
-    if (gm >= p.M) continue;
-#pragma unroll
-    for (int j = 0; j < WN; ++j) {
-#pragma unroll
-      for (int q = 0; q < 4; ++q) {
-        const int gn = n0 + (wn * WN + j) * 32 + q * 8 + (lane >> 5) * 4;
-        if (gn >= p.N) continue;
-        u16 h[4];
-#pragma unroll
-        for (int e = 0; e < 4; ++e) h[e] = f32_to_16(acc[i][j][q * 4 + e], BF16);
-        u16* dst = C + (size_t)gm * p.N + gn;
-        if (vec_ok) {
-          u32x2 w;
-          w.x = (unsigned)h[0] | ((unsigned)h[1] << 16);
-          w.y = (unsigned)h[2] | ((unsigned)h[3] << 16);
-          *reinterpret_cast<u32x2*>(dst) = w;
-        } else {
-#pragma unroll
-          for (int e = 0; e < 4; ++e)
-            if (gn + e < p.N) dst[e] = h[e];
-        }
-      }
-    }
-  }
+  gemm_store_tile<BF16, WM, WN>(p, acc, C, m0, n0, wm, wn, lane);
 }
 
 }  // namespace iex

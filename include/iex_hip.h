@@ -61,14 +61,15 @@ int iex_copy_bytes(void* dst, const void* src, size_t nbytes, void* stream);
 /* bits 16..19: force the kernel family: 1 = row kernel gathering from L2, 2 = LDS-staged
  * gather, 3 / 4 = matrix-core kernels (fp16 / bf16: A expanded to dense tiles in LDS; 4 waves
  * and 128 x 256 tiles / 8 waves and 128 x 512 tiles), 5 = matrix-core kernel for fp32
- * (v_mfma_f32_32x32x2, 32-row tiles).  0 = choose.
- * Families 2-5 rely on strictly ascending column indices inside a row (canonical CSR, what
+ * (v_mfma_f32_32x32x2, 32-row tiles), 6 = family 4's tile with the dense operand loaded from
+ * global memory straight into LDS and A expanded 64 columns at a time (fp16 / bf16).  0 = choose.
+ * Families 2-6 rely on strictly ascending column indices inside a row (canonical CSR, what
  * dense_to_sparse produces); family 1 accepts any order and duplicates -- force it for such
- * input.  Families 3-5 multiply explicit zeros with the dense operand, so a non-finite entry
+ * input.  Families 3-6 multiply explicit zeros with the dense operand, so a non-finite entry
  * in a row of `dense` that no nonzero references still reaches the output (0 * inf = NaN).
  * bits 20..23: rows per wavefront of family 2 (2, 4 or 8); windows of nonzeros held in
- * registers per row of family 4 (1, 2, 4 or 5 windows of 16) and 5 (2, 4 or 8 windows of 8).
- * 0 = choose.                                                                            */
+ * registers per row of family 4 (1, 2, 4 or 5 windows of 16), 5 (2, 4 or 8 windows of 8) and
+ * 6 (1, 2 or 4 windows of 16).  0 = choose.                                              */
 #define IEX_SPMM_FORCE_VARIANT(v) (((v) & 0xf) << 16)
 #define IEX_SPMM_FORCE_RPW(r) (((r) & 0xf) << 20)
 /* bits 24..27: adjacent 64-lane column tiles per wavefront of the row kernel (1 or 2); tile

@@ -2,6 +2,7 @@
 // the C entry points.  The device code is in spmm_device.cuh.
 #include "spmm_lds_device.cuh"
 #include "spmm_mfma2_device.cuh"
+#include "spmm_mfma3_device.cuh"
 #include "spmm_mfma_f32_device.cuh"
 
 namespace iex {
@@ -136,6 +137,41 @@ int launch_mfma2(const SpmmParams& p, int batch, int windows, hipStream_t stream
       case 5: return launch_mfma2_one<T, IT, 5>(p, batch, stream);
     }
     return fail(IEX_ERR_BAD_ARGUMENT, "spmm: windows of the matrix-core variant must be 1, 2, 4 or 5 (got %d)", windows);
+  } else {
+    return fail(IEX_ERR_UNSUPPORTED, "spmm: the matrix-core variant handles fp16 and bf16 only");
+  }
+}
+
+template <bool BF16, typename IT, int W>
+__global__ __launch_bounds__(kMfma3Threads, 2) void spmm_mfma3_kernel(SpmmParams p, int tiles_m) {
+  extern __shared__ __align__(16) unsigned char smem[];
+  spmm_mfma3_block<BF16, IT, W>(p, blockIdx.x % tiles_m, blockIdx.x / tiles_m, blockIdx.y, smem);
+}
+
+template <typename T, typename IT, int W>
+int launch_mfma3_one(const SpmmParams& p, int batch, hipStream_t stream) {
+  constexpr bool kBf16 = std::is_same<T, __hip_bfloat16>::value;
+  const int tiles_m = ceil_div(p.m, kMfmaBM), tiles_n = ceil_div(p.n, kMfma3BN);
+  auto kernel = spmm_mfma3_kernel<kBf16, IT, W>;
+  static thread_local bool raised = false;
+  if (!raised) {
+    if (int rc = check_hip(hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
+                                               hipFuncAttributeMaxDynamicSharedMemorySize, spmm_mfma3_lds_bytes()),
+                           "hipFuncSetAttribute(LDS size)"))
+      return rc;
+    raised = true;
+  }
+  hipLaunchKernelGGL(kernel, dim3(tiles_m * tiles_n, batch), dim3(kMfma3Threads), spmm_mfma3_lds_bytes(), stream, p, tiles_m);
+  return check_hip(hipGetLastError(), "spmm (matrix-core, direct loads) launch");
+}
+
+template <typename T, typename IT>
+int launch_mfma3(const SpmmParams& p, int batch, int windows, hipStream_t stream) {
+  if constexpr (sizeof(T) == 2) {
+    if (windows == 1) return launch_mfma3_one<T, IT, 1>(p, batch, stream);
+    if (windows == 2) return launch_mfma3_one<T, IT, 2>(p, batch, stream);
+    if (windows == 4) return launch_mfma3_one<T, IT, 4>(p, batch, stream);
+    return fail(IEX_ERR_BAD_ARGUMENT, "spmm: windows of the direct-load matrix-core variant must be 1, 2 or 4 (got %d)", windows);
   } else {
     return fail(IEX_ERR_UNSUPPORTED, "spmm: the matrix-core variant handles fp16 and bf16 only");
   }
@@ -299,6 +335,18 @@ int mfma_f32_variant(const SpmmParams& p, int batch, const Choice& ch, int& wind
   return 0;
 }
 
+// Windows of 16 nonzeros per row and half chunk of 64 columns for the direct-load matrix-core
+// kernel.  One window holds a row's share with a margin of three standard deviations up to 13 %
+// density (mean 8.3 of 64), two up to 33 % (mean 21) and exactly at 2:4 sparsity (32 of every 64,
+// recognised by nnz being exactly half of m * k); four always do.  A half chunk the windows do not
+// hold is multiplied twice, so a wrong guess costs time, not correctness.
+inline int mfma3_windows(const SpmmParams& p) {
+  const double cells = (double)p.m * p.k;
+  const double density = cells > 0 ? (double)p.nnz / cells : 0.0;
+  if (density <= 0.13) return 1;
+  return (density <= 0.33 || 2.0 * p.nnz == cells) ? 2 : 4;
+}
+
 template <typename T, typename IT>
 int launch_typed(const SpmmParams& p, int batch, const Choice& ch, hipStream_t stream) {
   constexpr int kMax = 16 / (int)sizeof(T);
@@ -306,7 +354,14 @@ int launch_typed(const SpmmParams& p, int batch, const Choice& ch, hipStream_t s
     int windows = 0;
     if (const int arr = mfma_f32_variant<T, IT>(p, batch, ch, windows)) return launch_mfma_f32(p, batch, arr, windows, ch.lpg != 8, stream);  // (lanes-per-group code 8 = no role split, for tuning)
   }
+  if (ch.variant == 6 && sizeof(T) == 2 && p.nnz > 0 && p.n % 8 == 0 && aligned(p.dense, 16) && aligned(p.out, 16))
+    return launch_mfma3<T, IT>(p, batch, ch.rpw ? ch.rpw : mfma3_windows(p), stream);
   const MfmaChoice mc = mfma_variant<T>(p, batch, ch);
+  // Where the 8-wave kernel would run and two windows per half chunk are the right size (13-33 %
+  // density, or 2:4), the direct-load kernel is faster (2:4 weights 4096 x 4096, n = 8192: 0.38
+  // against 0.45 ms; 80 % sparse 11008 x 4096: 0.99 against 1.03); with one window (sparser) it is
+  // slower (90 %: 0.32 against 0.27), and four spill registers.
+  if (mc.kind == 4 && ch.variant == 0 && mfma3_windows(p) == 2) return launch_mfma3<T, IT>(p, batch, 2, stream);
   if (mc.kind == 4) return launch_mfma2<T, IT>(p, batch, mc.param, stream);
   if (mc.kind == 3) return launch_mfma<T, IT>(p, batch, mc.param, stream);
   int lvec = 0, rpw = 0;

@@ -42,6 +42,9 @@ SPMM_KERNELS: dict[str, dict] = {
     "mfma8_windows2": {"force_variant": 4, "force_rpw": 2},
     "mfma8_windows4": {"force_variant": 4, "force_rpw": 4},
     "mfma8_windows5": {"force_variant": 4, "force_rpw": 5},
+    # the same tile with the dense operand loaded straight into LDS, A expanded 64 columns at a time
+    "mfma8_direct_windows1": {"force_variant": 6, "force_rpw": 1},
+    "mfma8_direct_windows2": {"force_variant": 6, "force_rpw": 2},
     # fp32 on the matrix cores: 32 x 128 tiles with 2, 4 or 8 windows, 16 x 128 tiles
     "mfma32_windows2": {"force_variant": 5, "force_nt": 4, "force_rpw": 2},
     "mfma32_windows4": {"force_variant": 5, "force_nt": 4, "force_rpw": 4},

@@ -309,7 +309,7 @@ def test_lds_staged_variant(oracle, dev, rpw, dtype, n):
                        pyops._spmm(bi, ri, v, ro_t, ci_t, m, force_variant=1, **kw))
 
 
-@pytest.mark.parametrize("family,knob", [(3, 8), (3, 16), (4, 1), (4, 2), (4, 4), (4, 5)])
+@pytest.mark.parametrize("family,knob", [(3, 8), (3, 16), (4, 1), (4, 2), (4, 4), (4, 5), (6, 1), (6, 2), (6, 4)])
 @pytest.mark.parametrize("dtype,n,itype", [(torch.float16, 264, torch.int16), (torch.float16, 512, torch.int32),
                                            (torch.bfloat16, 776, torch.int32), (torch.float16, 8, torch.int16)])
 def test_matrix_core_variants(oracle, dev, family, knob, dtype, n, itype):
@@ -449,10 +449,12 @@ def test_matrix_core_epilogue_options(oracle, dev, family):
 
 
 @pytest.mark.parametrize("dtype,k,n,density,family", [(torch.float16, 320, 2048, 0.5, 4), (torch.float16, 320, 1024, 0.5, 3),
+                                                      (torch.float16, 320, 2048, 0.25, 6), (torch.bfloat16, 512, 4096, 0.2, 6),
                                                       (torch.float32, 320, 1024, 0.5, 5), (torch.float32, 8192, 2048, 0.1, 2)])
 def test_automatic_choice_of_kernel_family(oracle, dev, dtype, k, n, density, family):
     """Shapes on which the library leaves the row kernel by itself: 16-bit operands of moderate
-    density go to the matrix-core kernels (8 waves when that still fills the chip, else 4),
+    density go to the matrix-core kernels (8 waves when that still fills the chip, else 4; the
+    direct-load kernel, family 6, between 13 and 33 % density),
     fp32 of high density to the fp32 matrix-core kernel, fp32 of low density with a long k
     (the slice of the dense operand outgrows an L2) to the LDS-staged gather.
     Checked against the oracle, and bit-equal to the forced family, which shows which one ran."""

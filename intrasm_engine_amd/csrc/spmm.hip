@@ -357,11 +357,11 @@ int launch_typed(const SpmmParams& p, int batch, const Choice& ch, hipStream_t s
   if (ch.variant == 6 && sizeof(T) == 2 && p.nnz > 0 && p.n % 8 == 0 && aligned(p.dense, 16) && aligned(p.out, 16))
     return launch_mfma3<T, IT>(p, batch, ch.rpw ? ch.rpw : mfma3_windows(p), stream);
   const MfmaChoice mc = mfma_variant<T>(p, batch, ch);
-  // Where the 8-wave kernel would run and two windows per half chunk are the right size (13-33 %
-  // density, or 2:4), the direct-load kernel is faster (2:4 weights 4096 x 4096, n = 8192: 0.38
-  // against 0.45 ms; 80 % sparse 11008 x 4096: 0.99 against 1.03); with one window (sparser) it is
-  // slower (90 %: 0.32 against 0.27), and four spill registers.
-  if (mc.kind == 4 && ch.variant == 0 && mfma3_windows(p) == 2) return launch_mfma3<T, IT>(p, batch, 2, stream);
+  // Where the 8-wave kernel would run: the direct-load kernel wins on 2:4 weights (4096 x 4096,
+  // n = 8192: 0.37 against 0.40-0.46 ms with five windows), ties at 80 % sparsity (11008 x 4096:
+  // 0.94 against 0.93; 4096 x 11008: 0.82 both) and loses at 90 % (n = 2048: 0.29 against 0.26);
+  // with four windows (denser than 33 %, not 2:4) it spills registers.
+  if (mc.kind == 4 && ch.variant == 0 && 2.0 * p.nnz == (double)p.m * p.k) return launch_mfma3<T, IT>(p, batch, 2, stream);
   if (mc.kind == 4) return launch_mfma2<T, IT>(p, batch, mc.param, stream);
   if (mc.kind == 3) return launch_mfma<T, IT>(p, batch, mc.param, stream);
   int lvec = 0, rpw = 0;

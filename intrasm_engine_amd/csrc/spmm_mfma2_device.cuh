@@ -24,7 +24,7 @@ constexpr int kMfma2BN = 512;
 constexpr int kMfma2LDB = kMfma2BN + kGemmLdbPad;
 constexpr int kMfma2Threads = 512;
 template <int BKA>
-constexpr int spmm_mfma2_lds_bytes() { return (2 * kMfmaBM * (BKA + 8) + 2 * kGemmBK * kMfma2LDB) * 2 + 16; }
+constexpr int spmm_mfma2_lds_bytes() { return (2 * kMfmaBM * (BKA + 8) + 2 * kGemmBK * kMfma2LDB) * 2 + 16 + kMfma2Threads * 4; }
 
 struct SpmmMfma2BStage {
   static constexpr int CHUNKS = kMfma2BN * kGemmBK / 8 / kMfma2Threads;  // 128-bit chunks per thread
@@ -67,6 +67,10 @@ __device__ __forceinline__ void spmm_mfma2_block(const SpmmParams& p, int tile_m
   u16* sA = reinterpret_cast<u16*>(smem);  // [2][BM][LDA]
   u16* sB = sA + 2 * BM * LDA;             // [2][BK][LDB]
   int* again = reinterpret_cast<int*>(sB + 2 * BK * LDB);  // [2], one per A buffer
+  // One word per lane that absorbs the writes of lanes with nothing to write: a predicated store is
+  // a branch around it, and branches cut the step into blocks across which the compiler cannot
+  // interleave the expansion with the MFMAs.
+  int* sink = again + 4 + threadIdx.x;
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
@@ -123,11 +127,15 @@ __device__ __forceinline__ void spmm_mfma2_block(const SpmmParams& p, int tile_m
     for (int w = 0; w < W; ++w) {
       const int c = (int)wcol[j][w];
       const bool in = pos[j] + w * LPR + sub < end[j] && c < kend;
-      if (in) rowp[c - ka0] = wval[j][w];
+      if constexpr (W < 5) {
+        *(in ? rowp + (c - ka0) : reinterpret_cast<u16*>(sink)) = wval[j][w];
+      } else {  // five windows: the unpredicated form keeps more registers live and spills
+        if (in) rowp[c - ka0] = wval[j][w];
+      }
       consumed += __popcll((__ballot(in) >> gshift) & 0xffffull);
     }
     pos[j] += consumed;
-    if (consumed == W * LPR) *again = 1;
+    *(consumed == W * LPR ? again : sink) = 1;
     load_windows(j);
   };
 

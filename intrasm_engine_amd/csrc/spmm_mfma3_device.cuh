@@ -32,7 +32,7 @@ constexpr int kMfma3Stages = 3;
 constexpr int kMfma3G = 64;                          // columns of A expanded at a time
 constexpr int kMfma3AStage = kMfmaBM * kMfma3G * 2;  // bytes of one A stage
 constexpr int kMfma3BStage = 32 * kMfma3BN * 2;      // bytes of one B stage
-constexpr int spmm_mfma3_lds_bytes() { return 2 * kMfma3AStage + kMfma3Stages * kMfma3BStage + 16; }
+constexpr int spmm_mfma3_lds_bytes() { return 2 * kMfma3AStage + kMfma3Stages * kMfma3BStage + 16 + kMfma3Threads * 4; }
 
 template <bool BF16, typename IT, int W>
 __device__ __forceinline__ void spmm_mfma3_block(const SpmmParams& p, int tile_m, int tile_n, int z, unsigned char* smem) {
@@ -54,6 +54,10 @@ __device__ __forceinline__ void spmm_mfma3_block(const SpmmParams& p, int tile_m
   unsigned char* sA = smem;                      // [2][BM][G] halves, chunk-permuted rows
   unsigned char* sB = smem + 2 * kMfma3AStage;   // [STAGES][32][BN] halves, chunk-permuted rows
   int* again = reinterpret_cast<int*>(sB + STAGES * kMfma3BStage);  // [3]: raised, read and cleared in turn
+  // One word per lane that absorbs the writes of lanes with nothing to write: a predicated store is a
+  // branch around it, and branches cut the step into blocks across which the compiler cannot
+  // interleave the expansion with the MFMAs.
+  int* sink = again + 4 + threadIdx.x;
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
@@ -127,11 +131,13 @@ __device__ __forceinline__ void spmm_mfma3_block(const SpmmParams& p, int tile_m
     for (int w = 0; w < W; ++w) {
       const int c = (int)wcol[j][w];
       const bool in = pos[j] + w * LPR + sub < end[j] && c < kend;
-      if (in) rowp[(c - k0) ^ asw8] = wval[j][w];
+      u16* dst = in ? rowp + ((c - k0) ^ asw8) : reinterpret_cast<u16*>(sink);
+      *dst = wval[j][w];
       consumed += __popcll((__ballot(in) >> gshift) & 0xffffull);
     }
     if constexpr (PEEK) {
-      if (consumed == W * LPR && pos[j] + W * LPR < end[j] && (int)wpeek[j] < kend) *flag = 1;
+      const bool more = consumed == W * LPR && pos[j] + W * LPR < end[j] && (int)wpeek[j] < kend;
+      *(more ? flag : sink) = 1;
     }
     pos[j] += consumed;
     load_windows(j);

@@ -19,7 +19,7 @@
 //              one launch and full tails, not complementary units.
 // The device code of both roles is the code of the stand-alone kernels, so results are
 // bit-identical to separate launches.
-#include "gemm_device.cuh"
+#include "gemm_dma_device.cuh"
 #include "spmm_mfma2_device.cuh"
 
 namespace iex {
@@ -83,7 +83,7 @@ __global__ __launch_bounds__(kMfma2Threads, 2) void fused_mc_kernel(FusedParams 
   if (is_gemm) {
     const int per_batch = p.g.tiles_m * p.g.tiles_n;
     const int z = idx / per_batch, t = idx % per_batch;
-    gemm_tile<BF16, TRANS_B, kFusedMcWM, kFusedMcWN, kGemmSets, kFusedMcWCN>(p.g, t / p.g.tiles_n, t % p.g.tiles_n, z, smem);
+    gemm_tile_dma<BF16, TRANS_B, kFusedMcWM, kFusedMcWN, kFusedMcWCN, 32, 4>(p.g, t / p.g.tiles_n, t % p.g.tiles_n, z, smem);
   } else {
     // p.spmm_by = row tiles here: consecutive ids walk the row blocks of one column panel
     spmm_mfma2_block<false, IT, W, 128>(p.s, idx % p.spmm_by, idx / p.spmm_by, 0, smem);
@@ -99,7 +99,7 @@ int launch_mc(FusedParams p, hipStream_t stream) {
   p.gemm_blocks = p.g.tiles_m * p.g.tiles_n * p.gemm_batch;
   p.spmm_by = ceil_div(p.s.m, kMfmaBM);
   p.spmm_blocks = p.spmm_by * ceil_div(p.s.n, kMfma2BN);
-  constexpr int lds_gemm = gemm_lds_bytes<TRANS_B, kFusedMcWM, kFusedMcWN, kFusedMcWCN>();
+  constexpr int lds_gemm = gemm_dma_lds_bytes<kFusedMcWM, kFusedMcWN, kFusedMcWCN, 32, 4>();
   constexpr int lds_spmm = spmm_mfma2_lds_bytes<128>();
   constexpr int lds = lds_gemm > lds_spmm ? lds_gemm : lds_spmm;
   auto kernel = fused_mc_kernel<BF16, TRANS_B, IT, W>;

@@ -363,6 +363,18 @@ def run_extras(torch, ops, dev, W, IL, mats, dens, csr_dev, time_cell, variant_o
     log(f"[bench] config 4: spmm {t_spmm:.3f} ms, gemm {t_gemm:.3f} ms, graph {t_graph:.3f} ms, fused {t_fused:.3f} ms")
     del w, x, ga, gb, riw, vw, row, ciw, xt, gat, gbt, spmm_execs, gemm_execs, fused_execs, fused_g_execs, gather_execs
 
+    # ---- the dense GEMM alone on larger shapes (bf16, B as (K, N)): how far the matrix cores are used
+    rows_gemm = []
+    for (gm, gn, gk) in ((8192, 8192, 8192), (4096, 8192, 4096), (11008, 8192, 4096)):
+        ga2 = torch.randn(gm, gk, device=dev).bfloat16()
+        gb2 = torch.randn(gk, gn, device=dev).bfloat16()
+        t = IL.run_non_interleaving([lambda: ops.gemm_mfma(ga2, gb2, False)] * reps) / reps
+        tf = IL.gemm_tflops(gm, gn, gk, t)
+        rows_gemm.append({"m": gm, "n": gn, "k": gk, "ms": round(t, 4), "TFLOPs": round(tf, 1),
+                          "mfma_frac": round(tf / MFMA_PEAK_TFLOPS_16BIT, 4)})
+        del ga2, gb2
+    out["gemm_bf16"] = rows_gemm
+
     # ---- config 5: LLaMA-7B-shaped sparse decoder layer, 16 sequences x 512 tokens, three variants
     from intrasm_engine_amd.decoder_layer import SparseDecoderLayer
     hidden, heads, mlp, seqs, L = 4096, 32, 11008, 16, 512

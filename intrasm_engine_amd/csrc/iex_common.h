@@ -43,13 +43,32 @@ template <> struct elem<__hip_bfloat16> {
 // A VEC-wide register vector of T moved with one load/store instruction.
 template <typename T, int VEC> struct alignas(sizeof(T) * VEC) vec_t { T v[VEC]; };
 
-template <typename T, int VEC>
+// The same vector at element alignment only: still one instruction (the hardware takes 128-bit
+// accesses at any dword / element boundary), for rows whose length is not a multiple of VEC.
+template <typename T, int VEC> struct alignas(sizeof(T)) vec_unaligned_t { T v[VEC]; };
+
+template <typename T, int VEC, bool ALIGNED = true>
 __device__ __forceinline__ vec_t<T, VEC> load_vec(const T* p) {
-  return *reinterpret_cast<const vec_t<T, VEC>*>(p);
+  if constexpr (ALIGNED) {
+    return *reinterpret_cast<const vec_t<T, VEC>*>(p);
+  } else {
+    const vec_unaligned_t<T, VEC> u = *reinterpret_cast<const vec_unaligned_t<T, VEC>*>(p);
+    vec_t<T, VEC> r;
+#pragma unroll
+    for (int i = 0; i < VEC; ++i) r.v[i] = u.v[i];
+    return r;
+  }
 }
-template <typename T, int VEC>
+template <typename T, int VEC, bool ALIGNED = true>
 __device__ __forceinline__ void store_vec(T* p, const vec_t<T, VEC>& x) {
-  *reinterpret_cast<vec_t<T, VEC>*>(p) = x;
+  if constexpr (ALIGNED) {
+    *reinterpret_cast<vec_t<T, VEC>*>(p) = x;
+  } else {
+    vec_unaligned_t<T, VEC> u;
+#pragma unroll
+    for (int i = 0; i < VEC; ++i) u.v[i] = x.v[i];
+    *reinterpret_cast<vec_unaligned_t<T, VEC>*>(p) = u;
+  }
 }
 
 // ---- wave64 cross-lane helpers --------------------------------------------------

@@ -24,6 +24,32 @@ int launch_one(const SpmmParams& p, int batch, hipStream_t stream) {
   return check_hip(hipGetLastError(), "spmm launch");
 }
 
+// n not a multiple of the 128-bit vector: full-width tiles with vectors at element alignment
+template <typename T, typename IT, int VEC, int WPR>
+__global__ __launch_bounds__((WPR > 4 ? WPR : 4) * 64) void spmm_ragged_kernel(SpmmParams p) {
+  __shared__ float red[spmm_lds_floats<VEC, WPR, 1>()];
+  spmm_block<T, IT, VEC, kWave, WPR, kSpmmUnroll, 1, true>(p, blockIdx.x, blockIdx.y, blockIdx.z, red);
+}
+
+template <typename T, typename IT, int VEC, int WPR>
+int launch_ragged_one(const SpmmParams& p, int batch, hipStream_t stream) {
+  constexpr int kWavesPerBlock = (WPR > 4) ? WPR : 4;
+  constexpr int kRowsPerBlock = kWavesPerBlock / WPR;
+  dim3 grid(ceil_div(p.m, kRowsPerBlock), ceil_div(p.n, kWave * VEC), batch);
+  hipLaunchKernelGGL((spmm_ragged_kernel<T, IT, VEC, WPR>), grid, dim3(kWavesPerBlock * kWave), 0, stream, p);
+  return check_hip(hipGetLastError(), "spmm (ragged rows) launch");
+}
+
+template <typename T, typename IT, int VEC>
+int launch_ragged(const SpmmParams& p, int batch, int wpr, hipStream_t stream) {
+  switch (wpr) {
+    case 1: return launch_ragged_one<T, IT, VEC, 1>(p, batch, stream);
+    case 4: return launch_ragged_one<T, IT, VEC, 4>(p, batch, stream);
+    case 8: return launch_ragged_one<T, IT, VEC, 8>(p, batch, stream);
+  }
+  return fail(IEX_ERR_BAD_ARGUMENT, "spmm: waves-per-row must be 1, 4 or 8 (got %d)", wpr);
+}
+
 template <typename T, typename IT, int VEC, int LPG>
 int launch_wpr(const SpmmParams& p, int batch, int wpr, int nt, hipStream_t stream) {
   if constexpr (LPG == kWave && VEC * sizeof(T) == 16) {
@@ -383,6 +409,11 @@ int launch_typed(const SpmmParams& p, int batch, const Choice& ch, hipStream_t s
       default: return launch_wpr<T, IT, kMax, 64>(p, batch, wpr, nt, stream);
     }
   }
+  // Rows whose length is not a multiple of the 128-bit vector (n = 785, 197 of the ViT shapes), at least
+  // half a tile wide: 128-bit accesses at element alignment instead of narrower vectors.  Measured on
+  // the reference's ViT sweep shapes (fp32, batch 384, 97 % sparse): 785 x 785 outputs 865 -> 516 us,
+  // 197 x 197 outputs 64 -> 33 us.
+  if (p.n % kMax != 0 && p.n >= kWave * kMax / 2 && ch.lpg == 0) return launch_ragged<T, IT, kMax>(p, batch, wpr, stream);
   if constexpr (kMax == 8) {
     if (sh.vec == 4) return launch_wpr<T, IT, 4, 64>(p, batch, wpr, nt, stream);
   }

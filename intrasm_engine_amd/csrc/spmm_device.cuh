@@ -60,8 +60,12 @@ struct row_slab {
 // NT  = adjacent 64*VEC-column tiles a wave covers (G == 1 only): per nonzero the wave then
 //       reads NT*64*VEC contiguous elements of one dense row, which amortises the broadcast
 //       of (column, value) and keeps very wide dense operands on fewer pages.
-template <typename T, typename IT, int VEC, int LPG, int WPR, int WIN = kSpmmUnroll, int NT = 1>
+// RAGGED = n is not a multiple of VEC: vectors are moved at element alignment, and the one lane of a
+//       row whose vector would reach past the row's end reads VEC elements ending at the row's end
+//       instead (shifted back by `shift`), sums all of them and stores only the ones it owns.
+template <typename T, typename IT, int VEC, int LPG, int WPR, int WIN = kSpmmUnroll, int NT = 1, bool RAGGED = false>
 __device__ __forceinline__ void spmm_block(const SpmmParams& p, int bx, int by, int bz, float* red) {
+  static_assert(!RAGGED || (NT == 1 && LPG == kWave), "ragged rows: one full-width tile per wave");
   constexpr int kWavesPerBlock = (WPR > 4) ? WPR : 4;
   constexpr int kRowsPerBlock = kWavesPerBlock / WPR;
   constexpr int G = kWave / LPG;
@@ -76,9 +80,10 @@ __device__ __forceinline__ void spmm_block(const SpmmParams& p, int bx, int by, 
   const int grp = lane / LPG;   // which nonzero of a step this lane works on (0 when G == 1)
 
   const int col0 = by * (NT * TW) + (lane % LPG) * VEC;  // first tile; tile t starts TW*t further
+  const int shift = (RAGGED && col0 < p.n && col0 + VEC > p.n) ? col0 + VEC - p.n : 0;  // (n >= VEC, checked by the host)
   int col_ld[NT];                                         // idle lanes gather a valid address, result unused
 #pragma unroll
-  for (int t = 0; t < NT; ++t) col_ld[t] = (col0 + t * TW < p.n) ? col0 + t * TW : 0;
+  for (int t = 0; t < NT; ++t) col_ld[t] = (col0 + t * TW < p.n) ? col0 + t * TW - shift : 0;
 
   float acc[NT][VEC];
 #pragma unroll
@@ -101,7 +106,7 @@ __device__ __forceinline__ void spmm_block(const SpmmParams& p, int bx, int by, 
       Slab s;
       const T* r = dense + (size_t)column * p.n;
 #pragma unroll
-      for (int t = 0; t < NT; ++t) s.t[t] = load_vec<T, VEC>(r + col_ld[t]);
+      for (int t = 0; t < NT; ++t) s.t[t] = load_vec<T, VEC, !RAGGED>(r + col_ld[t]);
       return s;
     };
     auto fma_row = [&](float a, const Slab& s) {
@@ -228,10 +233,10 @@ __device__ __forceinline__ void spmm_block(const SpmmParams& p, int bx, int by, 
   for (int t = 0; t < NT; ++t) {
     const int col = col0 + t * TW;
     if (col >= p.n) continue;
-    T* __restrict__ out = static_cast<T*>(p.out) + ((size_t)z * p.m + row) * p.n + col;
+    T* __restrict__ out = static_cast<T*>(p.out) + ((size_t)z * p.m + row) * p.n + col - shift;
     vec_t<T, VEC> o;
     if (p.accumulate) {
-      const vec_t<T, VEC> prev = load_vec<T, VEC>(out);
+      const vec_t<T, VEC> prev = load_vec<T, VEC, !RAGGED>(out);
 #pragma unroll
       for (int i = 0; i < VEC; ++i) acc[t][i] += elem<T>::to_float(prev.v[i]);
     }
@@ -241,7 +246,13 @@ __device__ __forceinline__ void spmm_block(const SpmmParams& p, int bx, int by, 
       if (p.relu) r = fmaxf(r, 0.f);
       o.v[i] = elem<T>::from_float(r);
     }
-    store_vec<T, VEC>(out, o);
+    if (RAGGED && shift > 0) {
+#pragma unroll
+      for (int i = 0; i < VEC; ++i)
+        if (i >= shift) out[i] = o.v[i];  // the elements before `shift` belong to the lane to the left
+    } else {
+      store_vec<T, VEC, !RAGGED>(out, o);
+    }
   }
 }
 

@@ -507,3 +507,44 @@ def test_two_tiles_per_wave(oracle, dev, dtype, n):
     # one and two tiles per wave sum a row in the same order: bit-equal
     assert torch.equal(out, pyops._spmm(b, ri, v, ro_t, ci_t, m, force_nt=1, force_wpr=4, **kw))
     assert torch.equal(out, pyops._spmm(b, ri, v, ro_t, ci_t, m, force_nt=2, force_wpr=4, **kw))
+
+
+@pytest.mark.parametrize("wpr", [1, 4, 8])
+@pytest.mark.parametrize("dtype,n", [(torch.float32, 785), (torch.float32, 197), (torch.float32, 130), (torch.float32, 257),
+                                     (torch.float16, 785), (torch.float16, 263), (torch.bfloat16, 513)])
+def test_rows_that_are_not_a_multiple_of_the_vector(oracle, dev, wpr, dtype, n):
+    """n = 785 and 197 are the ViT shapes of the reference's xformers sweep: wide rows whose length is no
+    multiple of the 128-bit vector run with 128-bit accesses at element alignment; the one lane per row whose
+    vector would pass the end of the row reads back-shifted and stores only its own elements.  Checked with a
+    batch (row starts at every alignment), accumulate mode and bias + ReLU, against the oracle, and bit for
+    bit against the narrow-vector kernel (force_lpg leaves the ragged path), which sums in the same order."""
+    from intrasm_engine_amd.pytorch import ops as pyops
+    rng = np.random.default_rng(n + wpr)
+    m, k, batch = 75, 300, 3
+    lens = np.clip(rng.geometric(1 / 40.0, m), 0, k)
+    lens[[0, 74]] = 0
+    lens[3] = k
+    ro, ci = W.csr_from_row_lengths(rng, m, k, lens)
+    csr = W.CSR(m, k, rng.standard_normal(ci.shape[0]).astype(np.float32), W.swizzle_from_offsets(ro), ro, ci)
+    b_np = rng.standard_normal((batch, k, n)).astype(np.float32)
+    bias_np = rng.standard_normal(m).astype(np.float32)
+    ri, v, ro_t, ci_t = to_dev(csr, dev, dtype)
+    b = torch.from_numpy(b_np).to(dev).to(dtype)
+    kw = dict(per_batch_values=False, dtypes=(dtype,), allow_i16=False, force_wpr=wpr)
+    vals_r, b_r = rounded(csr.values, dtype), rounded(b_np, dtype)
+    scale = oracle.spmm_abs_scale(b_r, csr.row_indices, vals_r, csr.row_offsets, csr.column_indices, m)
+    out = pyops._spmm(b, ri, v, ro_t, ci_t, m, accumulate=False, **kw)
+    want = oracle.spmm(b_r, csr.row_indices, vals_r, csr.row_offsets, csr.column_indices, m)
+    assert_close(out.float().cpu().numpy(), want, scale, RTOL[dtype], f"ragged rows {dtype} n={n} wpr={wpr}",
+                 atol=FP16_SUBNORMAL_HALF_STEP if dtype == torch.float16 else 0.0)
+    assert torch.equal(out, pyops._spmm(b, ri, v, ro_t, ci_t, m, accumulate=False, force_lpg=64, **kw))
+    # bias + ReLU
+    out = pyops._spmm(b, ri, v, ro_t, ci_t, m, accumulate=False, bias=torch.from_numpy(bias_np).to(dev), relu=True, **kw)
+    want = oracle.spmm(b_r, csr.row_indices, vals_r, csr.row_offsets, csr.column_indices, m, bias=bias_np, relu=True)
+    assert_close(out.float().cpu().numpy(), want, scale + np.abs(bias_np)[None, :, None], RTOL[dtype], "ragged rows, bias + ReLU")
+    # accumulate into a pre-filled output
+    init_np = rng.standard_normal((batch, m, n)).astype(np.float32)
+    init = torch.from_numpy(init_np).to(dev).to(dtype)
+    out = pyops._spmm(b, ri, v, ro_t, ci_t, m, accumulate=True, out=init.clone(), **kw)
+    want = oracle.spmm(b_r, csr.row_indices, vals_r, csr.row_offsets, csr.column_indices, m, out_init=rounded(init_np, dtype))
+    assert_close(out.float().cpu().numpy(), want, scale + np.abs(init_np), RTOL[dtype], "ragged rows, accumulate")

@@ -342,6 +342,12 @@ def run_extras(torch, ops, dev, W, IL, mats, dens, csr_dev, time_cell, variant_o
                                         dtypes=(torch.float16,), allow_i16=True, force_variant=1)] * reps
     t_gather = IL.run_non_interleaving(gather_execs) / reps
     t_graph_gather = IL.run_interleaving(gather_execs, gemm_execs) / reps
+    # the library's choice above has a workspace to use (the operator allocates one) and takes the dense-form
+    # path; without one the 8-wave matrix-core SpMM kernel runs, the kernel the fused launch shares its SpMM role with
+    mc_execs = [lambda: pyops._spmm(xt, riw, vw, row, ciw, w.m, per_batch_values=False, accumulate=False,
+                                    dtypes=(torch.float16,), allow_i16=True, no_workspace=True)] * reps
+    t_mc = IL.run_non_interleaving(mc_execs) / reps
+    t_graph_mc = IL.run_interleaving(mc_execs, gemm_execs) / reps
     fl_s, fl_g = W.spmm_flops(w.nnz, 2048), W.gemm_flops(4096, 2048, 4096)
     by_s = W.spmm_bytes(w.m, w.k, 2048, w.nnz, 1, 2, 2)
     out["config4"] = {
@@ -355,13 +361,16 @@ def run_extras(torch, ops, dev, W, IL, mats, dens, csr_dev, time_cell, variant_o
         "fused_launch_gemm_in_groups_of_64_ms": round(t_fused_g, 4),
         "graph_makespan_pct_of_serialized": round(100 * t_graph / (t_spmm + t_gemm), 1),
         "fused_makespan_pct_of_serialized": round(100 * t_fused / (t_spmm + t_gemm), 1),
+        "spmm_matrix_core_kernel_ms": round(t_mc, 4), "two_branch_graph_matrix_core_kernel_ms": round(t_graph_mc, 4),
+        "matrix_core_kernel_graph_makespan_pct_of_serialized": round(100 * t_graph_mc / (t_mc + t_gemm), 1),
+        "fused_makespan_pct_of_serialized_matrix_core_kernel": round(100 * t_fused / (t_mc + t_gemm), 1),
         "spmm_row_kernel_ms": round(t_gather, 4), "two_branch_graph_row_kernel_ms": round(t_graph_gather, 4),
         "row_kernel_graph_makespan_pct_of_serialized": round(100 * t_graph_gather / (t_gather + t_gemm), 1),
         "spmm_dense_equivalent_TFLOPs": round(2.0 * w.m * w.k * 2048 / t_spmm / 1e9, 1),
         "repeats_per_graph": reps,
     }
     log(f"[bench] config 4: spmm {t_spmm:.3f} ms, gemm {t_gemm:.3f} ms, graph {t_graph:.3f} ms, fused {t_fused:.3f} ms")
-    del w, x, ga, gb, riw, vw, row, ciw, xt, gat, gbt, spmm_execs, gemm_execs, fused_execs, fused_g_execs, gather_execs
+    del w, x, ga, gb, riw, vw, row, ciw, xt, gat, gbt, spmm_execs, gemm_execs, fused_execs, fused_g_execs, gather_execs, mc_execs
 
     # ---- the dense GEMM alone on larger shapes (bf16, B as (K, N)): how far the matrix cores are used
     rows_gemm = []
@@ -421,6 +430,7 @@ def run_extras(torch, ops, dev, W, IL, mats, dens, csr_dev, time_cell, variant_o
         row = {}
         for label, force in (("row_kernel_ms", dict(force_variant=1)), ("lds_staged_ms", dict(force_variant=2)),
                              ("matrix_core_4waves_ms", dict(force_variant=3)), ("matrix_core_8waves_ms", dict(force_variant=4)),
+                             ("no_workspace_choice_ms", dict(no_workspace=True)), ("dense_form_then_gemm_ms", dict(force_variant=7)),
                              ("library_choice_ms", {})):
             row[label] = round(IL.time_execs([lambda: pyops._spmm(xin, ri, v, ro, ci, c.m, **force, **kw)] * 2, repeats=3) / 2, 4)
         dense_flops = 2.0 * c.m * c.k * n_

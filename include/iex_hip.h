@@ -62,7 +62,8 @@ int iex_copy_bytes(void* dst, const void* src, size_t nbytes, void* stream);
  * gather, 3 / 4 = matrix-core kernels (fp16 / bf16: A expanded to dense tiles in LDS; 4 waves
  * and 128 x 256 tiles / 8 waves and 128 x 512 tiles), 5 = matrix-core kernel for fp32
  * (v_mfma_f32_32x32x2, 32-row tiles), 6 = family 4's tile with the dense operand loaded from
- * global memory straight into LDS and A expanded 64 columns at a time (fp16 / bf16).  0 = choose.
+ * global memory straight into LDS and A expanded 64 columns at a time (fp16 / bf16), 7 = dense
+ * form of A in the caller's workspace, then the dense GEMM (iex_spmm_ws only).  0 = choose.
  * Families 2-6 rely on strictly ascending column indices inside a row (canonical CSR, what
  * dense_to_sparse produces); family 1 accepts any order and duplicates -- force it for such
  * input.  Families 3-6 multiply explicit zeros with the dense operand, so a non-finite entry
@@ -89,6 +90,26 @@ int iex_spmm_ex(int dtype, int itype, int flags, int m, int k, int n, int nonzer
                 const int* row_indices, const void* values, const int* row_offsets,
                 const void* column_indices, const void* dense, const float* bias,
                 void* out, void* stream, int batch);
+
+/* iex_spmm_ex with a workspace in device memory that the call may use (and overwrite) until the
+ * work it puts on `stream` has run.  With `workspace_bytes` >= iex_spmm_workspace_bytes(...) and a
+ * 16-byte aligned `workspace`, fp16 / bf16 products that would run on a matrix-core SpMM kernel
+ * (families 3, 4, 6) instead write the dense form of A (m * k * 2 bytes) into the workspace and
+ * hand it to the dense GEMM (iex_gemm): the matrix-core SpMM kernels rebuild the dense form of
+ * their rows of A in LDS once per column tile of the output, the GEMM reads it ready-made (family
+ * 7; the caveat of families 3-6 about explicit zeros holds, and column indices inside a row must
+ * be distinct).  Needs values shared by the batch, plain store, no bias / ReLU, k and n multiples
+ * of 8; anything else, and a NULL or short workspace, runs exactly as iex_spmm_ex.
+ * IEX_SPMM_FORCE_VARIANT(7) asks for that path and fails where it cannot run.
+ * iex_spmm_workspace_bytes returns the size with which the call described would use the workspace,
+ * 0 when it would not whatever the size (has_bias: bias != NULL).  Neither call allocates.
+ * No counterpart in the reference: its launchers (csrc/extensions.h:28-30) take no workspace. */
+int iex_spmm_ws(int dtype, int itype, int flags, int m, int k, int n, int nonzeros,
+                const int* row_indices, const void* values, const int* row_offsets,
+                const void* column_indices, const void* dense, const float* bias,
+                void* out, void* stream, int batch, void* workspace, size_t workspace_bytes);
+size_t iex_spmm_workspace_bytes(int dtype, int itype, int flags, int m, int k, int n,
+                                int nonzeros, int batch, int has_bias);
 
 /* Drop-ins for the three launchers the reference declares in csrc/extensions.h:28-30.
  * CudaSpmm2: fp32, per-batch values (batch, nnz), accumulates into `out`

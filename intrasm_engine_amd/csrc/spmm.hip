@@ -1,9 +1,12 @@
 // Host side of the CSR SpMM: kernel wrappers, variant selection, argument checks and
 // the C entry points.  The device code is in spmm_device.cuh.
+#include <algorithm>
+#include <cmath>
 #include "spmm_lds_device.cuh"
 #include "spmm_mfma2_device.cuh"
 #include "spmm_mfma3_device.cuh"
 #include "spmm_mfma_f32_device.cuh"
+#include "spmm_dense_device.cuh"
 
 namespace iex {
 namespace {
@@ -253,6 +256,8 @@ struct Choice {
   int rpw = 0;      // rows per wavefront of the LDS-staged kernel (0 = choose)
   int nt = 0;       // adjacent column tiles per wavefront of the row kernel (0 = choose)
   int lpg = 0;      // lanes per nonzero of the row kernel: 8, 16, 32 or 64 (0 = choose)
+  void* ws = nullptr;   // caller's workspace for the dense form of A (variant 7), may be null
+  size_t ws_bytes = 0;
 };
 
 // The LDS-staged kernel needs a full-width tile (64 lanes x VEC, VEC the full or half 128-bit
@@ -373,6 +378,43 @@ inline int mfma3_windows(const SpmmParams& p) {
   return (density <= 0.33 || 2.0 * p.nnz == cells) ? 2 : 4;
 }
 
+// Dense form of A in the caller's workspace, then the dense GEMM (16-bit types, values shared by
+// the batch, plain store, no bias / ReLU).  What the shapes must satisfy, the workspace aside.
+inline bool dense_path_fits(int elem_size, const SpmmParams& p, bool flagged) {
+  return elem_size == 2 && !flagged && !p.bias && p.nnz > 0 && p.k % 8 == 0 && p.n % 8 == 0 &&
+         (long long)p.m * p.k < (1ll << 31) && aligned(p.dense, 16) && aligned(p.out, 16);
+}
+
+inline size_t dense_path_bytes(const SpmmParams& p) { return (size_t)p.m * p.k * 2; }
+
+// Whether the dense-form path is the faster one, from a time model fitted on MI355X (fp16):
+//   dense form + GEMM: two launches (8 us), m * k * 2 bytes written at 4 TB/s, the product at
+//     1000 TFLOP/s or, when the tiles are few, one round of 128 x 128 tiles per 512 tiles at 0.35 us
+//     per K step of 32 (4096^2, n <= 512: 58 us whatever the sparsity; 1024^2, n = 2048: 21 us);
+//   matrix-core SpMM kernels: 720 dense-equivalent TFLOP/s (2:4 4096^2, n = 8192: 0.40 against 0.27 ms
+//     for the dense form; 80 % 11008 x 4096: 0.93 / 0.69; 90 %, n = 2048: 0.27 / 0.23);
+//   gather kernels: nnz * n * 2 bytes through the L2 -> CU path at 26 TB/s (4096^2 at 70 %, n = 256:
+//     110 against 58 us; at 90 %, n = 256: 40 against 58; 11008 x 4096 at 95 %, n = 2048: 0.35 / 0.21 ms).
+// The dense form has to win by 15 % to be taken.
+inline bool dense_path_wins(const SpmmParams& p, int batch, int matrix_core_kind) {
+  const double cells = (double)p.m * p.k, flops = 2.0 * cells * p.n * batch;
+  const double tiles = (double)ceil_div(p.m, 128) * ceil_div(p.n, 128) * batch;
+  const double product = std::max(flops / 1000e12, std::ceil(tiles / 512.0) * (p.k / 32.0) * 0.35e-6);
+  const double dense_form = 8e-6 + cells * 2 / 4e12 + product;
+  const double other = matrix_core_kind ? 8e-6 + flops / 720e12 : 8e-6 + (double)p.nnz * p.n * batch * 2 / 26e12;
+  return 1.15 * dense_form < other;
+}
+
+template <typename T, typename IT>
+int launch_dense_path(const SpmmParams& p, int batch, const Choice& ch, hipStream_t stream) {
+  const int lds = min(p.k, kDenseSeg) * 2;
+  hipLaunchKernelGGL((csr_to_dense_kernel<IT>), dim3(p.m), dim3(kDenseThreads), lds, stream, p.k, p.row_offsets,
+                     static_cast<const IT*>(p.cols), static_cast<const uint16_t*>(p.values), static_cast<uint16_t*>(ch.ws));
+  if (int rc = check_hip(hipGetLastError(), "spmm dense-form launch")) return rc;
+  const int dtype = std::is_same<T, __half>::value ? IEX_F16 : IEX_BF16;
+  return iex_gemm(dtype, 0, p.m, p.n, p.k, ch.ws, p.dense, p.out, batch, 0, (long long)p.k * p.n, (long long)p.m * p.n, stream);
+}
+
 template <typename T, typename IT>
 int launch_typed(const SpmmParams& p, int batch, const Choice& ch, hipStream_t stream) {
   constexpr int kMax = 16 / (int)sizeof(T);
@@ -383,6 +425,16 @@ int launch_typed(const SpmmParams& p, int batch, const Choice& ch, hipStream_t s
   if (ch.variant == 6 && sizeof(T) == 2 && p.nnz > 0 && p.n % 8 == 0 && aligned(p.dense, 16) && aligned(p.out, 16))
     return launch_mfma3<T, IT>(p, batch, ch.rpw ? ch.rpw : mfma3_windows(p), stream);
   const MfmaChoice mc = mfma_variant<T>(p, batch, ch);
+  if constexpr (sizeof(T) == 2) {
+    const bool fits = dense_path_fits(2, p, p.per_batch_values || p.accumulate || p.relu);
+    const bool room = ch.ws && aligned(ch.ws, 16) && ch.ws_bytes >= dense_path_bytes(p);
+    if (ch.variant == 7) {
+      IEX_REQUIRE(fits, IEX_ERR_UNSUPPORTED, "spmm: the dense-form path needs 16-bit values shared by the batch, plain store, no bias, k and n multiples of 8 and 16-byte aligned operands");
+      IEX_REQUIRE(room, IEX_ERR_BAD_ARGUMENT, "spmm: the dense-form path needs a 16-byte aligned workspace of %zu bytes (iex_spmm_ws)", dense_path_bytes(p));
+      return launch_dense_path<T, IT>(p, batch, ch, stream);
+    }
+    if (ch.variant == 0 && fits && room && dense_path_wins(p, batch, mc.kind)) return launch_dense_path<T, IT>(p, batch, ch, stream);
+  }
   // Where the 8-wave kernel would run: the direct-load kernel wins on 2:4 weights (4096 x 4096,
   // n = 8192: 0.37 against 0.40-0.46 ms with five windows), ties at 80 % sparsity (11008 x 4096:
   // 0.94 against 0.93; 4096 x 11008: 0.82 both) and loses at 90 % (n = 2048: 0.29 against 0.26);
@@ -433,7 +485,7 @@ int spmm_matrix_core_windows(const SpmmParams& p) {
 int spmm_dispatch(int dtype, int itype, int flags, int m, int k, int n, int nonzeros,
                   const int* row_indices, const void* values, const int* row_offsets,
                   const void* column_indices, const void* dense, const float* bias, void* out,
-                  void* stream, int batch) {
+                  void* stream, int batch, void* workspace, size_t workspace_bytes) {
   IEX_REQUIRE(m >= 0 && k >= 0 && n >= 0 && nonzeros >= 0 && batch >= 0, IEX_ERR_BAD_ARGUMENT,
               "spmm: negative dimension (m=%d k=%d n=%d nnz=%d batch=%d)", m, k, n, nonzeros, batch);
   if (m == 0 || n == 0 || batch == 0) return 0;  // empty output: nothing to launch
@@ -453,6 +505,8 @@ int spmm_dispatch(int dtype, int itype, int flags, int m, int k, int n, int nonz
   ch.rpw = (flags >> 20) & 0xf;
   ch.nt = (flags >> 24) & 0xf;
   ch.lpg = ((flags >> 28) & 0x7) ? (4 << ((flags >> 28) & 0x7)) : 0;
+  ch.ws = workspace;
+  ch.ws_bytes = workspace ? workspace_bytes : 0;
   SpmmParams p{m, k, n, nonzeros, row_indices, values, row_offsets, column_indices, dense, bias, out,
                (flags & IEX_SPMM_PER_BATCH_VALUES) != 0, (flags & IEX_SPMM_ACCUMULATE) != 0,
                (flags & IEX_SPMM_RELU) != 0};
@@ -464,6 +518,25 @@ int spmm_dispatch(int dtype, int itype, int flags, int m, int k, int n, int nonz
   return fail(IEX_ERR_UNSUPPORTED, "spmm: no kernel for dtype=%d itype=%d", dtype, itype);
 }
 
+// Bytes of workspace with which iex_spmm_ws would take the dense-form path for this call (0: it
+// would not, whatever the workspace).  Pointers are taken to be 16-byte aligned.
+size_t spmm_workspace_bytes(int dtype, int itype, int flags, int m, int k, int n, int nonzeros, int batch, int has_bias) {
+  if (m <= 0 || k <= 0 || n <= 0 || nonzeros <= 0 || batch <= 0 || has_bias) return 0;
+  if (!(dtype == IEX_F16 || dtype == IEX_BF16) || !(itype == IEX_I32 || itype == IEX_I16)) return 0;
+  const int variant = (flags >> 16) & 0xf;
+  if (variant != 0 && variant != 7) return 0;
+  void* const some_aligned = reinterpret_cast<void*>(size_t(256));
+  SpmmParams p{m, k, n, nonzeros, nullptr, nullptr, nullptr, nullptr, some_aligned, nullptr, some_aligned, 0, 0, 0};
+  if (!dense_path_fits(2, p, (flags & (IEX_SPMM_PER_BATCH_VALUES | IEX_SPMM_ACCUMULATE | IEX_SPMM_RELU)) != 0)) return 0;
+  if (variant == 0) {
+    Choice ch;
+    ch.rpw = (flags >> 20) & 0xf;
+    ch.lpg = ((flags >> 28) & 0x7) ? (4 << ((flags >> 28) & 0x7)) : 0;
+    if (!dense_path_wins(p, batch, mfma_variant<__half>(p, batch, ch).kind)) return 0;
+  }
+  return dense_path_bytes(p);
+}
+
 }  // namespace iex
 
 extern "C" {
@@ -473,7 +546,19 @@ int iex_spmm_ex(int dtype, int itype, int flags, int m, int k, int n, int nonzer
                 const void* column_indices, const void* dense, const float* bias, void* out,
                 void* stream, int batch) {
   return iex::spmm_dispatch(dtype, itype, flags, m, k, n, nonzeros, row_indices, values, row_offsets,
-                            column_indices, dense, bias, out, stream, batch);
+                            column_indices, dense, bias, out, stream, batch, nullptr, 0);
+}
+
+int iex_spmm_ws(int dtype, int itype, int flags, int m, int k, int n, int nonzeros,
+                const int* row_indices, const void* values, const int* row_offsets,
+                const void* column_indices, const void* dense, const float* bias, void* out,
+                void* stream, int batch, void* workspace, size_t workspace_bytes) {
+  return iex::spmm_dispatch(dtype, itype, flags, m, k, n, nonzeros, row_indices, values, row_offsets,
+                            column_indices, dense, bias, out, stream, batch, workspace, workspace_bytes);
+}
+
+size_t iex_spmm_workspace_bytes(int dtype, int itype, int flags, int m, int k, int n, int nonzeros, int batch, int has_bias) {
+  return iex::spmm_workspace_bytes(dtype, itype, flags, m, k, n, nonzeros, batch, has_bias);
 }
 
 int iex_CudaSpmm2(int m, int k, int n, int nonzeros, const int* row_indices, const float* values,
@@ -481,21 +566,21 @@ int iex_CudaSpmm2(int m, int k, int n, int nonzeros, const int* row_indices, con
                   float* output_matrix, void* stream, int batch_size) {
   return iex::spmm_dispatch(IEX_F32, IEX_I32, IEX_SPMM_PER_BATCH_VALUES | IEX_SPMM_ACCUMULATE, m, k, n,
                             nonzeros, row_indices, values, row_offsets, column_indices, dense_matrix,
-                            nullptr, output_matrix, stream, batch_size);
+                            nullptr, output_matrix, stream, batch_size, nullptr, 0);
 }
 
 int iex_CudaSpmm3(int m, int k, int n, int nonzeros, const int* row_indices, const float* values,
                   const int* row_offsets, const int* column_indices, const float* dense_matrix,
                   float* output_matrix, void* stream, int batch_size) {
   return iex::spmm_dispatch(IEX_F32, IEX_I32, 0, m, k, n, nonzeros, row_indices, values, row_offsets,
-                            column_indices, dense_matrix, nullptr, output_matrix, stream, batch_size);
+                            column_indices, dense_matrix, nullptr, output_matrix, stream, batch_size, nullptr, 0);
 }
 
 int iex_CudaSpmm5(int m, int k, int n, int nonzeros, const int* row_indices, const uint16_t* values,
                   const int* row_offsets, const int16_t* column_indices, const uint16_t* dense_matrix,
                   uint16_t* output_matrix, void* stream, int batch_size) {
   return iex::spmm_dispatch(IEX_F16, IEX_I16, 0, m, k, n, nonzeros, row_indices, values, row_offsets,
-                            column_indices, dense_matrix, nullptr, output_matrix, stream, batch_size);
+                            column_indices, dense_matrix, nullptr, output_matrix, stream, batch_size, nullptr, 0);
 }
 
 }  // extern "C"

@@ -45,6 +45,8 @@ SPMM_KERNELS: dict[str, dict] = {
     # the same tile with the dense operand loaded straight into LDS, A expanded 64 columns at a time
     "mfma8_direct_windows1": {"force_variant": 6, "force_rpw": 1},
     "mfma8_direct_windows2": {"force_variant": 6, "force_rpw": 2},
+    # the dense form of the sparse operand written into a workspace (the operator allocates it), then the dense GEMM
+    "dense_form_gemm": {"force_variant": 7},
     # fp32 on the matrix cores: 32 x 128 tiles with 2, 4 or 8 windows, 16 x 128 tiles
     "mfma32_windows2": {"force_variant": 5, "force_nt": 4, "force_rpw": 2},
     "mfma32_windows4": {"force_variant": 5, "force_nt": 4, "force_rpw": 4},
@@ -53,12 +55,17 @@ SPMM_KERNELS: dict[str, dict] = {
 }
 
 
-def spmm_kernel_choices(dtype: torch.dtype, n: int) -> list[str]:
+def spmm_kernel_choices(dtype: torch.dtype, n: int, k: int | None = None, m: int | None = None) -> list[str]:
     """The entries of :data:`SPMM_KERNELS` that can run a product with ``n`` dense columns of
-    ``dtype`` (a family that cannot would silently fall back and only repeat a measurement)."""
+    ``dtype`` (a family that cannot would silently fall back and only repeat a measurement).
+    The dense-form path refuses shapes it cannot serve instead of falling back, and the backward
+    pass runs the same choice on the transposed matrix: it is offered when the sparse operand's
+    ``k`` and ``m`` are given and multiples of 8."""
     names = ["auto", "row", "row_wpr4", "row_wpr8", "lds_rows2", "lds_rows4", "lds_rows8"]
     if dtype in (torch.float16, torch.bfloat16) and n % 8 == 0:
-        names += [k for k in SPMM_KERNELS if k.startswith(("mfma4_", "mfma8_"))]
+        names += [k_ for k_ in SPMM_KERNELS if k_.startswith(("mfma4_", "mfma8_"))]
+        if k is not None and m is not None and k % 8 == 0 and m % 8 == 0:
+            names.append("dense_form_gemm")
     if dtype == torch.float32 and n % 4 == 0:
         names += [k for k in SPMM_KERNELS if k.startswith("mfma32_")]
     return names
@@ -109,7 +116,7 @@ class MySpMM(MyAutogradFunc):
     @classmethod
     def get_search_space(cls, sample_inputs, sample_grads=None):
         b, values = sample_inputs[0], sample_inputs[2]
-        names = spmm_kernel_choices(values.dtype, b.shape[-1])
+        names = spmm_kernel_choices(values.dtype, b.shape[-1], b.shape[-2], int(sample_inputs[5]))
         return {"spmm_kernel": TunableItemCfg("choice", names),
                 "grad_dense_kernel": TunableItemCfg("choice", names),
                 "grad_values_wpr": TunableItemCfg("choice", [0, 1, 4])}

@@ -91,7 +91,7 @@ def _check_index_dtypes(row_indices, row_offsets, column_indices, allow_i16=Fals
 
 def _spmm(b, row_indices, values, row_offsets, column_indices, m, *, per_batch_values,
           accumulate, dtypes, allow_i16, out=None, bias=None, relu=False, force_wpr=0, force_variant=0, force_rpw=0,
-          force_nt=0, force_lpg=0):
+          force_nt=0, force_lpg=0, no_workspace=False):
     tuned = getattr(_TUNING, "spmm", None)
     if tuned and not (force_wpr or force_variant or force_rpw or force_nt or force_lpg):
         force_wpr, force_variant, force_rpw, force_nt, force_lpg = (tuned.get(key, 0) for key in _SPMM_KEYS)
@@ -134,12 +134,19 @@ def _spmm(b, row_indices, values, row_offsets, column_indices, m, *, per_batch_v
             (_lib.SPMM_ACCUMULATE if accumulate else 0) | (_lib.SPMM_RELU if relu else 0) | \
             ((int(force_wpr) & 0xff) << 8) | ((int(force_variant) & 0xf) << 16) | ((int(force_rpw) & 0xf) << 20) | \
             ((int(force_nt) & 0xf) << 24) | ({0: 0, 8: 1, 16: 2, 32: 3, 64: 4}[int(force_lpg)] << 28)
+    lib = _lib.load()
     with torch.cuda.device(b.device):
-        rc = _lib.load().iex_spmm_ex(
+        # room for the dense form of the sparse operand where the library would rather hand the
+        # product to its dense GEMM (large 16-bit products): from torch's allocator, on the current
+        # stream, released (stream-ordered) when this call returns
+        ws_bytes = 0 if no_workspace else lib.iex_spmm_workspace_bytes(
+            _DT[b.dtype], _IT[column_indices.dtype], flags, m, k, n, nonzeros, batch, int(bias is not None))
+        ws = torch.empty(ws_bytes, dtype=torch.uint8, device=b.device) if ws_bytes else None
+        rc = lib.iex_spmm_ws(
             _DT[b.dtype], _IT[column_indices.dtype], flags, m, k, n, nonzeros,
             row_indices.data_ptr(), values.data_ptr(), row_offsets.data_ptr(),
             column_indices.data_ptr(), b.data_ptr(), bias.data_ptr() if bias is not None else None,
-            out.data_ptr(), _stream_ptr(b.device), batch)
+            out.data_ptr(), _stream_ptr(b.device), batch, ws.data_ptr() if ws is not None else None, ws_bytes)
     _lib.check(rc, "spmm")
     return out
 

@@ -67,6 +67,36 @@ def test_replay_own_operators_several_times(dev):
     constructor.destroy_graph_exec()
 
 
+def test_replay_spmm_that_uses_a_workspace(dev):
+    """A 16-bit product large enough for the dense-form path: the operator takes its workspace from
+    the allocator inside the capture, so it must come from the capture's pool and stay out of the
+    hands of tensors created between the replays."""
+    from intrasm_engine_amd import _lib
+    rng = np.random.default_rng(3)
+    m = k = 2048
+    n = 1024
+    ro, ci = W.csr_from_row_lengths(rng, m, k, rng.binomial(k, 0.2, m))
+    ri = torch.from_numpy(W.swizzle_from_offsets(ro)).to(dev)
+    ro_t, ci_t = torch.from_numpy(ro).to(dev), torch.from_numpy(ci.astype(np.int16)).to(dev)
+    v = torch.randn(ci.shape[0], device=dev).half()
+    b = torch.randn(1, k, n, device=dev).half()
+    assert _lib.load().iex_spmm_workspace_bytes(_lib.F16, _lib.I16, 0, m, k, n, ci.shape[0], 1, 0) == m * k * 2
+    constructor = TorchCUDAGraphConstructor()
+    with constructor.get_primary_stream():
+        with constructor:
+            out = ops.spmm_sputnik_reuse_weight_half(b, ri, v, ro_t, ci_t, m)
+    constructor.instantiate_graph_exec()
+    for it in range(4):
+        b.copy_(torch.randn(1, k, n, device=dev).half())
+        clutter = [torch.full((m * k,), float(it), device=dev, dtype=torch.float16) for _ in range(3)]
+        torch.cuda.synchronize()
+        constructor.execute_graph()
+        constructor.synchronize()
+        assert torch.equal(out, ops.spmm_sputnik_reuse_weight_half(b, ri, v, ro_t, ci_t, m)), it
+        assert all(bool((t == float(it)).all()) for t in clutter), it
+    constructor.destroy_graph_exec()
+
+
 def test_two_branches_join_structure_and_results(dev, tmp_path):
     a = W.config2_matrix(0.95, m=512, k=512)
     ri, v, ro, ci = to_dev(a, dev)

@@ -469,7 +469,8 @@ def test_automatic_choice_of_kernel_family(oracle, dev, dtype, k, n, density, fa
     b_np = rng.standard_normal((1, k, n)).astype(np.float32)
     ri, v, ro_t, ci_t = to_dev(csr, dev, dtype)
     b = torch.from_numpy(b_np).to(dev).to(dtype)
-    kw = dict(per_batch_values=False, accumulate=False, dtypes=(dtype,), allow_i16=False)
+    # (no workspace: the choice among the kernels that need none, what iex_spmm_ex does)
+    kw = dict(per_batch_values=False, accumulate=False, dtypes=(dtype,), allow_i16=False, no_workspace=True)
     out = pyops._spmm(b, ri, v, ro_t, ci_t, m, **kw)
     vals_r, b_r = rounded(csr.values, dtype), rounded(b_np, dtype)
     want = oracle.spmm(b_r, csr.row_indices, vals_r, csr.row_offsets, csr.column_indices, m)
@@ -548,3 +549,79 @@ def test_rows_that_are_not_a_multiple_of_the_vector(oracle, dev, wpr, dtype, n):
     out = pyops._spmm(b, ri, v, ro_t, ci_t, m, accumulate=True, out=init.clone(), **kw)
     want = oracle.spmm(b_r, csr.row_indices, vals_r, csr.row_offsets, csr.column_indices, m, out_init=rounded(init_np, dtype))
     assert_close(out.float().cpu().numpy(), want, scale + np.abs(init_np), RTOL[dtype], "ragged rows, accumulate")
+
+
+def _dense_form_case(rng, m, k, n, batch, dtype, itype, dev, mean_len=30.0):
+    lens = np.clip(rng.geometric(1 / mean_len, m), 0, k)
+    lens[0] = 0
+    lens[3] = k
+    ro, ci = W.csr_from_row_lengths(rng, m, k, lens)
+    csr = W.CSR(m, k, rng.standard_normal(ci.shape[0]).astype(np.float32), W.swizzle_from_offsets(ro), ro, ci)
+    b_np = rng.standard_normal((batch, k, n)).astype(np.float32)
+    ri, v, ro_t, ci_t = to_dev(csr, dev, dtype)
+    return csr, b_np, (ri, v, ro_t, ci_t.to(itype)), torch.from_numpy(b_np).to(dev).to(dtype)
+
+
+@pytest.mark.parametrize("dtype,itype,m,k,n,batch", [(torch.float16, torch.int16, 203, 160, 256, 2),
+                                                     (torch.bfloat16, torch.int32, 75, 304, 264, 1),
+                                                     (torch.float16, torch.int16, 130, 64, 8, 3),
+                                                     (torch.float16, torch.int32, 16, 16392, 512, 1)])
+def test_dense_form_path(oracle, dev, dtype, itype, m, k, n, batch):
+    """Family 7: the dense form of A written into a workspace, then the dense GEMM.  Empty rows, a
+    full row, a batch, a k beyond one segment of the row assembly (and no multiple of it)."""
+    from intrasm_engine_amd.pytorch import ops as pyops
+    csr, b_np, (ri, v, ro_t, ci_t), b = _dense_form_case(np.random.default_rng(m + n), m, k, n, batch, dtype, itype, dev)
+    out = pyops._spmm(b, ri, v, ro_t, ci_t, m, per_batch_values=False, accumulate=False, dtypes=(dtype,),
+                      allow_i16=True, force_variant=7)
+    vals_r, b_r = rounded(csr.values, dtype), rounded(b_np, dtype)
+    want = oracle.spmm(b_r, csr.row_indices, vals_r, csr.row_offsets, csr.column_indices, m)
+    scale = oracle.spmm_abs_scale(b_r, csr.row_indices, vals_r, csr.row_offsets, csr.column_indices, m)
+    assert_close(out.float().cpu().numpy(), want, scale, RTOL[dtype], f"dense form {dtype} {m}x{k}x{n}")
+
+
+def test_dense_form_path_is_chosen_with_a_workspace_and_only_then(oracle, dev):
+    """2048 x 2048 at 80 % sparsity times 2048 x 1024 in fp16: the time model prefers the dense form
+    (measured 34 against 71 us).  The operator asks the library for the workspace size, allocates it
+    and gets the dense-form result; the entry point without a workspace, a short workspace, and
+    shapes the path does not serve (fp32, per-batch values, a bias, a small product) run the other
+    kernels."""
+    from intrasm_engine_amd import _lib
+    from intrasm_engine_amd.pytorch import ops as pyops
+    lib = _lib.load()
+    m = k = 2048
+    n = 1024
+    dtype = torch.float16
+    rng = np.random.default_rng(12)
+    csr, b_np, (ri, v, ro_t, ci_t), b = _dense_form_case(rng, m, k, n, 1, dtype, torch.int16, dev, mean_len=0.2 * k)
+    nnz = csr.column_indices.shape[0]
+    need = lib.iex_spmm_workspace_bytes(_lib.F16, _lib.I16, 0, m, k, n, nnz, 1, 0)
+    assert need == m * k * 2
+    assert lib.iex_spmm_workspace_bytes(_lib.F32, _lib.I32, 0, m, k, n, nnz, 1, 0) == 0
+    assert lib.iex_spmm_workspace_bytes(_lib.F16, _lib.I16, _lib.SPMM_PER_BATCH_VALUES, m, k, n, nnz, 1, 0) == 0
+    assert lib.iex_spmm_workspace_bytes(_lib.F16, _lib.I16, _lib.SPMM_ACCUMULATE, m, k, n, nnz, 1, 0) == 0
+    assert lib.iex_spmm_workspace_bytes(_lib.F16, _lib.I16, 0, m, k, n, nnz, 1, 1) == 0      # bias
+    assert lib.iex_spmm_workspace_bytes(_lib.F16, _lib.I16, 0, 128, 128, 64, 1000, 1, 0) == 0  # too small to pay
+    assert lib.iex_spmm_workspace_bytes(_lib.F16, _lib.I16, 0, m, k, n - 4, nnz, 1, 0) == 0    # n no multiple of 8
+    assert lib.iex_spmm_workspace_bytes(_lib.F16, _lib.I16, 7 << 16, 128, 128, 64, 1000, 1, 0) == 128 * 128 * 2  # on request
+    kw = dict(per_batch_values=False, accumulate=False, dtypes=(dtype,), allow_i16=True)
+    auto = pyops._spmm(b, ri, v, ro_t, ci_t, m, **kw)
+    assert torch.equal(auto, pyops._spmm(b, ri, v, ro_t, ci_t, m, force_variant=7, **kw))
+    vals_r, b_r = rounded(csr.values, dtype), rounded(b_np, dtype)
+    want = oracle.spmm(b_r, csr.row_indices, vals_r, csr.row_offsets, csr.column_indices, m)
+    scale = oracle.spmm_abs_scale(b_r, csr.row_indices, vals_r, csr.row_offsets, csr.column_indices, m)
+    assert_close(auto.float().cpu().numpy(), want, scale, RTOL[dtype], "dense form, chosen")
+    # without a workspace, and with one that is too short, the gather kernel runs: bit-equal to family 1
+    row = pyops._spmm(b, ri, v, ro_t, ci_t, m, force_variant=1, **kw)
+    assert torch.equal(pyops._spmm(b, ri, v, ro_t, ci_t, m, no_workspace=True, **kw), row)
+    assert not torch.equal(auto, row)   # (the matrix cores sum in another order)
+    short = torch.empty(need - 16, dtype=torch.uint8, device=dev)
+    out = torch.empty_like(row)
+    args = (_lib.F16, _lib.I16, 0, m, k, n, nnz, ri.data_ptr(), v.data_ptr(), ro_t.data_ptr(), ci_t.data_ptr(),
+            b.data_ptr(), None, out.data_ptr(), torch.cuda.current_stream().cuda_stream, 1)
+    assert lib.iex_spmm_ws(*args, short.data_ptr(), need - 16) == 0, _lib.last_error()
+    assert torch.equal(out, row)
+    # the path on request where it cannot run: an error, not another kernel
+    forced = (_lib.F16, _lib.I16, 7 << 16) + args[3:]
+    assert lib.iex_spmm_ex(*forced) != 0 and "workspace" in _lib.last_error()
+    assert lib.iex_spmm_ws(*forced, short.data_ptr(), need - 16) != 0 and "workspace" in _lib.last_error()
+    torch.cuda.synchronize()

@@ -40,7 +40,9 @@ def test_every_kernel_choice_keeps_parity(oracle, dev, dtype):
     want_dv = oracle.sddmm(gr[None], br[None], a.row_indices, a.row_offsets, a.column_indices)
     scale_dv = oracle.sddmm_abs_scale(gr[None], br[None], a.row_indices, a.row_offsets, a.column_indices)
     outputs = {}
-    for i, kernel in enumerate(spmm_kernel_choices(dtype, b_np.shape[1])):
+    choices = spmm_kernel_choices(dtype, b_np.shape[1], a.k, a.m)
+    assert ("dense_form_gemm" in choices) == (dtype == torch.float16)
+    for i, kernel in enumerate(choices):
         b = inputs[0].detach().clone().requires_grad_(True)
         v = inputs[2].detach().clone().requires_grad_(True)
         params = {"spmm_kernel": kernel, "grad_dense_kernel": kernel, "grad_values_wpr": (0, 1, 4)[i % 3]}

@@ -101,8 +101,10 @@ def test_tune_my_autograd_function_front_end():
 
 
 def test_search_spaces_of_the_path():
-    half = spmm_kernel_choices(torch.float16, 128)
-    assert half[0] == "auto" and "mfma8_windows4" in half and "mfma4_lanes16" in half
+    half = spmm_kernel_choices(torch.float16, 128, 64, 256)
+    assert half[0] == "auto" and "mfma8_windows4" in half and "mfma4_lanes16" in half and half[-1] == "dense_form_gemm"
+    assert "dense_form_gemm" not in spmm_kernel_choices(torch.float16, 128)          # shape of the sparse operand unknown
+    assert "dense_form_gemm" not in spmm_kernel_choices(torch.float16, 128, 64, 100)  # m % 8 != 0 (k of the backward product)
     assert not any(k.startswith("mfma32") for k in half)
     assert not any(k.startswith("mfma") for k in spmm_kernel_choices(torch.float16, 100))    # n % 8 != 0
     single = spmm_kernel_choices(torch.float32, 64)

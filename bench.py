@@ -317,6 +317,22 @@ def run_extras(torch, ops, dev, W, IL, mats, dens, csr_dev, time_cell, variant_o
         "us": round(us_block, 2), "softmax_us": round(us_softmax, 2),
         "what": "SDDMM -> softmax over CSR rows -> SpMM, three launches; 16 heads x 4096 tokens x 64",
         "GFLOPs": round((W.sddmm_flops(pat.nnz, 64, 16) + W.spmm_flops(pat.nnz, 64, 16)) / us_block / 1e3, 1)}
+    # the weight gradient of a sparse linear layer is an SDDMM with k = tokens: config 4's weight (11008 x 4096 at
+    # 90 %) against 2048 tokens, fp16; the operator computes the dense product on the matrix cores and samples it
+    from intrasm_engine_amd.pytorch import ops as pyops_
+    w4g = W.config4()[0]
+    riw_, _, row_, ciw_ = csr_dev(w4g)
+    gy = (torch.randn(1, w4g.m, 2048, device=dev, generator=torch.Generator(dev).manual_seed(2)) * 0.1).half()
+    xx = torch.randn(1, w4g.k, 2048, device=dev, generator=torch.Generator(dev).manual_seed(3)).half()
+    kw_ = dict(sum_over_batch=False, dtypes=(torch.float16,))
+    us_g = time_cell(lambda: pyops_._sddmm(gy, xx, riw_, row_, ciw_, force_variant=1, **kw_), repeats=3, samples=3)
+    us_d = time_cell(lambda: ops.sddmm_sputnik_half(gy, xx, riw_, row_, ciw_), repeats=5)
+    out["sddmm_weight_gradient_c4_fp16"] = {
+        "what": "SDDMM on config 4's mask (11008 x 4096, 90 % sparse) with k = 2048 tokens",
+        "gather_kernel_us": round(us_g, 1), "operator_us": round(us_d, 1),
+        "operator_path": "dense product by the GEMM into a workspace, then sampling",
+        "operator_dense_equivalent_TFLOPs": round(2.0 * w4g.m * w4g.k * 2048 / us_d / 1e6, 1)}
+    del gy, xx, riw_, row_, ciw_, w4g
     log("[bench] SDDMM done")
 
     # ---- config 4: fp16 SpMM 11008x4096 @90% x 4096x2048  ||  bf16 GEMM 4096x4096x2048

@@ -135,6 +135,9 @@ int iex_CudaSpmm5(int m, int k, int n, int nonzeros, const int* row_indices,
 #define IEX_SDDMM_ACCUMULATE 0x2     /* out += ... instead of out = ...                   */
 /* bits 8..15: force wavefronts per row (1 or 4); 0 = choose from nnz/m.  For tuning.     */
 #define IEX_SDDMM_FORCE_WPR(w) (((w) & 0xff) << 8)
+/* bits 16..19: 1 = the gather kernel, 7 = dense product in the caller's workspace, then
+ * sampling (iex_sddmm_ws only; fails where it cannot run).  0 = choose.                  */
+#define IEX_SDDMM_FORCE_VARIANT(v) (((v) & 0xf) << 16)
 
 /* out[(z,) j] = sum_c lhs[z, row(j), c] * rhs[z, column_indices[j], c]
  * lhs is (batch, m, k), rhs is (batch, n, k) -- rhs rows are the sampled columns.
@@ -144,6 +147,24 @@ int iex_sddmm_ex(int dtype, int flags, int m, int k, int n, int nonzeros,
                  const int* row_indices, const int* row_offsets, const int* column_indices,
                  const void* lhs_matrix, const void* rhs_matrix, void* output_values,
                  void* stream, int batch);
+
+/* iex_sddmm_ex with a workspace in device memory that the call may use (and overwrite) until
+ * the work it puts on `stream` has run.  With `workspace_bytes` >= iex_sddmm_workspace_bytes(...)
+ * and a 16-byte aligned `workspace`, fp16 / bf16 calls with a long k and a mask that is not very
+ * sparse compute the whole product lhs * rhs^T (m * n * 2 bytes per batch entry, one entry at a
+ * time) with the dense GEMM and pick the nonzeros' entries: the gather kernel reads k * 2 bytes of
+ * rhs per nonzero, which costs more than all m * n dot products on the matrix cores (weight
+ * gradients of a sparse linear layer: k = tokens).  Same arithmetic per output (fp32 accumulation,
+ * one rounding).  Needs plain store, (batch, nnz) output or batch 1, k and n multiples of 8;
+ * anything else, and a NULL or short workspace, runs exactly as iex_sddmm_ex.
+ * iex_sddmm_workspace_bytes returns the size with which the call described would use the
+ * workspace, 0 when it would not whatever the size.  Neither call allocates.
+ * No counterpart in the reference: CudaSddmm2 (csrc/extensions.h:31) takes no workspace. */
+int iex_sddmm_ws(int dtype, int flags, int m, int k, int n, int nonzeros,
+                 const int* row_indices, const int* row_offsets, const int* column_indices,
+                 const void* lhs_matrix, const void* rhs_matrix, void* output_values,
+                 void* stream, int batch, void* workspace, size_t workspace_bytes);
+size_t iex_sddmm_workspace_bytes(int dtype, int flags, int m, int k, int n, int nonzeros, int batch);
 
 /* Drop-in for CudaSddmm2 (csrc/extensions.h:31; sddmm_sputnik_atomic_upd_weight,
  * sputnik_kernels.cpp:182-184): fp32, output (nnz) = sum over the batch, written

@@ -37,6 +37,8 @@ SIGNATURES = {
     "iex_CudaSpmm3": (_i, [_i, _i, _i, _i, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i]),
     "iex_CudaSpmm5": (_i, [_i, _i, _i, _i, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i]),
     "iex_sddmm_ex": (_i, [_i, _i, _i, _i, _i, _i, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i]),
+    "iex_sddmm_ws": (_i, [_i, _i, _i, _i, _i, _i, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _vp, _c.c_size_t]),
+    "iex_sddmm_workspace_bytes": (_c.c_size_t, [_i, _i, _i, _i, _i, _i, _i]),
     "iex_CudaSddmm2": (_i, [_i, _i, _i, _i, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i]),
     "iex_csr_softmax": (_i, [_i, _i, _i, _vp, _vp, _vp, _f, _vp, _i]),
     "iex_gemm": (_i, [_i, _i, _i, _i, _i, _vp, _vp, _vp, _i, _ll, _ll, _ll, _vp]),

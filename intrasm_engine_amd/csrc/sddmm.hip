@@ -16,6 +16,8 @@
 //     row_half_mirror, row_mirror): no LDS, no bpermute in the reduction.
 // Accumulation is fp32; with SUM_OVER_BATCH the batch loop runs inside the kernel so
 // the (nnz) output is a deterministic sum.
+#include <algorithm>
+#include <cmath>
 #include "iex_common.h"
 
 namespace iex {
@@ -205,11 +207,81 @@ int launch_typed(const SddmmParams& p, int wpr, hipStream_t stream) {
   return launch_passes<T, 1, 16>(p, wpr, stream);
 }
 
+// ---- dense product, then sampling (16-bit types, caller's workspace of m * n * 2 bytes) ----
+// A long k makes the gather kernel read k * 2 bytes of rhs per nonzero through the L2 -> CU path;
+// the dense GEMM computes all m * n dot products on the matrix cores in less time than that takes
+// once the mask is not very sparse, and a small kernel then picks the nonzeros' entries.
+// Same arithmetic per output (fp32 accumulation over k, one rounding to the 16-bit type).
+__global__ __launch_bounds__(256) void sample_dense_kernel(int m, int n, const int* __restrict__ row_offsets,
+                                                           const int* __restrict__ cols,
+                                                           const uint16_t* __restrict__ dense,
+                                                           uint16_t* __restrict__ out) {
+  const int row = blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (row >= m) return;
+  const int start = row_offsets[row], end = row_offsets[row + 1];
+  const uint16_t* drow = dense + (size_t)row * n;
+  for (int j = start + lane_id(); j < end; j += kWave) out[j] = drow[cols[j]];
+}
+
+inline bool sddmm_dense_fits(int dtype, const SddmmParams& p) {
+  return (dtype == IEX_F16 || dtype == IEX_BF16) && !p.accumulate && !(p.sum_over_batch && p.batch > 1) &&
+         p.k > 0 && p.k % 8 == 0 && p.n % 8 == 0 && (long long)p.m * p.n < (1ll << 31) && aligned(p.lhs, 16) &&
+         aligned(p.rhs, 16);
+}
+
+inline size_t sddmm_dense_bytes(const SddmmParams& p) { return (size_t)p.m * p.n * 2; }
+
+// Time model fitted on MI355X (fp16).  Dense product per batch entry: three launches, the GEMM at
+// 1000 TFLOP/s or, with few tiles, 0.35 us per K step of 32 per round of 512 tiles of 128 x 128,
+// m * n * 2 bytes written and nnz entries picked at 4 TB/s.  Gather kernel: nnz * k * 2 bytes at
+// 15 TB/s (16 heads of 4096 x 4096 at 93 % sparsity, k = 64: 125 us; 2048 x 1024 at 80 %, k = 2048:
+// 117 us), and with a k beyond the register-resident fragments no less than one wave's chain of
+// dependent loads (0.34 us per 128 elements of k and step of 4 nonzeros: 1024 x 1024 at 95 %,
+// k = 4096: 141 us).  Measured: 11008 x 4096 at 80 %, k = 8192 (weight gradient of an MLP
+// projection) 16.5 -> 0.77 ms; 4096 x 4096 at 50 %, k = 8192 9.7 -> 0.32 ms; 4096 x 4096 at 90 %,
+// k = 512 120 -> 55 us.  The dense product has to win by 15 %.
+inline bool sddmm_dense_wins(const SddmmParams& p) {
+  const double flops = 2.0 * p.m * p.n * p.k;
+  const double tiles = (double)ceil_div(p.m, 128) * ceil_div(p.n, 128);
+  const double product = std::max(flops / 1000e12, std::ceil(tiles / 512.0) * (p.k / 32.0) * 0.35e-6);
+  const double dense = p.batch * (16e-6 + product + ((double)p.m * p.n * 2 + (double)p.nnz * 8) / 4e12);
+  const double row_nnz = (double)p.nnz / p.m;
+  const double chain = p.k > 256 ? std::ceil(row_nnz / (row_nnz >= 64.0 ? 16.0 : 4.0)) * (p.k / 128.0) * 0.34e-6 : 0.0;
+  const double gather = std::max(8e-6 + (double)p.batch * p.nnz * p.k * 2 / 15e12, chain);
+  return 1.15 * dense < gather;
+}
+
+int launch_sddmm_dense(int dtype, const SddmmParams& p, void* ws, hipStream_t stream) {
+  for (int z = 0; z < p.batch; ++z) {
+    const uint16_t* lhs = static_cast<const uint16_t*>(p.lhs) + (size_t)z * p.m * p.k;
+    const uint16_t* rhs = static_cast<const uint16_t*>(p.rhs) + (size_t)z * p.n * p.k;
+    if (int rc = iex_gemm(dtype, 1, p.m, p.n, p.k, lhs, rhs, ws, 1, 0, 0, 0, stream)) return rc;
+    hipLaunchKernelGGL(sample_dense_kernel, dim3(ceil_div(p.m, 4)), dim3(256), 0, stream, p.m, p.n, p.row_offsets, p.cols,
+                       static_cast<const uint16_t*>(ws), static_cast<uint16_t*>(p.out) + (size_t)z * p.nnz);
+    if (int rc = check_hip(hipGetLastError(), "sddmm sampling launch")) return rc;
+  }
+  return 0;
+}
+
 }  // namespace
+
+// Bytes of workspace with which iex_sddmm_ws would compute the dense product and sample it (0: it
+// would not, whatever the workspace).  Pointers are taken to be 16-byte aligned.
+size_t sddmm_workspace_bytes(int dtype, int flags, int m, int k, int n, int nonzeros, int batch) {
+  if (m <= 0 || k <= 0 || n <= 0 || nonzeros <= 0 || batch <= 0) return 0;
+  const int variant = (flags >> 16) & 0xf;
+  if (variant != 0 && variant != 7) return 0;
+  void* const some_aligned = reinterpret_cast<void*>(size_t(256));
+  SddmmParams p{m, k, n, nonzeros, batch, nullptr, nullptr, nullptr, some_aligned, some_aligned, nullptr,
+                (flags & IEX_SDDMM_SUM_OVER_BATCH) != 0, (flags & IEX_SDDMM_ACCUMULATE) != 0};
+  if (!sddmm_dense_fits(dtype, p)) return 0;
+  if (variant == 0 && !sddmm_dense_wins(p)) return 0;
+  return sddmm_dense_bytes(p);
+}
 
 int sddmm_dispatch(int dtype, int flags, int m, int k, int n, int nonzeros, const int* row_indices,
                    const int* row_offsets, const int* column_indices, const void* lhs, const void* rhs,
-                   void* out, void* stream, int batch) {
+                   void* out, void* stream, int batch, void* workspace, size_t workspace_bytes) {
   IEX_REQUIRE(m >= 0 && k >= 0 && n >= 0 && nonzeros >= 0 && batch >= 0, IEX_ERR_BAD_ARGUMENT,
               "sddmm: negative dimension (m=%d k=%d n=%d nnz=%d batch=%d)", m, k, n, nonzeros, batch);
   if (m == 0 || nonzeros == 0 || batch == 0) return 0;
@@ -224,6 +296,16 @@ int sddmm_dispatch(int dtype, int flags, int m, int k, int n, int nonzeros, cons
   int wpr = (flags >> 8) & 0xff;  // forced (1 or 4), else from the mean row length
   if (wpr != 1 && wpr != 4) wpr = ((double)nonzeros / m >= 64.0) ? 4 : 1;
   hipStream_t s = static_cast<hipStream_t>(stream);
+  const int variant = (flags >> 16) & 0xf;  // 0 = choose, 1 = gather kernel, 7 = dense product then sampling
+  if (variant == 0 || variant == 7) {
+    const bool fits = sddmm_dense_fits(dtype, p);
+    const bool room = workspace && aligned(workspace, 16) && workspace_bytes >= sddmm_dense_bytes(p);
+    if (variant == 7) {
+      IEX_REQUIRE(fits, IEX_ERR_UNSUPPORTED, "sddmm: the dense-product path needs fp16 / bf16, plain store, one batch entry per output, k and n multiples of 8 and 16-byte aligned operands");
+      IEX_REQUIRE(room, IEX_ERR_BAD_ARGUMENT, "sddmm: the dense-product path needs a 16-byte aligned workspace of %zu bytes (iex_sddmm_ws)", sddmm_dense_bytes(p));
+    }
+    if (fits && room && (variant == 7 || sddmm_dense_wins(p))) return launch_sddmm_dense(dtype, p, workspace, s);
+  }
   switch (dtype) {
     case IEX_F32: return launch_typed<float>(p, wpr, s);
     case IEX_F16: return launch_typed<__half>(p, wpr, s);
@@ -240,7 +322,19 @@ int iex_sddmm_ex(int dtype, int flags, int m, int k, int n, int nonzeros, const 
                  const int* row_offsets, const int* column_indices, const void* lhs_matrix,
                  const void* rhs_matrix, void* output_values, void* stream, int batch) {
   return iex::sddmm_dispatch(dtype, flags, m, k, n, nonzeros, row_indices, row_offsets, column_indices,
-                             lhs_matrix, rhs_matrix, output_values, stream, batch);
+                             lhs_matrix, rhs_matrix, output_values, stream, batch, nullptr, 0);
+}
+
+int iex_sddmm_ws(int dtype, int flags, int m, int k, int n, int nonzeros, const int* row_indices,
+                 const int* row_offsets, const int* column_indices, const void* lhs_matrix,
+                 const void* rhs_matrix, void* output_values, void* stream, int batch, void* workspace,
+                 size_t workspace_bytes) {
+  return iex::sddmm_dispatch(dtype, flags, m, k, n, nonzeros, row_indices, row_offsets, column_indices,
+                             lhs_matrix, rhs_matrix, output_values, stream, batch, workspace, workspace_bytes);
+}
+
+size_t iex_sddmm_workspace_bytes(int dtype, int flags, int m, int k, int n, int nonzeros, int batch) {
+  return iex::sddmm_workspace_bytes(dtype, flags, m, k, n, nonzeros, batch);
 }
 
 int iex_CudaSddmm2(int m, int k, int n, int nonzeros, const int* row_indices, const int* row_offsets,
@@ -248,7 +342,7 @@ int iex_CudaSddmm2(int m, int k, int n, int nonzeros, const int* row_indices, co
                    float* output_values, void* stream, int batch_size) {
   return iex::sddmm_dispatch(IEX_F32, IEX_SDDMM_SUM_OVER_BATCH, m, k, n, nonzeros, row_indices,
                              row_offsets, column_indices, lhs_matrix, rhs_matrix, output_values, stream,
-                             batch_size);
+                             batch_size, nullptr, 0);
 }
 
 }  // extern "C"

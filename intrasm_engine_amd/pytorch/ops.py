@@ -152,10 +152,10 @@ def _spmm(b, row_indices, values, row_offsets, column_indices, m, *, per_batch_v
 
 
 def _sddmm(a, b, row_indices, row_offsets, column_indices, *, sum_over_batch, dtypes,
-           out=None, accumulate=False, force_wpr=0):
+           out=None, accumulate=False, force_wpr=0, force_variant=0, no_workspace=False):
     tuned = getattr(_TUNING, "sddmm", None)
-    if tuned and not force_wpr:
-        force_wpr = tuned.get("force_wpr", 0)
+    if tuned and not (force_wpr or force_variant):
+        force_wpr, force_variant = tuned.get("force_wpr", 0), tuned.get("force_variant", 0)
     _chk(a.dim() == b.dim())
     _chk(a.dim() == 3)
     _chk(a.size(0) == b.size(0))
@@ -180,12 +180,18 @@ def _sddmm(a, b, row_indices, row_offsets, column_indices, *, sum_over_batch, dt
         _chk(tuple(out.shape) == shape and out.dtype == a.dtype and out.is_contiguous()
              and out.device == a.device, "out has the wrong shape, dtype, layout or device")
     flags = (_lib.SDDMM_SUM_OVER_BATCH if sum_over_batch else 0) | \
-            (_lib.SDDMM_ACCUMULATE if accumulate else 0) | ((int(force_wpr) & 0xff) << 8)
+            (_lib.SDDMM_ACCUMULATE if accumulate else 0) | ((int(force_wpr) & 0xff) << 8) | \
+            ((int(force_variant) & 0xf) << 16)
+    lib = _lib.load()
     with torch.cuda.device(a.device):
-        rc = _lib.load().iex_sddmm_ex(
+        # room for the dense product where the library would rather compute all of it on the matrix
+        # cores and pick the nonzeros (16-bit, long k): from torch's allocator, on the current stream
+        ws_bytes = 0 if no_workspace else lib.iex_sddmm_workspace_bytes(_DT[a.dtype], flags, m, k, n, nonzeros, batch)
+        ws = torch.empty(ws_bytes, dtype=torch.uint8, device=a.device) if ws_bytes else None
+        rc = lib.iex_sddmm_ws(
             _DT[a.dtype], flags, m, k, n, nonzeros, row_indices.data_ptr(), row_offsets.data_ptr(),
             column_indices.data_ptr(), a.data_ptr(), b.data_ptr(), out.data_ptr(),
-            _stream_ptr(a.device), batch)
+            _stream_ptr(a.device), batch, ws.data_ptr() if ws is not None else None, ws_bytes)
     _lib.check(rc, "sddmm")
     return out
 

@@ -155,3 +155,72 @@ def test_operator_argument_checks(dev):
         ops.sddmm_sputnik_atomic_upd_weight(lhs, rhs[:, :, :32].contiguous(), ri, ro, ci)   # k mismatch
     with pytest.raises(RuntimeError, match="b must be a contiguous tensor"):
         ops.sddmm_sputnik_atomic_upd_weight(lhs, rhs.transpose(1, 2).contiguous().transpose(1, 2), ri, ro, ci)
+
+
+def _dense_product_case(rng, m, k, n, sparsity, batch, dtype, dev):
+    lens = rng.binomial(n, 1 - sparsity, m)
+    lens[0] = 0
+    lens[min(3, m - 1)] = n
+    ro, ci = W.csr_from_row_lengths(rng, m, n, lens)
+    csr = W.CSR(m, n, np.zeros(ci.shape[0], np.float32), W.swizzle_from_offsets(ro), ro, ci)
+    lhs_np = (rng.standard_normal((batch, m, k)) * 0.25).astype(np.float32)
+    rhs_np = rng.standard_normal((batch, n, k)).astype(np.float32)
+    t = lambda x: torch.from_numpy(x).to(dev).to(dtype)
+    return csr, lhs_np, rhs_np, t(lhs_np), t(rhs_np), to_dev(csr, dev)
+
+
+@pytest.mark.parametrize("dtype,m,k,n,batch", [(torch.float16, 203, 160, 256, 2), (torch.bfloat16, 75, 304, 264, 1),
+                                               (torch.float16, 130, 8, 8, 3), (torch.float16, 33, 1032, 520, 1)])
+def test_dense_product_path(oracle, dev, dtype, m, k, n, batch):
+    """The whole product lhs * rhs^T by the dense GEMM into a workspace, then the nonzeros' entries
+    picked: on request on small ragged shapes (an empty row, a full row, a batch), against the oracle."""
+    from intrasm_engine_amd.pytorch import ops as pyops
+    csr, lhs_np, rhs_np, lhs, rhs, (ri, _, ro, ci) = _dense_product_case(np.random.default_rng(m + k), m, k, n, 0.8, batch, dtype, dev)
+    out = pyops._sddmm(lhs, rhs, ri, ro, ci, sum_over_batch=False, dtypes=(dtype,), force_variant=7)
+    assert out.shape == (batch, csr.nnz) and out.dtype == dtype
+    l_r, r_r = rounded(lhs_np, dtype), rounded(rhs_np, dtype)
+    want = oracle.sddmm(l_r, r_r, csr.row_indices, csr.row_offsets, csr.column_indices, sum_over_batch=False)
+    scale = oracle.sddmm_abs_scale(l_r, r_r, csr.row_indices, csr.row_offsets, csr.column_indices, sum_over_batch=False)
+    assert_close(out.float().cpu().numpy(), want, scale, RTOL[dtype], f"dense product {dtype} {m}x{k}x{n}")
+
+
+def test_dense_product_path_is_chosen_with_a_workspace_and_only_then(oracle, dev):
+    """1024 x 1024 mask at 70 % sparsity, k = 4096, fp16: the time model prefers the dense product.
+    The operator asks for the workspace size, allocates it and gets that result; without a workspace,
+    with a short one, and for calls the path does not serve (fp32, batch-summed output of a batch,
+    accumulate, a short k with a sparse mask) the gather kernel runs."""
+    from intrasm_engine_amd import _lib
+    from intrasm_engine_amd.pytorch import ops as pyops
+    lib = _lib.load()
+    m = n = 1024
+    k = 4096
+    dtype = torch.float16
+    csr, lhs_np, rhs_np, lhs, rhs, (ri, _, ro, ci) = _dense_product_case(np.random.default_rng(8), m, k, n, 0.7, 1, dtype, dev)
+    nnz = csr.nnz
+    need = lib.iex_sddmm_workspace_bytes(_lib.F16, 0, m, k, n, nnz, 1)
+    assert need == m * n * 2
+    assert lib.iex_sddmm_workspace_bytes(_lib.F32, 0, m, k, n, nnz, 1) == 0
+    assert lib.iex_sddmm_workspace_bytes(_lib.F16, _lib.SDDMM_SUM_OVER_BATCH, m, k, n, nnz, 2) == 0
+    assert lib.iex_sddmm_workspace_bytes(_lib.F16, _lib.SDDMM_SUM_OVER_BATCH, m, k, n, nnz, 1) == need
+    assert lib.iex_sddmm_workspace_bytes(_lib.F16, _lib.SDDMM_ACCUMULATE, m, k, n, nnz, 1) == 0
+    assert lib.iex_sddmm_workspace_bytes(_lib.F16, 0, 4096, 64, 4096, 1150000, 16) == 0   # config 3: the gather kernel is faster
+    assert lib.iex_sddmm_workspace_bytes(_lib.F16, 7 << 16, 4096, 64, 4096, 1150000, 16) == 4096 * 4096 * 2  # on request
+    kw = dict(sum_over_batch=False, dtypes=(dtype,))
+    auto = pyops._sddmm(lhs, rhs, ri, ro, ci, **kw)
+    assert torch.equal(auto, pyops._sddmm(lhs, rhs, ri, ro, ci, force_variant=7, **kw))
+    l_r, r_r = rounded(lhs_np, dtype), rounded(rhs_np, dtype)
+    want = oracle.sddmm(l_r, r_r, csr.row_indices, csr.row_offsets, csr.column_indices, sum_over_batch=False)
+    scale = oracle.sddmm_abs_scale(l_r, r_r, csr.row_indices, csr.row_offsets, csr.column_indices, sum_over_batch=False)
+    assert_close(auto.float().cpu().numpy(), want, scale, RTOL[dtype], "dense product, chosen")
+    gather = pyops._sddmm(lhs, rhs, ri, ro, ci, force_variant=1, **kw)
+    assert torch.equal(pyops._sddmm(lhs, rhs, ri, ro, ci, no_workspace=True, **kw), gather)
+    assert not torch.equal(auto, gather)    # (another order of summation)
+    short = torch.empty(need - 16, dtype=torch.uint8, device=dev)
+    out = torch.empty_like(gather)
+    args = (_lib.F16, 0, m, k, n, nnz, ri.data_ptr(), ro.data_ptr(), ci.data_ptr(), lhs.data_ptr(), rhs.data_ptr(),
+            out.data_ptr(), torch.cuda.current_stream().cuda_stream, 1)
+    assert lib.iex_sddmm_ws(*args, short.data_ptr(), need - 16) == 0, _lib.last_error()
+    assert torch.equal(out, gather)
+    forced = (_lib.F16, 7 << 16) + args[2:]
+    assert lib.iex_sddmm_ex(*forced) != 0 and "workspace" in _lib.last_error()
+    torch.cuda.synchronize()

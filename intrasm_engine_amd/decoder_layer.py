@@ -51,11 +51,16 @@ class SparseDecoderLayer:
         ri, v, ro, ci, m = self.w[name]
         return ops.spmm_sputnik_reuse_weight_half(x.unsqueeze(0), ri, v, ro, ci, m)[0]
 
-    def _split_heads(self, t: torch.Tensor, seqs: int) -> torch.Tensor:
-        """(hidden, seqs*L) feature-major -> (seqs*heads, L, head_dim)."""
+    def _split_heads(self, t: torch.Tensor, seqs: int, scale: float = 1.0) -> torch.Tensor:
+        """(hidden, seqs*L) feature-major -> (seqs*heads, L, head_dim), times ``scale`` in the same pass."""
         L = t.shape[1] // seqs
-        return t.view(self.heads, self.head_dim, seqs, L).permute(2, 0, 3, 1).contiguous().view(
-            seqs * self.heads, L, self.head_dim)
+        src = t.view(self.heads, self.head_dim, seqs, L).permute(2, 0, 3, 1)
+        out = torch.empty((seqs, self.heads, L, self.head_dim), dtype=t.dtype, device=t.device)
+        if scale == 1.0:
+            out.copy_(src)
+        else:
+            torch.mul(src, scale, out=out)
+        return out.view(seqs * self.heads, L, self.head_dim)
 
     def _merge_heads(self, o: torch.Tensor, seqs: int) -> torch.Tensor:
         """(seqs*heads, L, head_dim) -> (hidden, seqs*L)."""
@@ -64,10 +69,16 @@ class SparseDecoderLayer:
             self.hidden, seqs * L)
 
     def _softmax(self, s: torch.Tensor) -> torch.Tensor:
-        return torch.softmax(s.float() * (1.0 / math.sqrt(self.head_dim)), dim=-1).half()
+        """Over keys; the scores arrive scaled (1/sqrt(d) is folded into Q where the heads are split),
+        so this is one pass: fp16 in, fp32 inside the kernel, fp16 out."""
+        return torch.softmax(s, dim=-1)
+
+    def _split_qkv(self, q, k, v, seqs: int):
+        return (self._split_heads(q, seqs, 1.0 / math.sqrt(self.head_dim)), self._split_heads(k, seqs),
+                self._split_heads(v, seqs))
 
     def attention(self, q, k, v, seqs: int) -> torch.Tensor:
-        Q, K, V = (self._split_heads(t, seqs) for t in (q, k, v))
+        Q, K, V = self._split_qkv(q, k, v, seqs)
         P = self._softmax(ops.gemm_mfma(Q, K, True))      # (B, L, L)
         return self._merge_heads(ops.gemm_mfma(P, V, False), seqs)
 
@@ -91,12 +102,12 @@ class SparseDecoderLayer:
         """Halves a and b of the batch; the dense GEMMs of one half ride along with sparse
         projections of the other half."""
         qa, ka, va = self.proj("q", xa), self.proj("k", xa), self.proj("v", xa)
-        Qa, Ka, Va = (self._split_heads(t, seqs_half) for t in (qa, ka, va))
+        Qa, Ka, Va = self._split_qkv(qa, ka, va, seqs_half)
         qb, Sa = self._fused("q", xb, Qa, Ka, True, group)              # b.q  ||  a.QK^T
         Pa = self._softmax(Sa)
         kb, Oa = self._fused("k", xb, Pa, Va, False, group)             # b.k  ||  a.PV
         vb = self.proj("v", xb)
-        Qb, Kb, Vb = (self._split_heads(t, seqs_half) for t in (qb, kb, vb))
+        Qb, Kb, Vb = self._split_qkv(qb, kb, vb, seqs_half)
         oa, Sb = self._fused("o", self._merge_heads(Oa, seqs_half), Qb, Kb, True, group)   # a.o  ||  b.QK^T
         ha = xa + oa
         Pb = self._softmax(Sb)

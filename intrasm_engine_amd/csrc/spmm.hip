@@ -407,9 +407,9 @@ inline bool dense_path_wins(const SpmmParams& p, int batch, int matrix_core_kind
 
 template <typename T, typename IT>
 int launch_dense_path(const SpmmParams& p, int batch, const Choice& ch, hipStream_t stream) {
-  const int lds = min(p.k, kDenseSeg) * 2;
-  hipLaunchKernelGGL((csr_to_dense_kernel<IT>), dim3(p.m), dim3(kDenseThreads), lds, stream, p.k, p.row_offsets,
-                     static_cast<const IT*>(p.cols), static_cast<const uint16_t*>(p.values), static_cast<uint16_t*>(ch.ws));
+  hipLaunchKernelGGL((csr_to_dense_kernel<IT>), dim3(ceil_div(p.m, kDenseWaves)), dim3(kDenseThreads), 0, stream, p.m, p.k,
+                     p.row_offsets, static_cast<const IT*>(p.cols), static_cast<const uint16_t*>(p.values),
+                     static_cast<uint16_t*>(ch.ws));
   if (int rc = check_hip(hipGetLastError(), "spmm dense-form launch")) return rc;
   const int dtype = std::is_same<T, __half>::value ? IEX_F16 : IEX_BF16;
   return iex_gemm(dtype, 0, p.m, p.n, p.k, ch.ws, p.dense, p.out, batch, 0, (long long)p.k * p.n, (long long)p.m * p.n, stream);

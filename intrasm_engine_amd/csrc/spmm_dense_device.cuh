@@ -4,42 +4,61 @@
 // tile of the output; when the output has many column tiles it is cheaper to build the dense
 // form once, in a workspace of m * k * 2 bytes that stays in L2 / MALL, and let the GEMM read it.
 //
-// One workgroup per row: the row is assembled in LDS (zeros, then the nonzeros scattered to their
-// columns) and written with 128-bit stores, so every byte of the workspace is written exactly
-// once, by one kind of store, whatever the sparsity.  Rows longer than kDenseSeg columns are done
-// in segments.  Needs k % 8 == 0 and a 16-byte aligned workspace; column indices inside a row
-// must be distinct (with duplicates the last writer wins instead of the sum).
+// One wavefront per row, four independent wavefronts per workgroup and no barrier: the row is
+// assembled in the wavefront's own slice of LDS (zeros, then the nonzeros scattered to their
+// columns; LDS operations of one wavefront execute in order, so the reads that follow see both)
+// and written with 128-bit stores, so every byte of the workspace is written exactly once, by one
+// kind of store, whatever the sparsity.  Rows longer than kDenseSeg columns are done in segments,
+// with a cursor into the row's ascending column indices.  Needs k % 8 == 0 and a 16-byte aligned
+// workspace; column indices inside a row must ascend strictly (canonical CSR).
 #pragma once
 #include "iex_common.h"
 
 namespace iex {
 
-constexpr int kDenseSeg = 16384;  // columns of a row assembled at a time (32 KB of LDS)
-constexpr int kDenseThreads = 256;
+constexpr int kDenseSeg = 4096;  // columns of a row assembled at a time (8 KB of LDS per wavefront)
+constexpr int kDenseWaves = 4;
+constexpr int kDenseThreads = kDenseWaves * kWave;
 
 template <typename IT>
-__global__ __launch_bounds__(kDenseThreads) void csr_to_dense_kernel(int k, const int* __restrict__ row_offsets,
+__global__ __launch_bounds__(kDenseThreads) void csr_to_dense_kernel(int m, int k, const int* __restrict__ row_offsets,
                                                                      const IT* __restrict__ cols,
                                                                      const uint16_t* __restrict__ values,
                                                                      uint16_t* __restrict__ out) {
-  extern __shared__ __align__(16) unsigned char smem[];
-  uint16_t* srow = reinterpret_cast<uint16_t*>(smem);
-  const int tid = threadIdx.x;
-  const int row = blockIdx.x;
-  const int start = row_offsets[row], end = row_offsets[row + 1];
+  __shared__ __align__(16) uint16_t smem[kDenseWaves][kDenseSeg];
+  const int lane = lane_id();
+  const int wave = uniform(threadIdx.x >> 6);
+  const int row = blockIdx.x * kDenseWaves + wave;
+  if (row >= m) return;  // (no barrier below)
+  uint16_t* srow = smem[wave];
+  int pos = uniform(row_offsets[row]);
+  const int end = uniform(row_offsets[row + 1]);
   uint16_t* orow = out + (size_t)row * k;
   for (int c0 = 0; c0 < k; c0 += kDenseSeg) {
     const int len = min(kDenseSeg, k - c0);  // a multiple of 8
-    for (int i = tid * 8; i < len; i += kDenseThreads * 8) *reinterpret_cast<uint4*>(srow + i) = uint4{0u, 0u, 0u, 0u};
-    __syncthreads();
-    for (int j = start + tid; j < end; j += kDenseThreads) {
-      const int c = (int)cols[j] - c0;
-      if ((unsigned)c < (unsigned)len) srow[c] = values[j];
+    for (int i = lane * 8; i < len; i += kWave * 8) *reinterpret_cast<uint4*>(srow + i) = uint4{0u, 0u, 0u, 0u};
+    // the nonzeros of this segment: 64 at a time from the cursor, four chunks in flight
+    for (bool more = pos < end; more;) {
+      int c[4];
+      uint16_t v[4];
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        const int j = min(pos + u * kWave + lane, end - 1);
+        c[u] = (int)cols[j] - c0;
+        v[u] = values[j];
+      }
+      int taken = 0;
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        const bool mine = pos + u * kWave + lane < end && c[u] < len;  // (c >= 0: earlier segments took what lies before c0)
+        if (mine) srow[c[u]] = v[u];
+        taken += __popcll(__ballot(mine));
+      }
+      pos += taken;
+      more = taken == 4 * kWave;  // a short take: the row ended or the next nonzero lies beyond this segment
     }
-    __syncthreads();
-    for (int i = tid * 8; i < len; i += kDenseThreads * 8)
+    for (int i = lane * 8; i < len; i += kWave * 8)
       *reinterpret_cast<uint4*>(orow + c0 + i) = *reinterpret_cast<const uint4*>(srow + i);
-    __syncthreads();  // the next segment clears the row again
   }
 }
 

@@ -32,6 +32,7 @@ struct SddmmParams {
   const void* rhs;
   void* out;
   int sum_over_batch, accumulate;
+  int deep = 0;  // generic-k path: keep four slices of both rows in flight (set by the launcher)
 };
 
 typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
@@ -151,7 +152,25 @@ __global__ __launch_bounds__(256) void sddmm_kernel(SddmmParams p) {
           for (int zz = 0; zz < zn; ++zz) {
             const T* l = lhs + (size_t)zz * lhs_zstride;
             const T* r = rhs + (size_t)zz * rhs_zstride + (size_t)col * p.k;
-            for (int kk = sl * VEC; kk < p.k; kk += KT)
+            int kk = sl * VEC;
+            if (p.deep) {
+              // few wavefronts on the chip: a long k is a chain of load -> multiply -> load with one
+              // memory latency per slice unless several slices are in flight.  (With the chip full,
+              // other wavefronts hide that latency and the extra rows in flight only cost cache hits:
+              // 4096 x 4096 at 90 %, k = 2048, fp32: 1.16 ms plain, 1.67 ms this way; 1024 x 1024 at
+              // 95 %, k = 4096: 0.36 ms plain, 0.13 ms this way.)
+              for (; kk + 3 * KT < p.k; kk += 4 * KT) {
+                vec_t<T, VEC> lv[4], rv[4];
+#pragma unroll
+                for (int u = 0; u < 4; ++u) {
+                  lv[u] = load_vec<T, VEC>(l + kk + u * KT);
+                  rv[u] = load_vec<T, VEC>(r + kk + u * KT);
+                }
+#pragma unroll
+                for (int u = 0; u < 4; ++u) acc = dot_vec<T, VEC>(lv[u], rv[u], acc);
+              }
+            }
+            for (; kk < p.k; kk += KT)
               acc = dot_vec<T, VEC>(load_vec<T, VEC>(l + kk), load_vec<T, VEC>(r + kk), acc);
           }
           acc = group_sum<LPN>(acc);
@@ -168,8 +187,10 @@ __global__ __launch_bounds__(256) void sddmm_kernel(SddmmParams p) {
 }
 
 template <typename T, int VEC, int LPN, int PASSES, int WPR, bool EXACT>
-int launch_one(const SddmmParams& p, hipStream_t stream) {
+int launch_one(const SddmmParams& p0, hipStream_t stream) {
+  SddmmParams p = p0;
   dim3 grid(ceil_div(p.m, 4 / WPR), 1, p.sum_over_batch ? 1 : ceil_div(p.batch, kSddmmZb));
+  p.deep = (long long)grid.x * grid.z * 4 <= 2048;  // at most two wavefronts per SIMD of the chip
   hipLaunchKernelGGL((sddmm_kernel<T, VEC, LPN, PASSES, WPR, EXACT>), grid, dim3(256), 0, stream, p);
   return check_hip(hipGetLastError(), "sddmm launch");
 }
@@ -236,8 +257,8 @@ inline size_t sddmm_dense_bytes(const SddmmParams& p) { return (size_t)p.m * p.n
 // m * n * 2 bytes written and nnz entries picked at 4 TB/s.  Gather kernel: nnz * k * 2 bytes at
 // 15 TB/s (16 heads of 4096 x 4096 at 93 % sparsity, k = 64: 125 us; 2048 x 1024 at 80 %, k = 2048:
 // 117 us), and with a k beyond the register-resident fragments no less than one wave's chain of
-// dependent loads (0.34 us per 128 elements of k and step of 4 nonzeros: 1024 x 1024 at 95 %,
-// k = 4096: 141 us).  Measured: 11008 x 4096 at 80 %, k = 8192 (weight gradient of an MLP
+// loads (0.12 us per 128 elements of k and step of 4 nonzeros with four slices in flight:
+// 1024 x 1024 at 95 %, k = 4096: 50 us).  Measured: 11008 x 4096 at 80 %, k = 8192 (weight gradient of an MLP
 // projection) 16.5 -> 0.77 ms; 4096 x 4096 at 50 %, k = 8192 9.7 -> 0.32 ms; 4096 x 4096 at 90 %,
 // k = 512 120 -> 55 us.  The dense product has to win by 15 %.
 inline bool sddmm_dense_wins(const SddmmParams& p) {
@@ -246,7 +267,7 @@ inline bool sddmm_dense_wins(const SddmmParams& p) {
   const double product = std::max(flops / 1000e12, std::ceil(tiles / 512.0) * (p.k / 32.0) * 0.35e-6);
   const double dense = p.batch * (16e-6 + product + ((double)p.m * p.n * 2 + (double)p.nnz * 8) / 4e12);
   const double row_nnz = (double)p.nnz / p.m;
-  const double chain = p.k > 256 ? std::ceil(row_nnz / (row_nnz >= 64.0 ? 16.0 : 4.0)) * (p.k / 128.0) * 0.34e-6 : 0.0;
+  const double chain = p.k > 256 ? std::ceil(row_nnz / (row_nnz >= 64.0 ? 16.0 : 4.0)) * (p.k / 128.0) * 0.12e-6 : 0.0;
   const double gather = std::max(8e-6 + (double)p.batch * p.nnz * p.k * 2 / 15e12, chain);
   return 1.15 * dense < gather;
 }

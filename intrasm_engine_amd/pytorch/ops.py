@@ -39,13 +39,14 @@ _SPMM_KEYS = ("force_wpr", "force_variant", "force_rpw", "force_nt", "force_lpg"
 def kernel_params(*, spmm: dict | None = None, sddmm: dict | None = None, gemm: dict | None = None):
     """Kernel choices for the operators called inside the block (this thread only), for tuning:
     ``spmm`` = any of force_variant / force_rpw / force_nt / force_lpg / force_wpr (the tuning
-    bits of ``iex_spmm_ex``), ``sddmm`` = force_wpr, ``gemm`` = tile (the shape code of
-    ``iex_gemm``: 5 = 128x128, 6 = 128x256, 7 = 256x256 tiles; 1..4 = the register-staged kernels).
+    bits of ``iex_spmm_ex``), ``sddmm`` = force_wpr / force_variant, ``gemm`` = tile (the shape code of
+    ``iex_gemm``: 5 = 128x128, 6 = 128x256, 7 = 256x256 tiles, 8 = 128x128 with eight stages; 1..4 = the
+    register-staged kernels).
     Without a block, or for a key left out, the library chooses.  A kernel family that cannot
     take the operands at hand (a matrix-core family for an n that is not a multiple of 8, say)
     falls back to a gather kernel, as the C entry points document: results stay correct, the
     timing is then that of the fallback."""
-    for name, given, known in (("spmm", spmm, _SPMM_KEYS), ("sddmm", sddmm, ("force_wpr",)), ("gemm", gemm, ("tile",))):
+    for name, given, known in (("spmm", spmm, _SPMM_KEYS), ("sddmm", sddmm, ("force_wpr", "force_variant")), ("gemm", gemm, ("tile",))):
         unknown = set(given or {}) - set(known)
         if unknown:
             raise TypeError(f"unknown {name} kernel parameters: {sorted(unknown)}")

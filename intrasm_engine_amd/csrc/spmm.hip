@@ -500,7 +500,7 @@ int spmm_dispatch(int dtype, int itype, int flags, int m, int k, int n, int nonz
               "spmm: int16 column indices need k <= 32768 (k=%d)", k);
   Choice ch;
   ch.wpr = (flags >> 8) & 0xff;
-  if (ch.wpr == 0) ch.wpr = spmm_pick_wpr(m, nonzeros);
+  if (ch.wpr == 0) ch.wpr = spmm_pick_wpr(m, nonzeros, dtype == IEX_F32 ? 4 : 2, n, batch);
   ch.variant = (flags >> 16) & 0xf;
   ch.rpw = (flags >> 20) & 0xf;
   ch.nt = (flags >> 24) & 0xf;

@@ -280,10 +280,24 @@ inline SpmmShape spmm_pick_shape(int n, const void* dense, const void* out) {
 // Waves per row from the mean row length.  Splitting a row over the 4 wavefronts of a
 // workgroup shortens the dependent chain "fetch 64 nonzeros -> gather" of the heaviest row,
 // which is what the kernel time of a skewed matrix follows; measured on MI355X it wins from
-// a mean of a few dozen nonzeros per row upwards (8 or 16 waves per row were slower).
-inline int spmm_pick_wpr(int m, int nnz) {
+// a mean of a few dozen nonzeros per row upwards (8 or 16 waves per row were slower) -- as long
+// as whole rows would leave the chip short of wavefronts.  With more than one full round of
+// wavefronts (256 CUs x 32) from whole rows alone, splitting only adds the partial sums' trip
+// through LDS: 16 heads of 4096 x 4096 at 93 % sparsity, n = 64, fp16: 163 us split, 93 us whole.
+// elem_size, n and batch size the launch: lanes per row = n / (elements per 128-bit vector),
+// at least 8; 64 / that many rows share a wavefront.
+inline int spmm_pick_wpr(int m, int nnz, int elem_size = 4, int n = 0, int batch = 1) {
   const double mean = m > 0 ? (double)nnz / m : 0.0;
-  return mean >= 24.0 ? 4 : 1;
+  if (mean < 24.0) return 1;
+  if (n > 0) {
+    const int vec = 16 / elem_size;
+    int lanes = 8;
+    while (lanes < kWave && lanes * vec < n) lanes <<= 1;
+    const long long tiles_n = (n + kWave * vec - 1) / (kWave * vec);
+    const long long waves = ((long long)m * lanes + kWave - 1) / kWave * tiles_n * batch;
+    if (waves >= 256 * 32) return 1;
+  }
+  return 4;
 }
 
 // Defined with the dispatcher (spmm.hip): register windows of the 8-wave matrix-core kernel if

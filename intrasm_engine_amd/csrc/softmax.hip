@@ -1,8 +1,8 @@
 // In-place row-wise softmax over the stored entries of a CSR matrix (wave64):
 // values[z, j] <- exp(scale*values[z, j] - max_row) / sum_row for j in row.
-// One wavefront per (row, batch entry); three strided passes over the row, the two
-// reductions done with DPP + readlane.  Rows are short (hundreds of entries) in sparse
-// attention, so the second and third pass hit L1/L2.
+// One wavefront per (row, batch entry), the two reductions done with DPP + readlane.  Rows of
+// up to 512 entries (sparse attention has hundreds) are held in registers between one read and
+// one write; longer rows take three strided passes, the second and third of which hit L1/L2.
 #include "iex_common.h"
 
 namespace iex {
@@ -20,6 +20,35 @@ __global__ __launch_bounds__(256) void csr_softmax_kernel(int m, int nnz, const 
   const int end = uniform(row_offsets[row + 1]);
   if (end <= start) return;
   T* v = values + (size_t)blockIdx.z * nnz;
+  // rows of up to 512 entries (sparse attention) stay in registers: one read, one write, one exp
+  // per entry, the same arithmetic in the same order as the three passes below
+  constexpr int R = 8;
+  if (end - start <= R * kWave) {
+    float x[R];
+    float mx = -INFINITY;
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+      const int j = start + r * kWave + lane;
+      x[r] = j < end ? scale * elem<T>::to_float(v[j]) : -INFINITY;
+      mx = fmaxf(mx, x[r]);
+    }
+    mx = wave_max(mx);
+    float sum = 0.f;
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+      const int j = start + r * kWave + lane;
+      x[r] = j < end ? __expf(x[r] - mx) : 0.f;
+      sum += x[r];
+    }
+    sum = wave_sum(sum);
+    const float inv = 1.f / sum;
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+      const int j = start + r * kWave + lane;
+      if (j < end) v[j] = elem<T>::from_float(x[r] * inv);
+    }
+    return;
+  }
   float mx = -INFINITY;
   for (int j = start + lane; j < end; j += kWave) mx = fmaxf(mx, scale * elem<T>::to_float(v[j]));
   mx = wave_max(mx);

@@ -145,6 +145,23 @@ def test_csr_softmax(oracle, dev, dtype):
     assert np.allclose(sums, 1.0, atol=1e-2 if dtype == torch.float16 else 1e-5)
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_csr_softmax_long_short_and_empty_rows(oracle, dev, dtype):
+    """Rows of 0, 1, 64, 65, 512 (the longest that stays in registers), 513 and 2000 entries."""
+    lens = np.array([0, 1, 64, 65, 512, 513, 2000, 0, 7, 300])
+    ro = np.concatenate([[0], np.cumsum(lens)]).astype(np.int32)
+    rng = np.random.default_rng(11)
+    vals = rng.standard_normal((3, int(ro[-1]))).astype(np.float32) * 4
+    ri = torch.from_numpy(W.swizzle_from_offsets(ro)).to(dev)
+    v = torch.from_numpy(vals).to(dev).to(dtype)
+    ops.csr_softmax_(v, ri, torch.from_numpy(ro).to(dev), 0.5)
+    want = oracle.csr_softmax(rounded(vals, dtype).astype(np.float64) * 0.5, ro)
+    got = v.float().cpu().numpy()
+    assert np.abs(got - want).max() <= (2e-6 if dtype == torch.float32 else 8e-3)
+    for r in np.nonzero(lens)[0]:
+        assert np.allclose(got[:, ro[r]:ro[r + 1]].sum(axis=1), 1.0, atol=1e-5 if dtype == torch.float32 else 2e-2), r
+
+
 def test_operator_argument_checks(dev):
     a, _, lhs_np, rhs_np = W.config1()
     ri, _, ro, ci = to_dev(a, dev)

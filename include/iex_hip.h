@@ -98,8 +98,9 @@ int iex_spmm_ex(int dtype, int itype, int flags, int m, int k, int n, int nonzer
  * hand it to the dense GEMM (iex_gemm): the matrix-core SpMM kernels rebuild the dense form of
  * their rows of A in LDS once per column tile of the output, the GEMM reads it ready-made (family
  * 7; the caveat of families 3-6 about explicit zeros holds, and column indices inside a row must
- * be distinct).  Needs values shared by the batch, plain store, no bias / ReLU, k and n multiples
- * of 8; anything else, and a NULL or short workspace, runs exactly as iex_spmm_ex.
+ * be distinct).  Needs values shared by the batch and k and n multiples of 8 (bias, ReLU and
+ * accumulation ride in the GEMM's epilogue); anything else, and a NULL or short workspace, runs
+ * exactly as iex_spmm_ex.
  * IEX_SPMM_FORCE_VARIANT(7) asks for that path and fails where it cannot run.
  * iex_spmm_workspace_bytes returns the size with which the call described would use the workspace,
  * 0 when it would not whatever the size (has_bias: bias != NULL).  Neither call allocates.

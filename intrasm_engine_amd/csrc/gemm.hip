@@ -127,7 +127,12 @@ int launch_shape(const GemmParams& p, int batch, int force, hipStream_t stream) 
 // straight into LDS: 5 = 128x128, 6 = 128x256, 7 = 256x256, 8 = 128x128 with eight stages.  0 = choose (one of 5..8).
 extern "C" int iex_gemm(int dtype, int trans_b_and_shape, int M, int N, int K, const void* A, const void* B, void* C, int batch,
                         long long stride_a, long long stride_b, long long stride_c, void* stream) {
-  using namespace iex;
+  return iex::gemm_dispatch(dtype, trans_b_and_shape, M, N, K, A, B, C, batch, stride_a, stride_b, stride_c, stream, nullptr, 0, 0);
+}
+
+int iex::gemm_dispatch(int dtype, int trans_b_and_shape, int M, int N, int K, const void* A, const void* B, void* C, int batch,
+                       long long stride_a, long long stride_b, long long stride_c, void* stream, const float* row_bias, int relu,
+                       int accumulate) {
   const int trans_b = trans_b_and_shape & 1, force = (trans_b_and_shape >> 4) & 0xf;
   IEX_REQUIRE(M >= 0 && N >= 0 && K >= 0 && batch >= 0, IEX_ERR_BAD_ARGUMENT, "gemm: negative dimension");
   if (M == 0 || N == 0 || batch == 0) return 0;
@@ -140,7 +145,7 @@ extern "C" int iex_gemm(int dtype, int trans_b_and_shape, int M, int N, int K, c
   IEX_REQUIRE(batch <= 65535, IEX_ERR_TOO_LARGE, "gemm: batch %d exceeds 65535", batch);
   IEX_REQUIRE((long long)M * K < (1ll << 31) && (long long)N * K < (1ll << 31) && (long long)M * N < (1ll << 31),
               IEX_ERR_TOO_LARGE, "gemm: an operand exceeds 2^31 elements per batch entry");
-  GemmParams p{M, N, K, A, B, C, stride_a, stride_b, stride_c, 0, 0};
+  GemmParams p{M, N, K, A, B, C, stride_a, stride_b, stride_c, 0, 0, row_bias, relu, accumulate};
   hipStream_t s = static_cast<hipStream_t>(stream);
   const bool bf = dtype == IEX_BF16;
   if (bf && trans_b) return launch_shape<true, true>(p, batch, force, s);

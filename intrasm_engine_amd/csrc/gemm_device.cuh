@@ -31,7 +31,16 @@ struct GemmParams {
   void* C;
   long long stride_a, stride_b, stride_c;
   int tiles_m, tiles_n;
+  // epilogue beyond C = A * B, for the SpMM path that hands its product to this kernel:
+  // C = relu?((accumulate ? C : 0) + A * B + row_bias[row])
+  const float* row_bias = nullptr;
+  int relu = 0, accumulate = 0;
 };
+
+// iex_gemm with the epilogue options above (gemm.hip).
+int gemm_dispatch(int dtype, int trans_b_and_shape, int M, int N, int K, const void* A, const void* B, void* C, int batch,
+                  long long stride_a, long long stride_b, long long stride_c, void* stream, const float* row_bias, int relu,
+                  int accumulate);
 
 typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
@@ -64,6 +73,11 @@ __device__ __forceinline__ f32x16 mfma_32x32x16(u32x4 a, u32x4 b, f32x16 c) {
     return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, a), __builtin_bit_cast(f16x8, b), c, 0, 0,
                                                   0);
   }
+}
+
+__device__ __forceinline__ float f16_to_32(unsigned short h, bool bf16) {
+  if (bf16) return __uint_as_float((unsigned)h << 16);
+  return (float)__builtin_bit_cast(_Float16, h);
 }
 
 __device__ __forceinline__ unsigned short f32_to_16(float v, bool bf16) {
@@ -167,16 +181,37 @@ __device__ __forceinline__ void gemm_store_tile(const GemmParams& p, const f32x1
   for (int i = 0; i < WM; ++i) {
     const int gm = m0 + (wm * WM + i) * 32 + (lane & 31);
     if (gm >= p.M) continue;
+    const float bias = p.row_bias ? p.row_bias[gm] : 0.f;
 #pragma unroll
     for (int j = 0; j < WN; ++j) {
 #pragma unroll
       for (int q = 0; q < 4; ++q) {
         const int gn = n0 + (wn * WN + j) * 32 + q * 8 + (lane >> 5) * 4;
         if (gn >= p.N) continue;
+        u16* dst = C + (size_t)gm * p.N + gn;
+        float x[4];
+#pragma unroll
+        for (int e = 0; e < 4; ++e) x[e] = acc[i][j][q * 4 + e];
+        if (p.accumulate) {
+          if (vec_ok) {
+            const u32x2 w = *reinterpret_cast<const u32x2*>(dst);
+            x[0] += f16_to_32((u16)(w.x & 0xffffu), BF16);
+            x[1] += f16_to_32((u16)(w.x >> 16), BF16);
+            x[2] += f16_to_32((u16)(w.y & 0xffffu), BF16);
+            x[3] += f16_to_32((u16)(w.y >> 16), BF16);
+          } else {
+#pragma unroll
+            for (int e = 0; e < 4; ++e)
+              if (gn + e < p.N) x[e] += f16_to_32(dst[e], BF16);
+          }
+        }
         u16 h[4];
 #pragma unroll
-        for (int e = 0; e < 4; ++e) h[e] = f32_to_16(acc[i][j][q * 4 + e], BF16);
-        u16* dst = C + (size_t)gm * p.N + gn;
+        for (int e = 0; e < 4; ++e) {
+          float y = x[e] + bias;
+          if (p.relu) y = fmaxf(y, 0.f);
+          h[e] = f32_to_16(y, BF16);
+        }
         if (vec_ok) {
           u32x2 w;
           w.x = (unsigned)h[0] | ((unsigned)h[1] << 16);

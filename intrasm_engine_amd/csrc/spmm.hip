@@ -381,7 +381,7 @@ inline int mfma3_windows(const SpmmParams& p) {
 // Dense form of A in the caller's workspace, then the dense GEMM (16-bit types, values shared by
 // the batch, plain store, no bias / ReLU).  What the shapes must satisfy, the workspace aside.
 inline bool dense_path_fits(int elem_size, const SpmmParams& p, bool flagged) {
-  return elem_size == 2 && !flagged && !p.bias && p.nnz > 0 && p.k % 8 == 0 && p.n % 8 == 0 &&
+  return elem_size == 2 && !flagged && p.nnz > 0 && p.k % 8 == 0 && p.n % 8 == 0 &&
          (long long)p.m * p.k < (1ll << 31) && aligned(p.dense, 16) && aligned(p.out, 16);
 }
 
@@ -412,7 +412,8 @@ int launch_dense_path(const SpmmParams& p, int batch, const Choice& ch, hipStrea
                      static_cast<uint16_t*>(ch.ws));
   if (int rc = check_hip(hipGetLastError(), "spmm dense-form launch")) return rc;
   const int dtype = std::is_same<T, __half>::value ? IEX_F16 : IEX_BF16;
-  return iex_gemm(dtype, 0, p.m, p.n, p.k, ch.ws, p.dense, p.out, batch, 0, (long long)p.k * p.n, (long long)p.m * p.n, stream);
+  return gemm_dispatch(dtype, 0, p.m, p.n, p.k, ch.ws, p.dense, p.out, batch, 0, (long long)p.k * p.n, (long long)p.m * p.n, stream,
+                       p.bias, p.relu, p.accumulate);
 }
 
 template <typename T, typename IT>
@@ -426,10 +427,10 @@ int launch_typed(const SpmmParams& p, int batch, const Choice& ch, hipStream_t s
     return launch_mfma3<T, IT>(p, batch, ch.rpw ? ch.rpw : mfma3_windows(p), stream);
   const MfmaChoice mc = mfma_variant<T>(p, batch, ch);
   if constexpr (sizeof(T) == 2) {
-    const bool fits = dense_path_fits(2, p, p.per_batch_values || p.accumulate || p.relu);
+    const bool fits = dense_path_fits(2, p, p.per_batch_values);
     const bool room = ch.ws && aligned(ch.ws, 16) && ch.ws_bytes >= dense_path_bytes(p);
     if (ch.variant == 7) {
-      IEX_REQUIRE(fits, IEX_ERR_UNSUPPORTED, "spmm: the dense-form path needs 16-bit values shared by the batch, plain store, no bias, k and n multiples of 8 and 16-byte aligned operands");
+      IEX_REQUIRE(fits, IEX_ERR_UNSUPPORTED, "spmm: the dense-form path needs 16-bit values shared by the batch, k and n multiples of 8 and 16-byte aligned operands");
       IEX_REQUIRE(room, IEX_ERR_BAD_ARGUMENT, "spmm: the dense-form path needs a 16-byte aligned workspace of %zu bytes (iex_spmm_ws)", dense_path_bytes(p));
       return launch_dense_path<T, IT>(p, batch, ch, stream);
     }
@@ -521,13 +522,14 @@ int spmm_dispatch(int dtype, int itype, int flags, int m, int k, int n, int nonz
 // Bytes of workspace with which iex_spmm_ws would take the dense-form path for this call (0: it
 // would not, whatever the workspace).  Pointers are taken to be 16-byte aligned.
 size_t spmm_workspace_bytes(int dtype, int itype, int flags, int m, int k, int n, int nonzeros, int batch, int has_bias) {
-  if (m <= 0 || k <= 0 || n <= 0 || nonzeros <= 0 || batch <= 0 || has_bias) return 0;
+  (void)has_bias;  // the GEMM's epilogue adds it
+  if (m <= 0 || k <= 0 || n <= 0 || nonzeros <= 0 || batch <= 0) return 0;
   if (!(dtype == IEX_F16 || dtype == IEX_BF16) || !(itype == IEX_I32 || itype == IEX_I16)) return 0;
   const int variant = (flags >> 16) & 0xf;
   if (variant != 0 && variant != 7) return 0;
   void* const some_aligned = reinterpret_cast<void*>(size_t(256));
   SpmmParams p{m, k, n, nonzeros, nullptr, nullptr, nullptr, nullptr, some_aligned, nullptr, some_aligned, 0, 0, 0};
-  if (!dense_path_fits(2, p, (flags & (IEX_SPMM_PER_BATCH_VALUES | IEX_SPMM_ACCUMULATE | IEX_SPMM_RELU)) != 0)) return 0;
+  if (!dense_path_fits(2, p, (flags & IEX_SPMM_PER_BATCH_VALUES) != 0)) return 0;
   if (variant == 0) {
     Choice ch;
     ch.rpw = (flags >> 20) & 0xf;

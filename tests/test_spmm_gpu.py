@@ -579,12 +579,40 @@ def test_dense_form_path(oracle, dev, dtype, itype, m, k, n, batch):
     assert_close(out.float().cpu().numpy(), want, scale, RTOL[dtype], f"dense form {dtype} {m}x{k}x{n}")
 
 
+def test_dense_form_path_epilogue_options(oracle, dev):
+    """bias + ReLU and accumulation into the output ride in the GEMM's epilogue; per-batch values have
+    no single dense form and are refused on request."""
+    from intrasm_engine_amd.pytorch import ops as pyops
+    rng = np.random.default_rng(77)
+    m, k, n, batch = 200, 304, 136, 3
+    csr = W.pruned_weight(47, m, k, 0.8)
+    ri, v, ro_t, ci_t = to_dev(csr, dev, torch.bfloat16)
+    b_np = rng.standard_normal((batch, k, n)).astype(np.float32)
+    b = torch.from_numpy(b_np).to(dev).bfloat16()
+    b_r, vals_r = rounded(b_np, torch.bfloat16), rounded(csr.values, torch.bfloat16)
+    base = oracle.spmm(b_r, csr.row_indices, vals_r, csr.row_offsets, csr.column_indices, m)
+    scale = oracle.spmm_abs_scale(b_r, csr.row_indices, vals_r, csr.row_offsets, csr.column_indices, m)
+    kw = dict(dtypes=(torch.bfloat16,), allow_i16=False, force_variant=7)
+    bias_np = rng.standard_normal(m).astype(np.float32)
+    out = pyops._spmm(b, ri, v, ro_t, ci_t, m, per_batch_values=False, accumulate=False,
+                      bias=torch.from_numpy(bias_np).to(dev), relu=True, **kw)
+    assert_close(out.float().cpu().numpy(), np.maximum(base + bias_np[None, :, None], 0.0), scale + np.abs(bias_np)[None, :, None],
+                 RTOL[torch.bfloat16], "bias+relu")
+    prev_np = rounded(rng.standard_normal((batch, m, n)).astype(np.float32), torch.bfloat16)
+    prev = torch.from_numpy(prev_np).to(dev).bfloat16()
+    out = pyops._spmm(b, ri, v, ro_t, ci_t, m, per_batch_values=False, accumulate=True, out=prev, **kw)
+    assert out.data_ptr() == prev.data_ptr()
+    assert_close(out.float().cpu().numpy(), base + prev_np, scale + np.abs(prev_np), RTOL[torch.bfloat16], "accumulate")
+    vb = torch.randn(batch, csr.nnz, device=dev).bfloat16()
+    with pytest.raises(RuntimeError, match="dense-form path needs"):
+        pyops._spmm(b, ri, vb, ro_t, ci_t, m, per_batch_values=True, accumulate=False, **kw)
+
+
 def test_dense_form_path_is_chosen_with_a_workspace_and_only_then(oracle, dev):
     """2048 x 2048 at 80 % sparsity times 2048 x 1024 in fp16: the time model prefers the dense form
     (measured 34 against 71 us).  The operator asks the library for the workspace size, allocates it
     and gets the dense-form result; the entry point without a workspace, a short workspace, and
-    shapes the path does not serve (fp32, per-batch values, a bias, a small product) run the other
-    kernels."""
+    shapes the path does not serve (fp32, per-batch values, a small product) run the other kernels."""
     from intrasm_engine_amd import _lib
     from intrasm_engine_amd.pytorch import ops as pyops
     lib = _lib.load()
@@ -598,8 +626,7 @@ def test_dense_form_path_is_chosen_with_a_workspace_and_only_then(oracle, dev):
     assert need == m * k * 2
     assert lib.iex_spmm_workspace_bytes(_lib.F32, _lib.I32, 0, m, k, n, nnz, 1, 0) == 0
     assert lib.iex_spmm_workspace_bytes(_lib.F16, _lib.I16, _lib.SPMM_PER_BATCH_VALUES, m, k, n, nnz, 1, 0) == 0
-    assert lib.iex_spmm_workspace_bytes(_lib.F16, _lib.I16, _lib.SPMM_ACCUMULATE, m, k, n, nnz, 1, 0) == 0
-    assert lib.iex_spmm_workspace_bytes(_lib.F16, _lib.I16, 0, m, k, n, nnz, 1, 1) == 0      # bias
+    assert lib.iex_spmm_workspace_bytes(_lib.F16, _lib.I16, _lib.SPMM_ACCUMULATE | _lib.SPMM_RELU, m, k, n, nnz, 1, 1) == need
     assert lib.iex_spmm_workspace_bytes(_lib.F16, _lib.I16, 0, 128, 128, 64, 1000, 1, 0) == 0  # too small to pay
     assert lib.iex_spmm_workspace_bytes(_lib.F16, _lib.I16, 0, m, k, n - 4, nnz, 1, 0) == 0    # n no multiple of 8
     assert lib.iex_spmm_workspace_bytes(_lib.F16, _lib.I16, 7 << 16, 128, 128, 64, 1000, 1, 0) == 128 * 128 * 2  # on request

@@ -103,14 +103,14 @@ int iex_spmm_ex(int dtype, int itype, int flags, int m, int k, int n, int nonzer
  * exactly as iex_spmm_ex.
  * IEX_SPMM_FORCE_VARIANT(7) asks for that path and fails where it cannot run.
  * iex_spmm_workspace_bytes returns the size with which the call described would use the workspace,
- * 0 when it would not whatever the size (has_bias: bias != NULL).  Neither call allocates.
+ * 0 when it would not whatever the size.  Neither call allocates.
  * No counterpart in the reference: its launchers (csrc/extensions.h:28-30) take no workspace. */
 int iex_spmm_ws(int dtype, int itype, int flags, int m, int k, int n, int nonzeros,
                 const int* row_indices, const void* values, const int* row_offsets,
                 const void* column_indices, const void* dense, const float* bias,
                 void* out, void* stream, int batch, void* workspace, size_t workspace_bytes);
 size_t iex_spmm_workspace_bytes(int dtype, int itype, int flags, int m, int k, int n,
-                                int nonzeros, int batch, int has_bias);
+                                int nonzeros, int batch);
 
 /* Drop-ins for the three launchers the reference declares in csrc/extensions.h:28-30.
  * CudaSpmm2: fp32, per-batch values (batch, nnz), accumulates into `out`

@@ -521,8 +521,7 @@ int spmm_dispatch(int dtype, int itype, int flags, int m, int k, int n, int nonz
 
 // Bytes of workspace with which iex_spmm_ws would take the dense-form path for this call (0: it
 // would not, whatever the workspace).  Pointers are taken to be 16-byte aligned.
-size_t spmm_workspace_bytes(int dtype, int itype, int flags, int m, int k, int n, int nonzeros, int batch, int has_bias) {
-  (void)has_bias;  // the GEMM's epilogue adds it
+size_t spmm_workspace_bytes(int dtype, int itype, int flags, int m, int k, int n, int nonzeros, int batch) {
   if (m <= 0 || k <= 0 || n <= 0 || nonzeros <= 0 || batch <= 0) return 0;
   if (!(dtype == IEX_F16 || dtype == IEX_BF16) || !(itype == IEX_I32 || itype == IEX_I16)) return 0;
   const int variant = (flags >> 16) & 0xf;
@@ -559,8 +558,8 @@ int iex_spmm_ws(int dtype, int itype, int flags, int m, int k, int n, int nonzer
                             column_indices, dense, bias, out, stream, batch, workspace, workspace_bytes);
 }
 
-size_t iex_spmm_workspace_bytes(int dtype, int itype, int flags, int m, int k, int n, int nonzeros, int batch, int has_bias) {
-  return iex::spmm_workspace_bytes(dtype, itype, flags, m, k, n, nonzeros, batch, has_bias);
+size_t iex_spmm_workspace_bytes(int dtype, int itype, int flags, int m, int k, int n, int nonzeros, int batch) {
+  return iex::spmm_workspace_bytes(dtype, itype, flags, m, k, n, nonzeros, batch);
 }
 
 int iex_CudaSpmm2(int m, int k, int n, int nonzeros, const int* row_indices, const float* values,

@@ -141,7 +141,7 @@ def _spmm(b, row_indices, values, row_offsets, column_indices, m, *, per_batch_v
         # product to its dense GEMM (large 16-bit products): from torch's allocator, on the current
         # stream, released (stream-ordered) when this call returns
         ws_bytes = 0 if no_workspace else lib.iex_spmm_workspace_bytes(
-            _DT[b.dtype], _IT[column_indices.dtype], flags, m, k, n, nonzeros, batch, int(bias is not None))
+            _DT[b.dtype], _IT[column_indices.dtype], flags, m, k, n, nonzeros, batch)
         ws = torch.empty(ws_bytes, dtype=torch.uint8, device=b.device) if ws_bytes else None
         rc = lib.iex_spmm_ws(
             _DT[b.dtype], _IT[column_indices.dtype], flags, m, k, n, nonzeros,

@@ -80,7 +80,7 @@ def test_replay_spmm_that_uses_a_workspace(dev):
     ro_t, ci_t = torch.from_numpy(ro).to(dev), torch.from_numpy(ci.astype(np.int16)).to(dev)
     v = torch.randn(ci.shape[0], device=dev).half()
     b = torch.randn(1, k, n, device=dev).half()
-    assert _lib.load().iex_spmm_workspace_bytes(_lib.F16, _lib.I16, 0, m, k, n, ci.shape[0], 1, 0) == m * k * 2
+    assert _lib.load().iex_spmm_workspace_bytes(_lib.F16, _lib.I16, 0, m, k, n, ci.shape[0], 1) == m * k * 2
     constructor = TorchCUDAGraphConstructor()
     with constructor.get_primary_stream():
         with constructor:

@@ -622,14 +622,14 @@ def test_dense_form_path_is_chosen_with_a_workspace_and_only_then(oracle, dev):
     rng = np.random.default_rng(12)
     csr, b_np, (ri, v, ro_t, ci_t), b = _dense_form_case(rng, m, k, n, 1, dtype, torch.int16, dev, mean_len=0.2 * k)
     nnz = csr.column_indices.shape[0]
-    need = lib.iex_spmm_workspace_bytes(_lib.F16, _lib.I16, 0, m, k, n, nnz, 1, 0)
+    need = lib.iex_spmm_workspace_bytes(_lib.F16, _lib.I16, 0, m, k, n, nnz, 1)
     assert need == m * k * 2
-    assert lib.iex_spmm_workspace_bytes(_lib.F32, _lib.I32, 0, m, k, n, nnz, 1, 0) == 0
-    assert lib.iex_spmm_workspace_bytes(_lib.F16, _lib.I16, _lib.SPMM_PER_BATCH_VALUES, m, k, n, nnz, 1, 0) == 0
-    assert lib.iex_spmm_workspace_bytes(_lib.F16, _lib.I16, _lib.SPMM_ACCUMULATE | _lib.SPMM_RELU, m, k, n, nnz, 1, 1) == need
-    assert lib.iex_spmm_workspace_bytes(_lib.F16, _lib.I16, 0, 128, 128, 64, 1000, 1, 0) == 0  # too small to pay
-    assert lib.iex_spmm_workspace_bytes(_lib.F16, _lib.I16, 0, m, k, n - 4, nnz, 1, 0) == 0    # n no multiple of 8
-    assert lib.iex_spmm_workspace_bytes(_lib.F16, _lib.I16, 7 << 16, 128, 128, 64, 1000, 1, 0) == 128 * 128 * 2  # on request
+    assert lib.iex_spmm_workspace_bytes(_lib.F32, _lib.I32, 0, m, k, n, nnz, 1) == 0
+    assert lib.iex_spmm_workspace_bytes(_lib.F16, _lib.I16, _lib.SPMM_PER_BATCH_VALUES, m, k, n, nnz, 1) == 0
+    assert lib.iex_spmm_workspace_bytes(_lib.F16, _lib.I16, _lib.SPMM_ACCUMULATE | _lib.SPMM_RELU, m, k, n, nnz, 1) == need
+    assert lib.iex_spmm_workspace_bytes(_lib.F16, _lib.I16, 0, 128, 128, 64, 1000, 1) == 0  # too small to pay
+    assert lib.iex_spmm_workspace_bytes(_lib.F16, _lib.I16, 0, m, k, n - 4, nnz, 1) == 0    # n no multiple of 8
+    assert lib.iex_spmm_workspace_bytes(_lib.F16, _lib.I16, 7 << 16, 128, 128, 64, 1000, 1) == 128 * 128 * 2  # on request
     kw = dict(per_batch_values=False, accumulate=False, dtypes=(dtype,), allow_i16=True)
     auto = pyops._spmm(b, ri, v, ro_t, ci_t, m, **kw)
     assert torch.equal(auto, pyops._spmm(b, ri, v, ro_t, ci_t, m, force_variant=7, **kw))

@@ -332,7 +332,26 @@ def run_extras(torch, ops, dev, W, IL, mats, dens, csr_dev, time_cell, variant_o
         "gather_kernel_us": round(us_g, 1), "operator_us": round(us_d, 1),
         "operator_path": "dense product by the GEMM into a workspace, then sampling",
         "operator_dense_equivalent_TFLOPs": round(2.0 * w4g.m * w4g.k * 2048 / us_d / 1e6, 1)}
-    del gy, xx, riw_, row_, ciw_, w4g
+    # the same layer as an autograd function: forward SpMM, backward SpMM with the transposed weight (gradient of
+    # the activation) + that SDDMM (gradient of the values); one training step of a sparse linear layer, eager
+    from intrasm_engine_amd.pytorch.cpp_extensions.layers_and_funcs.sputnik import spmm as spmm_fn
+    from intrasm_engine_amd.pytorch import utils as U_
+    vals_ = torch.from_numpy(w4g.values).to(dev).half().requires_grad_(True)
+    info_ = U_.transpose_info(w4g.m, w4g.k, row_, ciw_)
+    x2 = xx[0].detach().clone().requires_grad_(True)          # (k, tokens)
+    g2 = gy[0].detach().clone()                               # (m, tokens)
+
+    def train_step():
+        vals_.grad = None
+        x2.grad = None
+        spmm_fn(x2, riw_, vals_, row_, ciw_, w4g.m, info_).backward(g2)
+
+    us_step = time_cell(train_step, repeats=3, samples=3)
+    out["sparse_linear_training_step_c4_fp16"] = {
+        "what": "MySpMM forward + backward on config 4's weight, 2048 tokens, fp16, int32 indices, eager",
+        "us": round(us_step, 1), "nonzero_GFLOP": round(3 * 2.0 * w4g.nnz * 2048 / 1e9, 2),
+        "dense_equivalent_TFLOPs": round(3 * 2.0 * w4g.m * w4g.k * 2048 / us_step / 1e6, 1)}
+    del gy, xx, riw_, row_, ciw_, w4g, vals_, info_, x2, g2
     log("[bench] SDDMM done")
 
     # ---- config 4: fp16 SpMM 11008x4096 @90% x 4096x2048  ||  bf16 GEMM 4096x4096x2048

@@ -260,6 +260,34 @@ def test_full_size_config4_integer_exact(dev):
     assert torch.equal(out[0].double(), want)
 
 
+@pytest.mark.parametrize("shape", ["config4", "q_2to4"])
+def test_full_size_dense_form_agrees_with_the_other_families(dev, shape):
+    """At the full sizes of config 4 (11008 x 4096 at 90 %, 2048 tokens) and of a 2:4 projection of the
+    decoder layer (4096 x 4096, 8192 tokens), random fp16 operands: the operator's result (dense form + GEMM)
+    equals the matrix-core SpMM kernel's bit for bit -- two independent ways to the same MFMA sequence
+    over k -- and the gather kernel's to the fp16 tolerance, on a strided sample of rows."""
+    from intrasm_engine_amd.pytorch import ops as pyops
+    rng = np.random.default_rng(21)
+    if shape == "config4":
+        w, n = W.pruned_weight(21, 11008, 4096, 0.90), 2048
+    else:
+        m = k = 4096
+        keep = np.argsort(rng.random((m, k // 4, 4)), axis=2)[:, :, :2] + 4 * np.arange(k // 4)[None, :, None]
+        ci = np.sort(keep.reshape(m, k // 2), axis=1).reshape(-1).astype(np.int32)
+        ro = (np.arange(m + 1) * (k // 2)).astype(np.int32)
+        w, n = W.CSR(m, k, rng.standard_normal(ci.shape[0]).astype(np.float32), W.swizzle_from_offsets(ro), ro, ci), 8192
+    ri, v, ro_t, ci_t = to_dev(w, dev, torch.float16, torch.int16)
+    x = torch.randn(1, w.k, n, device=dev, generator=torch.Generator(dev).manual_seed(5)).half()
+    kw = dict(per_batch_values=False, accumulate=False, dtypes=(torch.float16,), allow_i16=True)
+    auto = pyops._spmm(x, ri, v, ro_t, ci_t, w.m, **kw)
+    assert torch.equal(auto, pyops._spmm(x, ri, v, ro_t, ci_t, w.m, force_variant=7, **kw))     # the dense form is what ran
+    assert torch.equal(auto, pyops._spmm(x, ri, v, ro_t, ci_t, w.m, force_variant=4, **kw))
+    rows = slice(0, w.m, 37)
+    gather = pyops._spmm(x, ri, v, ro_t, ci_t, w.m, force_variant=1, **kw)[0, rows].float()
+    scale = float(gather.abs().max())
+    assert torch.allclose(auto[0, rows].float(), gather, rtol=1e-2, atol=1e-2 * scale)
+
+
 def test_operator_argument_checks(dev):
     a, b_np, _, _ = W.config1()
     ri, v, ro, ci = to_dev(a, dev)

@@ -63,7 +63,10 @@ int iex_copy_bytes(void* dst, const void* src, size_t nbytes, void* stream);
  * and 128 x 256 tiles / 8 waves and 128 x 512 tiles), 5 = matrix-core kernel for fp32
  * (v_mfma_f32_32x32x2, 32-row tiles), 6 = family 4's tile with the dense operand loaded from
  * global memory straight into LDS and A expanded 64 columns at a time (fp16 / bf16), 7 = dense
- * form of A in the caller's workspace, then the dense GEMM (iex_spmm_ws only).  0 = choose.
+ * form of A in the caller's workspace, then the dense GEMM (iex_spmm_ws only), 8 = A with at most
+ * 128 columns and an output at least one tile (64 128-bit vectors) wide: the dense operand's tile
+ * in LDS, rows streamed in natural order (bit-equal to family 1 with one wavefront per row; fails
+ * on other shapes).  0 = choose.
  * Families 2-6 rely on strictly ascending column indices inside a row (canonical CSR, what
  * dense_to_sparse produces); family 1 accepts any order and duplicates -- force it for such
  * input.  Families 3-6 multiply explicit zeros with the dense operand, so a non-finite entry

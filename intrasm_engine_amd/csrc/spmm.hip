@@ -7,6 +7,7 @@
 #include "spmm_mfma3_device.cuh"
 #include "spmm_mfma_f32_device.cuh"
 #include "spmm_dense_device.cuh"
+#include "spmm_smallk_device.cuh"
 
 namespace iex {
 namespace {
@@ -51,6 +52,55 @@ int launch_ragged(const SpmmParams& p, int batch, int wpr, hipStream_t stream) {
     case 8: return launch_ragged_one<T, IT, VEC, 8>(p, batch, stream);
   }
   return fail(IEX_ERR_BAD_ARGUMENT, "spmm: waves-per-row must be 1, 4 or 8 (got %d)", wpr);
+}
+
+// ---- few columns in A, wide output: the dense operand's tile lives in LDS ---------------------
+template <typename T, typename IT, int VEC>
+__global__ __launch_bounds__(kSmallKThreads) void spmm_smallk_kernel(SpmmParams p, int rows_per_wave) {
+  extern __shared__ __align__(16) unsigned char smem[];
+  spmm_smallk_block<T, IT, VEC>(p, rows_per_wave, blockIdx.x, blockIdx.y, blockIdx.z, smem);
+}
+
+template <typename T>
+bool smallk_fits(const SpmmParams& p) {
+  constexpr int kMax = 16 / (int)sizeof(T);
+  return p.k >= 1 && p.k <= kSmallKMax && p.n % kMax == 0 && p.n >= kWave * kMax && aligned(p.dense, 16) && aligned(p.out, 16);
+}
+
+// ... and where the library takes it by itself: enough rows for the tile load (k KB per workgroup) to be a
+// fraction of what the workgroup writes, and enough work to pay for it -- on small, almost empty products
+// the row kernel is a plain writer of zeros at 5 TB/s and stays ahead (32 x 1024 x 1024 outputs, k = 32,
+// 95-99.9 % sparse: 26-33 us against 34-36; 8 x 4096 x 4096, k = 128 at 99.9 %: 114 against 128).
+template <typename T>
+bool smallk_wanted(const SpmmParams& p, int batch) {
+  if (!smallk_fits<T>(p) || p.m < (p.k <= 64 ? 8 : 32) * p.k) return false;
+  const double mean_row = (double)p.nnz / p.m, out_bytes = (double)p.m * p.n * batch * sizeof(T);
+  return p.k <= 64 ? (out_bytes >= 256e6 || mean_row >= 3.0) : mean_row >= 0.4;
+}
+
+template <typename T, typename IT>
+int launch_smallk(const SpmmParams& p, int batch, hipStream_t stream) {
+  constexpr int kMax = 16 / (int)sizeof(T);
+  // rows per wavefront: enough for the tile load (k KB per workgroup) to be a fraction of the output
+  // (8 * rows KB), as long as that leaves every CU several workgroups
+  const long long tiles = (long long)ceil_div(p.n, kWave * kMax) * batch;
+  int rows = std::min(64, std::max(16, p.k / 2));
+  while (rows > 4 && (long long)ceil_div(p.m, kSmallKWaves * rows) * tiles < 1024) rows >>= 1;
+  const int lds = p.k * kWave * 16;
+  auto kern = spmm_smallk_kernel<T, IT, kMax>;
+  if (lds > 64 * 1024) {
+    static thread_local bool raised = false;  // per instantiation
+    if (!raised) {
+      if (int rc = check_hip(hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                                 kSmallKMax * kWave * 16),
+                             "hipFuncSetAttribute(LDS size)"))
+        return rc;
+      raised = true;
+    }
+  }
+  dim3 grid(ceil_div(p.m, kSmallKWaves * rows), ceil_div(p.n, kWave * kMax), batch);
+  hipLaunchKernelGGL(kern, grid, dim3(kSmallKThreads), lds, stream, p, rows);
+  return check_hip(hipGetLastError(), "spmm (few columns) launch");
 }
 
 template <typename T, typename IT, int VEC, int LPG>
@@ -395,13 +445,21 @@ inline size_t dense_path_bytes(const SpmmParams& p) { return (size_t)p.m * p.k *
 //     for the dense form; 80 % 11008 x 4096: 0.93 / 0.69; 90 %, n = 2048: 0.27 / 0.23);
 //   gather kernels: nnz * n * 2 bytes through the L2 -> CU path at 26 TB/s (4096^2 at 70 %, n = 256:
 //     110 against 58 us; at 90 %, n = 256: 40 against 58; 11008 x 4096 at 95 %, n = 2048: 0.35 / 0.21 ms).
-// The dense form has to win by 15 % to be taken.
-inline bool dense_path_wins(const SpmmParams& p, int batch, int matrix_core_kind) {
+//   a short K makes the GEMM a writer of its output at 2 TB/s (16 x 4096 x 4096, k = 64: 0.31 ms), the
+//     gather kernels write it at 4 TB/s, the few-columns kernel at 4.5 TB/s plus 10 clocks of a CU's LDS
+//     per nonzero and tile (same shape at 93 % sparsity: 0.15 ms; 8 x 4096 x 4096, k = 128 at 50 %: 0.58
+//     against 0.17 for the dense form).
+// The dense form has to win by 15 % to be taken.  `few_columns`: the alternative is the few-columns kernel.
+inline bool dense_path_wins(const SpmmParams& p, int batch, int matrix_core_kind, bool few_columns) {
   const double cells = (double)p.m * p.k, flops = 2.0 * cells * p.n * batch;
+  const double out_bytes = (double)p.m * p.n * batch * 2;
   const double tiles = (double)ceil_div(p.m, 128) * ceil_div(p.n, 128) * batch;
-  const double product = std::max(flops / 1000e12, std::ceil(tiles / 512.0) * (p.k / 32.0) * 0.35e-6);
+  const double product = std::max({flops / 1000e12, std::ceil(tiles / 512.0) * (p.k / 32.0) * 0.35e-6, out_bytes / 2e12});
   const double dense_form = 8e-6 + cells * 2 / 4e12 + product;
-  const double other = matrix_core_kind ? 8e-6 + flops / 720e12 : 8e-6 + (double)p.nnz * p.n * batch * 2 / 26e12;
+  double other;
+  if (few_columns) other = 8e-6 + out_bytes / 4.5e12 + (double)p.nnz * batch * ceil_div(p.n, 512) * 10.0 / (256 * 2.1e9);
+  else if (matrix_core_kind) other = 8e-6 + flops / 720e12;
+  else other = 8e-6 + (double)p.nnz * p.n * batch * 2 / 26e12 + out_bytes / 4e12;
   return 1.15 * dense_form < other;
 }
 
@@ -419,6 +477,22 @@ int launch_dense_path(const SpmmParams& p, int batch, const Choice& ch, hipStrea
 template <typename T, typename IT>
 int launch_typed(const SpmmParams& p, int batch, const Choice& ch, hipStream_t stream) {
   constexpr int kMax = 16 / (int)sizeof(T);
+  // A with few columns and many rows, wide output: the tile of the dense operand in LDS, rows streamed
+  // (spmm_smallk_device.cuh).  Measured on the shapes of the reference's sweep (fp32, per-batch values):
+  // 96 x 3136 x 3136 outputs, k = 32, 98 % sparse 1033 -> 837 us (4.5 TB/s of output); 192 x 784 x 784
+  // 226 -> 145; 8 x 4096 x 4096, k = 64 at 90 % 262 -> 175, at 50 % 564 -> 354 (the fp32 matrix-core
+  // kernel, which the density would pick, takes 1282: its K loop is two chunks long); k = 128 with
+  // 4096 rows 264 -> 237, with 1024 rows 79 -> 99 (a 128 KB tile per 128 rows): hence m >= 32 k.
+  // 192 x 784 x 784, k = 32: 226 -> 145 us: hence m >= 8 k up to k = 64.  16-bit products that are dense
+  // enough go to the dense-form path first (time model above).
+  if (ch.variant == 0 && smallk_wanted<T>(p, batch)) {
+    if constexpr (sizeof(T) == 2) {
+      const bool room = ch.ws && aligned(ch.ws, 16) && ch.ws_bytes >= dense_path_bytes(p);
+      if (room && dense_path_fits(2, p, p.per_batch_values) && dense_path_wins(p, batch, 0, true))
+        return launch_dense_path<T, IT>(p, batch, ch, stream);
+    }
+    return launch_smallk<T, IT>(p, batch, stream);
+  }
   if constexpr (std::is_same<T, float>::value && std::is_same<IT, int>::value) {
     int windows = 0;
     if (const int arr = mfma_f32_variant<T, IT>(p, batch, ch, windows)) return launch_mfma_f32(p, batch, arr, windows, ch.lpg != 8, stream);  // (lanes-per-group code 8 = no role split, for tuning)
@@ -434,7 +508,7 @@ int launch_typed(const SpmmParams& p, int batch, const Choice& ch, hipStream_t s
       IEX_REQUIRE(room, IEX_ERR_BAD_ARGUMENT, "spmm: the dense-form path needs a 16-byte aligned workspace of %zu bytes (iex_spmm_ws)", dense_path_bytes(p));
       return launch_dense_path<T, IT>(p, batch, ch, stream);
     }
-    if (ch.variant == 0 && fits && room && dense_path_wins(p, batch, mc.kind)) return launch_dense_path<T, IT>(p, batch, ch, stream);
+    if (ch.variant == 0 && fits && room && dense_path_wins(p, batch, mc.kind, false)) return launch_dense_path<T, IT>(p, batch, ch, stream);
   }
   // Where the 8-wave kernel would run: the direct-load kernel wins on 2:4 weights (4096 x 4096,
   // n = 8192: 0.37 against 0.40-0.46 ms with five windows), ties at 80 % sparsity (11008 x 4096:
@@ -443,6 +517,10 @@ int launch_typed(const SpmmParams& p, int batch, const Choice& ch, hipStream_t s
   if (mc.kind == 4 && ch.variant == 0 && 2.0 * p.nnz == (double)p.m * p.k) return launch_mfma3<T, IT>(p, batch, 2, stream);
   if (mc.kind == 4) return launch_mfma2<T, IT>(p, batch, mc.param, stream);
   if (mc.kind == 3) return launch_mfma<T, IT>(p, batch, mc.param, stream);
+  if (ch.variant == 8) {
+    IEX_REQUIRE(smallk_fits<T>(p), IEX_ERR_UNSUPPORTED, "spmm: the few-columns kernel needs k <= %d, n a multiple of the 128-bit vector and at least one tile wide, 16-byte aligned operands", kSmallKMax);
+    return launch_smallk<T, IT>(p, batch, stream);
+  }
   int lvec = 0, rpw = 0;
   if (lds_variant<T>(p, batch, ch, lvec, rpw)) {
     if (lvec == kMax) return launch_lds_rpw<T, IT, kMax>(p, batch, rpw, stream);
@@ -533,7 +611,8 @@ size_t spmm_workspace_bytes(int dtype, int itype, int flags, int m, int k, int n
     Choice ch;
     ch.rpw = (flags >> 20) & 0xf;
     ch.lpg = ((flags >> 28) & 0x7) ? (4 << ((flags >> 28) & 0x7)) : 0;
-    if (!dense_path_wins(p, batch, mfma_variant<__half>(p, batch, ch).kind)) return 0;
+    const bool few = smallk_wanted<__half>(p, batch);
+    if (!dense_path_wins(p, batch, few ? 0 : mfma_variant<__half>(p, batch, ch).kind, few)) return 0;
   }
   return dense_path_bytes(p);
 }

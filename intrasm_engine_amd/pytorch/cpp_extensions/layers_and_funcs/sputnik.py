@@ -47,6 +47,8 @@ SPMM_KERNELS: dict[str, dict] = {
     "mfma8_direct_windows2": {"force_variant": 6, "force_rpw": 2},
     # the dense form of the sparse operand written into a workspace (the operator allocates it), then the dense GEMM
     "dense_form_gemm": {"force_variant": 7},
+    # A with at most 128 columns and a wide output: the dense operand's tile in LDS, rows streamed
+    "few_columns": {"force_variant": 8},
     # fp32 on the matrix cores: 32 x 128 tiles with 2, 4 or 8 windows, 16 x 128 tiles
     "mfma32_windows2": {"force_variant": 5, "force_nt": 4, "force_rpw": 2},
     "mfma32_windows4": {"force_variant": 5, "force_nt": 4, "force_rpw": 4},
@@ -62,6 +64,9 @@ def spmm_kernel_choices(dtype: torch.dtype, n: int, k: int | None = None, m: int
     pass runs the same choice on the transposed matrix: it is offered when the sparse operand's
     ``k`` and ``m`` are given and multiples of 8."""
     names = ["auto", "row", "row_wpr4", "row_wpr8", "lds_rows2", "lds_rows4", "lds_rows8"]
+    vec = 4 if dtype == torch.float32 else 8
+    if k is not None and m is not None and max(k, m) <= 128 and n % vec == 0 and n >= 64 * vec:
+        names.append("few_columns")      # (refuses other shapes; the backward product has m columns)
     if dtype in (torch.float16, torch.bfloat16) and n % 8 == 0:
         names += [k_ for k_ in SPMM_KERNELS if k_.startswith(("mfma4_", "mfma8_"))]
         if k is not None and m is not None and k % 8 == 0 and m % 8 == 0:

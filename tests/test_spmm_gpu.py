@@ -607,6 +607,66 @@ def test_dense_form_path(oracle, dev, dtype, itype, m, k, n, batch):
     assert_close(out.float().cpu().numpy(), want, scale, RTOL[dtype], f"dense form {dtype} {m}x{k}x{n}")
 
 
+@pytest.mark.parametrize("dtype,itype,batch,m,k,n,sparsity", [
+    (torch.float32, torch.int32, 2, 203, 32, 256, 0.9), (torch.float32, torch.int32, 3, 1000, 128, 516, 0.5),
+    (torch.float32, torch.int32, 1, 77, 1, 1024, 0.0), (torch.float16, torch.int16, 2, 300, 100, 520, 0.7),
+    (torch.bfloat16, torch.int32, 1, 130, 64, 2048, 0.95), (torch.float32, torch.int32, 1, 5000, 16, 260, 0.99)])
+def test_few_columns_kernel(oracle, dev, dtype, itype, batch, m, k, n, sparsity):
+    """Family 8 (A with at most 128 columns, wide output: the dense operand's tile in LDS, rows streamed in
+    natural order): per-batch values and shared values with bias + ReLU + accumulate, an empty first row,
+    a single column, a last tile that is partly outside the matrix.  Against the oracle, and bit-equal to
+    the row kernel with one wavefront per row (same order of summation)."""
+    from intrasm_engine_amd.pytorch import ops as pyops
+    rng = np.random.default_rng(m + k)
+    mask = rng.random((m, k)) >= sparsity
+    mask[0] = False
+    ro, ci, _ = W.csr_from_mask(mask)
+    csr = W.CSR(m, k, rng.standard_normal(ci.shape[0]).astype(np.float32), W.swizzle_from_offsets(ro), ro, ci)
+    ri, v, ro_t, ci_t = to_dev(csr, dev, dtype, itype)
+    b_np = rng.standard_normal((batch, k, n)).astype(np.float32)
+    b = torch.from_numpy(b_np).to(dev).to(dtype)
+    vb_np = rng.standard_normal((batch, csr.nnz)).astype(np.float32)
+    vb = torch.from_numpy(vb_np).to(dev).to(dtype)
+    kw = dict(dtypes=(dtype,), allow_i16=True)
+    out = pyops._spmm(b, ri, vb, ro_t, ci_t, m, per_batch_values=True, accumulate=False, force_variant=8, **kw)
+    assert torch.equal(out, pyops._spmm(b, ri, vb, ro_t, ci_t, m, per_batch_values=True, accumulate=False,
+                                        force_variant=1, force_wpr=1, **kw))
+    b_r, vb_r = rounded(b_np, dtype), rounded(vb_np, dtype)
+    for z in range(batch):
+        want = oracle.spmm(b_r[z:z + 1], csr.row_indices, vb_r[z], csr.row_offsets, csr.column_indices, m)
+        sc = oracle.spmm_abs_scale(b_r[z:z + 1], csr.row_indices, vb_r[z], csr.row_offsets, csr.column_indices, m)
+        assert_close(out[z:z + 1].float().cpu().numpy(), want, sc, RTOL[dtype], f"few columns, per-batch values z={z}")
+    bias = torch.randn(m, device=dev)
+    prev = torch.randn(batch, m, n, device=dev).to(dtype)
+    kw2 = dict(per_batch_values=False, accumulate=True, bias=bias, relu=True, **kw)
+    got = pyops._spmm(b, ri, v, ro_t, ci_t, m, force_variant=8, out=prev.clone(), **kw2)
+    assert torch.equal(got, pyops._spmm(b, ri, v, ro_t, ci_t, m, force_variant=1, force_wpr=1, out=prev.clone(), **kw2))
+
+
+def test_few_columns_kernel_long_runs_of_rows_and_refusals(dev):
+    """40000 rows, k = 128: a wavefront walks 64 rows (two groups of row offsets), the nonzeros of a group
+    span several 64-entry reads.  The library takes the kernel by itself here (bit-equal to forcing it);
+    shapes it cannot serve are refused on request."""
+    from intrasm_engine_amd.pytorch import ops as pyops
+    rng = np.random.default_rng(9)
+    m, k, n, batch = 40000, 128, 512, 8
+    mask = rng.random((m, k)) >= 0.97
+    ro, ci, _ = W.csr_from_mask(mask)
+    ri = torch.from_numpy(W.swizzle_from_offsets(ro)).to(dev)
+    ro_t, ci_t = torch.from_numpy(ro).to(dev), torch.from_numpy(ci).to(dev)
+    v = torch.randn(ci.shape[0], device=dev)
+    b = torch.randn(batch, k, n, device=dev)
+    kw = dict(per_batch_values=False, accumulate=False, dtypes=(torch.float32,), allow_i16=False)
+    row = pyops._spmm(b, ri, v, ro_t, ci_t, m, force_variant=1, force_wpr=1, **kw)
+    assert torch.equal(pyops._spmm(b, ri, v, ro_t, ci_t, m, force_variant=8, **kw), row)
+    assert torch.equal(pyops._spmm(b, ri, v, ro_t, ci_t, m, **kw), row)
+    with pytest.raises(RuntimeError, match="few-columns kernel needs"):
+        pyops._spmm(b[:, :, :130].contiguous(), ri, v, ro_t, ci_t, m, force_variant=8, **kw)      # n = 130
+    wide = torch.randn(1, 256, 512, device=dev)
+    with pytest.raises(RuntimeError, match="few-columns kernel needs"):
+        pyops._spmm(wide, ri[:8], v[:1], torch.zeros(9, dtype=torch.int32, device=dev), ci_t[:1], 8, force_variant=8, **kw)  # k = 256
+
+
 def test_dense_form_path_epilogue_options(oracle, dev):
     """bias + ReLU and accumulation into the output ride in the GEMM's epilogue; per-batch values have
     no single dense form and are refused on request."""

@@ -71,6 +71,28 @@ __device__ __forceinline__ void store_vec(T* p, const vec_t<T, VEC>& x) {
   }
 }
 
+// The same store with the streaming hint: for outputs far larger than the caches, written once
+// and not read again by the kernel (measured on 3.8 GB of SpMM output: 4.5 -> 5.3 TB/s).
+template <int BYTES> struct stream_word;
+template <> struct stream_word<16> { typedef unsigned int type __attribute__((ext_vector_type(4))); };
+template <> struct stream_word<8> { typedef unsigned int type __attribute__((ext_vector_type(2))); };
+template <> struct stream_word<4> { typedef unsigned int type; };
+template <> struct stream_word<2> { typedef unsigned short type; };
+template <typename T, int VEC, bool ALIGNED = true>
+__device__ __forceinline__ void store_vec_stream(T* p, const vec_t<T, VEC>& x) {
+  typedef typename stream_word<sizeof(T) * VEC>::type W;
+  // The pointer passes through an empty asm so that the compiler sees another address than in the plain
+  // store of the other branch: it would otherwise merge the two stores of an `if (stream) ... else ...`
+  // into one and drop the hint, which only one of them carries.
+  asm volatile("" : "+v"(p));
+  if constexpr (ALIGNED) {
+    __builtin_nontemporal_store(__builtin_bit_cast(W, x), reinterpret_cast<W*>(p));
+  } else {
+    typedef W WU __attribute__((aligned(sizeof(T))));
+    __builtin_nontemporal_store(__builtin_bit_cast(W, x), reinterpret_cast<WU*>(p));
+  }
+}
+
 // ---- wave64 cross-lane helpers --------------------------------------------------
 __device__ __forceinline__ int lane_id() { return threadIdx.x & (kWave - 1); }
 

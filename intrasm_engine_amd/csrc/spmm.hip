@@ -67,15 +67,16 @@ bool smallk_fits(const SpmmParams& p) {
   return p.k >= 1 && p.k <= kSmallKMax && p.n % kMax == 0 && p.n >= kWave * kMax && aligned(p.dense, 16) && aligned(p.out, 16);
 }
 
-// ... and where the library takes it by itself: enough rows for the tile load (k KB per workgroup) to be a
-// fraction of what the workgroup writes, and enough work to pay for it -- on small, almost empty products
-// the row kernel is a plain writer of zeros at 5 TB/s and stays ahead (32 x 1024 x 1024 outputs, k = 32,
-// 95-99.9 % sparse: 26-33 us against 34-36; 8 x 4096 x 4096, k = 128 at 99.9 %: 114 against 128).
+// ... and where the library takes it by itself: up to 64 columns (two workgroups per CU), enough rows for
+// the tile load (k KB per workgroup) to be a fraction of what the workgroup writes, and rows that gather:
+// from 1.5 nonzeros per row the LDS gather wins (fp32, per-batch values: 192 x 784 x 784 outputs,
+// k = 32, 2 per row: 107 against 127 us; 8 x 4096 x 4096, k = 64, 6 per row: 126 / 172, 32 per row: 344 / 535);
+// almost empty rows are a plain write, which the row kernel does at 6 TB/s with streaming stores
+// (96 x 3136 x 3136, 0.5 per row: 627 against 711), and k = 128 leaves one workgroup per CU (6 per row: 197 / 176).
 template <typename T>
 bool smallk_wanted(const SpmmParams& p, int batch) {
-  if (!smallk_fits<T>(p) || p.m < (p.k <= 64 ? 8 : 32) * p.k) return false;
-  const double mean_row = (double)p.nnz / p.m, out_bytes = (double)p.m * p.n * batch * sizeof(T);
-  return p.k <= 64 ? (out_bytes >= 256e6 || mean_row >= 3.0) : mean_row >= 0.4;
+  (void)batch;
+  return smallk_fits<T>(p) && p.k <= 64 && p.m >= 8 * p.k && (double)p.nnz >= 1.5 * p.m;
 }
 
 template <typename T, typename IT>
@@ -477,14 +478,9 @@ int launch_dense_path(const SpmmParams& p, int batch, const Choice& ch, hipStrea
 template <typename T, typename IT>
 int launch_typed(const SpmmParams& p, int batch, const Choice& ch, hipStream_t stream) {
   constexpr int kMax = 16 / (int)sizeof(T);
-  // A with few columns and many rows, wide output: the tile of the dense operand in LDS, rows streamed
-  // (spmm_smallk_device.cuh).  Measured on the shapes of the reference's sweep (fp32, per-batch values):
-  // 96 x 3136 x 3136 outputs, k = 32, 98 % sparse 1033 -> 837 us (4.5 TB/s of output); 192 x 784 x 784
-  // 226 -> 145; 8 x 4096 x 4096, k = 64 at 90 % 262 -> 175, at 50 % 564 -> 354 (the fp32 matrix-core
-  // kernel, which the density would pick, takes 1282: its K loop is two chunks long); k = 128 with
-  // 4096 rows 264 -> 237, with 1024 rows 79 -> 99 (a 128 KB tile per 128 rows): hence m >= 32 k.
-  // 192 x 784 x 784, k = 32: 226 -> 145 us: hence m >= 8 k up to k = 64.  16-bit products that are dense
-  // enough go to the dense-form path first (time model above).
+  // A with few columns and rows that gather, wide output: the tile of the dense operand in LDS, rows
+  // streamed (spmm_smallk_device.cuh; smallk_wanted has the measurements).  16-bit products that are
+  // dense enough go to the dense-form path first (time model above).
   if (ch.variant == 0 && smallk_wanted<T>(p, batch)) {
     if constexpr (sizeof(T) == 2) {
       const bool room = ch.ws && aligned(ch.ws, 16) && ch.ws_bytes >= dense_path_bytes(p);
@@ -589,6 +585,8 @@ int spmm_dispatch(int dtype, int itype, int flags, int m, int k, int n, int nonz
   SpmmParams p{m, k, n, nonzeros, row_indices, values, row_offsets, column_indices, dense, bias, out,
                (flags & IEX_SPMM_PER_BATCH_VALUES) != 0, (flags & IEX_SPMM_ACCUMULATE) != 0,
                (flags & IEX_SPMM_RELU) != 0};
+  // beyond the 256 MB last-level cache an output can only stream; the hint is worth 15-25 % of the write rate
+  p.stream_out = (double)m * n * batch * (dtype == IEX_F32 ? 4 : 2) >= 128e6;
   hipStream_t s = static_cast<hipStream_t>(stream);
   if (dtype == IEX_F32 && itype == IEX_I32) return launch_typed<float, int>(p, batch, ch, s);
   if (dtype == IEX_F16 && itype == IEX_I32) return launch_typed<__half, int>(p, batch, ch, s);

@@ -33,6 +33,7 @@ struct SpmmParams {
   const float* bias;
   void* out;
   int per_batch_values, accumulate, relu;
+  int stream_out = 0;  // the output is far larger than the caches: store it with the streaming hint
 };
 
 constexpr int kSpmmUnroll = 8;
@@ -250,6 +251,8 @@ __device__ __forceinline__ void spmm_block(const SpmmParams& p, int bx, int by, 
 #pragma unroll
       for (int i = 0; i < VEC; ++i)
         if (i >= shift) out[i] = o.v[i];  // the elements before `shift` belong to the lane to the left
+    } else if (p.stream_out) {
+      store_vec_stream<T, VEC, !RAGGED>(out, o);
     } else {
       store_vec<T, VEC, !RAGGED>(out, o);
     }

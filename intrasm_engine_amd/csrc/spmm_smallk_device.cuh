@@ -92,7 +92,8 @@ __device__ __forceinline__ void spmm_smallk_block(const SpmmParams& p, int rows_
         if (p.relu) r = fmaxf(r, 0.f);
         o.v[u] = elem<T>::from_float(r);
       }
-      store_vec<T, VEC>(out, o);
+      if (p.stream_out) store_vec_stream<T, VEC>(out, o);  // leaves L2 to the tile loads
+      else store_vec<T, VEC>(out, o);
     }
   }
 }

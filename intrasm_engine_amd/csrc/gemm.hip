@@ -146,6 +146,7 @@ int iex::gemm_dispatch(int dtype, int trans_b_and_shape, int M, int N, int K, co
   IEX_REQUIRE((long long)M * K < (1ll << 31) && (long long)N * K < (1ll << 31) && (long long)M * N < (1ll << 31),
               IEX_ERR_TOO_LARGE, "gemm: an operand exceeds 2^31 elements per batch entry");
   GemmParams p{M, N, K, A, B, C, stride_a, stride_b, stride_c, 0, 0, row_bias, relu, accumulate};
+  p.stream_out = (double)M * N * batch * 2 >= 128e6;
   hipStream_t s = static_cast<hipStream_t>(stream);
   const bool bf = dtype == IEX_BF16;
   if (bf && trans_b) return launch_shape<true, true>(p, batch, force, s);

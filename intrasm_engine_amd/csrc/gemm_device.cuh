@@ -35,6 +35,7 @@ struct GemmParams {
   // C = relu?((accumulate ? C : 0) + A * B + row_bias[row])
   const float* row_bias = nullptr;
   int relu = 0, accumulate = 0;
+  int stream_out = 0;  // C is far larger than the caches: store it with the streaming hint
 };
 
 // iex_gemm with the epilogue options above (gemm.hip).
@@ -221,6 +222,67 @@ __device__ __forceinline__ void gemm_store_tile(const GemmParams& p, const f32x1
 #pragma unroll
           for (int e = 0; e < 4; ++e)
             if (gn + e < p.N) dst[e] = h[e];
+        }
+      }
+    }
+  }
+}
+
+// The same, through LDS: a lane's accumulators are 4 adjacent columns of 32 different rows, so the
+// direct store writes 32 pieces of 16 bytes per instruction; here each 32-row block of the wavefront's
+// tile is laid out in the wavefront's own slice of LDS (rows padded by 16 bytes) and read back 16 lanes
+// per row, so a store instruction writes 4 rows of WN * 64 contiguous bytes.  A GEMM with a short K is a
+// writer of its output: 16 x 4096 x 4096 outputs with K = 64 went from 1.7 TB/s to the rate of a fill.
+// `lds` = this wavefront's slice, gemm_store_lds_bytes<WN>() bytes, nobody else touches it (no barrier
+// needed: the LDS operations of one wavefront execute in order).  Needs N % 8 == 0, a 16-byte aligned
+// C and no accumulation; `stream`: store with the streaming hint.
+template <int WN>
+constexpr int gemm_store_lds_bytes() { return 32 * (WN * 64 + 16); }
+
+template <bool BF16, int WM, int WN>
+__device__ __forceinline__ void gemm_store_tile_lds(const GemmParams& p, const f32x16 (&acc)[WM][WN], unsigned short* __restrict__ C,
+                                                    int m0, int n0, int wm, int wn, int lane, unsigned char* lds, bool stream) {
+  typedef unsigned short u16;
+  constexpr int ROWB = WN * 64 + 16;   // bytes of a padded row
+  constexpr int CPR = WN * 4;          // 16-byte chunks per row
+  constexpr int RPI = kWave / CPR;     // rows a store instruction covers
+  static_assert(kWave % CPR == 0 && 32 % RPI == 0, "whole rows per instruction");
+#pragma unroll
+  for (int i = 0; i < WM; ++i) {
+    const int row0 = m0 + (wm * WM + i) * 32;
+    if (row0 >= p.M) break;  // (uniform)
+    const int gm_w = min(row0 + (lane & 31), p.M - 1);
+    const float bias = p.row_bias ? p.row_bias[gm_w] : 0.f;
+#pragma unroll
+    for (int j = 0; j < WN; ++j) {
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        u16 h[4];
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          float y = acc[i][j][q * 4 + e] + bias;
+          if (p.relu) y = fmaxf(y, 0.f);
+          h[e] = f32_to_16(y, BF16);
+        }
+        u32x2 w;
+        w.x = (unsigned)h[0] | ((unsigned)h[1] << 16);
+        w.y = (unsigned)h[2] | ((unsigned)h[3] << 16);
+        *reinterpret_cast<u32x2*>(lds + (lane & 31) * ROWB + (j * 32 + q * 8 + (lane >> 5) * 4) * 2) = w;
+      }
+    }
+    const int chunk = lane % CPR;
+    const int gn = n0 + wn * WN * 32 + chunk * 8;
+#pragma unroll
+    for (int t = 0; t < 32 / RPI; ++t) {
+      const int r = t * RPI + lane / CPR;
+      const u32x4 v = *reinterpret_cast<const u32x4*>(lds + r * ROWB + chunk * 16);
+      if (row0 + r < p.M && gn < p.N) {
+        u16* dst = C + (size_t)(row0 + r) * p.N + gn;
+        if (stream) {
+          asm volatile("" : "+v"(dst));  // (keeps the compiler from merging this store with the plain one and dropping the hint)
+          __builtin_nontemporal_store(v, reinterpret_cast<u32x4*>(dst));
+        } else {
+          *reinterpret_cast<u32x4*>(dst) = v;
         }
       }
     }

@@ -233,7 +233,14 @@ __device__ __forceinline__ void gemm_tile_dma(const GemmParams& p, int tile_m, i
   }
   wait_vmcnt<0>();  // the re-fetched last tiles: nothing may still be writing LDS when the workgroup ends
 
-  gemm_store_tile<BF16, WM, WN>(p, acc, C, m0, n0, wm, wn, lane);
+  // the stages are free now: row-contiguous stores through LDS where the shape allows
+  static_assert(WAVES * gemm_store_lds_bytes<WN>() <= gemm_dma_lds_bytes<WM, WN, WCN, BK, STAGES>(), "the epilogue fits the stages");
+  if (!p.accumulate && p.N % 8 == 0 && (reinterpret_cast<uintptr_t>(C) & 15) == 0) {
+    __syncthreads();  // everybody has read its last fragments
+    gemm_store_tile_lds<BF16, WM, WN>(p, acc, C, m0, n0, wm, wn, lane, smem + wave * gemm_store_lds_bytes<WN>(), p.stream_out != 0);
+  } else {
+    gemm_store_tile<BF16, WM, WN>(p, acc, C, m0, n0, wm, wn, lane);
+  }
 }
 
 }  // namespace iex

@@ -446,8 +446,8 @@ inline size_t dense_path_bytes(const SpmmParams& p) { return (size_t)p.m * p.k *
 //     for the dense form; 80 % 11008 x 4096: 0.93 / 0.69; 90 %, n = 2048: 0.27 / 0.23);
 //   gather kernels: nnz * n * 2 bytes through the L2 -> CU path at 26 TB/s (4096^2 at 70 %, n = 256:
 //     110 against 58 us; at 90 %, n = 256: 40 against 58; 11008 x 4096 at 95 %, n = 2048: 0.35 / 0.21 ms).
-//   a short K makes the GEMM a writer of its output at 2 TB/s (16 x 4096 x 4096, k = 64: 0.31 ms), the
-//     gather kernels write it at 4 TB/s, the few-columns kernel at 4.5 TB/s plus 10 clocks of a CU's LDS
+//   a short K makes the GEMM a writer of its output at 3 TB/s (16 x 4096 x 4096, k = 64: 0.18 ms) and the
+//     matrix-core SpMM kernels at 1.2 TB/s (8 x 4096 x 4096, k = 128: 0.24 ms), the gather kernels write it at 4 TB/s, the few-columns kernel at 4.5 TB/s plus 10 clocks of a CU's LDS
 //     per nonzero and tile (same shape at 93 % sparsity: 0.15 ms; 8 x 4096 x 4096, k = 128 at 50 %: 0.58
 //     against 0.17 for the dense form).
 // The dense form has to win by 15 % to be taken.  `few_columns`: the alternative is the few-columns kernel.
@@ -455,11 +455,11 @@ inline bool dense_path_wins(const SpmmParams& p, int batch, int matrix_core_kind
   const double cells = (double)p.m * p.k, flops = 2.0 * cells * p.n * batch;
   const double out_bytes = (double)p.m * p.n * batch * 2;
   const double tiles = (double)ceil_div(p.m, 128) * ceil_div(p.n, 128) * batch;
-  const double product = std::max({flops / 1000e12, std::ceil(tiles / 512.0) * (p.k / 32.0) * 0.35e-6, out_bytes / 2e12});
+  const double product = std::max({flops / 1000e12, std::ceil(tiles / 512.0) * (p.k / 32.0) * 0.35e-6, out_bytes / 3e12});
   const double dense_form = 8e-6 + cells * 2 / 4e12 + product;
   double other;
   if (few_columns) other = 8e-6 + out_bytes / 4.5e12 + (double)p.nnz * batch * ceil_div(p.n, 512) * 10.0 / (256 * 2.1e9);
-  else if (matrix_core_kind) other = 8e-6 + flops / 720e12;
+  else if (matrix_core_kind) other = 8e-6 + std::max(flops / 720e12, out_bytes / 1.2e12);
   else other = 8e-6 + (double)p.nnz * p.n * batch * 2 / 26e12 + out_bytes / 4e12;
   return 1.15 * dense_form < other;
 }

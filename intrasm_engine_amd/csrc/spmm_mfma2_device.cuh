@@ -212,7 +212,7 @@ __device__ __forceinline__ void spmm_mfma2_block(const SpmmParams& p, int tile_m
     cur = nxt;
   }
 
-  spmm_mfma_epilogue<BF16, WM, WN>(p, acc, C, m0, n0, wm, wn, lane);
+  spmm_mfma_epilogue<BF16, WM, WN>(p, acc, C, m0, n0, wm, wn, lane, smem);
 }
 
 }  // namespace iex

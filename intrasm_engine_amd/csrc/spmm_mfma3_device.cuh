@@ -250,7 +250,7 @@ __device__ __forceinline__ void spmm_mfma3_block(const SpmmParams& p, int tile_m
   }
   wait_vmcnt<0>();  // the re-fetched last tiles: nothing may still be writing LDS when the workgroup ends
 
-  spmm_mfma_epilogue<BF16, WM, WN>(p, acc, C, m0, n0, wm, wn, lane);
+  spmm_mfma_epilogue<BF16, WM, WN>(p, acc, C, m0, n0, wm, wn, lane, smem);
 }
 
 }  // namespace iex

@@ -107,6 +107,10 @@ int launch_shape(const GemmParams& p, int batch, int force, hipStream_t stream) 
   //   8192^3: 256x256 1200, 128x256 1040, register-staged 256x256 980;   4096 x 8192 x 4096: 1140 / 1000 / 920
   //   config 4's 4096 x 2048 x 4096 (128 tiles of 256x256): 620 / 860 / 470, 128x128 750
   //   2048^3: 290 / 420 / 220, 128x128 550
+  // A short K (at most 8 steps) is prologue and epilogue: small tiles, two workgroups per CU that cover for
+  // each other (512 x (512 x 512 x 128), the attention scores of the decoder layer: 229 -> 123 us; 8192 x 8192 x
+  // 128: 59 -> 48; from K = 512 the large tiles are ahead again).
+  if (p.K <= 256) return launch_dma<BF16, TRANS_B, 2, 2, 32, 4>(p, batch, stream);
   auto fill = [](int n, int tile) { return (double)n / ((double)ceil_div(n, tile) * tile); };
   const long long huge_tiles = (long long)ceil_div(p.M, 256) * ceil_div(p.N, 256) * batch;
   if (huge_tiles >= 512 && fill(p.M, 256) * fill(p.N, 256) >= 0.8) return launch_dma<BF16, TRANS_B, 4, 4, 32, 4>(p, batch, stream);

@@ -55,16 +55,23 @@ int launch_ragged(const SpmmParams& p, int batch, int wpr, hipStream_t stream) {
 }
 
 // ---- few columns in A, wide output: the dense operand's tile lives in LDS ---------------------
-template <typename T, typename IT, int VEC>
+template <typename T, typename IT, int VEC, bool RAGGED>
 __global__ __launch_bounds__(kSmallKThreads) void spmm_smallk_kernel(SpmmParams p, int rows_per_wave) {
   extern __shared__ __align__(16) unsigned char smem[];
-  spmm_smallk_block<T, IT, VEC>(p, rows_per_wave, blockIdx.x, blockIdx.y, blockIdx.z, smem);
+  spmm_smallk_block<T, IT, VEC, RAGGED>(p, rows_per_wave, blockIdx.x, blockIdx.y, blockIdx.z, smem);
+}
+
+// full vectors at their natural alignment, or (ragged) any n at element alignment
+template <typename T>
+bool smallk_aligned(const SpmmParams& p) {
+  constexpr int kMax = 16 / (int)sizeof(T);
+  return p.n % kMax == 0 && aligned(p.dense, 16) && aligned(p.out, 16);
 }
 
 template <typename T>
 bool smallk_fits(const SpmmParams& p) {
   constexpr int kMax = 16 / (int)sizeof(T);
-  return p.k >= 1 && p.k <= kSmallKMax && p.n % kMax == 0 && p.n >= kWave * kMax && aligned(p.dense, 16) && aligned(p.out, 16);
+  return p.k >= 1 && p.k <= kSmallKMax && p.n >= kWave * kMax && aligned(p.dense, sizeof(T)) && aligned(p.out, sizeof(T));
 }
 
 // ... and where the library takes it by itself: up to 64 columns (two workgroups per CU), enough rows for
@@ -76,7 +83,9 @@ bool smallk_fits(const SpmmParams& p) {
 template <typename T>
 bool smallk_wanted(const SpmmParams& p, int batch) {
   (void)batch;
-  return smallk_fits<T>(p) && p.k <= 64 && p.m >= 8 * p.k && (double)p.nnz >= 1.5 * p.m;
+  // (rows that are no multiple of the vector: from 2.5 per row -- 384 x 785 x 785, k = 64: 3.2 per row 377 -> 322 us,
+  // 1.9 per row 290 -> 313)
+  return smallk_fits<T>(p) && p.k <= 64 && p.m >= 8 * p.k && (double)p.nnz >= (smallk_aligned<T>(p) ? 1.5 : 2.5) * p.m;
 }
 
 template <typename T, typename IT>
@@ -88,15 +97,16 @@ int launch_smallk(const SpmmParams& p, int batch, hipStream_t stream) {
   int rows = std::min(64, std::max(16, p.k / 2));
   while (rows > 4 && (long long)ceil_div(p.m, kSmallKWaves * rows) * tiles < 1024) rows >>= 1;
   const int lds = p.k * kWave * 16;
-  auto kern = spmm_smallk_kernel<T, IT, kMax>;
+  const bool ragged = !smallk_aligned<T>(p);
+  auto kern = ragged ? spmm_smallk_kernel<T, IT, kMax, true> : spmm_smallk_kernel<T, IT, kMax, false>;
   if (lds > 64 * 1024) {
-    static thread_local bool raised = false;  // per instantiation
-    if (!raised) {
+    static thread_local bool raised[2] = {false, false};  // per instantiation and alignment variant
+    if (!raised[ragged]) {
       if (int rc = check_hip(hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
                                                  kSmallKMax * kWave * 16),
                              "hipFuncSetAttribute(LDS size)"))
         return rc;
-      raised = true;
+      raised[ragged] = true;
     }
   }
   dim3 grid(ceil_div(p.m, kSmallKWaves * rows), ceil_div(p.n, kWave * kMax), batch);
@@ -514,7 +524,7 @@ int launch_typed(const SpmmParams& p, int batch, const Choice& ch, hipStream_t s
   if (mc.kind == 4) return launch_mfma2<T, IT>(p, batch, mc.param, stream);
   if (mc.kind == 3) return launch_mfma<T, IT>(p, batch, mc.param, stream);
   if (ch.variant == 8) {
-    IEX_REQUIRE(smallk_fits<T>(p), IEX_ERR_UNSUPPORTED, "spmm: the few-columns kernel needs k <= %d, n a multiple of the 128-bit vector and at least one tile wide, 16-byte aligned operands", kSmallKMax);
+    IEX_REQUIRE(smallk_fits<T>(p), IEX_ERR_UNSUPPORTED, "spmm: the few-columns kernel needs k <= %d and an output at least one tile (64 128-bit vectors) wide", kSmallKMax);
     return launch_smallk<T, IT>(p, batch, stream);
   }
   int lvec = 0, rpw = 0;

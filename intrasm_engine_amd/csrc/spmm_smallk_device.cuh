@@ -16,7 +16,11 @@
 //   * what is left per row is the store of its 64 * VEC outputs, and stores do not wait.
 // Accumulation is fp32, in ascending nonzero order (the order of the row kernel with one wavefront
 // per row, so results are bit-equal to it); the swizzle (row_indices) is ignored: it only
-// schedules.  Needs n % VEC == 0 and 16-byte aligned dense operand and output (full vectors).
+// schedules.  Needs n % VEC == 0 and 16-byte aligned dense operand and output (full vectors), or
+// RAGGED: any n >= VEC at element alignment -- rows then start at any element, vectors are moved with
+// element-aligned 128-bit accesses, and the one lane per row whose vector would pass the row's end
+// works on the last VEC elements of the row instead (shifted back), computes all of them and stores
+// only the ones it owns (the others belong to the lane to its left, which stores the same values).
 #pragma once
 #include "spmm_device.cuh"
 
@@ -26,7 +30,7 @@ constexpr int kSmallKMax = 128;   // dense rows (KB of LDS) a tile may have
 constexpr int kSmallKWaves = 8;
 constexpr int kSmallKThreads = kSmallKWaves * kWave;
 
-template <typename T, typename IT, int VEC>
+template <typename T, typename IT, int VEC, bool RAGGED = false>
 __device__ __forceinline__ void spmm_smallk_block(const SpmmParams& p, int rows_per_wave, int bx, int by, int bz,
                                                   unsigned char* smem) {
   typedef vec_t<T, VEC> V;
@@ -36,8 +40,9 @@ __device__ __forceinline__ void spmm_smallk_block(const SpmmParams& p, int rows_
   const int z = bz;
   const int col0 = by * (kWave * VEC) + lane * VEC;
   const bool lane_live = col0 < p.n;
-  const T* __restrict__ dense = static_cast<const T*>(p.dense) + (size_t)z * p.k * p.n + min(col0, p.n - VEC);
-  for (int kr = wave; kr < p.k; kr += kSmallKWaves) tile[kr * kWave + lane] = load_vec<T, VEC>(dense + (size_t)kr * p.n);
+  const int shift = (RAGGED && lane_live && col0 + VEC > p.n) ? col0 + VEC - p.n : 0;
+  const T* __restrict__ dense = static_cast<const T*>(p.dense) + (size_t)z * p.k * p.n + min(col0 - shift, p.n - VEC);
+  for (int kr = wave; kr < p.k; kr += kSmallKWaves) tile[kr * kWave + lane] = load_vec<T, VEC, !RAGGED>(dense + (size_t)kr * p.n);
   __syncthreads();
 
   const T* __restrict__ values = static_cast<const T*>(p.values) + (p.per_batch_values ? (size_t)z * p.nnz : (size_t)0);
@@ -78,9 +83,9 @@ __device__ __forceinline__ void spmm_smallk_block(const SpmmParams& p, int rows_
         j = cbase + tl;
       }
       if (!lane_live) continue;
-      T* __restrict__ out = static_cast<T*>(p.out) + ((size_t)z * p.m + row) * p.n + col0;
+      T* __restrict__ out = static_cast<T*>(p.out) + ((size_t)z * p.m + row) * p.n + col0 - shift;
       if (p.accumulate) {
-        const V prev = load_vec<T, VEC>(out);
+        const V prev = load_vec<T, VEC, !RAGGED>(out);
 #pragma unroll
         for (int u = 0; u < VEC; ++u) acc[u] += elem<T>::to_float(prev.v[u]);
       }
@@ -92,8 +97,15 @@ __device__ __forceinline__ void spmm_smallk_block(const SpmmParams& p, int rows_
         if (p.relu) r = fmaxf(r, 0.f);
         o.v[u] = elem<T>::from_float(r);
       }
-      if (p.stream_out) store_vec_stream<T, VEC>(out, o);  // leaves L2 to the tile loads
-      else store_vec<T, VEC>(out, o);
+      if (RAGGED && shift > 0) {
+#pragma unroll
+        for (int u = 0; u < VEC; ++u)
+          if (u >= shift) out[u] = o.v[u];
+      } else if (p.stream_out) {
+        store_vec_stream<T, VEC, !RAGGED>(out, o);  // leaves L2 to the tile loads
+      } else {
+        store_vec<T, VEC, !RAGGED>(out, o);
+      }
     }
   }
 }

@@ -156,7 +156,13 @@ __device__ __forceinline__ void spmm_mfma_epilogue_lds(const SpmmParams& p, cons
       const u32x4 v = *reinterpret_cast<const u32x4*>(lds + r * ROWB + chunk * 16);
       if (slot0 + r < p.m && gn < p.n) {
         const int row = p.row_indices[slot0 + r];
-        *reinterpret_cast<u32x4*>(C + (size_t)row * p.n + gn) = v;
+        u16* dst = C + (size_t)row * p.n + gn;
+        if (p.stream_out) {
+          asm volatile("" : "+v"(dst));  // (or the compiler merges this store with the plain one and drops the hint)
+          __builtin_nontemporal_store(v, reinterpret_cast<u32x4*>(dst));
+        } else {
+          *reinterpret_cast<u32x4*>(dst) = v;
+        }
       }
     }
   }

@@ -76,7 +76,7 @@ bool smallk_fits(const SpmmParams& p) {
 
 // ... and where the library takes it by itself: up to 64 columns (two workgroups per CU), enough rows for
 // the tile load (k KB per workgroup) to be a fraction of what the workgroup writes, and rows that gather:
-// from 1.5 nonzeros per row the LDS gather wins (fp32, per-batch values: 192 x 784 x 784 outputs,
+// from 1.8 nonzeros per row the LDS gather wins (fp32, per-batch values: 192 x 784 x 784 outputs,
 // k = 32, 2 per row: 107 against 127 us; 8 x 4096 x 4096, k = 64, 6 per row: 126 / 172, 32 per row: 344 / 535);
 // almost empty rows are a plain write, which the row kernel does at 6 TB/s with streaming stores
 // (96 x 3136 x 3136, 0.5 per row: 627 against 711), and k = 128 leaves one workgroup per CU (6 per row: 197 / 176).
@@ -85,7 +85,7 @@ bool smallk_wanted(const SpmmParams& p, int batch) {
   (void)batch;
   // (rows that are no multiple of the vector: from 2.5 per row -- 384 x 785 x 785, k = 64: 3.2 per row 377 -> 322 us,
   // 1.9 per row 290 -> 313)
-  return smallk_fits<T>(p) && p.k <= 64 && p.m >= 8 * p.k && (double)p.nnz >= (smallk_aligned<T>(p) ? 1.5 : 2.5) * p.m;
+  return smallk_fits<T>(p) && p.k <= 64 && p.m >= 8 * p.k && (double)p.nnz >= (smallk_aligned<T>(p) ? 1.8 : 2.5) * p.m;
 }
 
 template <typename T, typename IT>

@@ -99,7 +99,7 @@ int launch_shape(const GemmParams& p, int batch, int force, hipStream_t stream) 
   if (force == 5) return launch_dma<BF16, TRANS_B, 2, 2, 32, 4>(p, batch, stream);
   if (force == 6) return launch_dma<BF16, TRANS_B, 2, 4, 32, 4>(p, batch, stream);
   if (force == 7) return launch_dma<BF16, TRANS_B, 4, 4, 32, 4>(p, batch, stream);
-  if (force == 8) return launch_dma<BF16, TRANS_B, 2, 1, 32, 8, 4>(p, batch, stream);
+  if (force == 8) return launch_dma<BF16, TRANS_B, 2, 1, 64, 4, 4>(p, batch, stream);
   // Default: operands straight from global memory into LDS (gemm_dma_device.cuh).  The larger the
   // tile of a wave, the fewer LDS bytes each MFMA needs, and LDS time is what the main loop runs
   // against; the smaller the tile, the more workgroups there are to fill 256 CUs, and a tile wider
@@ -116,12 +116,12 @@ int launch_shape(const GemmParams& p, int batch, int force, hipStream_t stream) 
   if (huge_tiles >= 512 && fill(p.M, 256) * fill(p.N, 256) >= 0.8) return launch_dma<BF16, TRANS_B, 4, 4, 32, 4>(p, batch, stream);
   const long long wide_tiles = (long long)ceil_div(p.M, 128) * ceil_div(p.N, 256) * batch;
   if (wide_tiles >= 256 && fill(p.N, 256) >= 0.8) return launch_dma<BF16, TRANS_B, 2, 4, 32, 4>(p, batch, stream);
-  // One round of at most one 128 x 128 tile per CU and a long K: eight waves (64 x 32 each) and eight stages
-  // instead of four and four (10-14 %: 4096 x 512 x 4096 44 -> 38.6 us).  What bounds these is the LDS of the CUs
-  // that have a tile -- 273 clocks of direct-load writes and 170-250 of fragment reads per step of 8 MFMAs per
-  // wave -- while the other CUs idle; only a K split over workgroups (partial sums in a workspace) would change that.
+  // One round of at most one 128 x 128 tile per CU and a long K: eight waves (64 x 32 each) and K steps of 64
+  // (4096 x 512 x 4096: 44 -> 34.5 us; eight waves with steps of 32 and eight stages 38.6; 64 x 128 tiles 36.8).
+  // Such a product is one chain of dependent steps per CU, 0.3 us per 32 of K whatever the tile shape, while
+  // most CUs idle; only a K split over workgroups (partial sums in a workspace) would change that.
   const long long small_tiles = (long long)ceil_div(p.M, 128) * ceil_div(p.N, 128) * batch;
-  if (small_tiles <= 256 && p.K >= 2048) return launch_dma<BF16, TRANS_B, 2, 1, 32, 8, 4>(p, batch, stream);
+  if (small_tiles <= 256 && p.K >= 2048) return launch_dma<BF16, TRANS_B, 2, 1, 64, 4, 4>(p, batch, stream);
   return launch_dma<BF16, TRANS_B, 2, 2, 32, 4>(p, batch, stream);
 }
 
@@ -130,7 +130,7 @@ int launch_shape(const GemmParams& p, int batch, int force, hipStream_t stream) 
 
 // trans_b: bit 0 = B is (N, K); bits 4..7 force the kernel for tuning.  Register-staged operands:
 // 1 = 128x128 tiles, 2 = 128x256, 3 = 256x256, 4 = 128x128 with K steps of 64.  Operands loaded
-// straight into LDS: 5 = 128x128, 6 = 128x256, 7 = 256x256, 8 = 128x128 by eight waves with eight stages.  0 = choose (one of 5..8).
+// straight into LDS: 5 = 128x128, 6 = 128x256, 7 = 256x256, 8 = 128x128 by eight waves with K steps of 64.  0 = choose (one of 5..8).
 extern "C" int iex_gemm(int dtype, int trans_b_and_shape, int M, int N, int K, const void* A, const void* B, void* C, int batch,
                         long long stride_a, long long stride_b, long long stride_c, void* stream) {
   return iex::gemm_dispatch(dtype, trans_b_and_shape, M, N, K, A, B, C, batch, stride_a, stride_b, stride_c, stream, nullptr, 0, 0);

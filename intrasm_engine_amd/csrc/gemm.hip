@@ -118,8 +118,9 @@ int launch_shape(const GemmParams& p, int batch, int force, hipStream_t stream) 
   if (wide_tiles >= 256 && fill(p.N, 256) >= 0.8) return launch_dma<BF16, TRANS_B, 2, 4, 32, 4>(p, batch, stream);
   // One round of at most one 128 x 128 tile per CU and a long K: eight waves (64 x 32 each) and K steps of 64
   // (4096 x 512 x 4096: 44 -> 34.5 us; eight waves with steps of 32 and eight stages 38.6; 64 x 128 tiles 36.8).
-  // Such a product is one chain of dependent steps per CU, 0.3 us per 32 of K whatever the tile shape, while
-  // most CUs idle; only a K split over workgroups (partial sums in a workspace) would change that.
+  // Such a product runs on the few CUs that have a tile (128 x 128 x 4096 is 16 us of one CU's matrix cores at
+  // their peak and takes 34) while the others idle; only a K split over workgroups (partial sums in a
+  // workspace) would change that.
   const long long small_tiles = (long long)ceil_div(p.M, 128) * ceil_div(p.N, 128) * batch;
   if (small_tiles <= 256 && p.K >= 2048) return launch_dma<BF16, TRANS_B, 2, 1, 64, 4, 4>(p, batch, stream);
   return launch_dma<BF16, TRANS_B, 2, 2, 32, 4>(p, batch, stream);

@@ -100,6 +100,7 @@ int launch_shape(const GemmParams& p, int batch, int force, hipStream_t stream) 
   if (force == 6) return launch_dma<BF16, TRANS_B, 2, 4, 32, 4>(p, batch, stream);
   if (force == 7) return launch_dma<BF16, TRANS_B, 4, 4, 32, 4>(p, batch, stream);
   if (force == 8) return launch_dma<BF16, TRANS_B, 2, 1, 64, 4, 4>(p, batch, stream);
+  if (force == 9) return launch_dma<BF16, TRANS_B, 1, 1, 64, 4, 4>(p, batch, stream);
   // Default: operands straight from global memory into LDS (gemm_dma_device.cuh).  The larger the
   // tile of a wave, the fewer LDS bytes each MFMA needs, and LDS time is what the main loop runs
   // against; the smaller the tile, the more workgroups there are to fill 256 CUs, and a tile wider
@@ -121,6 +122,10 @@ int launch_shape(const GemmParams& p, int batch, int force, hipStream_t stream) 
   // Such a product runs on the few CUs that have a tile (128 x 128 x 4096 is 16 us of one CU's matrix cores at
   // their peak and takes 34) while the others idle; only a K split over workgroups (partial sums in a
   // workspace) would change that.
+  // Half as tall (64 x 128) where even that leaves at most one tile per CU: twice the CUs at work
+  // (4096 x 256 x 4096: 35 -> 27.5 us, 4096 x 512 x 4096: 35 -> 30, 1024 x 2048 x 1024: 13.9 -> 12.4).
+  const long long half_tiles = (long long)ceil_div(p.M, 64) * ceil_div(p.N, 128) * batch;
+  if (half_tiles <= 256 && p.K >= 512) return launch_dma<BF16, TRANS_B, 1, 1, 64, 4, 4>(p, batch, stream);
   const long long small_tiles = (long long)ceil_div(p.M, 128) * ceil_div(p.N, 128) * batch;
   if (small_tiles <= 256 && p.K >= 2048) return launch_dma<BF16, TRANS_B, 2, 1, 64, 4, 4>(p, batch, stream);
   return launch_dma<BF16, TRANS_B, 2, 2, 32, 4>(p, batch, stream);
@@ -131,7 +136,7 @@ int launch_shape(const GemmParams& p, int batch, int force, hipStream_t stream) 
 
 // trans_b: bit 0 = B is (N, K); bits 4..7 force the kernel for tuning.  Register-staged operands:
 // 1 = 128x128 tiles, 2 = 128x256, 3 = 256x256, 4 = 128x128 with K steps of 64.  Operands loaded
-// straight into LDS: 5 = 128x128, 6 = 128x256, 7 = 256x256, 8 = 128x128 by eight waves with K steps of 64.  0 = choose (one of 5..8).
+// straight into LDS: 5 = 128x128, 6 = 128x256, 7 = 256x256, 8 = 128x128, 9 = 64x128 by eight waves with K steps of 64.  0 = choose (one of 5..9).
 extern "C" int iex_gemm(int dtype, int trans_b_and_shape, int M, int N, int K, const void* A, const void* B, void* C, int batch,
                         long long stride_a, long long stride_b, long long stride_c, void* stream) {
   return iex::gemm_dispatch(dtype, trans_b_and_shape, M, N, K, A, B, C, batch, stride_a, stride_b, stride_c, stream, nullptr, 0, 0);

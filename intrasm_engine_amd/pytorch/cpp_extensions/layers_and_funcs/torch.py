@@ -15,7 +15,7 @@ from .utils import MyAutogradFunc, TunableItemCfg, maybe_captured
 ops = torch.ops.iex_ops
 
 # name -> tile-shape code of the GEMM entry point (workgroup tile, K step)
-GEMM_TILES: dict[str, int] = {"auto": 0, "128x128": 5, "128x256": 6, "256x256": 7, "128x128_8waves_k64": 8,
+GEMM_TILES: dict[str, int] = {"auto": 0, "128x128": 5, "128x256": 6, "256x256": 7, "128x128_8waves_k64": 8, "64x128_8waves_k64": 9,
                               # operands staged through registers on their way to LDS
                               "staged_128x128": 1, "staged_128x256": 2, "staged_256x256": 3, "staged_128x128_k64": 4}
 

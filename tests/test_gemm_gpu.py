@@ -38,13 +38,13 @@ def test_gemm_ragged_n_with_transposed_b(oracle, dev, shape):
         ops.gemm_mfma(torch.zeros(8, 8, device=dev).half(), torch.zeros(8, shape[1] | 1, device=dev).half(), False)
 
 
-@pytest.mark.parametrize("shape_code", [1, 2, 3, 4, 5, 6, 7, 8])
+@pytest.mark.parametrize("shape_code", [1, 2, 3, 4, 5, 6, 7, 8, 9])
 @pytest.mark.parametrize("trans_b", [False, True])
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
 @pytest.mark.parametrize("mnk", [(300, 520, 200), (129, 136, 8), (260, 264, 1000)])
 def test_every_tile_shape(oracle, dev, shape_code, trans_b, dtype, mnk):
     """Every kernel of the GEMM entry point forced through the C ABI (register-staged 128x128, 128x256, 256x256 tiles
-    and 128x128 with K steps of 64; 128x128, 128x256, 256x256 and 128x128 by eight waves with K steps of 64, operands loaded straight
+    and 128x128 with K steps of 64; 128x128, 128x256, 256x256, and 128x128 and 64x128 by eight waves with K steps of 64, operands loaded straight
     into LDS) on ragged
     problems: m, n and k leave partial tiles and a partial last K step; k = 8 is a single, mostly empty step;
     k = 1000 runs the load pipeline through many steps and ends on a partial one."""

@@ -253,7 +253,7 @@ inline bool sddmm_dense_fits(int dtype, const SddmmParams& p) {
 inline size_t sddmm_dense_bytes(const SddmmParams& p) { return (size_t)p.m * p.n * 2; }
 
 // Time model fitted on MI355X (fp16).  Dense product per batch entry: three launches, the GEMM at
-// 1000 TFLOP/s or, with few tiles, 0.28 us per K step of 32 per round of 512 tiles of 128 x 128,
+// 1000 TFLOP/s or, with few tiles, 0.23 us per K step of 32 per round of 512 tiles of 128 x 128,
 // m * n * 2 bytes written and nnz entries picked at 4 TB/s.  Gather kernel: nnz * k * 2 bytes at
 // 15 TB/s (16 heads of 4096 x 4096 at 93 % sparsity, k = 64: 125 us; 2048 x 1024 at 80 %, k = 2048:
 // 117 us), and with a k beyond the register-resident fragments no less than one wave's chain of
@@ -264,7 +264,7 @@ inline size_t sddmm_dense_bytes(const SddmmParams& p) { return (size_t)p.m * p.n
 inline bool sddmm_dense_wins(const SddmmParams& p) {
   const double flops = 2.0 * p.m * p.n * p.k;
   const double tiles = (double)ceil_div(p.m, 128) * ceil_div(p.n, 128);
-  const double product = std::max(flops / 1000e12, std::ceil(tiles / 512.0) * (p.k / 32.0) * 0.28e-6);
+  const double product = std::max(flops / 1000e12, std::ceil(tiles / 512.0) * (p.k / 32.0) * 0.23e-6);
   const double dense = p.batch * (16e-6 + product + ((double)p.m * p.n * 2 + (double)p.nnz * 8) / 4e12);
   const double row_nnz = (double)p.nnz / p.m;
   const double chain = p.k > 256 ? std::ceil(row_nnz / (row_nnz >= 64.0 ? 16.0 : 4.0)) * (p.k / 128.0) * 0.12e-6 : 0.0;

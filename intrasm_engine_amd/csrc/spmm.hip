@@ -450,8 +450,8 @@ inline size_t dense_path_bytes(const SpmmParams& p) { return (size_t)p.m * p.k *
 
 // Whether the dense-form path is the faster one, from a time model fitted on MI355X (fp16):
 //   dense form + GEMM: two launches (8 us), m * k * 2 bytes written at 4 TB/s, the product at
-//     1000 TFLOP/s or, when the tiles are few, one round of 128 x 128 tiles per 512 tiles at 0.28 us
-//     per K step of 32 (4096^2, n <= 512: 47-50 us whatever the sparsity; 1024^2, n = 2048: 21 us);
+//     1000 TFLOP/s or, when the tiles are few, one round of 128 x 128 tiles per 512 tiles at 0.23 us
+//     per K step of 32 (4096^2, n <= 512: 40-45 us whatever the sparsity; 1024^2, n = 2048: 21 us);
 //   matrix-core SpMM kernels: 720 dense-equivalent TFLOP/s (2:4 4096^2, n = 8192: 0.40 against 0.27 ms
 //     for the dense form; 80 % 11008 x 4096: 0.93 / 0.69; 90 %, n = 2048: 0.27 / 0.23);
 //   gather kernels: nnz * n * 2 bytes through the L2 -> CU path at 26 TB/s (4096^2 at 70 %, n = 256:
@@ -465,7 +465,7 @@ inline bool dense_path_wins(const SpmmParams& p, int batch, int matrix_core_kind
   const double cells = (double)p.m * p.k, flops = 2.0 * cells * p.n * batch;
   const double out_bytes = (double)p.m * p.n * batch * 2;
   const double tiles = (double)ceil_div(p.m, 128) * ceil_div(p.n, 128) * batch;
-  const double product = std::max({flops / 1000e12, std::ceil(tiles / 512.0) * (p.k / 32.0) * 0.28e-6, out_bytes / 3e12});
+  const double product = std::max({flops / 1000e12, std::ceil(tiles / 512.0) * (p.k / 32.0) * 0.23e-6, out_bytes / 3e12});
   const double dense_form = 8e-6 + cells * 2 / 4e12 + product;
   double other;
   if (few_columns) other = 8e-6 + out_bytes / 4.5e12 + (double)p.nnz * batch * ceil_div(p.n, 512) * 10.0 / (256 * 2.1e9);

@@ -18,6 +18,7 @@ MFMA GEMM and the sparse+dense co-run of config 4 (serialized / two-branch graph
 from __future__ import annotations
 
 import argparse
+import contextlib
 import json
 import os
 import statistics
@@ -353,6 +354,18 @@ def run_extras(torch, ops, dev, W, IL, mats, dens, csr_dev, time_cell, variant_o
         "dense_equivalent_TFLOPs": round(3 * 2.0 * w4g.m * w4g.k * 2048 / us_step / 1e6, 1)}
     del gy, xx, riw_, row_, ciw_, w4g, vals_, info_, x2, g2
     log("[bench] SDDMM done")
+
+    # ---- where the HBM roof binds: two points of the reference's xformers-style SpMM sweep (fp32, per-batch values;
+    # a sparse M x K pattern with a small K times a dense K x M operand: the M x M output per batch entry is the traffic)
+    from intrasm_engine_amd.benchmarks import benchmark_spmm as xf
+    pts = {}
+    for label, cfg in (("swin_t_stage1_B96_M3136_K32_s0.9844", ((96, 3136, 32), 0.9844)),
+                       ("basic_B8_M4096_K32_s0.90", ((8, 4096, 32), 0.90))):
+        with contextlib.redirect_stdout(sys.stderr):     # (the sweep prints its own line; stdout carries only the JSON line)
+            r = xf.bench_spmm([cfg], repeats=4, check=False)[0]
+        pts[label] = {"us": round(r["us"], 1), "GBps": round(r["GBps"], 1), "hbm_frac": round(r["GBps"] / HBM_PEAK_GBPS, 4),
+                      "output_GB": round(cfg[0][0] * cfg[0][1] * cfg[0][1] * 4 / 1e9, 2)}
+    out["output_bound_sweep_points_fp32"] = pts
 
     # ---- config 4: fp16 SpMM 11008x4096 @90% x 4096x2048  ||  bf16 GEMM 4096x4096x2048
     w, x, ga, gb = W.config4()

@@ -55,10 +55,10 @@ int launch_ragged(const SpmmParams& p, int batch, int wpr, hipStream_t stream) {
 }
 
 // ---- few columns in A, wide output: the dense operand's tile lives in LDS ---------------------
-template <typename T, typename IT, int VEC, bool RAGGED>
-__global__ __launch_bounds__(kSmallKThreads) void spmm_smallk_kernel(SpmmParams p, int rows_per_wave) {
+template <typename T, typename IT, int VEC, bool RAGGED, int WAVES>
+__global__ __launch_bounds__(WAVES * kWave) void spmm_smallk_kernel(SpmmParams p, int rows_per_wave) {
   extern __shared__ __align__(16) unsigned char smem[];
-  spmm_smallk_block<T, IT, VEC, RAGGED>(p, rows_per_wave, blockIdx.x, blockIdx.y, blockIdx.z, smem);
+  spmm_smallk_block<T, IT, VEC, RAGGED, WAVES>(p, rows_per_wave, blockIdx.x, blockIdx.y, blockIdx.z, smem);
 }
 
 // full vectors at their natural alignment, or (ragged) any n at element alignment
@@ -79,13 +79,17 @@ bool smallk_fits(const SpmmParams& p) {
 // from 1.8 nonzeros per row the LDS gather wins (fp32, per-batch values: 192 x 784 x 784 outputs,
 // k = 32, 2 per row: 107 against 127 us; 8 x 4096 x 4096, k = 64, 6 per row: 126 / 172, 32 per row: 344 / 535);
 // almost empty rows are a plain write, which the row kernel does at 6 TB/s with streaming stores
-// (96 x 3136 x 3136, 0.5 per row: 627 against 711), and k = 128 leaves one workgroup per CU (6 per row: 197 / 176).
+// (96 x 3136 x 3136, 0.5 per row: 627 against 711).
 template <typename T>
 bool smallk_wanted(const SpmmParams& p, int batch) {
   (void)batch;
   // (rows that are no multiple of the vector: from 2.5 per row -- 384 x 785 x 785, k = 64: 3.2 per row 377 -> 322 us,
   // 1.9 per row 290 -> 313)
-  return smallk_fits<T>(p) && p.k <= 64 && p.m >= 8 * p.k && (double)p.nnz >= (smallk_aligned<T>(p) ? 1.8 : 2.5) * p.m;
+  // k = 65 .. 128 (one workgroup of 16 wavefronts per CU): from 4 per row and 32 k rows -- 8 x 4096 x 4096, k = 128:
+  // 6.4 per row 166 -> 137 us, 1.3 per row 102 -> 120.
+  if (!smallk_fits<T>(p)) return false;
+  if (p.k > 64) return p.m >= 32 * p.k && (double)p.nnz >= 4.0 * p.m;
+  return p.m >= 8 * p.k && (double)p.nnz >= (smallk_aligned<T>(p) ? 1.8 : 2.5) * p.m;
 }
 
 template <typename T, typename IT>
@@ -94,11 +98,13 @@ int launch_smallk(const SpmmParams& p, int batch, hipStream_t stream) {
   // rows per wavefront: enough for the tile load (k KB per workgroup) to be a fraction of the output
   // (8 * rows KB), as long as that leaves every CU several workgroups
   const long long tiles = (long long)ceil_div(p.n, kWave * kMax) * batch;
+  const int waves = smallk_waves(p.k);
   int rows = std::min(64, std::max(16, p.k / 2));
-  while (rows > 4 && (long long)ceil_div(p.m, kSmallKWaves * rows) * tiles < 1024) rows >>= 1;
+  while (rows > 4 && (long long)ceil_div(p.m, waves * rows) * tiles < 1024) rows >>= 1;
   const int lds = p.k * kWave * 16;
   const bool ragged = !smallk_aligned<T>(p);
-  auto kern = ragged ? spmm_smallk_kernel<T, IT, kMax, true> : spmm_smallk_kernel<T, IT, kMax, false>;
+  auto kern = waves == 8 ? (ragged ? spmm_smallk_kernel<T, IT, kMax, true, 8> : spmm_smallk_kernel<T, IT, kMax, false, 8>)
+                         : (ragged ? spmm_smallk_kernel<T, IT, kMax, true, 16> : spmm_smallk_kernel<T, IT, kMax, false, 16>);
   if (lds > 64 * 1024) {
     static thread_local bool raised[2] = {false, false};  // per instantiation and alignment variant
     if (!raised[ragged]) {
@@ -109,8 +115,8 @@ int launch_smallk(const SpmmParams& p, int batch, hipStream_t stream) {
       raised[ragged] = true;
     }
   }
-  dim3 grid(ceil_div(p.m, kSmallKWaves * rows), ceil_div(p.n, kWave * kMax), batch);
-  hipLaunchKernelGGL(kern, grid, dim3(kSmallKThreads), lds, stream, p, rows);
+  dim3 grid(ceil_div(p.m, waves * rows), ceil_div(p.n, kWave * kMax), batch);
+  hipLaunchKernelGGL(kern, grid, dim3(waves * kWave), lds, stream, p, rows);
   return check_hip(hipGetLastError(), "spmm (few columns) launch");
 }
 

@@ -6,7 +6,7 @@
 // The row kernel spends a wavefront per (row, 64 * VEC columns): three dependent memory latencies
 // (row offsets -> column indices / values -> dense row) to write one kilobyte, and every nonzero
 // gathers its dense row segment from L2 although all rows of A share the same k dense rows.
-// Here a workgroup of 8 wavefronts owns one tile of 64 * VEC columns, one batch entry and a long
+// Here a workgroup of 8 (k <= 64) or 16 wavefronts owns one tile of 64 * VEC columns, one batch entry and a long
 // run of consecutive rows:
 //   * the k x (64 * VEC) tile of the dense operand is loaded into LDS once (k KB), lane i's
 //     vector of every dense row at [row][i]: the layout the gather reads;
@@ -27,10 +27,11 @@
 namespace iex {
 
 constexpr int kSmallKMax = 128;   // dense rows (KB of LDS) a tile may have
-constexpr int kSmallKWaves = 8;
-constexpr int kSmallKThreads = kSmallKWaves * kWave;
+// 8 wavefronts per workgroup up to 64 dense rows (two workgroups per CU), 16 beyond (the 65-128 KB tile
+// leaves room for one workgroup per CU only, which then brings the wavefronts)
+constexpr int smallk_waves(int k) { return k <= 64 ? 8 : 16; }
 
-template <typename T, typename IT, int VEC, bool RAGGED = false>
+template <typename T, typename IT, int VEC, bool RAGGED = false, int WAVES = 8>
 __device__ __forceinline__ void spmm_smallk_block(const SpmmParams& p, int rows_per_wave, int bx, int by, int bz,
                                                   unsigned char* smem) {
   typedef vec_t<T, VEC> V;
@@ -42,12 +43,12 @@ __device__ __forceinline__ void spmm_smallk_block(const SpmmParams& p, int rows_
   const bool lane_live = col0 < p.n;
   const int shift = (RAGGED && lane_live && col0 + VEC > p.n) ? col0 + VEC - p.n : 0;
   const T* __restrict__ dense = static_cast<const T*>(p.dense) + (size_t)z * p.k * p.n + min(col0 - shift, p.n - VEC);
-  for (int kr = wave; kr < p.k; kr += kSmallKWaves) tile[kr * kWave + lane] = load_vec<T, VEC, !RAGGED>(dense + (size_t)kr * p.n);
+  for (int kr = wave; kr < p.k; kr += WAVES) tile[kr * kWave + lane] = load_vec<T, VEC, !RAGGED>(dense + (size_t)kr * p.n);
   __syncthreads();
 
   const T* __restrict__ values = static_cast<const T*>(p.values) + (p.per_batch_values ? (size_t)z * p.nnz : (size_t)0);
   const IT* __restrict__ cols = static_cast<const IT*>(p.cols);
-  const int r_begin = min(p.m, (bx * kSmallKWaves + wave) * rows_per_wave);
+  const int r_begin = min(p.m, (bx * WAVES + wave) * rows_per_wave);
   const int r_end = min(p.m, r_begin + rows_per_wave);
   int cbase = -kWave;  // first nonzero held in (cc, vv); none yet
   int cc = 0;

@@ -206,7 +206,8 @@ int iex_gemm(int dtype, int trans_b, int M, int N, int K, const void* A, const v
  * (as iex_gemm: gemm_batch entries, element strides stride_*) and row blocks of the fp16 CSR
  * SpMM (as iex_spmm_ex with dtype IEX_F16, batch 1, no flags).  interleave == 0: the GEMM
  * workgroups come first; interleave == g > 0: they are spread through the grid in groups of
- * g.  Both results are identical to the separate launches.  No counterpart in the reference
+ * g, each group followed by an even share of the SpMM blocks (any g >= 1 is valid; a negative
+ * value is refused).  Both results are identical to the separate launches.  No counterpart in the reference
  * (the name survives only as the unused HORIZONTAL_GRAINED flag, tests/test_interleaving.py:441). */
 int iex_fused_spmm_gemm(int spmm_itype, int m, int k, int n, int nonzeros,
                         const int* row_indices, const void* values, const int* row_offsets,
@@ -214,6 +215,12 @@ int iex_fused_spmm_gemm(int spmm_itype, int m, int k, int n, int nonzeros,
                         int gemm_dtype, int trans_b, int M, int N, int K, const void* A,
                         const void* B, void* C, int gemm_batch, long long stride_a,
                         long long stride_b, long long stride_c, int interleave, void* stream);
+/* The workgroup-id -> role map of that launch, evaluated on the host: for a grid of gemm_blocks +
+ * spmm_blocks workgroups and group size `interleave`, workgroup `id` runs GEMM tile *index
+ * (*is_gemm = 1) or SpMM block *index (*is_gemm = 0).  Every tile and every block is the role of
+ * exactly one id for any counts and any interleave >= 0; the device code calls the same function.
+ * No launch, no GPU needed.  No counterpart in the reference. */
+int iex_fused_role(int gemm_blocks, int spmm_blocks, int interleave, int id, int* is_gemm, int* index);
 
 /* ------------------------------------------------------------ graph builder ---- */
 /* Opaque builder of ONE hipGraph from per-stream captures; mirrors

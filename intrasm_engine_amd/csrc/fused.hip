@@ -5,10 +5,10 @@
 //
 // Workgroup roles
 //   interleave == 0 : ids [0, G) run GEMM tiles, ids [G, G+S) run SpMM blocks;
-//   interleave == g : the G GEMM workgroups are spread through the id range in groups of g
-//                     consecutive ids (group q starts at id q*T/ceil(G/g)), so both kinds are
-//                     dispatched side by side from start to end while the tiles of a group
-//                     still share their operand panels in L2.
+//   interleave == g : the G GEMM workgroups are spread through the id range in ceil(G/g) groups of g
+//                     consecutive ids, each followed by its even share of the SpMM blocks, so both
+//                     kinds are dispatched side by side from start to end while the tiles of a
+//                     group still share their operand panels in L2.
 // The GEMM may be batched (tiles of all batch entries are enumerated).
 // Two kernels, picked by what the stand-alone SpMM of the same shape would run on:
 //   gather     256 threads; GEMM tiles of 128 x 128 beside row blocks of the row kernel (at most 4
@@ -36,24 +36,33 @@ constexpr int kFusedWM = 2, kFusedWN = 2;
 // missing waves by keeping four times as many gathers in flight per wave.
 constexpr int kFusedWin = 32;
 
-// Role of workgroup b: GEMM tile `idx` or SpMM block `idx`.
-__device__ __forceinline__ void fused_role(const FusedParams& p, int b, bool& is_gemm, int& idx) {
-  const long long total = (long long)p.gemm_blocks + p.spmm_blocks;
-  if (p.interleave > 0) {
-    // GEMM tiles in groups of `interleave` consecutive ids; group q starts at id q*total/groups
-    const int gsz = p.interleave;
-    const long long groups = (p.gemm_blocks + gsz - 1) / gsz;
-    long long q = ((long long)b * groups) / total;
-    if ((q + 1) * total / groups <= b) ++q;
-    const long long start = q * total / groups;
-    const int in_group = min(gsz, p.gemm_blocks - (int)q * gsz);
-    const int off = b - (int)start;
-    is_gemm = off < in_group;
-    idx = is_gemm ? (int)q * gsz + off : b - ((int)q * gsz + in_group);
-  } else {
-    is_gemm = b < p.gemm_blocks;
-    idx = is_gemm ? b : b - p.gemm_blocks;
+// Role of workgroup b: GEMM tile `idx` or SpMM block `idx`.  A bijection between the ids [0, G + S) and
+// the G tiles plus the S blocks for every G >= 0, S >= 0 and group size g >= 0:
+//   g == 0: ids [0, G) are the tiles, [G, G + S) the blocks;
+//   g >= 1: Q = ceil(G / g) groups, each "its tiles, then its share of the blocks"; group q holds the
+//           tiles [q g, min(G, (q + 1) g)) and floor(S / Q) blocks, one more in the first S mod Q groups
+//           (the last group, the only one that can be short of tiles, never gets the extra block).
+// Host and device: the host side is exported as iex_fused_role for the CPU test of this mapping.
+__host__ __device__ inline void fused_role_of(int gemm_blocks, int spmm_blocks, int interleave, int b, bool& is_gemm, int& idx) {
+  const int G = gemm_blocks, S = spmm_blocks, g = interleave;
+  if (g <= 0 || G == 0) {
+    is_gemm = b < G;
+    idx = is_gemm ? b : b - G;
+    return;
   }
+  const int Q = (G + g - 1) / g;          // groups
+  const int s0 = S / Q, r = S % Q;        // blocks per group, groups with one more
+  const long long u1 = (long long)g + s0 + 1, u0 = (long long)g + s0;
+  const int q = (b < r * u1) ? (int)(b / u1) : r + (int)((b - r * u1) / u0);
+  const long long blocks_before = (long long)q * s0 + (q < r ? q : r);
+  const int off = (int)(b - ((long long)q * g + blocks_before));
+  const int tiles_here = (G - q * g < g) ? G - q * g : g;
+  is_gemm = off < tiles_here;
+  idx = is_gemm ? q * g + off : (int)(blocks_before + off - tiles_here);
+}
+
+__device__ __forceinline__ void fused_role(const FusedParams& p, int b, bool& is_gemm, int& idx) {
+  fused_role_of(p.gemm_blocks, p.spmm_blocks, p.interleave, b, is_gemm, idx);
 }
 
 template <bool BF16, bool TRANS_B, typename IT, int VEC, int LPG, int WPR>
@@ -190,6 +199,20 @@ int launch_gemm_kind(const FusedParams& p, SpmmShape vec, bool bf16, bool trans_
 }  // namespace
 }  // namespace iex
 
+extern "C" int iex_fused_role(int gemm_blocks, int spmm_blocks, int interleave, int id, int* is_gemm, int* index) {
+  using namespace iex;
+  IEX_REQUIRE(gemm_blocks >= 0 && spmm_blocks >= 0 && interleave >= 0 && is_gemm && index, IEX_ERR_BAD_ARGUMENT,
+              "fused role: negative count or null pointer");
+  IEX_REQUIRE(id >= 0 && (long long)id < (long long)gemm_blocks + spmm_blocks, IEX_ERR_BAD_ARGUMENT,
+              "fused role: id %d outside the grid of %lld workgroups", id, (long long)gemm_blocks + spmm_blocks);
+  bool ig;
+  int idx;
+  fused_role_of(gemm_blocks, spmm_blocks, interleave, id, ig, idx);
+  *is_gemm = ig ? 1 : 0;
+  *index = idx;
+  return 0;
+}
+
 extern "C" int iex_fused_spmm_gemm(int spmm_itype, int m, int k, int n, int nonzeros, const int* row_indices,
                                    const void* values, const int* row_offsets, const void* column_indices,
                                    const void* dense, void* spmm_out, int gemm_dtype, int trans_b, int M, int N, int K,
@@ -198,6 +221,7 @@ extern "C" int iex_fused_spmm_gemm(int spmm_itype, int m, int k, int n, int nonz
   using namespace iex;
   IEX_REQUIRE(m > 0 && k > 0 && n > 0 && nonzeros >= 0, IEX_ERR_BAD_ARGUMENT, "fused: SpMM dimensions must be positive");
   IEX_REQUIRE(M > 0 && N > 0 && K > 0 && gemm_batch > 0, IEX_ERR_BAD_ARGUMENT, "fused: GEMM dimensions must be positive");
+  IEX_REQUIRE(interleave >= 0, IEX_ERR_BAD_ARGUMENT, "fused: interleave must be 0 (GEMM workgroups first) or a group size >= 1 (got %d)", interleave);
   IEX_REQUIRE(stride_a % 8 == 0 && stride_b % 8 == 0, IEX_ERR_UNSUPPORTED, "fused: GEMM batch strides must be multiples of 8");
   IEX_REQUIRE(row_indices && row_offsets && dense && spmm_out && A && B && C, IEX_ERR_BAD_ARGUMENT,
               "fused: null pointer argument");

@@ -50,7 +50,9 @@ __global__ __launch_bounds__(kDenseThreads) void csr_to_dense_kernel(int m, int 
       int taken = 0;
 #pragma unroll
       for (int u = 0; u < 4; ++u) {
-        const bool mine = pos + u * kWave + lane < end && c[u] < len;  // (c >= 0: earlier segments took what lies before c0)
+        // (canonical CSR: c >= 0, earlier segments took what lies before c0; the test keeps a row whose
+        // columns do not ascend inside the wavefront's slice of LDS -- its result is then undefined, not a fault)
+        const bool mine = pos + u * kWave + lane < end && c[u] < len && c[u] >= 0;
         if (mine) srow[c[u]] = v[u];
         taken += __popcll(__ballot(mine));
       }

@@ -77,14 +77,14 @@ def spmm_kernel_choices(dtype: torch.dtype, n: int, k: int | None = None, m: int
 
 
 def _spmm(b3, row_indices, values, row_offsets, column_indices, m, kernel="auto"):
-    with _ops.kernel_params(spmm=SPMM_KERNELS[kernel]):
+    with _ops.kernel_params(spmm=SPMM_KERNELS[kernel] or None):   # "auto" keeps an enclosing block's choice
         if values.dtype == torch.float32:
             return ops.spmm_sputnik_reuse_weight(b3, row_indices, values, row_offsets, column_indices, m)
         return ops.spmm_sputnik_reuse_weight_half(b3, row_indices, values, row_offsets, column_indices, m)
 
 
 def _sddmm(a3, b3, row_indices, row_offsets, column_indices, wpr=0):
-    with _ops.kernel_params(sddmm={"force_wpr": wpr}):
+    with _ops.kernel_params(sddmm={"force_wpr": wpr} if wpr else None):
         if a3.dtype == torch.float32:
             return ops.sddmm_sputnik_atomic_upd_weight(a3, b3, row_indices, row_offsets, column_indices)
         return ops.sddmm_sputnik_half(a3, b3, row_indices, row_offsets, column_indices)[0]

@@ -21,7 +21,7 @@ GEMM_TILES: dict[str, int] = {"auto": 0, "128x128": 5, "128x256": 6, "256x256": 
 
 
 def _gemm(a, b, trans_b, tile="auto"):
-    with _ops.kernel_params(gemm={"tile": GEMM_TILES[tile]}):
+    with _ops.kernel_params(gemm={"tile": GEMM_TILES[tile]} if GEMM_TILES[tile] else None):
         return ops.gemm_mfma(a, b, trans_b)
 
 

@@ -42,7 +42,8 @@ def kernel_params(*, spmm: dict | None = None, sddmm: dict | None = None, gemm: 
     bits of ``iex_spmm_ex``), ``sddmm`` = force_wpr / force_variant, ``gemm`` = tile (the shape code of
     ``iex_gemm``: 5 = 128x128, 6 = 128x256, 7 = 256x256 tiles, 8 = 128x128 and 9 = 64x128 by eight waves with K steps of 64; 1..4 = the
     register-staged kernels).
-    Without a block, or for a key left out, the library chooses.  A kernel family that cannot
+    Without a block, or for a key left out, the library chooses; a category left out (None) keeps
+    what an enclosing block set for it.  A kernel family that cannot
     take the operands at hand (a matrix-core family for an n that is not a multiple of 8, say)
     falls back to a gather kernel, as the C entry points document: results stay correct, the
     timing is then that of the fallback."""
@@ -51,7 +52,11 @@ def kernel_params(*, spmm: dict | None = None, sddmm: dict | None = None, gemm: 
         if unknown:
             raise TypeError(f"unknown {name} kernel parameters: {sorted(unknown)}")
     before = {k: getattr(_TUNING, k, None) for k in ("spmm", "sddmm", "gemm")}
-    _TUNING.spmm, _TUNING.sddmm, _TUNING.gemm = spmm or None, sddmm or None, gemm or None
+    # only the categories that were passed are replaced: a nested block for one category keeps
+    # what an outer block set for the others (an empty dict hands that category back to the library)
+    for name, given in (("spmm", spmm), ("sddmm", sddmm), ("gemm", gemm)):
+        if given is not None:
+            setattr(_TUNING, name, given or None)
     try:
         yield
     finally:

@@ -1,15 +1,36 @@
 """The sparse decoder layer of configuration 5 at a small shape: the operator chain against
 a dense fp32 PyTorch reference, and the three execution variants against each other."""
+import math
+
 import numpy as np
 import pytest
 import torch
 
 from intrasm_engine_amd import workloads as W
-from intrasm_engine_amd.decoder_layer import SparseDecoderLayer, reference_forward
+from intrasm_engine_amd.decoder_layer import SparseDecoderLayer
 from intrasm_engine_amd.pytorch.utils import sparse_to_dense
 
 pytestmark = pytest.mark.gpu
 HIDDEN, HEADS, MLP, SEQS, L = 256, 4, 512, 4, 64
+
+
+def reference_forward(weights_dense: dict, x: torch.Tensor, heads: int, seqs: int) -> torch.Tensor:
+    """The same layer with dense fp32 matrices and plain PyTorch (for tests at small sizes).
+    weights_dense: name -> (m, k) fp32 tensor; x: (hidden, tokens) fp32."""
+    hidden = x.shape[0]
+    hd = hidden // heads
+    L = x.shape[1] // seqs
+
+    def split(t):
+        return t.view(heads, hd, seqs, L).permute(2, 0, 3, 1).reshape(seqs * heads, L, hd)
+
+    q, k, v = (weights_dense[n] @ x for n in ("q", "k", "v"))
+    Q, K, V = split(q), split(k), split(v)
+    P = torch.softmax((Q @ K.transpose(1, 2)) / math.sqrt(hd), dim=-1)
+    O = (P @ V).view(seqs, heads, L, hd).permute(1, 3, 0, 2).reshape(hidden, seqs * L)
+    h = x + weights_dense["o"] @ O
+    act = torch.nn.functional.silu(weights_dense["gate"] @ h) * (weights_dense["up"] @ h)
+    return h + weights_dense["down"] @ act
 
 
 def _layer(dev):

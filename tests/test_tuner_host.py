@@ -142,3 +142,19 @@ def test_search_spaces_of_the_path():
         pair.check_params_sanity({"space_2.gemm_tile": "row"})
     with pytest.raises(ValueError, match="third operator"):
         pair.check_params_sanity({"space_3.gemm_tile": "auto"})
+
+
+def test_nested_kernel_params_keep_the_other_categories():
+    """A block for one category leaves what an enclosing block set for the others; an "auto" choice inside
+    the autograd functions does not erase a caller's choice."""
+    from intrasm_engine_amd.pytorch import ops as pyops
+    seen = lambda: tuple(getattr(pyops._TUNING, k, None) for k in ("spmm", "sddmm", "gemm"))
+    with pyops.kernel_params(spmm={"force_variant": 1}, gemm={"tile": 6}):
+        with pyops.kernel_params(sddmm={"force_wpr": 4}):
+            assert seen() == ({"force_variant": 1}, {"force_wpr": 4}, {"tile": 6})
+            with pyops.kernel_params(spmm=None, gemm={"tile": 5}):
+                assert seen() == ({"force_variant": 1}, {"force_wpr": 4}, {"tile": 5})
+            with pyops.kernel_params(spmm={}):               # an empty dict hands the category back to the library
+                assert seen() == (None, {"force_wpr": 4}, {"tile": 6})
+        assert seen() == ({"force_variant": 1}, None, {"tile": 6})
+    assert seen() == (None, None, None)

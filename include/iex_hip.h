@@ -115,6 +115,24 @@ int iex_spmm_ws(int dtype, int itype, int flags, int m, int k, int n, int nonzer
 size_t iex_spmm_workspace_bytes(int dtype, int itype, int flags, int m, int k, int n,
                                 int nonzeros, int batch);
 
+/* iex_spmm_ws for callers that cannot allocate device memory (code under hipGraph capture, tight serving
+ * loops, harnesses that forbid hipMalloc): same arguments as iex_spmm_ex, same results as iex_spmm_ws with a
+ * workspace of the size iex_spmm_workspace_bytes asks for, but the workspace is an array of
+ * IEX_SPMM_STATIC_SCRATCH_BYTES that the library itself holds on every GPU it runs on, from the moment the
+ * library is loaded there until the process ends.  The call allocates and frees nothing (the first call on a
+ * device looks the array's address up once).  A call whose workspace would exceed the array fails with
+ * IEX_ERR_TOO_LARGE before anything is launched; a call that would not use a workspace runs as iex_spmm_ex.
+ * All calls on one GPU share that GPU's array: two calls whose work may overlap in time (different streams,
+ * different threads) race on it -- order them, or give one of them iex_spmm_ws with memory of its own.  The
+ * array keeps the previous call's contents; every kernel that reads it writes what it reads first.
+ * No counterpart in the reference (its launchers take no workspace, csrc/extensions.h:28-30). */
+#define IEX_SPMM_STATIC_SCRATCH_BYTES ((size_t)96 << 20)
+int iex_spmm_static(int dtype, int itype, int flags, int m, int k, int n, int nonzeros,
+                    const int* row_indices, const void* values, const int* row_offsets,
+                    const void* column_indices, const void* dense, const float* bias,
+                    void* out, void* stream, int batch);
+size_t iex_spmm_static_scratch_bytes(void);
+
 /* Drop-ins for the three launchers the reference declares in csrc/extensions.h:28-30.
  * CudaSpmm2: fp32, per-batch values (batch, nnz), accumulates into `out`
  *            (spmm_sputnik_atomic, sputnik_kernels.cpp:170-172);

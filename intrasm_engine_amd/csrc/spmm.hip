@@ -2,6 +2,7 @@
 // the C entry points.  The device code is in spmm_device.cuh.
 #include <algorithm>
 #include <cmath>
+#include <mutex>
 #include "spmm_lds_device.cuh"
 #include "spmm_mfma2_device.cuh"
 #include "spmm_mfma3_device.cuh"
@@ -631,9 +632,58 @@ size_t spmm_workspace_bytes(int dtype, int itype, int flags, int m, int k, int n
   return dense_path_bytes(p);
 }
 
+// ---- the library's own scratch memory, for callers that cannot allocate ---------------------------------
+// One array per GPU, placed when the code object is loaded on it and held until the process ends.  In host
+// code the array's name is only a handle for hipGetSymbolAddress: every use of the memory below goes through
+// the per-device pointer that call returned.
+constexpr size_t kStaticScratchBytes = IEX_SPMM_STATIC_SCRATCH_BYTES;
+static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
+
+namespace {
+constexpr int kMaxDevices = 64;
+std::mutex scratch_mutex;
+void* scratch_ptr[kMaxDevices] = {};   // per device: each GPU holds its own copy of the array at its own address
+
+// The calling thread's current device's copy of `scratch` (looked up once per device, with that device current).
+int static_scratch(void** ptr) {
+  int device = -1;
+  if (int rc = check_hip(hipGetDevice(&device), "hipGetDevice")) return rc;
+  IEX_REQUIRE(device >= 0 && device < kMaxDevices, IEX_ERR_UNSUPPORTED, "spmm: device ordinal %d beyond %d", device, kMaxDevices - 1);
+  std::lock_guard<std::mutex> lock(scratch_mutex);
+  if (!scratch_ptr[device]) {
+    void* p = nullptr;
+    if (int rc = check_hip(hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)), "hipGetSymbolAddress(scratch)")) return rc;
+    IEX_REQUIRE(p != nullptr && aligned(p, 256), IEX_ERR_STATE, "spmm: the library's scratch array has no usable device address");
+    scratch_ptr[device] = p;
+  }
+  *ptr = scratch_ptr[device];
+  return 0;
+}
+}  // namespace
+
 }  // namespace iex
 
 extern "C" {
+
+int iex_spmm_static(int dtype, int itype, int flags, int m, int k, int n, int nonzeros,
+                    const int* row_indices, const void* values, const int* row_offsets,
+                    const void* column_indices, const void* dense, const float* bias, void* out,
+                    void* stream, int batch) {
+  using namespace iex;
+  const size_t need = spmm_workspace_bytes(dtype, itype, flags, m, k, n, nonzeros, batch);
+  if (need == 0)  // a call that would not touch a workspace runs as iex_spmm_ex does (a forced family 7 fails there)
+    return spmm_dispatch(dtype, itype, flags, m, k, n, nonzeros, row_indices, values, row_offsets, column_indices, dense,
+                         bias, out, stream, batch, nullptr, 0);
+  IEX_REQUIRE(need <= kStaticScratchBytes, IEX_ERR_TOO_LARGE,
+              "spmm (static scratch): this call needs %zu bytes of scratch memory, the library's array holds %zu "
+              "(pass a workspace of your own to iex_spmm_ws, or call iex_spmm_ex)", need, kStaticScratchBytes);
+  void* ws = nullptr;
+  if (int rc = static_scratch(&ws)) return rc;
+  return spmm_dispatch(dtype, itype, flags, m, k, n, nonzeros, row_indices, values, row_offsets, column_indices, dense,
+                       bias, out, stream, batch, ws, kStaticScratchBytes);
+}
+
+size_t iex_spmm_static_scratch_bytes(void) { return iex::kStaticScratchBytes; }
 
 int iex_spmm_ex(int dtype, int itype, int flags, int m, int k, int n, int nonzeros,
                 const int* row_indices, const void* values, const int* row_offsets,

@@ -66,8 +66,13 @@ int iex_copy_bytes(void* dst, const void* src, size_t nbytes, void* stream);
  * form of A in the caller's workspace, then the dense GEMM (iex_spmm_ws only), 8 = A with at most
  * 128 columns and an output at least one tile (64 128-bit vectors) wide: the dense operand's tile
  * in LDS, rows streamed in natural order (bit-equal to family 1 with one wavefront per row; fails
- * on other shapes).  0 = choose.
- * Families 2-6 rely on strictly ascending column indices inside a row (canonical CSR, what
+ * on other shapes), 9 = fp32 with int32 indices only, on request only: a slice of the dense operand resident in
+ * LDS (direct-to-LDS loads, double-buffered stages), k split over workgroups, fp32 partial sums added by a second
+ * kernel in slice order (deterministic); needs n a multiple of 4, 16-byte aligned dense operands, k <= 262144 and,
+ * for more than one slice, iex_spmm_ws with the workspace iex_spmm_workspace_bytes reports (bits 20..23: slices,
+ * 0 = choose; bits 24..27 = 2: workgroups of 16 wavefronts and 128 rows instead of 8 and 64); fails on other
+ * shapes.  0 = choose.
+ * Families 2-6 and 9 rely on strictly ascending column indices inside a row (canonical CSR, what
  * dense_to_sparse produces); family 1 accepts any order and duplicates -- force it for such
  * input.  Families 3-6 multiply explicit zeros with the dense operand, so a non-finite entry
  * in a row of `dense` that no nonzero references still reaches the output (0 * inf = NaN).

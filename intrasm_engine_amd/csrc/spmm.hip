@@ -9,6 +9,7 @@
 #include "spmm_mfma_f32_device.cuh"
 #include "spmm_dense_device.cuh"
 #include "spmm_smallk_device.cuh"
+#include "spmm_ksplit_device.cuh"
 
 namespace iex {
 namespace {
@@ -318,6 +319,93 @@ inline int launch_mfma_f32(const SpmmParams& p, int batch, int arrangement, int 
   return fail(IEX_ERR_BAD_ARGUMENT, "spmm: arrangement of the fp32 matrix-core variant must be 1, 2, 4, 5 or 6 (got %d)", arrangement);
 }
 
+// ---- slice of the dense operand resident in LDS, k split over workgroups ------------------------------
+template <typename T, typename IT, int VEC, int RPW, int WAVES, int KB>
+__global__ __launch_bounds__(WAVES * kWave, WAVES == 8 ? 2 : 1) void spmm_ksplit_kernel(KsplitParams q) {
+  extern __shared__ __align__(16) unsigned char smem[];
+  spmm_ksplit_block<T, IT, VEC, RPW, WAVES, KB>(q, blockIdx.x / q.slices, blockIdx.x % q.slices, blockIdx.y, blockIdx.z, smem);
+}
+
+struct KsplitPlan {
+  int vec = 0;        // elements per lane: the tile is 64 * vec columns (0 = the shape does not fit)
+  int waves = 8;      // wavefronts per workgroup: 8 (two workgroups per CU) or 16 (one, stages twice as long)
+  int slices = 1;     // k slices
+  int slice_rows = 0; // dense rows per slice
+  size_t partial_bytes = 0;
+};
+
+constexpr int kKsplitRpw = 8;
+
+template <typename T>
+constexpr int ksplit_kb(int vec, int waves) {
+  // 32 KB stages (64 KB with 16 wavefronts), at most 64 dense rows (one window of nonzeros per row and stage)
+  const int rb = kWave * vec * (int)sizeof(T);
+  const int kb = (waves == 16 ? 65536 : 32768) / rb;
+  return kb > 64 ? 64 : kb;
+}
+
+// Tile width, slices and partial-sum bytes for a shape; plan.vec == 0 when the kernel cannot take it.
+template <typename T>
+KsplitPlan ksplit_plan(const SpmmParams& p, int batch, int force_slices, int force_waves) {
+  KsplitPlan pl;
+  constexpr int kMax = 16 / (int)sizeof(T);
+  if (!(p.nnz > 0 && p.n >= kMax && p.n % kMax == 0 && p.k <= 262144 && aligned(p.dense, 16) && aligned(p.out, 16))) return pl;
+  int vec = kMax;
+  while (vec > kMax / 4 && kWave * (vec / 2) >= p.n) vec >>= 1;   // the narrowest tile that holds n
+  pl.vec = vec;
+  pl.waves = force_waves == 16 && vec == kMax ? 16 : 8;
+  const int kb = ksplit_kb<T>(vec, pl.waves);
+  const long long row_blocks = ceil_div(p.m, pl.waves * kKsplitRpw);
+  const long long cells = row_blocks * ceil_div(p.n, kWave * vec) * batch;
+  // two workgroups of 8 wavefronts (one of 16) per CU, and the slices a multiple of the 8 XCDs where that is
+  // possible: consecutive workgroup ids go to consecutive XCDs, so each L2 then holds one slice of the operand
+  const long long want = pl.waves == 16 ? 256 : 512;
+  int slices = force_slices > 0 ? force_slices : (int)std::min<long long>(16, std::max<long long>(1, (want + cells - 1) / cells));
+  if (force_slices == 0 && slices > 4 && slices < 8) slices = 8;
+  slices = std::min(slices, ceil_div(p.k, kb));
+  pl.slice_rows = ceil_div(ceil_div(p.k, slices), kb) * kb;
+  pl.slices = ceil_div(p.k, pl.slice_rows);
+  pl.partial_bytes = pl.slices > 1 ? (size_t)pl.slices * batch * p.m * p.n * sizeof(float) : 0;
+  return pl;
+}
+
+template <typename T, typename IT, int VEC, int WAVES>
+int launch_ksplit_one(const SpmmParams& p, int batch, const KsplitPlan& pl, float* partial, hipStream_t stream) {
+  constexpr int KB = ksplit_kb<T>(VEC, WAVES);
+  constexpr int lds = spmm_ksplit_lds_bytes<VEC, T, KB>();
+  KsplitParams q{p, ceil_div(p.m, WAVES * kKsplitRpw), pl.slices, pl.slice_rows, partial};
+  IEX_REQUIRE((long long)q.row_blocks * q.slices < (1ll << 31), IEX_ERR_TOO_LARGE, "spmm (k split): grid too large");
+  auto kernel = spmm_ksplit_kernel<T, IT, VEC, kKsplitRpw, WAVES, KB>;
+  if (lds >= 64 * 1024) {
+    static thread_local bool raised = false;   // per instantiation
+    if (!raised) {
+      if (int rc = check_hip(hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, lds),
+                             "hipFuncSetAttribute(LDS size)"))
+        return rc;
+      raised = true;
+    }
+  }
+  hipLaunchKernelGGL(kernel, dim3(q.row_blocks * q.slices, ceil_div(p.n, kWave * VEC), batch), dim3(WAVES * kWave), lds, stream, q);
+  if (int rc = check_hip(hipGetLastError(), "spmm (k split) launch")) return rc;
+  if (pl.slices > 1) {
+    const size_t quads = (size_t)batch * p.m * p.n / 4;
+    const int blocks = (int)std::min<size_t>((quads + 255) / 256, 256 * 16);
+    hipLaunchKernelGGL((spmm_ksplit_reduce_kernel<T>), dim3(blocks), dim3(256), 0, stream, p, partial, pl.slices, batch);
+    return check_hip(hipGetLastError(), "spmm (k split) reduction launch");
+  }
+  return 0;
+}
+
+template <typename T, typename IT>
+int launch_ksplit(const SpmmParams& p, int batch, const KsplitPlan& pl, void* ws, hipStream_t stream) {
+  constexpr int kMax = 16 / (int)sizeof(T);
+  float* partial = static_cast<float*>(ws);
+  if (pl.vec == kMax && pl.waves == 16) return launch_ksplit_one<T, IT, kMax, 16>(p, batch, pl, partial, stream);
+  if (pl.vec == kMax) return launch_ksplit_one<T, IT, kMax, 8>(p, batch, pl, partial, stream);
+  if (pl.vec == kMax / 2) return launch_ksplit_one<T, IT, kMax / 2, 8>(p, batch, pl, partial, stream);
+  return launch_ksplit_one<T, IT, kMax / 4, 8>(p, batch, pl, partial, stream);
+}
+
 struct Choice {
   int wpr = 0;      // wavefronts per row of the row kernel
   int variant = 0;  // 0 = choose, 1 = row kernel, 2 = LDS-staged kernel, 3 / 4 = matrix-core kernels (16-bit), 5 = (fp32)
@@ -507,6 +595,13 @@ int launch_typed(const SpmmParams& p, int batch, const Choice& ch, hipStream_t s
     return launch_smallk<T, IT>(p, batch, stream);
   }
   if constexpr (std::is_same<T, float>::value && std::is_same<IT, int>::value) {
+    if (ch.variant == 9) {
+      const KsplitPlan pl = ksplit_plan<T>(p, batch, ch.rpw, ch.nt == 2 ? 16 : 8);
+      IEX_REQUIRE(pl.vec > 0, IEX_ERR_UNSUPPORTED, "spmm: the k-split kernel needs n a multiple of the 128-bit vector, 16-byte aligned dense operands and k <= 262144");
+      IEX_REQUIRE(pl.partial_bytes == 0 || (ch.ws && aligned(ch.ws, 16) && ch.ws_bytes >= pl.partial_bytes), IEX_ERR_BAD_ARGUMENT,
+                  "spmm: the k-split kernel needs a 16-byte aligned workspace of %zu bytes for its partial sums (iex_spmm_ws)", pl.partial_bytes);
+      return launch_ksplit<T, IT>(p, batch, pl, ch.ws, stream);
+    }
     int windows = 0;
     if (const int arr = mfma_f32_variant<T, IT>(p, batch, ch, windows)) return launch_mfma_f32(p, batch, arr, windows, ch.lpg != 8, stream);  // (lanes-per-group code 8 = no role split, for tuning)
   }
@@ -616,10 +711,15 @@ int spmm_dispatch(int dtype, int itype, int flags, int m, int k, int n, int nonz
 // would not, whatever the workspace).  Pointers are taken to be 16-byte aligned.
 size_t spmm_workspace_bytes(int dtype, int itype, int flags, int m, int k, int n, int nonzeros, int batch) {
   if (m <= 0 || k <= 0 || n <= 0 || nonzeros <= 0 || batch <= 0) return 0;
-  if (!(dtype == IEX_F16 || dtype == IEX_BF16) || !(itype == IEX_I32 || itype == IEX_I16)) return 0;
   const int variant = (flags >> 16) & 0xf;
-  if (variant != 0 && variant != 7) return 0;
   void* const some_aligned = reinterpret_cast<void*>(size_t(256));
+  if (dtype == IEX_F32 && itype == IEX_I32) {
+    SpmmParams p{m, k, n, nonzeros, nullptr, nullptr, nullptr, nullptr, some_aligned, nullptr, some_aligned, 0, 0, 0};
+    if (variant == 9) return ksplit_plan<float>(p, batch, (flags >> 20) & 0xf, ((flags >> 24) & 0xf) == 2 ? 16 : 8).partial_bytes;
+    return 0;
+  }
+  if (!(dtype == IEX_F16 || dtype == IEX_BF16) || !(itype == IEX_I32 || itype == IEX_I16)) return 0;
+  if (variant != 0 && variant != 7) return 0;
   SpmmParams p{m, k, n, nonzeros, nullptr, nullptr, nullptr, nullptr, some_aligned, nullptr, some_aligned, 0, 0, 0};
   if (!dense_path_fits(2, p, (flags & IEX_SPMM_PER_BATCH_VALUES) != 0)) return 0;
   if (variant == 0) {

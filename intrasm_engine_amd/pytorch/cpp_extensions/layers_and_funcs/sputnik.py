@@ -54,6 +54,9 @@ SPMM_KERNELS: dict[str, dict] = {
     "mfma32_windows4": {"force_variant": 5, "force_nt": 4, "force_rpw": 4},
     "mfma32_windows8": {"force_variant": 5, "force_nt": 4, "force_rpw": 8},
     "mfma32_rows16": {"force_variant": 5, "force_nt": 6, "force_rpw": 4},
+    # fp32: a slice of the dense operand resident in LDS, k split over workgroups (the operator allocates the partial sums)
+    "ksplit_lds": {"force_variant": 9},
+    "ksplit_lds_16waves": {"force_variant": 9, "force_nt": 2},
 }
 
 
@@ -73,6 +76,7 @@ def spmm_kernel_choices(dtype: torch.dtype, n: int, k: int | None = None, m: int
             names.append("dense_form_gemm")
     if dtype == torch.float32 and n % 4 == 0:
         names += [k for k in SPMM_KERNELS if k.startswith("mfma32_")]
+        names += ["ksplit_lds", "ksplit_lds_16waves"]          # (the backward product has the same n)
     return names
 
 

@@ -108,7 +108,8 @@ def test_search_spaces_of_the_path():
     assert not any(k.startswith("mfma32") for k in half)
     assert not any(k.startswith("mfma") for k in spmm_kernel_choices(torch.float16, 100))    # n % 8 != 0
     single = spmm_kernel_choices(torch.float32, 64)
-    assert "mfma32_windows4" in single and not any(k.startswith(("mfma4", "mfma8")) for k in single)
+    assert "mfma32_windows4" in single and "ksplit_lds" in single and not any(k.startswith(("mfma4", "mfma8")) for k in single)
+    assert "ksplit_lds" not in half and "ksplit_lds" not in spmm_kernel_choices(torch.float32, 66)
     assert "few_columns" in spmm_kernel_choices(torch.float32, 256, 64, 128) and "few_columns" not in single
     assert set(half) | set(single) | {"few_columns"} == set(SPMM_KERNELS)
     for flags in SPMM_KERNELS.values():                       # every name maps to legal tuning keys

@@ -11,7 +11,9 @@ in HBM before the timed region; CSR construction is set-up work and is not timed
 
 One JSON line is printed.  ``value`` = algorithmic GB of one sweep / seconds per sweep.
 ``roofline`` describes the SpMM kernel instantiation that takes the most time in the
-sweep; ``cpu_baseline`` is the single-core C port of the same sweep timed on this host;
+sweep (its name is read from the library, its HBM traffic from the committed counter
+summary taken on that same kernel); ``cpu_baseline`` is torch.sparse CSR on the host cores
+over the same 15 cells (median of 5 per cell);
 ``extras`` holds the per-cell table, the fp16 sweep, SDDMM (configs 1 and 3), the bf16
 MFMA GEMM and the sparse+dense co-run of config 4 (serialized / two-branch graph / fused).
 """
@@ -34,15 +36,27 @@ HBM_PEAK_GBPS = 8000.0           # MI355X HBM3E
 MFMA_PEAK_TFLOPS_16BIT = 2500.0  # dense bf16 / fp16
 VALU_PEAK_TFLOPS_FP32 = 78.6     # vector fp32 FMA without packed math (the build disables v_pk_*_f32)
 CELL_REPEATS = 20                # launches of one cell inside its timing graph
-# HBM-side bytes per launch (L2 misses + write-backs), mean over the five sparsities a kernel serves in
-# the sweep, from two `rocprofv3 --pmc` runs (FETCH_SIZE, WRITE_SIZE) of `bench.py --pmc-probe`, each
-# scaled by the counter's reading for a plain 256 MiB copy (x2.000 and x1.000): see
-# profiles/spmm_fp32_config2_hbm_traffic_pmc.txt.  Counters cannot be read inside a timing run.
-MEASURED_TRAFFIC_MB = {   # (sparsity, n) -> MB per launch of the row kernel
-    (0.7, 64): 51.30, (0.7, 128): 61.56, (0.7, 256): 174.86, (0.8, 64): 37.78, (0.8, 128): 47.37, (0.8, 256): 134.22,
-    (0.9, 64): 24.31, (0.9, 128): 33.78, (0.9, 256): 83.51, (0.95, 64): 17.59, (0.95, 128): 27.04, (0.95, 256): 61.88,
-    (0.98, 64): 13.56, (0.98, 128): 23.01, (0.98, 256): 49.03,
-}
+TRAFFIC_PROFILE = os.path.join(ROOT, "profiles", "spmm_fp32_config2_hbm_traffic_pmc.txt")
+COLD_SCRATCH_BYTES = 512 << 20   # written between cold-cache samples (> the 256 MB last-level cache)
+
+
+def read_traffic_profile():
+    """HBM-side bytes per launch (L2 misses + write-backs) of every fp32 cell, from the committed summary of two
+    `rocprofv3 --pmc` runs (FETCH_SIZE, WRITE_SIZE) of `bench.py --pmc-probe`, each scaled by the counter's reading for
+    a plain 256 MiB copy.  Counters cannot be read inside a timing run, so the figure is tied to the kernel it was
+    measured on: each line carries the kernel name the library reported for that cell, and a cell whose kernel has
+    changed since is not used.  Returns ({(sparsity, n): (kernel, bytes)}, commit)."""
+    cells, commit = {}, None
+    try:
+        for line in open(TRAFFIC_PROFILE):
+            if line.startswith("measured_at_commit"):
+                commit = line.split()[1]
+            if line.startswith("cell "):
+                f = {k.strip(): v.strip() for k, v in (kv.split("=", 1) for kv in line.split("|")[1:])}
+                cells[(float(f["sparsity"]), int(f["n"]))] = (f["kernel"], float(f["traffic_bytes"]))
+    except (OSError, KeyError, ValueError):
+        pass
+    return cells, commit
 
 
 def log(*a):
@@ -57,9 +71,17 @@ def main():
     ap.add_argument("--no-extras", action="store_true", help="skip fp16 / SDDMM / GEMM / co-run sections")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
     ap.add_argument("--pmc-probe", action="store_true",
-                    help="for `rocprofv3 --pmc FETCH_SIZE|WRITE_SIZE`: 3 plain copies of 256 MiB (iex_copy_bytes), then "
-                         "3 launches of each cell of the dominant SpMM kernel, and exit")
+                    help="for `rocprofv3 --pmc ...`: 3 plain copies of 256 MiB (iex_copy_bytes), then 3 launches of each "
+                         "fp32 cell, and exit")
+    ap.add_argument("--overlap-probe", action="store_true",
+                    help="for `rocprofv3 --kernel-trace`: 3 replays of config 4's two-branch graph, and exit")
+    ap.add_argument("--summarize-pmc", nargs=3, metavar=("FETCH_CSV", "WRITE_CSV", "CELLS_JSON"),
+                    help="turn the counter_collection.csv of the FETCH_SIZE and of the WRITE_SIZE run of --pmc-probe and its "
+                         "pmc_probe_cells.json into profiles/spmm_fp32_config2_hbm_traffic_pmc.txt (no GPU needed)")
     args = ap.parse_args()
+    if args.summarize_pmc:
+        summarize_pmc(*args.summarize_pmc)
+        return
     if args.gpus != 1:
         log("bench.py measures one GPU: every box of this build has a single MI355X and the path has no "
             "cross-GPU step (rows of A shard with no exchange). Run with --gpus 1.")
@@ -98,8 +120,17 @@ def main():
         c = mats[s]
         return W.spmm_bytes(c.m, c.k, n, c.nnz, 1, sv, si)
 
+    from intrasm_engine_amd import _lib
+
+    def kernel_of(fn):
+        """Kernel name(s) the library launches for this call: asked of the library after one eager call."""
+        fn()
+        torch.cuda.synchronize()
+        return _lib.last_kernels()
+
     if args.pmc_probe:
-        from intrasm_engine_amd import _lib
+        # for `rocprofv3 --pmc ...`: 3 plain copies of 256 MiB (the calibration of FETCH_SIZE / WRITE_SIZE), then every
+        # fp32 cell 3 times in cell order; the kernel names go to stderr and to gpurun_out/pmc_probe_cells.json
         nbytes = 256 << 20
         src = torch.zeros(nbytes // 4, dtype=torch.float32, device=dev)
         dst = torch.empty_like(src)
@@ -107,13 +138,36 @@ def main():
             _lib.check(_lib.load().iex_copy_bytes(dst.data_ptr(), src.data_ptr(), nbytes,
                                                   torch.cuda.current_stream().cuda_stream), "copy")
         torch.cuda.synchronize()
+        names = []
         for s_, n_ in cells:       # dispatch order = cell order, 3 launches each
             fn = spmm32(s_, n_)
             for _ in range(3):
                 fn()
             torch.cuda.synchronize()
-        log(f"[bench] pmc probe done: copy of {nbytes} bytes x3 (copy_kernel), then every fp32 cell x3 in the order "
-            + " ".join(f"({s_},{n_}):{cell_bytes(s_, n_)}B" for s_, n_ in cells))
+            names.append({"sparsity": s_, "n": n_, "kernel": _lib.last_kernels(), "algorithmic_bytes": cell_bytes(s_, n_)})
+        os.makedirs(os.path.join(ROOT, "gpurun_out"), exist_ok=True)
+        json.dump({"copy_bytes": nbytes, "cells": names}, open(os.path.join(ROOT, "gpurun_out", "pmc_probe_cells.json"), "w"))
+        log("[bench] pmc probe done: copy of %d bytes x3 (copy_kernel), then every fp32 cell x3" % nbytes)
+        return
+
+    if args.overlap_probe:
+        # for `rocprofv3 --kernel-trace`: config 4's two-branch graph (SpMM kernel || GEMM), 3 replays
+        from intrasm_engine_amd.pytorch import ops as pyops
+        w, x, ga, gb = W.config4()
+        riw, vw, row, ciw = csr_dev(w, torch.float16, torch.int16)
+        xt = torch.from_numpy(x).to(dev).half()
+        gat, gbt = torch.from_numpy(ga).to(dev).bfloat16(), torch.from_numpy(gb).to(dev).bfloat16()
+        kw = dict(per_batch_values=False, accumulate=False, dtypes=(torch.float16,), allow_i16=True)
+        for label, extra in (("matrix-core SpMM kernel || GEMM", dict(no_workspace=True)), ("row-kernel SpMM || GEMM", dict(force_variant=1))):
+            constructor, keep = IL.capture_interleaved([lambda: pyops._spmm(xt, riw, vw, row, ciw, w.m, **extra, **kw)] * 2,
+                                                       [lambda: ops.gemm_mfma(gat, gbt, False)] * 2)
+            constructor.instantiate_graph_exec()
+            for _ in range(3):
+                constructor.execute_graph()
+                constructor.synchronize()
+            constructor.destroy_graph_exec()
+            log(f"[bench] overlap probe: {label}, 3 replays of a graph with 2 + 2 kernels on two branches")
+            del keep
         return
 
     sweep_bytes = sum(cell_bytes(s, n) for s, n in cells)
@@ -143,42 +197,42 @@ def main():
 
     # ------------------------------------------- per-cell launch durations (HIP events)
     def time_cell(fn, repeats=CELL_REPEATS, samples=5):
-        """Average duration of one launch: `repeats` launches in one graph on the current
+        """Average duration of one launch, caches warm: `repeats` launches in one graph on the current
         stream, events around the graph launch, median of `samples`."""
         ms = IL.time_execs([fn] * repeats, repeats=samples, warmup=1)
         return ms / repeats * 1e3  # us
 
-    def variant_of(csr, n, sv):
-        """(VEC, LPG, WPR) of the row kernel for an aligned operand (spmm_pick_shape / pick_wpr)."""
-        mean = csr.nnz / csr.m
-        wpr = 4 if mean >= 24 else 1
-        kmax = 16 // sv
-        vec, lpg = kmax, 64
-        while vec > 1 and n % vec:
-            vec //= 2
-        if vec == kmax:
-            while lpg > 8 and (lpg // 2) * vec >= n:
-                lpg //= 2
-        else:
-            while vec > 1 and 64 * vec // 2 >= n:
-                vec //= 2
-        return vec, lpg, wpr
+    cold_scratch = torch.empty(COLD_SCRATCH_BYTES // 4, dtype=torch.float32, device=dev)
+
+    def time_cold(fn, samples=7):
+        """Duration of one launch with cold caches: 512 MB are written between samples (more than the 256 MB
+        last-level cache, the reference's protocol: benchmark/utils_bench_transformer.py:60,73-75), one eager launch
+        between two events on the current stream, median of `samples`.  Includes the few us of an eager launch."""
+        fn()
+        times = []
+        for i in range(samples):
+            cold_scratch.fill_(float(i))
+            torch.cuda.synchronize()
+            a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            a.record()
+            fn()
+            b.record()
+            torch.cuda.synchronize()
+            times.append(a.elapsed_time(b))
+        return statistics.median(times) * 1e3  # us
 
     table = []
     for s, n in cells:
+        kernel = kernel_of(spmm32(s, n))
         us = time_cell(spmm32(s, n))
+        cold = time_cold(spmm32(s, n))
         by, fl = cell_bytes(s, n), W.spmm_flops(mats[s].nnz, n)
-        vec, lpg, wpr = variant_of(mats[s], n, 4)
-        kernel = f"spmm_kernel<float, int, {vec}, {lpg}, {wpr}>"
-        c = mats[s]
-        # the dispatcher's rule for the fp32 matrix-core kernel (spmm.hip, mfma_f32_variant)
-        if c.nnz / (c.m * c.k) >= 0.27 and n % 4 == 0 and -(-c.m // 32) * -(-n // 128) >= 200 and n / (-(-n // 128) * 128) >= 0.75:
-            kernel = "spmm_mfma_f32_kernel<32, 4, 1, 16, true>"
-        table.append({"sparsity": s, "n": n, "nnz": mats[s].nnz, "us": round(us, 2), "GBps": round(by / us / 1e3, 1),
+        table.append({"sparsity": s, "n": n, "nnz": mats[s].nnz, "us": round(us, 2), "cold_us": round(cold, 2),
+                      "GBps": round(by / us / 1e3, 1), "cold_GBps": round(by / cold / 1e3, 1),
                       "hbm_frac": round(by / us / 1e3 / HBM_PEAK_GBPS, 4), "GFLOPs": round(fl / us / 1e3, 1),
                       "valu_frac": round(fl / us / 1e6 / VALU_PEAK_TFLOPS_FP32, 4),
                       "kernel": kernel, "bytes": by})
-        log(f"[bench] fp32 s={s} n={n}: {us:.2f} us  {by / us / 1e3:.0f} GB/s  {fl / us / 1e3:.0f} GFLOP/s")
+        log(f"[bench] fp32 s={s} n={n}: {us:.2f} us warm, {cold:.2f} us cold  {by / us / 1e3:.0f} GB/s  {fl / us / 1e3:.0f} GFLOP/s  {kernel}")
 
     by_kernel = {}
     for row in table:
@@ -186,12 +240,17 @@ def main():
     dom_name, dom_rows = max(by_kernel.items(), key=lambda kv: sum(r["us"] for r in kv[1]))
     dom_bytes = statistics.mean(r["bytes"] for r in dom_rows)
     dom_us = statistics.mean(r["us"] for r in dom_rows)
+    measured, measured_commit = read_traffic_profile()
+    usable = [measured.get((r["sparsity"], r["n"])) for r in dom_rows]
+    traffic_ok = all(u is not None and u[0] == dom_name for u in usable)
     roofline = {"bound": "hbm", "achieved": round(dom_bytes / dom_us / 1e3, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                 "frac": round(dom_bytes / dom_us / 1e3 / HBM_PEAK_GBPS, 4),
-                "traffic": (round(statistics.mean(MEASURED_TRAFFIC_MB[(r["sparsity"], r["n"])] for r in dom_rows) * 1e6)
-                            if dom_name.startswith("spmm_kernel<float") and all((r["sparsity"], r["n"]) in MEASURED_TRAFFIC_MB for r in dom_rows)
-                            else None),
-                "kernel": dom_name, "avg_launch_us": round(dom_us, 2),
+                "traffic": round(statistics.mean(u[1] for u in usable)) if traffic_ok else None,
+                "traffic_source": (f"profiles/{os.path.basename(TRAFFIC_PROFILE)}, measured at commit {measured_commit} on the same "
+                                   "kernel instantiation (name compared with what the library reports now)") if traffic_ok else
+                                  "none: the committed counter summary was taken on another kernel than the one the library launches now",
+                "kernel": dom_name, "kernel_name_from": "iex_last_kernels() after an eager call of each cell",
+                "avg_launch_us": round(dom_us, 2),
                 "algorithmic_bytes_per_launch": int(dom_bytes),
                 "cells": [[r["sparsity"], r["n"]] for r in dom_rows],
                 "gather_bytes_per_launch": int(statistics.mean(r["nnz"] * r["n"] * 4 for r in dom_rows)),
@@ -200,6 +259,7 @@ def main():
                         "kernel is bound by that L2->CU bandwidth (gather_TBps), not by HBM, so frac stays small; "
                         "traffic = HBM-side bytes per launch from rocprofv3 --pmc FETCH_SIZE + WRITE_SIZE"}
 
+    cold_sweep_us = sum(r["cold_us"] for r in table)
     result = {
         "metric": "SpMM/SDDMM GB/s and % HBM peak; co-run makespan vs serialized (%) on 1 GPU",
         "value": round(value, 1), "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
@@ -208,62 +268,46 @@ def main():
         "config": {"workload": "config 2: fp32 CSR SpMM sweep, A 4096x4096 at {70,80,90,95,98}% sparsity (geometric "
                                "row lengths), B 4096x{64,128,256}; one step = the 15 launches in one hipGraph",
                    "value_is": "algorithmic bytes of the sweep / time per sweep",
-                   "pct_hbm_peak": round(100 * value / HBM_PEAK_GBPS, 2), "cache": "warm (operands stay in L2 / MALL between steps)"},
+                   "pct_hbm_peak": round(100 * value / HBM_PEAK_GBPS, 2), "cache": "warm (operands stay in L2 / MALL between steps)",
+                   "cold_cache_sweep_us": round(cold_sweep_us, 1),
+                   "cold_cache_GBps": round(sweep_bytes / cold_sweep_us / 1e3, 1),
+                   "cold_cache_protocol": "per cell: 512 MB written, then one eager launch between two events; sum of the 15 medians of 7"},
         "roofline": roofline,
     }
     extras = {"cells_fp32": [{k: v for k, v in r.items() if k != "bytes"} for r in table],
               "sweep_GFLOPs": round(sweep_flops / (ms_per_step * 1e-3) / 1e9, 1)}
 
-    # ------------------------------------------------------------------ CPU baseline
+    # ------------------------------------------------------------------ CPU baselines
     if not args.no_cpu:
-        import oracle  # test infrastructure, used here only as the measured CPU port
-        oracle.build()
-        t0 = time.perf_counter()
-        passes = 0
-        while passes < 3 or time.perf_counter() - t0 < 12.0:   # about 12 s of CPU work
-            for s, n in cells:
-                c = mats[s]
-                oracle.spmm_f32(dens[n], c.row_indices, c.values, c.row_offsets, c.column_indices, c.m)
-            passes += 1
-        cpu_s = (time.perf_counter() - t0) / passes
-        result["cpu_baseline"] = {"value": round(sweep_bytes / 1e9 / cpu_s, 3), "unit": "GB/s", "cores": 1, "kind": "port",
-                                  "sample": f"{passes} full passes over the same 15 fp32 cells (single-threaded C port "
-                                            f"of the oracle, gcc -O3), {cpu_s:.2f} s per pass",
-                                  "host_cpu_count": os.cpu_count()}
-        log(f"[bench] CPU port: {cpu_s:.2f} s per sweep ({passes} passes) -> {sweep_bytes / 1e9 / cpu_s:.2f} GB/s on 1 core")
-        # the library baselines the task names: torch.sparse CSR and scipy CSR on the host cores
-        try:
-            tcpu = {}
-            sample = [(s, 128) for s in W.C2_SPARSITIES]
-            nthreads = torch.get_num_threads()
-            t0 = time.perf_counter()
-            for s, n in sample:
-                c = mats[s]
-                a_t = torch.sparse_csr_tensor(torch.from_numpy(c.row_offsets), torch.from_numpy(c.column_indices),
-                                              torch.from_numpy(c.values), size=(c.m, c.k))
-                _ = a_t @ torch.from_numpy(dens[n][0])
-            tcpu["torch_sparse_csr_s"] = round(time.perf_counter() - t0, 3)
-            tcpu["torch_threads"] = nthreads
-            import scipy.sparse as sp
-            t0 = time.perf_counter()
-            for s, n in sample:
-                c = mats[s]
-                _ = sp.csr_matrix((c.values, c.column_indices, c.row_offsets), shape=(c.m, c.k)) @ dens[n][0]
-            tcpu["scipy_csr_s"] = round(time.perf_counter() - t0, 3)
-            sample_bytes = sum(cell_bytes(s, n) for s, n in sample)
-            tcpu["sample"] = "the five n=128 cells"
-            tcpu["torch_sparse_csr_GBps"] = round(sample_bytes / 1e9 / tcpu["torch_sparse_csr_s"], 3)
-            tcpu["scipy_csr_GBps"] = round(sample_bytes / 1e9 / tcpu["scipy_csr_s"], 3)
-            gpu_sample_us = sum(r["us"] for r in table if r["n"] == 128)
-            tcpu["gpu_same_sample_GBps"] = round(sample_bytes / gpu_sample_us / 1e3, 1)
-            extras["cpu_libraries"] = tcpu
-        except Exception as e:  # a library baseline must not take the bench down
-            extras["cpu_libraries"] = {"error": repr(e)}
+        # the reference's CPU path for this metric: torch.sparse CSR @ dense on the host cores, every one of the
+        # 15 cells, median of 5 runs per cell after one untimed run
+        nthreads = torch.get_num_threads()
+        cpu_cells = []
+        for s, n in cells:
+            c = mats[s]
+            a_t = torch.sparse_csr_tensor(torch.from_numpy(c.row_offsets), torch.from_numpy(c.column_indices),
+                                          torch.from_numpy(c.values), size=(c.m, c.k))
+            b_t = torch.from_numpy(dens[n][0])
+            _ = a_t @ b_t
+            ts = []
+            for _ in range(5):
+                t0 = time.perf_counter()
+                _ = a_t @ b_t
+                ts.append(time.perf_counter() - t0)
+            cpu_cells.append(statistics.median(ts))
+        cpu_s = sum(cpu_cells)
+        result["cpu_baseline"] = {"value": round(sweep_bytes / 1e9 / cpu_s, 3), "unit": "GB/s", "cores": nthreads, "kind": "reference",
+                                  "library": "torch.sparse_csr_tensor @ dense (fp32), the CPU path the metric names; the reference's own "
+                                             "native path is CUDA-only and cannot be built here",
+                                  "sample": f"all 15 fp32 cells of the same sweep, median of 5 runs per cell, {cpu_s * 1e3:.1f} ms per sweep",
+                                  "torch_num_threads": nthreads, "host_cpu_count": os.cpu_count()}
+        log(f"[bench] torch.sparse CSR on {nthreads} threads: {cpu_s * 1e3:.1f} ms per sweep -> {sweep_bytes / 1e9 / cpu_s:.2f} GB/s")
+        extras["cpu"] = cpu_extras(torch, W, mats, dens, cells, cell_bytes, sweep_bytes, nthreads, log)
 
     # ------------------------------------------------------------------------ extras
     if not args.no_extras:
         try:
-            extras.update(run_extras(torch, ops, dev, W, IL, mats, dens, csr_dev, time_cell, variant_of, log))
+            extras.update(run_extras(torch, ops, dev, W, IL, mats, dens, csr_dev, time_cell, time_cold, kernel_of, log))
         except Exception as e:
             import traceback
             traceback.print_exc(file=sys.stderr)
@@ -272,7 +316,128 @@ def main():
     print(json.dumps(result), flush=True)
 
 
-def run_extras(torch, ops, dev, W, IL, mats, dens, csr_dev, time_cell, variant_of, log):
+def summarize_pmc(fetch_csv, write_csv, cells_json):
+    """Writes profiles/spmm_fp32_config2_hbm_traffic_pmc.txt from the two counter runs of `--pmc-probe`."""
+    import csv
+    import subprocess
+
+    def per_dispatch(path, counter):
+        out = {}
+        for r in csv.DictReader(open(path)):
+            if r["Counter_Name"] == counter:
+                out[int(r["Dispatch_Id"])] = (r["Kernel_Name"], float(r["Counter_Value"]))
+        return [out[k] for k in sorted(out)]
+
+    probe = json.load(open(cells_json))
+    cells, nbytes = probe["cells"], probe["copy_bytes"]
+    readings = {}
+    for counter, path in (("FETCH_SIZE", fetch_csv), ("WRITE_SIZE", write_csv)):
+        d = per_dispatch(path, counter)
+        copies = [v for name, v in d if "copy_kernel" in name]
+        last_copy = max(i for i, (name, _) in enumerate(d) if "copy_kernel" in name)
+        spmm = [(name, v) for name, v in d[last_copy + 1:] if "spmm" in name]
+        assert len(copies) == 3 and len(spmm) == 3 * len(cells), (counter, len(copies), len(spmm))
+        readings[counter] = (statistics.median(copies), [statistics.median(v for _, v in spmm[3 * i: 3 * i + 3]) for i in range(len(cells))],
+                             [spmm[3 * i][0] for i in range(len(cells))])
+    f_copy, f_cells, f_names = readings["FETCH_SIZE"]
+    w_copy, w_cells, _ = readings["WRITE_SIZE"]
+    f_scale, w_scale = nbytes / (f_copy * 1024.0), nbytes / (w_copy * 1024.0)
+    commit = subprocess.run(["git", "-C", ROOT, "rev-parse", "--short", "HEAD"], stdout=subprocess.PIPE, text=True).stdout.strip() or "unknown"
+    lines = [
+        "HBM-side traffic (L2 misses + write-backs) of the 15 fp32 cells of config 2, one MI355X, per launch.",
+        "Two counter runs of the same committed command (rocprofv3 does not split counters over passes), then this summary:",
+        "  rocprofv3 --pmc FETCH_SIZE -d gpurun_out/pmc_fetch -o p --output-format csv -- python3 bench.py --pmc-probe",
+        "  rocprofv3 --pmc WRITE_SIZE -d gpurun_out/pmc_write -o p --output-format csv -- python3 bench.py --pmc-probe",
+        "  python3 bench.py --summarize-pmc gpurun_out/pmc_fetch/p_counter_collection.csv gpurun_out/pmc_write/p_counter_collection.csv gpurun_out/pmc_probe_cells.json",
+        "Both counters read KiB per dispatch; each is scaled by what it reads for a plain copy of known size (iex_copy_bytes,",
+        "256 MiB read and 256 MiB written, three dispatches, median).  Every cell: three dispatches, median.  `kernel` is what",
+        "the library reported for the cell in the probe run (iex_last_kernels); bench.py uses a line only while that still",
+        "holds.  traffic_bytes = fetch_kib * 1024 * fetch_scale + write_kib * 1024 * write_scale.",
+        f"measured_at_commit {commit}",
+        f"calibration | copy_bytes={nbytes} | fetch_kib={f_copy:.0f} | fetch_scale={f_scale:.3f} | write_kib={w_copy:.0f} | write_scale={w_scale:.3f}",
+    ]
+    for i, c in enumerate(cells):
+        traffic = f_cells[i] * 1024 * f_scale + w_cells[i] * 1024 * w_scale
+        assert c["kernel"].split("<")[0] in f_names[i], (c["kernel"], f_names[i])
+        lines.append(f"cell | sparsity={c['sparsity']} | n={c['n']} | kernel={c['kernel']} | fetch_kib={f_cells[i]:.0f} | write_kib={w_cells[i]:.0f} | "
+                     f"traffic_bytes={traffic:.0f} | algorithmic_bytes={c['algorithmic_bytes']} | ratio={traffic / c['algorithmic_bytes']:.2f}")
+    open(TRAFFIC_PROFILE, "w").write("\n".join(lines) + "\n")
+    print("\n".join(lines))
+
+
+def cpu_extras(torch, W, mats, dens, cells, cell_bytes, sweep_bytes, nthreads, log):
+    """The other CPU legs: the single-core C port of the oracle and scipy CSR on the same sweep, the SDDMM of config 1
+    (gather form in numpy, torch.sparse.sampled_addmm) and the GEMM of config 4 (torch.matmul, fp32)."""
+    out = {}
+    import oracle  # test infrastructure, used here only as a measured CPU port
+    oracle.build()
+    t0, passes = time.perf_counter(), 0
+    while passes < 2 or time.perf_counter() - t0 < 6.0:
+        for s, n in cells:
+            c = mats[s]
+            oracle.spmm_f32(dens[n], c.row_indices, c.values, c.row_offsets, c.column_indices, c.m)
+        passes += 1
+    port_s = (time.perf_counter() - t0) / passes
+    out["c_port_single_core"] = {"GBps": round(sweep_bytes / 1e9 / port_s, 3), "s_per_sweep": round(port_s, 3), "passes": passes,
+                                 "what": "oracle.c compiled with gcc -O3, one thread, all 15 cells"}
+    try:
+        import scipy.sparse as sp
+        ts = []
+        for s, n in cells:
+            c = mats[s]
+            a_s = sp.csr_matrix((c.values, c.column_indices, c.row_offsets), shape=(c.m, c.k))
+            reps = []
+            for _ in range(3):
+                t0 = time.perf_counter()
+                _ = a_s @ dens[n][0]
+                reps.append(time.perf_counter() - t0)
+            ts.append(statistics.median(reps))
+        out["scipy_csr"] = {"GBps": round(sweep_bytes / 1e9 / sum(ts), 3), "s_per_sweep": round(sum(ts), 3),
+                            "what": "scipy.sparse.csr_matrix @ dense, all 15 cells, median of 3 per cell (single-threaded)"}
+    except Exception as e:  # a library baseline must not take the bench down
+        out["scipy_csr"] = {"error": repr(e)}
+    # SDDMM, config 1: mask 1024 x 1024 at 90 %, k = 64, fp32
+    try:
+        a1, _, lhs1, rhs1 = W.config1()
+        rows = np.repeat(np.arange(a1.m), np.diff(a1.row_offsets))
+        reps = []
+        for _ in range(5):
+            t0 = time.perf_counter()
+            _ = np.einsum("ij,ij->i", lhs1[0][rows], rhs1[0][a1.column_indices])
+            reps.append(time.perf_counter() - t0)
+        by = W.sddmm_bytes(a1.m, 64, a1.k, a1.nnz, 1, 4, True)
+        out["sddmm_c1_numpy_gather"] = {"ms": round(statistics.median(reps) * 1e3, 3), "GBps": round(by / statistics.median(reps) / 1e9, 3)}
+        mask = torch.sparse_csr_tensor(torch.from_numpy(a1.row_offsets), torch.from_numpy(a1.column_indices),
+                                       torch.zeros(a1.nnz), size=(a1.m, a1.k))
+        lt, rt = torch.from_numpy(lhs1[0]), torch.from_numpy(rhs1[0]).t().contiguous()
+        _ = torch.sparse.sampled_addmm(mask, lt, rt, beta=0.0)
+        reps = []
+        for _ in range(5):
+            t0 = time.perf_counter()
+            _ = torch.sparse.sampled_addmm(mask, lt, rt, beta=0.0)
+            reps.append(time.perf_counter() - t0)
+        out["sddmm_c1_torch_sampled_addmm"] = {"ms": round(statistics.median(reps) * 1e3, 3), "threads": nthreads,
+                                               "GBps": round(by / statistics.median(reps) / 1e9, 3)}
+    except Exception as e:
+        out["sddmm_c1_cpu"] = {"error": repr(e)}
+    # GEMM, config 4's shape (4096 x 4096 x 2048), torch.matmul in fp32 on the host
+    try:
+        ga, gb = torch.randn(4096, 4096), torch.randn(4096, 2048)
+        _ = ga @ gb
+        reps = []
+        for _ in range(3):
+            t0 = time.perf_counter()
+            _ = ga @ gb
+            reps.append(time.perf_counter() - t0)
+        out["gemm_c4_torch_matmul_fp32"] = {"ms": round(statistics.median(reps) * 1e3, 1), "threads": nthreads,
+                                            "TFLOPs": round(2.0 * 4096 * 4096 * 2048 / statistics.median(reps) / 1e12, 3)}
+    except Exception as e:
+        out["gemm_c4_cpu"] = {"error": repr(e)}
+    log(f"[bench] CPU legs: {json.dumps(out)}")
+    return out
+
+
+def run_extras(torch, ops, dev, W, IL, mats, dens, csr_dev, time_cell, time_cold, kernel_of, log):
     out = {}
     # ---- fp16 sweep (int16 column indices, the reference's half layout)
     rows = []
@@ -303,12 +468,16 @@ def run_extras(torch, ops, dev, W, IL, mats, dens, csr_dev, time_cell, variant_o
     us = time_cell(lambda: ops.sddmm_sputnik_half(qt, kt, ri3, ro3, ci3), repeats=10)
     by = W.sddmm_bytes(pat.m, 64, pat.k, pat.nnz, 16, 2, False)
     out["sddmm_c3_fp16_16heads"] = {"nnz": pat.nnz, "sparsity": round(pat.sparsity, 4), "us": round(us, 2),
+                                    "cold_us": round(time_cold(lambda: ops.sddmm_sputnik_half(qt, kt, ri3, ro3, ci3)), 2),
+                                    "kernel": kernel_of(lambda: ops.sddmm_sputnik_half(qt, kt, ri3, ro3, ci3)),
                                     "GBps": round(by / us / 1e3, 1), "hbm_frac": round(by / us / 1e3 / HBM_PEAK_GBPS, 4),
                                     "GFLOPs": round(W.sddmm_flops(pat.nnz, 64, 16) / us / 1e3, 1)}
     scores = ops.sddmm_sputnik_half(qt, kt, ri3, ro3, ci3)
     us = time_cell(lambda: ops.spmm_sputnik_batched_values(vt, ri3, scores, ro3, ci3, pat.m), repeats=10)
     by = W.spmm_bytes(pat.m, pat.k, 64, pat.nnz, 16, 2, 4, True)
     out["spmm_c3_fp16_16heads"] = {"us": round(us, 2), "GBps": round(by / us / 1e3, 1),
+                                   "cold_us": round(time_cold(lambda: ops.spmm_sputnik_batched_values(vt, ri3, scores, ro3, ci3, pat.m)), 2),
+                                   "kernel": kernel_of(lambda: ops.spmm_sputnik_batched_values(vt, ri3, scores, ro3, ci3, pat.m)),
                                    "hbm_frac": round(by / us / 1e3 / HBM_PEAK_GBPS, 4),
                                    "GFLOPs": round(W.spmm_flops(pat.nnz, 64, 16) / us / 1e3, 1)}
     from intrasm_engine_amd.pytorch.sparse_attention import sparse_attention
@@ -368,15 +537,30 @@ def run_extras(torch, ops, dev, W, IL, mats, dens, csr_dev, time_cell, variant_o
     out["output_bound_sweep_points_fp32"] = pts
 
     # ---- config 4: fp16 SpMM 11008x4096 @90% x 4096x2048  ||  bf16 GEMM 4096x4096x2048
+    # Eight distinct operand sets per branch, as the reference's harness runs them (tests/test_interleaving.py:544,617):
+    # every repetition reads its own copy of the weight (same pattern, values of its own), activation and GEMM
+    # operands, so no repetition finds the previous one's operands in the caches.
+    from intrasm_engine_amd.pytorch import ops as pyops
     w, x, ga, gb = W.config4()
+    reps = 8
     riw, vw, row, ciw = csr_dev(w, torch.float16, torch.int16)
-    xt = torch.from_numpy(x).to(dev).half()
-    gat, gbt = torch.from_numpy(ga).to(dev).bfloat16(), torch.from_numpy(gb).to(dev).bfloat16()
-    reps = 4
-    spmm_execs = [lambda: ops.spmm_sputnik_reuse_weight_half(xt, riw, vw, row, ciw, w.m)] * reps
-    gemm_execs = [lambda: ops.gemm_mfma(gat, gbt, False)] * reps
-    fused_execs = [lambda: ops.fused_spmm_gemm(xt, riw, vw, row, ciw, w.m, gat, gbt, False, 0)] * reps
-    fused_g_execs = [lambda: ops.fused_spmm_gemm(xt, riw, vw, row, ciw, w.m, gat, gbt, False, 64)] * reps
+    gen = torch.Generator(dev).manual_seed(4)
+    sets = []
+    for i in range(reps):
+        sign = (torch.randint(0, 2, vw.shape, device=dev, generator=gen) * 2 - 1).to(vw.dtype)
+        sets.append((riw.clone(), vw * sign if i else vw, row.clone(), ciw.clone(),
+                     torch.randn(1, w.k, 2048, device=dev, generator=gen).half() if i else torch.from_numpy(x).to(dev).half(),
+                     torch.randn(4096, 4096, device=dev, generator=gen).bfloat16() if i else torch.from_numpy(ga).to(dev).bfloat16(),
+                     torch.randn(4096, 2048, device=dev, generator=gen).bfloat16() if i else torch.from_numpy(gb).to(dev).bfloat16()))
+    kw4 = dict(per_batch_values=False, accumulate=False, dtypes=(torch.float16,), allow_i16=True)
+
+    def spmm_list(**extra):
+        return [(lambda t=t: pyops._spmm(t[4], t[0], t[1], t[2], t[3], w.m, **extra, **kw4)) for t in sets]
+
+    spmm_execs = [(lambda t=t: ops.spmm_sputnik_reuse_weight_half(t[4], t[0], t[1], t[2], t[3], w.m)) for t in sets]
+    gemm_execs = [(lambda t=t: ops.gemm_mfma(t[5], t[6], False)) for t in sets]
+    fused_execs = [(lambda t=t: ops.fused_spmm_gemm(t[4], t[0], t[1], t[2], t[3], w.m, t[5], t[6], False, 0)) for t in sets]
+    fused_g_execs = [(lambda t=t: ops.fused_spmm_gemm(t[4], t[0], t[1], t[2], t[3], w.m, t[5], t[6], False, 64)) for t in sets]
     t_spmm = IL.run_non_interleaving(spmm_execs) / reps
     t_gemm = IL.run_non_interleaving(gemm_execs) / reps
     t_serial = IL.run_non_interleaving(spmm_execs, gemm_execs) / reps
@@ -385,23 +569,24 @@ def run_extras(torch, ops, dev, W, IL, mats, dens, csr_dev, time_cell, variant_o
     t_fused_g = IL.run_non_interleaving(fused_g_execs) / reps
     # the same pair with the SpMM forced onto the gather (row) kernel: vector ALU + L2 beside the matrix cores,
     # the resource split the reference's co-run experiment is about
-    from intrasm_engine_amd.pytorch import ops as pyops
-    gather_execs = [lambda: pyops._spmm(xt, riw, vw, row, ciw, w.m, per_batch_values=False, accumulate=False,
-                                        dtypes=(torch.float16,), allow_i16=True, force_variant=1)] * reps
+    gather_execs = spmm_list(force_variant=1)
     t_gather = IL.run_non_interleaving(gather_execs) / reps
     t_graph_gather = IL.run_interleaving(gather_execs, gemm_execs) / reps
     # the library's choice above has a workspace to use (the operator allocates one) and takes the dense-form
     # path; without one the 8-wave matrix-core SpMM kernel runs, the kernel the fused launch shares its SpMM role with
-    mc_execs = [lambda: pyops._spmm(xt, riw, vw, row, ciw, w.m, per_batch_values=False, accumulate=False,
-                                    dtypes=(torch.float16,), allow_i16=True, no_workspace=True)] * reps
+    mc_execs = spmm_list(no_workspace=True)
     t_mc = IL.run_non_interleaving(mc_execs) / reps
     t_graph_mc = IL.run_interleaving(mc_execs, gemm_execs) / reps
+    k_spmm, k_gemm, k_fused = kernel_of(spmm_execs[0]), kernel_of(gemm_execs[0]), kernel_of(fused_execs[0])
+    cold_spmm, cold_gemm = time_cold(spmm_execs[0]) / 1e3, time_cold(gemm_execs[0]) / 1e3
     fl_s, fl_g = W.spmm_flops(w.nnz, 2048), W.gemm_flops(4096, 2048, 4096)
     by_s = W.spmm_bytes(w.m, w.k, 2048, w.nnz, 1, 2, 2)
     out["config4"] = {
         "spmm_ms": round(t_spmm, 4), "spmm_GBps": round(by_s / t_spmm / 1e6, 1), "spmm_GFLOPs": round(fl_s / t_spmm / 1e6, 1),
         "spmm_hbm_frac": round(by_s / t_spmm / 1e6 / HBM_PEAK_GBPS, 4),
         "spmm_valu_frac": round(fl_s / t_spmm / 1e9 / VALU_PEAK_TFLOPS_FP32, 4),
+        "spmm_kernels": k_spmm, "gemm_kernels": k_gemm, "fused_kernels": k_fused,
+        "spmm_cold_ms": round(cold_spmm, 4), "gemm_cold_ms": round(cold_gemm, 4),
         "gemm_ms": round(t_gemm, 4), "gemm_TFLOPs": round(IL.gemm_tflops(4096, 2048, 4096, t_gemm), 1),
         "gemm_mfma_frac": round(IL.gemm_tflops(4096, 2048, 4096, t_gemm) / MFMA_PEAK_TFLOPS_16BIT, 4),
         "serialized_sum_ms": round(t_spmm + t_gemm, 4), "serialized_one_stream_ms": round(t_serial, 4),
@@ -415,20 +600,34 @@ def run_extras(torch, ops, dev, W, IL, mats, dens, csr_dev, time_cell, variant_o
         "spmm_row_kernel_ms": round(t_gather, 4), "two_branch_graph_row_kernel_ms": round(t_graph_gather, 4),
         "row_kernel_graph_makespan_pct_of_serialized": round(100 * t_graph_gather / (t_gather + t_gemm), 1),
         "spmm_dense_equivalent_TFLOPs": round(2.0 * w.m * w.k * 2048 / t_spmm / 1e9, 1),
-        "repeats_per_graph": reps,
+        "repeats_per_graph": reps, "operand_sets": f"{reps} distinct (own copies of the CSR arrays, values, activation and GEMM operands per repetition)",
     }
     log(f"[bench] config 4: spmm {t_spmm:.3f} ms, gemm {t_gemm:.3f} ms, graph {t_graph:.3f} ms, fused {t_fused:.3f} ms")
-    del w, x, ga, gb, riw, vw, row, ciw, xt, gat, gbt, spmm_execs, gemm_execs, fused_execs, fused_g_execs, gather_execs, mc_execs
+    del w, x, ga, gb, riw, vw, row, ciw, sets, spmm_execs, gemm_execs, fused_execs, fused_g_execs, gather_execs, mc_execs
+    reps = 4
 
     # ---- the dense GEMM alone on larger shapes (bf16, B as (K, N)): how far the matrix cores are used
     rows_gemm = []
-    for (gm, gn, gk) in ((8192, 8192, 8192), (4096, 8192, 4096), (11008, 8192, 4096)):
+    for (gm, gn, gk) in ((8192, 8192, 8192), (4096, 8192, 4096), (11008, 8192, 4096), (4096, 2048, 4096)):
         ga2 = torch.randn(gm, gk, device=dev).bfloat16()
         gb2 = torch.randn(gk, gn, device=dev).bfloat16()
         t = IL.run_non_interleaving([lambda: ops.gemm_mfma(ga2, gb2, False)] * reps) / reps
         tf = IL.gemm_tflops(gm, gn, gk, t)
+        # the vendor library on the same operands in the same run, as a comparator (never on the product path)
+        # (eagerly, between two events: the vendor library refuses to run under stream capture)
+        for _ in range(2):
+            torch.matmul(ga2, gb2)
+        ev0, ev1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        ev0.record()
+        for _ in range(2 * reps):
+            torch.matmul(ga2, gb2)
+        ev1.record()
+        torch.cuda.synchronize()
+        t_lib = ev0.elapsed_time(ev1) / (2 * reps)
         rows_gemm.append({"m": gm, "n": gn, "k": gk, "ms": round(t, 4), "TFLOPs": round(tf, 1),
-                          "mfma_frac": round(tf / MFMA_PEAK_TFLOPS_16BIT, 4)})
+                          "mfma_frac": round(tf / MFMA_PEAK_TFLOPS_16BIT, 4), "kernel": kernel_of(lambda: ops.gemm_mfma(ga2, gb2, False)),
+                          "torch_matmul_is": "torch.matmul (hipBLASLt) on the same operands, eager, a comparator only",
+                          "torch_matmul_ms": round(t_lib, 4), "torch_matmul_TFLOPs": round(IL.gemm_tflops(gm, gn, gk, t_lib), 1)})
         del ga2, gb2
     out["gemm_bf16"] = rows_gemm
 

@@ -43,6 +43,11 @@ enum {
 int iex_abi_version(void);
 /* Text of the most recent failure on this thread ("" when none). */
 const char* iex_last_error(void);
+/* Names (with template arguments) of the kernels that the most recent SpMM / SDDMM / GEMM / fused entry point
+ * launched on this thread, joined by " + " ("" before the first call or when nothing was launched): what a
+ * profile of the same call lists, read from the library instead of re-derived from its selection rules.
+ * No counterpart in the reference. */
+const char* iex_last_kernels(void);
 /* 1 when a gfx950 device is visible to the HIP runtime, else 0. */
 int iex_device_ok(void);
 

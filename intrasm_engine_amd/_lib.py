@@ -28,6 +28,7 @@ _vp, _i, _ll, _f = _c.c_void_p, _c.c_int, _c.c_longlong, _c.c_float
 SIGNATURES = {
     "iex_abi_version": (_i, []),
     "iex_last_error": (_c.c_char_p, []),
+    "iex_last_kernels": (_c.c_char_p, []),
     "iex_device_ok": (_i, []),
     "iex_copy_bytes": (_i, [_vp, _vp, _c.c_size_t, _vp]),
     "iex_spmm_ex": (_i, [_i, _i, _i, _i, _i, _i, _i, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i]),
@@ -95,6 +96,11 @@ def load() -> ctypes.CDLL:
         raise ImportError(f"{LIB_PATH}: ABI version {lib.iex_abi_version()} != 1")
     _lib = lib
     return lib
+
+
+def last_kernels() -> str:
+    """Kernels launched by the most recent compute entry point on this thread."""
+    return load().iex_last_kernels().decode("utf-8", "replace")
 
 
 def last_error() -> str:

@@ -18,6 +18,26 @@ int fail(int code, const char* fmt, ...) {
   return code;
 }
 
+static char* trail_buffer() {
+  static thread_local char buf[512] = {0};
+  return buf;
+}
+
+void trail_reset() { trail_buffer()[0] = 0; }
+
+void note_kernel(const char* fmt, ...) {
+  char* buf = trail_buffer();
+  size_t used = std::strlen(buf);
+  if (used > 0 && used + 4 < 512) {
+    std::memcpy(buf + used, " + ", 4);
+    used += 3;
+  }
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(buf + used, 512 - used, fmt, ap);
+  va_end(ap);
+}
+
 int check_hip(hipError_t err, const char* what) {
   if (err == hipSuccess) return 0;
   snprintf(last_error_buffer(), 512, "%s: %s (hipError_t %d)", what, hipGetErrorString(err), (int)err);
@@ -50,6 +70,8 @@ int iex_copy_bytes(void* dst, const void* src, size_t nbytes, void* stream) {
 int iex_abi_version(void) { return IEX_ABI_VERSION; }
 
 const char* iex_last_error(void) { return iex::last_error_buffer(); }
+
+const char* iex_last_kernels(void) { return iex::trail_buffer(); }
 
 int iex_device_ok(void) {
   int count = 0;

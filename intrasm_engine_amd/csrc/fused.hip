@@ -120,6 +120,9 @@ int launch_mc(FusedParams p, hipStream_t stream) {
       return rc;
     raised = true;
   }
+  trail_reset();
+  note_kernel("fused_mc_kernel<%s, %s, %s, %d> (%d GEMM tiles, %d SpMM tiles)", BF16 ? "true" : "false", TRANS_B ? "true" : "false", type_name<IT>(), W,
+              p.gemm_blocks, p.spmm_blocks);
   hipLaunchKernelGGL(kernel, dim3(p.gemm_blocks + p.spmm_blocks), dim3(kMfma2Threads), lds, stream, p);
   return check_hip(hipGetLastError(), "fused (matrix-core) launch");
 }
@@ -158,6 +161,9 @@ int launch(FusedParams p, hipStream_t stream) {
   constexpr int lds_gemm = gemm_lds_bytes<TRANS_B, kFusedWM, kFusedWN>();
   constexpr int lds_spmm = spmm_lds_floats<VEC, WPR>() * 4;
   constexpr int lds = lds_gemm > lds_spmm ? lds_gemm : lds_spmm;
+  trail_reset();
+  note_kernel("fused_kernel<%s, %s, %s, %d, %d, %d> (%d GEMM tiles, %d SpMM blocks)", BF16 ? "true" : "false", TRANS_B ? "true" : "false",
+              type_name<IT>(), VEC, LPG, WPR, p.gemm_blocks, p.spmm_blocks);
   hipLaunchKernelGGL((fused_kernel<BF16, TRANS_B, IT, VEC, LPG, WPR>), dim3(p.gemm_blocks + p.spmm_blocks), dim3(256), lds, stream,
                      p);
   return check_hip(hipGetLastError(), "fused launch");

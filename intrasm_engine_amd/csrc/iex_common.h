@@ -19,6 +19,16 @@ constexpr int kWave = 64;
 char* last_error_buffer();
 int fail(int code, const char* fmt, ...);
 int check_hip(hipError_t err, const char* what);
+// Names of the kernels the current entry point has launched on this thread (iex_last_kernels):
+// trail_reset() at the start of an entry point, note_kernel() beside every launch.
+void trail_reset();
+void note_kernel(const char* fmt, ...);
+template <typename T> inline const char* type_name();
+template <> inline const char* type_name<float>() { return "float"; }
+template <> inline const char* type_name<__half>() { return "__half"; }
+template <> inline const char* type_name<__hip_bfloat16>() { return "__hip_bfloat16"; }
+template <> inline const char* type_name<int>() { return "int"; }
+template <> inline const char* type_name<short>() { return "short"; }
 
 #define IEX_REQUIRE(cond, code, ...)                 \
   do {                                               \

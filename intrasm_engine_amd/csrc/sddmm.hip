@@ -191,6 +191,7 @@ int launch_one(const SddmmParams& p0, hipStream_t stream) {
   SddmmParams p = p0;
   dim3 grid(ceil_div(p.m, 4 / WPR), 1, p.sum_over_batch ? 1 : ceil_div(p.batch, kSddmmZb));
   p.deep = (long long)grid.x * grid.z * 4 <= 2048;  // at most two wavefronts per SIMD of the chip
+  note_kernel("sddmm_kernel<%s, %d, %d, %d, %d, %s>", type_name<T>(), VEC, LPN, PASSES, WPR, EXACT ? "true" : "false");
   hipLaunchKernelGGL((sddmm_kernel<T, VEC, LPN, PASSES, WPR, EXACT>), grid, dim3(256), 0, stream, p);
   return check_hip(hipGetLastError(), "sddmm launch");
 }
@@ -277,6 +278,7 @@ int launch_sddmm_dense(int dtype, const SddmmParams& p, void* ws, hipStream_t st
     const uint16_t* lhs = static_cast<const uint16_t*>(p.lhs) + (size_t)z * p.m * p.k;
     const uint16_t* rhs = static_cast<const uint16_t*>(p.rhs) + (size_t)z * p.n * p.k;
     if (int rc = iex_gemm(dtype, 1, p.m, p.n, p.k, lhs, rhs, ws, 1, 0, 0, 0, stream)) return rc;
+    note_kernel("sample_dense_kernel");
     hipLaunchKernelGGL(sample_dense_kernel, dim3(ceil_div(p.m, 4)), dim3(256), 0, stream, p.m, p.n, p.row_offsets, p.cols,
                        static_cast<const uint16_t*>(ws), static_cast<uint16_t*>(p.out) + (size_t)z * p.nnz);
     if (int rc = check_hip(hipGetLastError(), "sddmm sampling launch")) return rc;
@@ -305,6 +307,7 @@ int sddmm_dispatch(int dtype, int flags, int m, int k, int n, int nonzeros, cons
                    void* out, void* stream, int batch, void* workspace, size_t workspace_bytes) {
   IEX_REQUIRE(m >= 0 && k >= 0 && n >= 0 && nonzeros >= 0 && batch >= 0, IEX_ERR_BAD_ARGUMENT,
               "sddmm: negative dimension (m=%d k=%d n=%d nnz=%d batch=%d)", m, k, n, nonzeros, batch);
+  trail_reset();
   if (m == 0 || nonzeros == 0 || batch == 0) return 0;
   IEX_REQUIRE(row_indices && row_offsets && column_indices && out, IEX_ERR_BAD_ARGUMENT,
               "sddmm: null pointer argument");

@@ -26,6 +26,7 @@ int launch_one(const SpmmParams& p, int batch, hipStream_t stream) {
   constexpr int kRowsPerBlock = kWavesPerBlock / WPR;
   dim3 grid(ceil_div(p.m, kRowsPerBlock), ceil_div(p.n, NT * LPG * VEC), batch);
   dim3 block(kWavesPerBlock * kWave);
+  note_kernel("spmm_kernel<%s, %s, %d, %d, %d, %d>", type_name<T>(), type_name<IT>(), VEC, LPG, WPR, NT);
   hipLaunchKernelGGL((spmm_kernel<T, IT, VEC, LPG, WPR, NT>), grid, block, 0, stream, p);
   return check_hip(hipGetLastError(), "spmm launch");
 }
@@ -42,6 +43,7 @@ int launch_ragged_one(const SpmmParams& p, int batch, hipStream_t stream) {
   constexpr int kWavesPerBlock = (WPR > 4) ? WPR : 4;
   constexpr int kRowsPerBlock = kWavesPerBlock / WPR;
   dim3 grid(ceil_div(p.m, kRowsPerBlock), ceil_div(p.n, kWave * VEC), batch);
+  note_kernel("spmm_ragged_kernel<%s, %s, %d, %d>", type_name<T>(), type_name<IT>(), VEC, WPR);
   hipLaunchKernelGGL((spmm_ragged_kernel<T, IT, VEC, WPR>), grid, dim3(kWavesPerBlock * kWave), 0, stream, p);
   return check_hip(hipGetLastError(), "spmm (ragged rows) launch");
 }
@@ -118,6 +120,7 @@ int launch_smallk(const SpmmParams& p, int batch, hipStream_t stream) {
     }
   }
   dim3 grid(ceil_div(p.m, waves * rows), ceil_div(p.n, kWave * kMax), batch);
+  note_kernel("spmm_smallk_kernel<%s, %s, %d, %s, %d>", type_name<T>(), type_name<IT>(), kMax, ragged ? "true" : "false", waves);
   hipLaunchKernelGGL(kern, grid, dim3(waves * kWave), lds, stream, p, rows);
   return check_hip(hipGetLastError(), "spmm (few columns) launch");
 }
@@ -146,6 +149,7 @@ __global__ __launch_bounds__(kLdsThreads, 4) void spmm_lds_kernel(SpmmParams p) 
 template <typename T, typename IT, int VEC, int RPW>
 int launch_lds_one(const SpmmParams& p, int batch, hipStream_t stream) {
   dim3 grid(ceil_div(p.m, kLdsWaves * RPW), ceil_div(p.n, kWave * VEC), batch);
+  note_kernel("spmm_lds_kernel<%s, %s, %d, %d>", type_name<T>(), type_name<IT>(), VEC, RPW);
   hipLaunchKernelGGL((spmm_lds_kernel<T, IT, VEC, RPW>), grid, dim3(kLdsThreads), kLdsTileBytes, stream, p);
   return check_hip(hipGetLastError(), "spmm (LDS-staged) launch");
 }
@@ -184,6 +188,7 @@ int launch_mfma_one(const SpmmParams& p, int batch, hipStream_t stream) {
       return rc;
     raised = true;
   }
+  note_kernel("spmm_mfma_kernel<%s, %s, %d>", kBf16 ? "true" : "false", type_name<IT>(), LPR);
   hipLaunchKernelGGL(kernel, dim3(tiles_m * tiles_n, batch), dim3(kMfmaThreads), kMfmaLdsBytes, stream, p, tiles_m);
   return check_hip(hipGetLastError(), "spmm (matrix-core) launch");
 }
@@ -221,6 +226,7 @@ int launch_mfma2_one(const SpmmParams& p, int batch, hipStream_t stream) {
       return rc;
     raised = true;
   }
+  note_kernel("spmm_mfma2_kernel<%s, %s, %d, %d>", kBf16 ? "true" : "false", type_name<IT>(), W, BKA);
   hipLaunchKernelGGL(kernel, dim3(tiles_m * tiles_n, batch), dim3(kMfma2Threads), kMfma2LdsBytes, stream, p, tiles_m);
   return check_hip(hipGetLastError(), "spmm (matrix-core, 8 waves) launch");
 }
@@ -259,6 +265,7 @@ int launch_mfma3_one(const SpmmParams& p, int batch, hipStream_t stream) {
       return rc;
     raised = true;
   }
+  note_kernel("spmm_mfma3_kernel<%s, %s, %d>", kBf16 ? "true" : "false", type_name<IT>(), W);
   hipLaunchKernelGGL(kernel, dim3(tiles_m * tiles_n, batch), dim3(kMfma3Threads), spmm_mfma3_lds_bytes(), stream, p, tiles_m);
   return check_hip(hipGetLastError(), "spmm (matrix-core, direct loads) launch");
 }
@@ -290,6 +297,7 @@ int launch_mfma_f32_one(const SpmmParams& p, int batch, hipStream_t stream) {
   constexpr int kBN = MT * NJ * WAVES_N;
   const int tiles_m = ceil_div(p.m, MT), tiles_n = ceil_div(p.n, kBN);
   constexpr int kLds = spmm_mfma_f32_lds_bytes<MT, NJ, WAVES_N>();
+  note_kernel("spmm_mfma_f32_kernel<%d, %d, %d, %d, %s>", MT, NJ, WAVES_N, W, SPLIT ? "true" : "false");
   hipLaunchKernelGGL((spmm_mfma_f32_kernel<MT, NJ, WAVES_N, W, SPLIT>), dim3(tiles_m * tiles_n, batch),
                      dim3(kF32Threads + (SPLIT ? MT * 8 : 0)), kLds, stream, p, tiles_m);
   return check_hip(hipGetLastError(), "spmm (matrix-core, fp32) launch");
@@ -385,11 +393,13 @@ int launch_ksplit_one(const SpmmParams& p, int batch, const KsplitPlan& pl, floa
       raised = true;
     }
   }
+  note_kernel("spmm_ksplit_kernel<%s, %s, %d, %d, %d, %d> (%d slices)", type_name<T>(), type_name<IT>(), VEC, kKsplitRpw, WAVES, KB, pl.slices);
   hipLaunchKernelGGL(kernel, dim3(q.row_blocks * q.slices, ceil_div(p.n, kWave * VEC), batch), dim3(WAVES * kWave), lds, stream, q);
   if (int rc = check_hip(hipGetLastError(), "spmm (k split) launch")) return rc;
   if (pl.slices > 1) {
     const size_t quads = (size_t)batch * p.m * p.n / 4;
     const int blocks = (int)std::min<size_t>((quads + 255) / 256, 256 * 16);
+    note_kernel("spmm_ksplit_reduce_kernel<%s>", type_name<T>());
     hipLaunchKernelGGL((spmm_ksplit_reduce_kernel<T>), dim3(blocks), dim3(256), 0, stream, p, partial, pl.slices, batch);
     return check_hip(hipGetLastError(), "spmm (k split) reduction launch");
   }
@@ -571,6 +581,7 @@ inline bool dense_path_wins(const SpmmParams& p, int batch, int matrix_core_kind
 
 template <typename T, typename IT>
 int launch_dense_path(const SpmmParams& p, int batch, const Choice& ch, hipStream_t stream) {
+  note_kernel("csr_to_dense_kernel<%s>", type_name<IT>());
   hipLaunchKernelGGL((csr_to_dense_kernel<IT>), dim3(ceil_div(p.m, kDenseWaves)), dim3(kDenseThreads), 0, stream, p.m, p.k,
                      p.row_offsets, static_cast<const IT*>(p.cols), static_cast<const uint16_t*>(p.values),
                      static_cast<uint16_t*>(ch.ws));
@@ -675,6 +686,7 @@ int spmm_dispatch(int dtype, int itype, int flags, int m, int k, int n, int nonz
                   void* stream, int batch, void* workspace, size_t workspace_bytes) {
   IEX_REQUIRE(m >= 0 && k >= 0 && n >= 0 && nonzeros >= 0 && batch >= 0, IEX_ERR_BAD_ARGUMENT,
               "spmm: negative dimension (m=%d k=%d n=%d nnz=%d batch=%d)", m, k, n, nonzeros, batch);
+  trail_reset();
   if (m == 0 || n == 0 || batch == 0) return 0;  // empty output: nothing to launch
   IEX_REQUIRE(row_indices && row_offsets && dense && out, IEX_ERR_BAD_ARGUMENT,
               "spmm: null pointer argument");

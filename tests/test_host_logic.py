@@ -91,3 +91,23 @@ def test_forward_options_are_validated():
         normalise_kwargs({"bogus": 1})
     with pytest.raises(ValueError):
         normalise_kwargs({"constructor_enabled": True})
+
+
+@pytest.mark.gpu
+def test_dense_to_sparse_on_a_device_tensor(oracle, dev):
+    """The CSR build run on the GPU (torch kernels on a device tensor, as the reference calls it,
+    pytorch/utils.py:143-153): values, offsets, column indices and the swizzle bit-equal to the oracle's, for a
+    ragged matrix with empty rows and ties in row length."""
+    import torch
+    from intrasm_engine_amd.pytorch.utils import dense_to_sparse, sparse_to_dense
+    rng = np.random.default_rng(5)
+    dense = rng.standard_normal((197, 301)).astype(np.float32)
+    dense[rng.random(dense.shape) < 0.83] = 0.0
+    dense[[0, 50, 196]] = 0.0
+    dense[7] = dense[9]                                   # equal lengths: the swizzle must keep row order
+    values, row_indices, row_offsets, column_indices = dense_to_sparse(torch.from_numpy(dense), device=dev)
+    assert all(t.is_cuda for t in (values, row_indices, row_offsets, column_indices))
+    want = oracle.dense_to_csr(dense)
+    for got, ref in zip((values, row_indices, row_offsets, column_indices), want):
+        assert np.array_equal(got.cpu().numpy(), ref)
+    assert torch.equal(sparse_to_dense(197, 301, values, row_offsets, column_indices).cpu(), torch.from_numpy(dense))

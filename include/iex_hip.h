@@ -165,10 +165,20 @@ int iex_CudaSpmm5(int m, int k, int n, int nonzeros, const int* row_indices,
 /* ----------------------------------------------------------------- SDDMM ---- */
 #define IEX_SDDMM_SUM_OVER_BATCH 0x1 /* one (nnz) output summed over the batch            */
 #define IEX_SDDMM_ACCUMULATE 0x2     /* out += ... instead of out = ...                   */
-/* bits 8..15: force wavefronts per row (1 or 4); 0 = choose from nnz/m.  For tuning.     */
+/* bits 8..15: force wavefronts per row (1 or 4); 0 = choose from nnz/m.  For tuning.
+ * With variant 3 the same bits set the number of nonzeros from which a 128 x 128 block of the
+ * mask counts as dense: 0 = built in, 1 = every block, 255 = none, else 64 * value.       */
 #define IEX_SDDMM_FORCE_WPR(w) (((w) & 0xff) << 8)
-/* bits 16..19: 1 = the gather kernel, 7 = dense product in the caller's workspace, then
- * sampling (iex_sddmm_ws only; fails where it cannot run).  0 = choose.                  */
+/* bits 16..19: 1 = the gather kernel; 3 = the kernel for masks with structure (attention: bands,
+ * blocks, windows): per 128 rows, the dense 128 x 128 blocks of the mask get their scores from the
+ * matrix cores, sampled inside the workgroup and never stored, the nonzeros elsewhere one dot
+ * product each (fp16 / bf16, k = 32, 64 or 128, n <= 65536, plain store, one output per batch
+ * entry, strictly ascending columns inside a row; iex_sddmm_ws only: the workspace holds
+ * (6 ceil(n / 128) + 1) * m words -- per row and block of columns a cursor, a packed word and a
+ * 128-bit mask -- that a small kernel writes first, once for all batch entries); 7 = dense
+ * product in the caller's workspace, then sampling (iex_sddmm_ws only).
+ * 3 and 7 fail where they cannot run.  0 = choose: 3 when the mask is at least 3 % dense and
+ * batch * m * n is at least 2^25, else 7 or 1 by a time model.                              */
 #define IEX_SDDMM_FORCE_VARIANT(v) (((v) & 0xf) << 16)
 
 /* out[(z,) j] = sum_c lhs[z, row(j), c] * rhs[z, column_indices[j], c]
@@ -189,6 +199,7 @@ int iex_sddmm_ex(int dtype, int flags, int m, int k, int n, int nonzeros,
  * gradients of a sparse linear layer: k = tokens).  Same arithmetic per output (fp32 accumulation,
  * one rounding).  Needs plain store, (batch, nnz) output or batch 1, k and n multiples of 8;
  * anything else, and a NULL or short workspace, runs exactly as iex_sddmm_ex.
+ * The workspace also serves variant 3 above (short k, masks with structure), which 0 = choose picks first.
  * iex_sddmm_workspace_bytes returns the size with which the call described would use the
  * workspace, 0 when it would not whatever the size.  Neither call allocates.
  * No counterpart in the reference: CudaSddmm2 (csrc/extensions.h:31) takes no workspace. */

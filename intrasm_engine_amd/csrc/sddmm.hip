@@ -19,6 +19,7 @@
 #include <algorithm>
 #include <cmath>
 #include "iex_common.h"
+#include "sddmm_mfma_device.cuh"
 
 namespace iex {
 namespace {
@@ -286,6 +287,68 @@ int launch_sddmm_dense(int dtype, const SddmmParams& p, void* ws, hipStream_t st
   return 0;
 }
 
+// ---- score tiles on the matrix cores, sampled inside the workgroup (sddmm_mfma_device.cuh) ----
+// 16-bit types, k = 32, 64 or 128, plain store, one output per batch entry, canonical CSR (columns ascending and
+// distinct inside a row), n <= 128 * kSdMaxTiles; the workspace holds (6 ceil(n / 128) + 1) * m words (per row and
+// column tile: a 128-bit mask, a cursor, a packed word).
+inline bool sddmm_mfma_fits(int dtype, const SddmmParams& p) {
+  return (dtype == IEX_F16 || dtype == IEX_BF16) && !p.accumulate && !(p.sum_over_batch && p.batch > 1) &&
+         (p.k == 32 || p.k == 64 || p.k == 128) && aligned(p.lhs, 16) && aligned(p.rhs, 16) &&
+         ceil_div(p.n, kSdBN) <= kSdMaxTiles && (long long)(ceil_div(p.n, kSdBN) + 1) * p.m < (1ll << 28);
+}
+
+inline size_t sddmm_mfma_bytes(const SddmmParams& p) { return sddmm_mfma_words(p.m, ceil_div(p.n, kSdBN)) * sizeof(int); }
+
+// The host does not look at the pattern, so the choice goes by the mask's overall density.  Measured on MI355X
+// (fp16, 16 heads of 4096 x 4096, k = 64, microseconds, gather kernel / this kernel):
+//   band of 256 + 32 scattered per row (7 %)  119 /  64      band of 512 + 32 (13 %)      232 /  81
+//   band of 128 + 16 scattered (3.5 %)          74 /  53      block diagonal 256 (6 %)     102 /  38
+//   causal window of 512 (12 %)                191 /  62      band 256 + 128 scattered     150 / 109
+//   equal rows, columns at random:  1 %  32 / 40    3 %  57 / 80    5 %  98 / 120    10 %  171 / 225
+//                                  15 % 252 / 237  20 % 334 / 243
+// Masks with structure (what per-entry SDDMM is used for: attention) gain 1.4x to 3x from 3 % up; a mask without
+// any loses 1.2x to 1.3x below 15 %.  IEX_SDDMM_FORCE_VARIANT(1) keeps the gather kernel.
+inline bool sddmm_mfma_wins(const SddmmParams& p) {
+  const double density = (double)p.nnz / ((double)p.m * p.n);
+  return density >= 0.03 && (double)p.batch * p.m * p.n >= 32.0 * 1024 * 1024;
+}
+
+template <bool BF16, int KS>
+int launch_sddmm_mfma_ks(const SddmmMfmaParams& q, int batch, hipStream_t stream) {
+  constexpr int lds = sddmm_mfma_lds_bytes<KS>();
+  auto kernel = sddmm_mfma_kernel<BF16, KS>;
+  static thread_local bool raised = false;   // per instantiation: more than 64 KB of dynamic LDS
+  if (!raised) {
+    if (int rc = check_hip(hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, lds),
+                           "hipFuncSetAttribute(LDS size)"))
+      return rc;
+    raised = true;
+  }
+  note_kernel("sddmm_mfma_kernel<%s, %d>", BF16 ? "true" : "false", KS);
+  hipLaunchKernelGGL(kernel, dim3(ceil_div(q.m, kSdBM), batch), dim3(kSdThreads), lds, stream, q);
+  return check_hip(hipGetLastError(), "sddmm (matrix-core) launch");
+}
+
+int launch_sddmm_mfma(int dtype, const SddmmParams& p, void* ws, int dense_code, hipStream_t stream) {
+  const int tiles_n = ceil_div(p.n, kSdBN);
+  u32x4* mask = static_cast<u32x4*>(ws);
+  int* tile_ptr = reinterpret_cast<int*>(mask + (size_t)tiles_n * p.m);
+  int* brief = tile_ptr + (size_t)(tiles_n + 1) * p.m;
+  note_kernel("sddmm_tile_ptr_kernel");
+  hipLaunchKernelGGL(sddmm_tile_ptr_kernel, dim3(ceil_div(p.m, 4)), dim3(256), 0, stream, p.m, tiles_n, p.row_offsets, p.cols, tile_ptr, brief, mask);
+  if (int rc = check_hip(hipGetLastError(), "sddmm row-cursor launch")) return rc;
+  // dense_code (for tests and tuning): 0 = the built-in threshold, 1 = every tile on the matrix cores, 255 = none,
+  // else 64 * code nonzeros per 128 x 128 block
+  const int dense_min = dense_code == 0 ? kSdDenseMin : dense_code == 1 ? 0 : dense_code == 255 ? kSdBM * kSdBN + 1 : 64 * dense_code;
+  SddmmMfmaParams q{p.m, p.k, p.n, p.nnz, p.cols, p.lhs, p.rhs, p.out, mask, tile_ptr, brief, tiles_n, dense_min};
+  const bool bf16 = dtype == IEX_BF16;
+  switch (p.k) {
+    case 32: return bf16 ? launch_sddmm_mfma_ks<true, 2>(q, p.batch, stream) : launch_sddmm_mfma_ks<false, 2>(q, p.batch, stream);
+    case 64: return bf16 ? launch_sddmm_mfma_ks<true, 4>(q, p.batch, stream) : launch_sddmm_mfma_ks<false, 4>(q, p.batch, stream);
+    default: return bf16 ? launch_sddmm_mfma_ks<true, 8>(q, p.batch, stream) : launch_sddmm_mfma_ks<false, 8>(q, p.batch, stream);
+  }
+}
+
 }  // namespace
 
 // Bytes of workspace with which iex_sddmm_ws would compute the dense product and sample it (0: it
@@ -293,10 +356,12 @@ int launch_sddmm_dense(int dtype, const SddmmParams& p, void* ws, hipStream_t st
 size_t sddmm_workspace_bytes(int dtype, int flags, int m, int k, int n, int nonzeros, int batch) {
   if (m <= 0 || k <= 0 || n <= 0 || nonzeros <= 0 || batch <= 0) return 0;
   const int variant = (flags >> 16) & 0xf;
-  if (variant != 0 && variant != 7) return 0;
+  if (variant != 0 && variant != 7 && variant != 3) return 0;
   void* const some_aligned = reinterpret_cast<void*>(size_t(256));
   SddmmParams p{m, k, n, nonzeros, batch, nullptr, nullptr, nullptr, some_aligned, some_aligned, nullptr,
                 (flags & IEX_SDDMM_SUM_OVER_BATCH) != 0, (flags & IEX_SDDMM_ACCUMULATE) != 0};
+  if (variant != 7 && sddmm_mfma_fits(dtype, p) && (variant == 3 || sddmm_mfma_wins(p))) return sddmm_mfma_bytes(p);
+  if (variant == 3) return 0;
   if (!sddmm_dense_fits(dtype, p)) return 0;
   if (variant == 0 && !sddmm_dense_wins(p)) return 0;
   return sddmm_dense_bytes(p);
@@ -320,7 +385,16 @@ int sddmm_dispatch(int dtype, int flags, int m, int k, int n, int nonzeros, cons
   int wpr = (flags >> 8) & 0xff;  // forced (1 or 4), else from the mean row length
   if (wpr != 1 && wpr != 4) wpr = ((double)nonzeros / m >= 64.0) ? 4 : 1;
   hipStream_t s = static_cast<hipStream_t>(stream);
-  const int variant = (flags >> 16) & 0xf;  // 0 = choose, 1 = gather kernel, 7 = dense product then sampling
+  const int variant = (flags >> 16) & 0xf;  // 0 = choose, 1 = gather kernel, 3 = score tiles on the matrix cores, 7 = dense product then sampling
+  if (variant == 0 || variant == 3) {
+    const bool fits = sddmm_mfma_fits(dtype, p);
+    const bool room = workspace && aligned(workspace, 16) && workspace_bytes >= sddmm_mfma_bytes(p);
+    if (variant == 3) {
+      IEX_REQUIRE(fits, IEX_ERR_UNSUPPORTED, "sddmm: the matrix-core kernel needs fp16 / bf16, k = 32, 64 or 128, plain store, one output per batch entry and 16-byte aligned operands");
+      IEX_REQUIRE(room, IEX_ERR_BAD_ARGUMENT, "sddmm: the matrix-core kernel needs a 16-byte aligned workspace of %zu bytes (iex_sddmm_ws)", sddmm_mfma_bytes(p));
+    }
+    if (fits && room && (variant == 3 || sddmm_mfma_wins(p))) return launch_sddmm_mfma(dtype, p, workspace, variant == 3 ? (flags >> 8) & 0xff : 0, s);
+  }
   if (variant == 0 || variant == 7) {
     const bool fits = sddmm_dense_fits(dtype, p);
     const bool room = workspace && aligned(workspace, 16) && workspace_bytes >= sddmm_dense_bytes(p);

@@ -1,0 +1,527 @@
+// CSR SDDMM for attention-like masks (gfx950, fp16 / bf16, k = 32, 64 or 128): where the mask is dense the scores
+// come from the matrix cores, tile by tile, and are sampled inside the workgroup without ever being stored; where it
+// is thin the few dot products are computed one by one.
+//
+// The gather kernel (sddmm.hip) reads k * 2 bytes of rhs per nonzero through the L2 -> CU path; for an attention
+// mask (a dense band plus scattered entries, 5-10 % dense) that is 2.4 GB per 16 heads and that path is what bounds
+// it.  A dense product of everything (34 GFLOP) is cheap on the matrix cores but wasted on the nine tenths of the
+// 128 x 128 tiles that hold one entry per row.  So a workgroup (4 wavefronts) owns 128 consecutive rows of one batch
+// entry and sorts the column tiles (128 columns each) of its rows by how many nonzeros they hold:
+//   * dense tiles (dense_min nonzeros or more in the 128 x 128 block): the rhs rows of the tile come from global
+//     memory straight into LDS (global_load_lds_dwordx4, double-buffered, 16-byte chunks permuted so that the
+//     operand reads are conflict-free), 2 x 2 x k/16 MFMAs of 32 x 32 x 16 per wavefront (each owns 64 x 64 of the
+//     tile; the lhs fragments stay in registers for the whole phase), operands swapped so that a lane ends up with
+//     4 adjacent columns of one row and writes them to the score tile in LDS with one 64-bit store, already rounded
+//     to the element type.  Sampling, two ways per (row, tile): up to 4 nonzeros -> the row's own lane (threads
+//     0..127) copies the scores named by a packed word; more -> a wavefront takes the row: a 128-bit mask of the
+//     row's columns in the tile tells each lane whether its two columns are present and, by a population count
+//     of the bits below, where in the row's output they go; the stores of a row are contiguous.  No column index
+//     is read from memory in this phase.
+//   * thin tiles: a wavefront lays the nonzeros that its 32 rows have there end to end (a list in LDS, so that rows
+//     of different lengths cost no idle lanes) and takes them 64 at a time, k/8 lanes per nonzero: 16 bytes of
+//     the rhs row per lane from memory, of the lhs row from LDS, v_dot2 in fp32, summed across the lanes, rounded
+//     once; the results are stored 64 at a time.
+// What the kernel needs to know about the mask comes from a small kernel that runs first, once per call for all
+// batch entries, into the caller's workspace: tile_ptr[t][row] = position of the row's first nonzero with column
+// >= 128 t (columns ascend inside a row), brief[t][row] = count and in-tile columns of up to 4 nonzeros, packed in
+// one word, and mask[t][row] for the pairs with more.
+// The dense phase runs on a hand-counted pipeline: all its global reads (rhs rows for the next dense tile, the
+// per-row words two dense tiles ahead) are direct-to-LDS loads in inline assembly, invisible to the compiler's
+// wait-count pass; each wavefront issues a fixed number of them per tile and waits with s_waitcnt vmcnt(N), N =
+// the loads it issued after the ones it needs (the counter retires loads in order, and the stores of the previous
+// tile's sampling are older than these loads, so nothing ever waits for the current tile's stores).  The
+// workgroup barriers in that loop wait for LDS traffic only.
+#pragma once
+#include "gemm_dma_device.cuh"
+
+namespace iex {
+
+constexpr int kSdBM = 128, kSdBN = 128, kSdThreads = 256;
+constexpr int kSdShort = 4;           // nonzeros of a (row, tile) pair that the row's own lane samples
+constexpr int kSdLd = kSdBN + 8;      // halves per row of the score tile (272 bytes)
+constexpr int kSdMaxTiles = 512;      // column tiles per row (n <= 65536): the tile list lives in LDS
+constexpr int kSdDenseMin = 2048;     // nonzeros in a 128 x 128 block from which its scores come from the matrix cores
+constexpr int kSdSlot = kSdBM * (4 + 4 + 16);   // bytes of per-row words of one dense tile: cursor, packed word, mask
+
+struct SddmmMfmaParams {
+  int m, k, n, nnz;
+  const int* cols;
+  const void* lhs;
+  const void* rhs;
+  void* out;
+  const u32x4* mask;     // [tiles_n][m], written only where brief says "more than kSdShort"
+  const int* tile_ptr;   // [(tiles_n + 1)][m]
+  const int* brief;      // [tiles_n][m]
+  int tiles_n;
+  int dense_min;
+};
+
+// Workgroup barrier for LDS traffic only.  __syncthreads() also waits until the thread's global stores have
+// reached L2; in a loop that stores every iteration that is a round trip to L2 per iteration.
+__device__ __forceinline__ void lds_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
+
+// 4 bytes per lane from global memory straight into LDS at lds_base_uniform + 4 * lane.
+__device__ __forceinline__ void lds_dma4(const void* g, unsigned lds_base_uniform) {
+  asm volatile("s_mov_b32 m0, %1\n\tglobal_load_lds_dword %0, off" ::"v"(g), "s"(lds_base_uniform) : "memory", "m0");
+}
+
+template <int CTRL>
+__device__ __forceinline__ unsigned dpp_u(unsigned v) {
+  return (unsigned)__builtin_amdgcn_update_dpp(0, (int)v, CTRL, 0xf, 0xf, true);
+}
+__device__ __forceinline__ unsigned wave_sum_u(unsigned v) {
+  v += dpp_u<0xB1>(v);
+  v += dpp_u<0x4E>(v);
+  v += dpp_u<0x141>(v);
+  v += dpp_u<0x140>(v);
+  return (unsigned)bcast_i((int)v, 0) + (unsigned)bcast_i((int)v, 16) + (unsigned)bcast_i((int)v, 32) + (unsigned)bcast_i((int)v, 48);
+}
+
+template <int KS>
+constexpr int sddmm_mfma_lds_bytes() {
+  return kSdBM * kSdLd * 2 + 2 * kSdBN * KS * 32 + 3 * kSdSlot + 16 + kSdMaxTiles * 2 + 16;
+}
+
+// Words of workspace per call: masks first (16-byte entries), then the cursors, then the packed words.
+inline size_t sddmm_mfma_words(int m, int tiles_n) { return (size_t)m * (4 * (size_t)tiles_n + (tiles_n + 1) + tiles_n); }
+
+// tile_ptr[t][row] for t = 0 .. tiles_n, brief[t][row] and (where needed) mask[t][row] for t < tiles_n: one
+// wavefront per row.  brief packs what a lane needs to sample a (row, tile) pair without touching the column indices
+// again: bits 28..30 = number of nonzeros of the row in the tile (0..4, or 7 for "more"), bits 7u .. 7u + 6 =
+// column of nonzero u inside the tile.  The mask of a pair with more has bit c set when column 128 t + c is present.
+// The row's columns are first marked in a bit map in LDS (n bits); counts, cursors and packed words come from the
+// map, 64 tiles at a time, one tile per lane.
+__global__ __launch_bounds__(256) void sddmm_tile_ptr_kernel(int m, int tiles_n, const int* __restrict__ row_offsets,
+                                                             const int* __restrict__ cols, int* __restrict__ tile_ptr,
+                                                             int* __restrict__ brief, u32x4* __restrict__ mask) {
+  __shared__ unsigned bits[4][kSdMaxTiles * 4];
+  const int lane = lane_id();
+  const int wave = threadIdx.x >> 6;
+  const int r = blockIdx.x * 4 + wave;
+  if (r >= m) return;   // (no workgroup barrier below: every wavefront works alone)
+  unsigned* mine = bits[wave];
+  const int s = uniform(row_offsets[r]), e = uniform(row_offsets[r + 1]);
+  for (int i = lane; i < tiles_n * 4; i += kWave) mine[i] = 0;
+  __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+  __builtin_amdgcn_wave_barrier();
+  for (int base = s; base < e; base += 4 * kWave) {   // four loads in flight
+    int c[4];
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      const int j = base + u * kWave + lane;
+      c[u] = j < e ? cols[j] : -1;
+    }
+#pragma unroll
+    for (int u = 0; u < 4; ++u)
+      if (c[u] >= 0) atomicOr(&mine[min(c[u] >> 5, tiles_n * 4 - 1)], 1u << (c[u] & 31));
+  }
+  __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+  __builtin_amdgcn_wave_barrier();
+  int running = s;   // position of the first nonzero of tile base_t
+  for (int base_t = 0; base_t < tiles_n; base_t += kWave) {
+    const int t = base_t + lane;
+    const bool in = t < tiles_n;
+    u32x4 w = {0u, 0u, 0u, 0u};
+    if (in) w.x = mine[t * 4], w.y = mine[t * 4 + 1], w.z = mine[t * 4 + 2], w.w = mine[t * 4 + 3];
+    const int count = __popc(w.x) + __popc(w.y) + __popc(w.z) + __popc(w.w);
+    int upto = count;   // inclusive prefix sum over the 64 tiles
+#pragma unroll
+    for (int d = 1; d < kWave; d <<= 1) {
+      const int v = __shfl_up(upto, d, kWave);
+      if (lane >= d) upto += v;
+    }
+    if (in) {
+      tile_ptr[(size_t)t * m + r] = running + upto - count;
+      int word = (count <= kSdShort ? count : 7) << 28;
+      if (count > kSdShort) {
+        mask[(size_t)t * m + r] = w;
+      } else {
+        unsigned left[4] = {w.x, w.y, w.z, w.w};
+#pragma unroll
+        for (int u = 0; u < kSdShort; ++u) {   // the u-th lowest set bit of the 128
+          int at = -1;
+#pragma unroll
+          for (int q = 3; q >= 0; --q)
+            if (left[q]) at = q;
+          if (at >= 0) {
+            const unsigned v = at == 0 ? left[0] : at == 1 ? left[1] : at == 2 ? left[2] : left[3];
+            word |= (at * 32 + __builtin_ctz(v)) << (7 * u);
+#pragma unroll
+            for (int q = 0; q < 4; ++q)
+              if (q == at) left[q] = v & (v - 1);
+          }
+        }
+      }
+      brief[(size_t)t * m + r] = word;
+    }
+    running += __builtin_amdgcn_readlane(upto, kWave - 1);
+  }
+  if (lane == 0) tile_ptr[(size_t)tiles_n * m + r] = e;
+}
+
+// acc + <a, b> over 8 elements of 16 bits, products and sums in fp32
+template <bool BF16>
+__device__ __forceinline__ float dot8(u32x4 a, u32x4 b, float acc) {
+  typedef _Float16 h2 __attribute__((ext_vector_type(2)));
+  typedef __bf16 b2 __attribute__((ext_vector_type(2)));
+  const unsigned aw[4] = {a.x, a.y, a.z, a.w}, bw[4] = {b.x, b.y, b.z, b.w};
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    if constexpr (BF16)
+      acc = __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(b2, aw[i]), __builtin_bit_cast(b2, bw[i]), acc, false);
+    else
+      acc = __builtin_amdgcn_fdot2(__builtin_bit_cast(h2, aw[i]), __builtin_bit_cast(h2, bw[i]), acc, false);
+  }
+  return acc;
+}
+
+template <bool BF16, int KS>
+__global__ __launch_bounds__(kSdThreads, KS == 8 ? 1 : 2) void sddmm_mfma_kernel(SddmmMfmaParams p) {
+  constexpr int RB = KS * 32;            // bytes of a k row
+  constexpr int CH = RB / 16;            // 16-byte chunks per k row
+  constexpr int RPI = kWave / CH;        // rhs rows per direct load
+  constexpr int STAGE = kSdBN * RB;
+  static_assert(KS == 2 || KS == 4 || KS == 8, "k = 32, 64 or 128");
+  typedef unsigned short u16;
+  typedef __attribute__((address_space(3))) unsigned char lds_u8;
+  extern __shared__ __align__(16) unsigned char smem[];
+  u16* S = reinterpret_cast<u16*>(smem);                                      // [128][kSdLd]; before the loop: column sums
+  unsigned char* sR = smem + kSdBM * kSdLd * 2;                               // [2][128][RB]
+  unsigned char* sM = sR + 2 * STAGE;                                         // [3] slots of per-row words
+  unsigned long long* long_rows = reinterpret_cast<unsigned long long*>(sM + 3 * kSdSlot);   // [2] rows with more than kSdShort
+  u16* list = reinterpret_cast<u16*>(long_rows + 2);                          // [tiles_n] dense tiles from the front, thin from the back
+  int* n_dense = reinterpret_cast<int*>(list + kSdMaxTiles);
+  const unsigned ldsR = (unsigned)(size_t)(lds_u8*)sR;
+  const unsigned ldsM = (unsigned)(size_t)(lds_u8*)sM;
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int wr = wave >> 1, wc = wave & 1;
+  // Workgroups go to the 8 XCDs round-robin by their linear id; renumbered so that an XCD gets all row blocks of
+  // a batch entry (and then of the next): the rhs rows they all read stay in that XCD's L2.
+  const int row_blocks = gridDim.x, total = row_blocks * gridDim.y;
+  int id = blockIdx.x + row_blocks * blockIdx.y;
+  // The two workgroups that share a CU take the two phases below in opposite order, so that one phase's matrix-core
+  // and LDS work runs beside the other's waiting for memory.  (Which two share a CU is the dispatcher's business:
+  // neighbours in launch order on the XCD, or 32 apart; the parity below differs in both cases.)
+  const int launch_slot = id / 8;
+  const bool thin_first = ((launch_slot ^ (launch_slot >> 5)) & 1) != 0;
+  if (total % 8 == 0) id = (id % 8) * (total / 8) + id / 8;
+  const int z = id / row_blocks;
+  const int row0 = (id % row_blocks) * kSdBM;
+  const u16* __restrict__ lhs = static_cast<const u16*>(p.lhs) + (size_t)z * p.m * p.k;
+  const unsigned char* rhs = reinterpret_cast<const unsigned char*>(static_cast<const u16*>(p.rhs) + (size_t)z * p.n * p.k);
+  u16* __restrict__ out = static_cast<u16*>(p.out) + (size_t)z * p.nnz;
+  const int tiles_n = p.tiles_n;
+
+  // ---- which tiles are dense: nonzeros of the 128 rows in tile t = sum over rows of tile_ptr[t + 1] - tile_ptr[t]
+  {
+    unsigned* colsum = reinterpret_cast<unsigned*>(S);
+    const int ra = min(row0 + lane, p.m - 1), rb = min(row0 + kWave + lane, p.m - 1);
+    for (int t0 = wave; t0 <= tiles_n; t0 += 32) {   // 8 tiles per step: 16 loads in flight
+      unsigned v[8];
+#pragma unroll
+      for (int u = 0; u < 8; ++u) {
+        const int t = min(t0 + 4 * u, tiles_n);
+        v[u] = (unsigned)p.tile_ptr[(size_t)t * p.m + ra] + (unsigned)p.tile_ptr[(size_t)t * p.m + rb];
+      }
+#pragma unroll
+      for (int u = 0; u < 8; ++u) {
+        const unsigned sum = wave_sum_u(v[u]);
+        if (lane == 0 && t0 + 4 * u <= tiles_n) colsum[t0 + 4 * u] = sum;
+      }
+    }
+    __syncthreads();
+    if (wave == 0) {
+      int nd = 0, ns = 0;
+      for (int base = 0; base < tiles_n; base += kWave) {
+        const int t = base + lane;
+        const bool in = t < tiles_n;
+        const int tc = min(t, tiles_n - 1);
+        const bool dense = in && (int)(colsum[tc + 1] - colsum[tc]) >= p.dense_min;
+        const unsigned long long dm = __ballot(dense), sm = __ballot(in && !dense);
+        const unsigned long long below = (1ull << lane) - 1;
+        if (dense) list[nd + __popcll(dm & below)] = (u16)t;
+        if (in && !dense) list[tiles_n - 1 - ns - __popcll(sm & below)] = (u16)t;
+        nd += __popcll(dm);
+        ns += __popcll(sm);
+      }
+      if (lane == 0) *n_dense = nd;
+    }
+    __syncthreads();
+  }
+  const int nd = __builtin_amdgcn_readfirstlane(*n_dense);
+
+  for (int phase = 0; phase < 2; ++phase) {
+  // ---- dense tiles
+  if ((phase == 0) != thin_first) {
+   if (nd > 0) {
+    auto sw = [](int row) { return CH == 4 ? (row >> 2) & 3 : CH == 8 ? (row >> 1) & 7 : row & 15; };
+    // direct loads of one tile of rhs rows: instruction g = wave * KS + q fills rows g * RPI .. + RPI - 1
+    const int dl_row = lane / CH, dl_slot = lane % CH;
+    auto issue_rows = [&](int i) {   // the i-th dense tile (past the end the last one again, into a stage nobody reads)
+      const int ct = __builtin_amdgcn_readfirstlane((int)list[min(i, nd - 1)]);
+      const unsigned base = ldsR + (i & 1) * STAGE;
+#pragma unroll
+      for (int q = 0; q < KS; ++q) {
+        const int row = (wave * KS + q) * RPI + dl_row;
+        const int grow = min(ct * kSdBN + row, p.n - 1);   // past the last column: a valid row nobody samples
+        lds_dma16(rhs + (size_t)grow * RB + ((dl_slot ^ sw(row)) << 4), __builtin_amdgcn_readfirstlane(base + (wave * KS + q) * 1024));
+      }
+    };
+    // per-row words of the i-th dense tile: wavefronts 0, 1 fetch cursor and packed word of their 64 rows (two
+    // loads each), wavefronts 2, 3 the masks of 64 rows (one load each)
+    const int meta_row = min(row0 + (wave & 1) * kWave + lane, p.m - 1);
+    auto issue_words = [&](int i) {
+      const int ct = __builtin_amdgcn_readfirstlane((int)list[min(i, nd - 1)]);
+      const unsigned base = ldsM + (i % 3) * kSdSlot;
+      if (wave < 2) {
+        lds_dma4(p.tile_ptr + (size_t)ct * p.m + meta_row, __builtin_amdgcn_readfirstlane(base + wave * 256));
+        lds_dma4(p.brief + (size_t)ct * p.m + meta_row, __builtin_amdgcn_readfirstlane(base + 512 + wave * 256));
+      } else {
+        lds_dma16(p.mask + (size_t)ct * p.m + meta_row, __builtin_amdgcn_readfirstlane(base + 1024 + (wave - 2) * 1024));
+      }
+    };
+    issue_rows(0);
+    issue_words(0);
+    issue_rows(1);
+    issue_words(1);
+
+    // this wavefront's lhs fragments: rows wr * 64 + i * 32 + lane % 32, k entries ks * 16 + (lane / 32) * 8 .. + 7
+    const int frag_row = lane & 31, frag_k = (lane >> 5) * 8;
+    u32x4 fl[2][KS];
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+      const int row = min(row0 + wr * 64 + i * 32 + frag_row, p.m - 1);
+#pragma unroll
+      for (int ks = 0; ks < KS; ++ks) fl[i][ks] = *reinterpret_cast<const u32x4*>(lhs + (size_t)row * p.k + ks * 16 + frag_k);
+    }
+    const bool owner = tid < kSdBM && row0 + tid < p.m;   // threads 0..127: one row each
+
+    wait_vmcnt<0>();        // the first tile's rhs rows, the first words and the lhs fragments have landed
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+      for (int ks = 0; ks < KS; ++ks) asm volatile("" : "+v"(fl[i][ks]));
+
+    for (int i = 0; i < nd; ++i) {
+      lds_barrier();        // everybody's loads for this tile have landed; the previous tile's sampling is over
+      const unsigned char* slot = sM + (i % 3) * kSdSlot;
+      int pk = 0, tp = 0;
+      if (tid < kSdBM) {
+        tp = reinterpret_cast<const int*>(slot)[tid];
+        pk = reinterpret_cast<const int*>(slot + 512)[tid];
+      }
+      const int count = owner ? (pk >> 28) & 7 : 0;
+      const unsigned long long longs = __ballot(count == 7);
+      if (tid < kSdBM && lane == 0) long_rows[wave] = longs;
+
+      // ---- scores of the tile: S[r][c] = <lhs[r], rhs[c0 + c]>, rounded to the element type
+      f32x16 acc[2][2];
+#pragma unroll
+      for (int a = 0; a < 2; ++a)
+#pragma unroll
+        for (int b = 0; b < 2; ++b)
+#pragma unroll
+          for (int r = 0; r < 16; ++r) acc[a][b][r] = 0.f;
+      const unsigned char* stage = sR + (i & 1) * STAGE;
+#pragma unroll
+      for (int ks = 0; ks < KS; ++ks) {
+        u32x4 fr[2];
+#pragma unroll
+        for (int b = 0; b < 2; ++b) {
+          const int c = wc * 64 + b * 32 + frag_row;
+          fr[b] = *reinterpret_cast<const u32x4*>(stage + c * RB + (((ks * 2 + (lane >> 5)) ^ sw(c)) << 4));
+        }
+#pragma unroll
+        for (int a = 0; a < 2; ++a)
+#pragma unroll
+          for (int b = 0; b < 2; ++b) acc[a][b] = mfma_32x32x16<BF16>(fr[b], fl[a][ks], acc[a][b]);
+      }
+#pragma unroll
+      for (int a = 0; a < 2; ++a)
+#pragma unroll
+        for (int b = 0; b < 2; ++b)
+#pragma unroll
+          for (int q = 0; q < 4; ++q) {
+            u16 h[4];
+#pragma unroll
+            for (int e = 0; e < 4; ++e) h[e] = f32_to_16(acc[a][b][q * 4 + e], BF16);
+            u32x2 w;
+            w.x = (unsigned)h[0] | ((unsigned)h[1] << 16);
+            w.y = (unsigned)h[2] | ((unsigned)h[3] << 16);
+            *reinterpret_cast<u32x2*>(S + (wr * 64 + a * 32 + frag_row) * kSdLd + wc * 64 + b * 32 + q * 8 + (lane >> 5) * 4) = w;
+          }
+      // The next tile's rhs rows and words, asked for a whole tile ago (below, before the previous tile's
+      // sampling), must have landed before the barrier.
+      wait_vmcnt<0>();
+      lds_barrier();
+      issue_rows(i + 2);    // into the stage whose MFMAs everybody has just finished
+      issue_words(i + 2);   // into the slot of the tile before this one
+
+      // ---- sampling: short runs by the row's own lane
+      if (count >= 1 && count <= kSdShort) {
+#pragma unroll
+        for (int u = 0; u < kSdShort; ++u)
+          if (u < count) out[tp + u] = S[tid * kSdLd + ((pk >> (7 * u)) & 127)];
+      }
+      // long runs: this wavefront takes rows 32 * wave .. + 31, four at a time; every lane reads the row's mask and
+      // cursor itself (the same LDS address for all lanes: a broadcast)
+      unsigned todo = (unsigned)(long_rows[wave >> 1] >> ((wave & 1) * 32));
+      todo = __builtin_amdgcn_readfirstlane(todo);
+      while (todo) {
+        int rr[4];
+        bool on[4];
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+          on[u] = todo != 0;
+          rr[u] = wave * 32 + (todo ? __builtin_ctz(todo) : 0);
+          todo &= todo - 1;
+        }
+        u32x4 mk[4];
+        int start[4];
+        u16 lo[4], hi[4];
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+          mk[u] = *reinterpret_cast<const u32x4*>(slot + 1024 + rr[u] * 16);
+          start[u] = reinterpret_cast<const int*>(slot)[rr[u]];
+          lo[u] = S[rr[u] * kSdLd + lane];
+          hi[u] = S[rr[u] * kSdLd + kWave + lane];
+        }
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+          if (!on[u]) continue;
+          const int half = __popc(mk[u].x) + __popc(mk[u].y);
+          const int rank_lo = __builtin_amdgcn_mbcnt_hi(mk[u].y, __builtin_amdgcn_mbcnt_lo(mk[u].x, 0));
+          const int rank_hi = __builtin_amdgcn_mbcnt_hi(mk[u].w, __builtin_amdgcn_mbcnt_lo(mk[u].z, 0)) + half;
+          const unsigned word_lo = lane < 32 ? mk[u].x : mk[u].y, word_hi = lane < 32 ? mk[u].z : mk[u].w;
+          if ((word_lo >> (lane & 31)) & 1) out[min(start[u] + rank_lo, p.nnz - 1)] = lo[u];
+          if ((word_hi >> (lane & 31)) & 1) out[min(start[u] + rank_hi, p.nnz - 1)] = hi[u];
+        }
+      }
+    }
+    wait_vmcnt<0>();   // the loads issued past the last dense tile: nothing may still be writing LDS when the phase ends
+   }
+  } else {
+
+  // ---- thin tiles.  A wavefront serves its 32 rows.  The nonzeros of a row between two dense tiles are
+  // consecutive in the row (columns ascend): one stretch of the CSR arrays per row and run of thin tiles.  The
+  // stretches of the 32 rows and of as many runs as fit (at most 32 nonzeros per row and run at a time) are laid
+  // end to end as a list of (column, row) entries in LDS, with the position of each in the output beside it, so
+  // that the work is the same for every lane whatever the rows' lengths; then, 64 entries per step, LPN lanes per
+  // entry: each lane reads 16 bytes of the entry's rhs row from memory (a load instruction covers whole rows) and
+  // of its lhs row from LDS, v_dot2 in fp32, summed over the LPN lanes, and lane i keeps the result of entry i of
+  // the step.  Results replace their entries and go to memory 64 at a time at the end: the loop holds no global
+  // store (its waits for loads never sit out a store's round trip) and the loads of the next step are in flight
+  // while this one computes.
+  {
+    constexpr int LPN = CH;              // lanes per nonzero
+    constexpr int LROW = RB + 16;        // bytes per lhs row in LDS (padded: rows start 4 banks apart)
+    constexpr int CAP = 1024;            // entries of a wavefront's list
+    constexpr int CAPR = 32;             // nonzeros a row contributes per run and round
+    const int sl = lane % LPN, g = lane / LPN;
+    unsigned* ent = reinterpret_cast<unsigned*>(smem) + wave * (2 * CAP);          // in the score tile: [CAP] entries,
+    int* pos = reinterpret_cast<int*>(ent + CAP);                                  // [CAP] output positions
+    unsigned char* lrows = sR + wave * (32 * LROW);
+    for (int i = lane; i < 32 * CH; i += kWave) {
+      const int r = i / CH, ch = i % CH;
+      const int gr = min(row0 + wave * 32 + r, p.m - 1);
+      *reinterpret_cast<u32x4*>(lrows + r * LROW + ch * 16) = *reinterpret_cast<const u32x4*>(lhs + (size_t)gr * p.k + ch * 8);
+    }
+    const int* __restrict__ cols = p.cols;
+    // lanes 0..31 hold the bounds of the wavefront's rows; when the list is built, lanes 0..31 serve an even row
+    // and lanes 32..63 the odd row after it
+    const int hl = lane & 31, hsel = lane >> 5;
+    const int my_row = row0 + wave * 32 + hl;
+    const bool valid = lane < 32 && my_row < p.m;
+    const int grow = min(my_row, p.m - 1);
+    int T = 0;   // entries in the list
+
+    auto fetch = [&](int base, unsigned& w, u32x4 (&rv)[LPN]) {
+      w = ent[min(base + lane, T - 1)];
+#pragma unroll
+      for (int u = 0; u < LPN; ++u) {
+        const unsigned wu = (unsigned)__shfl((int)w, g * LPN + u, kWave);
+        rv[u] = *reinterpret_cast<const u32x4*>(rhs + (size_t)(wu >> 5) * RB + sl * 16);
+      }
+    };
+    auto finish = [&](int base, unsigned w, u32x4 (&rv)[LPN]) {
+      float res = 0.f;
+#pragma unroll
+      for (int u = 0; u < LPN; ++u) {
+        const unsigned wu = (unsigned)__shfl((int)w, g * LPN + u, kWave);
+        const u32x4 lf = *reinterpret_cast<const u32x4*>(lrows + (wu & 31) * LROW + sl * 16);
+        const float acc = group_sum<LPN>(dot8<BF16>(lf, rv[u], 0.f));
+        res = sl == u ? acc : res;
+      }
+      if (base + lane < T) ent[base + lane] = (unsigned)f32_to_16(res, BF16);
+    };
+    auto work_off = [&]() {   // the list: compute, store, empty
+      if (T > 0) {
+        __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        unsigned wa, wb;
+        u32x4 rva[LPN], rvb[LPN];
+        fetch(0, wa, rva);
+        for (int base = 0; base < T; base += 2 * kWave) {
+          const bool second = base + kWave < T;
+          if (second) fetch(base + kWave, wb, rvb);
+          finish(base, wa, rva);
+          if (second) {
+            if (base + 2 * kWave < T) fetch(base + 2 * kWave, wa, rva);
+            finish(base + kWave, wb, rvb);
+          }
+        }
+        __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        for (int i = lane; i < T; i += kWave) out[pos[i]] = (u16)ent[i];
+        __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+      }
+      T = 0;
+    };
+
+    for (int run = 0; run <= nd; ++run) {
+      const int a = run == 0 ? 0 : __builtin_amdgcn_readfirstlane((int)list[run - 1]) + 1;
+      const int b = run == nd ? tiles_n : __builtin_amdgcn_readfirstlane((int)list[run]);
+      if (a >= b) continue;   // two dense tiles side by side
+      int s = p.tile_ptr[(size_t)a * p.m + grow];
+      const int e = valid ? p.tile_ptr[(size_t)b * p.m + grow] : s;
+      while (__ballot(s < e)) {
+        const int len = min(max(e - s, 0), CAPR);
+        int upto = len;   // inclusive prefix sum over lanes 0..31
+#pragma unroll
+        for (int d = 1; d < 32; d <<= 1) {
+          const int t = __shfl_up(upto, d, kWave);
+          if (lane >= d) upto += t;
+        }
+        const int before = upto - len;
+        const int round_total = __builtin_amdgcn_readlane(upto, 31);
+        if (T + round_total > CAP) work_off();
+        int sr[16], cv[16];
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+          sr[i] = __shfl(s, 2 * i + hsel, kWave);
+          cv[i] = cols[min(sr[i] + hl, p.nnz - 1)];
+        }
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+          const int lr = __shfl(len, 2 * i + hsel, kWave), pr = __shfl(before, 2 * i + hsel, kWave);
+          if (hl < lr) {
+            ent[T + pr + hl] = ((unsigned)cv[i] << 5) | (unsigned)(2 * i + hsel);
+            pos[T + pr + hl] = sr[i] + hl;
+          }
+        }
+        T += round_total;
+        s += len;
+      }
+    }
+    work_off();
+  }
+  }
+  __syncthreads();   // the score tile changes hands: sampled by one phase, collecting results in the other
+  }
+}
+
+}  // namespace iex

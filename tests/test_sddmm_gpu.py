@@ -53,13 +53,18 @@ def test_config3_fp16_per_head_then_spmm(oracle, dev):
 
 def test_full_size_config3_properties(dev):
     """All 16 heads: (a) every head of the batched launch equals the same head launched alone
-    (bit-exact), (b) the diagonal entries equal the row-wise dot products <q_i, k_i>."""
+    (bit-exact, kernel by kernel: which one the library picks by itself depends on the amount of work),
+    (b) the diagonal entries equal the row-wise dot products <q_i, k_i>."""
+    from intrasm_engine_amd.pytorch import ops as pyops
     pattern, q, k, _ = W.config3()
     ri, _, ro, ci = to_dev(pattern, dev)
     qt, kt = torch.from_numpy(q).to(dev).half(), torch.from_numpy(k).to(dev).half()
+    for variant in (1, 3):
+        with pyops.kernel_params(sddmm={"force_variant": variant}):
+            out = ops.sddmm_sputnik_half(qt, kt, ri, ro, ci)
+            for h in (0, 7, 15):
+                assert torch.equal(ops.sddmm_sputnik_half(qt[h:h + 1].contiguous(), kt[h:h + 1].contiguous(), ri, ro, ci)[0], out[h]), (variant, h)
     out = ops.sddmm_sputnik_half(qt, kt, ri, ro, ci)
-    for h in (0, 7, 15):
-        assert torch.equal(ops.sddmm_sputnik_half(qt[h:h + 1].contiguous(), kt[h:h + 1].contiguous(), ri, ro, ci)[0], out[h])
     rows = torch.repeat_interleave(torch.arange(pattern.m, device=dev), torch.diff(ro.long()))
     diag = (rows == ci.long()).nonzero().squeeze(1)
     assert diag.numel() == pattern.m
@@ -220,7 +225,9 @@ def test_dense_product_path_is_chosen_with_a_workspace_and_only_then(oracle, dev
     assert lib.iex_sddmm_workspace_bytes(_lib.F16, _lib.SDDMM_SUM_OVER_BATCH, m, k, n, nnz, 2) == 0
     assert lib.iex_sddmm_workspace_bytes(_lib.F16, _lib.SDDMM_SUM_OVER_BATCH, m, k, n, nnz, 1) == need
     assert lib.iex_sddmm_workspace_bytes(_lib.F16, _lib.SDDMM_ACCUMULATE, m, k, n, nnz, 1) == 0
-    assert lib.iex_sddmm_workspace_bytes(_lib.F16, 0, 4096, 64, 4096, 1150000, 16) == 0   # config 3: the gather kernel is faster
+    # config 3: not the dense product; the tables of the kernel that samples score tiles inside the workgroup
+    assert lib.iex_sddmm_workspace_bytes(_lib.F16, 0, 4096, 64, 4096, 1150000, 16) == (6 * 32 + 1) * 4096 * 4
+    assert lib.iex_sddmm_workspace_bytes(_lib.F16, 0, 4096, 64, 4096, 1150000 // 4, 16) == 0   # a mask this thin: the gather kernel
     assert lib.iex_sddmm_workspace_bytes(_lib.F16, 7 << 16, 4096, 64, 4096, 1150000, 16) == 4096 * 4096 * 2  # on request
     kw = dict(sum_over_batch=False, dtypes=(dtype,))
     auto = pyops._sddmm(lhs, rhs, ri, ro, ci, **kw)

@@ -1,0 +1,117 @@
+"""The SDDMM kernel for attention-like masks (variant 3: score tiles of the dense blocks on the matrix cores,
+sampled inside the workgroup; the nonzeros of thin blocks one dot product at a time): parity with the CPU oracle on
+ragged shapes and on config 3, forced and where the library picks it, with every block treated as dense, every
+block as thin, and with the built-in threshold."""
+import numpy as np
+import pytest
+import torch
+
+from intrasm_engine_amd import workloads as W
+from _util import FP16_SUBNORMAL_HALF_STEP, RTOL, assert_close, rounded, to_dev
+
+pytestmark = pytest.mark.gpu
+ops = torch.ops.iex_ops
+
+
+def _run(dev, csr, lhs, rhs, dtype, **force):
+    from intrasm_engine_amd.pytorch import ops as pyops
+    ri, _, ro, ci = to_dev(csr, dev)
+    lt, rt = torch.from_numpy(lhs).to(dev).to(dtype), torch.from_numpy(rhs).to(dev).to(dtype)
+    return pyops._sddmm(lt, rt, ri, ro, ci, sum_over_batch=False, dtypes=(dtype,), **force)
+
+
+def _want(oracle, csr, lhs, rhs, dtype):
+    l16, r16 = rounded(lhs, dtype), rounded(rhs, dtype)
+    want = oracle.sddmm(l16, r16, csr.row_indices, csr.row_offsets, csr.column_indices, sum_over_batch=False)
+    scale = oracle.sddmm_abs_scale(l16, r16, csr.row_indices, csr.row_offsets, csr.column_indices, sum_over_batch=False)
+    return want, scale
+
+
+@pytest.mark.parametrize("k", [32, 64, 128])
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("m,n", [(131, 97), (300, 517), (128, 128)])
+@pytest.mark.parametrize("blocks", [0, 1, 255, 2])      # threshold: built-in, all dense, all thin, 128 nonzeros
+def test_ragged_shapes_forced(oracle, dev, k, dtype, m, n, blocks):
+    """m and n that are no multiples of the 128 x 128 tile, empty rows, a completely dense row (more than 64
+    nonzeros in one tile: both sampling steps), rows of 1 to 4 nonzeros per tile (the row's own lane) and of 5 and
+    more (the wavefront), two batch entries."""
+    rng = np.random.default_rng(k + m)
+    lens = rng.integers(0, min(n, 40), m)
+    lens[[0, 9, m - 1]] = 0
+    lens[5] = n
+    lens[6] = min(n, 70)
+    ro, ci = W.csr_from_row_lengths(rng, m, n, lens)
+    csr = W.CSR(m, n, np.ones(ci.shape[0], np.float32), W.swizzle_from_offsets(ro), ro, ci)
+    lhs = rng.standard_normal((2, m, k)).astype(np.float32)
+    rhs = rng.standard_normal((2, n, k)).astype(np.float32)
+    out = _run(dev, csr, lhs, rhs, dtype, force_variant=3, force_wpr=blocks)
+    want, scale = _want(oracle, csr, lhs, rhs, dtype)
+    assert_close(out.float().cpu().numpy(), want, scale, RTOL[dtype], f"matrix-core SDDMM {m}x{n} k={k} {dtype} blocks={blocks}",
+                 atol=FP16_SUBNORMAL_HALF_STEP if dtype == torch.float16 else 0.0)
+    assert torch.equal(out, _run(dev, csr, lhs, rhs, dtype, force_variant=3, force_wpr=blocks))         # same call, same bits
+
+
+def test_integer_operands_agree_with_the_gather_kernel_exactly(dev):
+    rng = np.random.default_rng(8)
+    m, n, k = 260, 390, 64
+    lens = rng.integers(0, 200, m)
+    ro, ci = W.csr_from_row_lengths(rng, m, n, lens)
+    csr = W.CSR(m, n, np.ones(ci.shape[0], np.float32), W.swizzle_from_offsets(ro), ro, ci)
+    lhs = rng.integers(-3, 4, (3, m, k)).astype(np.float32)
+    rhs = rng.integers(-3, 4, (3, n, k)).astype(np.float32)
+    want = _run(dev, csr, lhs, rhs, torch.float16, force_variant=1)
+    for blocks in (0, 1, 255, 3):
+        assert torch.equal(_run(dev, csr, lhs, rhs, torch.float16, force_variant=3, force_wpr=blocks), want), blocks
+
+
+def test_band_plus_scattered_mask_mixes_both_kinds_of_block(oracle, dev):
+    """A 640 x 1100 mask with a band of 96 columns and 3 scattered entries per row: band blocks go to the matrix
+    cores, the others are sampled entry by entry, within one workgroup; bf16 and fp16, three batch entries."""
+    rng = np.random.default_rng(77)
+    m, n, k = 640, 1100, 64
+    idx = np.arange(m)
+    mask = np.abs(idx[:, None] * n // m - np.arange(n)[None, :]) < 48
+    mask[np.repeat(idx, 3), rng.integers(0, n, (m, 3)).ravel()] = True
+    ro, ci, _ = W.csr_from_mask(mask)
+    csr = W.CSR(m, n, np.ones(ci.shape[0], np.float32), W.swizzle_from_offsets(ro), ro, ci)
+    lhs = rng.standard_normal((3, m, k)).astype(np.float32)
+    rhs = rng.standard_normal((3, n, k)).astype(np.float32)
+    for dtype in (torch.float16, torch.bfloat16):
+        out = _run(dev, csr, lhs, rhs, dtype, force_variant=3)
+        want, scale = _want(oracle, csr, lhs, rhs, dtype)
+        assert_close(out.float().cpu().numpy(), want, scale, RTOL[dtype], f"band + scattered {dtype}",
+                     atol=FP16_SUBNORMAL_HALF_STEP if dtype == torch.float16 else 0.0)
+
+
+def test_config3_four_heads_against_the_oracle_and_sixteen_against_the_gather_kernel(oracle, dev):
+    from intrasm_engine_amd import _lib
+    pattern, q, k, _ = W.config3(heads=4)
+    out = _run(dev, pattern, q, k, torch.float16, force_variant=3)
+    want, scale = _want(oracle, pattern, q, k, torch.float16)
+    assert_close(out.float().cpu().numpy(), want, scale, 1e-2, "config 3, 4 heads, matrix cores", atol=FP16_SUBNORMAL_HALF_STEP)
+    # all 16 heads: what the operator picks by itself for this shape is this kernel, each head equals the head alone,
+    # and the gather kernel agrees to the tolerance
+    pattern, q, k, _ = W.config3()
+    ri, _, ro, ci = to_dev(pattern, dev)
+    qt, kt = torch.from_numpy(q).to(dev).half(), torch.from_numpy(k).to(dev).half()
+    auto = ops.sddmm_sputnik_half(qt, kt, ri, ro, ci)
+    assert "sddmm_mfma_kernel" in _lib.last_kernels()
+    assert torch.equal(auto, _run(dev, pattern, q, k, torch.float16, force_variant=3))
+    for h in (0, 15):           # (a single head alone is too little work for this kernel to be picked: forced)
+        alone = _run(dev, pattern, q[h:h + 1], k[h:h + 1], torch.float16, force_variant=3)
+        assert torch.equal(alone[0], auto[h])
+    gather = _run(dev, pattern, q, k, torch.float16, force_variant=1).float()
+    assert torch.allclose(auto.float(), gather, rtol=1e-2, atol=1e-2 * 8.0 * 0.1)
+
+
+def test_refusals(dev):
+    from intrasm_engine_amd import _lib
+    rng = np.random.default_rng(1)
+    ro, ci = W.csr_from_row_lengths(rng, 64, 64, np.full(64, 8))
+    csr = W.CSR(64, 64, np.ones(ci.shape[0], np.float32), W.swizzle_from_offsets(ro), ro, ci)
+    with pytest.raises(RuntimeError, match="k = 32, 64 or 128"):
+        _run(dev, csr, rng.standard_normal((1, 64, 48)).astype(np.float32), rng.standard_normal((1, 64, 48)).astype(np.float32),
+             torch.float16, force_variant=3)
+    lib = _lib.load()
+    assert lib.iex_sddmm_workspace_bytes(_lib.F16, 3 << 16, 4096, 64, 4096, 1000, 16) == (6 * 32 + 1) * 4096 * 4
+    assert lib.iex_sddmm_workspace_bytes(_lib.F32, 3 << 16, 4096, 64, 4096, 1000, 16) == 0

@@ -231,8 +231,9 @@ int iex_csr_softmax(int dtype, int m, int nonzeros, const int* row_indices,
  * dtype is IEX_F16 or IEX_BF16 for A, B and C; accumulation is fp32 on the matrix cores.
  * stride_* are element strides between batch entries (0 = operand shared by the batch).
  * Bits 4..7 of trans_b force the kernel for tuning: 5 = 128x128, 6 = 128x256, 7 = 256x256 tiles,
- * 8 = 128x128 and 9 = 64x128 by eight waves with K steps of 64 (few tiles, long K), all with the operands loaded
- * from global memory straight into LDS (what 0 = choose picks from);
+ * 8 = 128x128 and 9 = 64x128 by eight waves with K steps of 64 (few tiles, long K), 10 = 128x256 by eight waves
+ * (11: with K steps of 64), all with the operands loaded from global memory straight into LDS (0 = choose picks
+ * among 5 and 7..10);
  * 1 = 128x128, 2 = 128x256, 3 = 256x256, 4 = 128x128 with K steps of 64, operands staged through
  * registers.  K % 8 == 0, N % 8 == 0 for a (K,N) B, 16-byte aligned operands.
  * Replaces the cuBLAS / CUTLASS / Triton companions of tests/test_interleaving.py:26-345. */

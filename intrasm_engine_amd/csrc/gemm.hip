@@ -101,22 +101,36 @@ int launch_shape(const GemmParams& p, int batch, int force, hipStream_t stream) 
   if (force == 7) return launch_dma<BF16, TRANS_B, 4, 4, 32, 4>(p, batch, stream);
   if (force == 8) return launch_dma<BF16, TRANS_B, 2, 1, 64, 4, 4>(p, batch, stream);
   if (force == 9) return launch_dma<BF16, TRANS_B, 1, 1, 64, 4, 4>(p, batch, stream);
+  if (force == 10) return launch_dma<BF16, TRANS_B, 2, 2, 32, 4, 4>(p, batch, stream);
+  if (force == 11) return launch_dma<BF16, TRANS_B, 2, 2, 64, 3, 4>(p, batch, stream);
   // Default: operands straight from global memory into LDS (gemm_dma_device.cuh).  The larger the
   // tile of a wave, the fewer LDS bytes each MFMA needs, and LDS time is what the main loop runs
   // against; the smaller the tile, the more workgroups there are to fill 256 CUs, and a tile wider
-  // than what is left of the matrix computes columns nobody stores.  Measured (bf16, TFLOP/s):
-  //   8192^3: 256x256 1200, 128x256 1040, register-staged 256x256 980;   4096 x 8192 x 4096: 1140 / 1000 / 920
-  //   config 4's 4096 x 2048 x 4096 (128 tiles of 256x256): 620 / 860 / 470, 128x128 750
-  //   2048^3: 290 / 420 / 220, 128x128 550
+  // than what is left of the matrix computes columns nobody stores.  (Register-staged operands, codes 1..4:
+  // 8192^3 256x256 980 TFLOP/s against 1200 here.)
   // A short K (at most 8 steps) is prologue and epilogue: small tiles, two workgroups per CU that cover for
   // each other (512 x (512 x 512 x 128), the attention scores of the decoder layer: 229 -> 123 us; 8192 x 8192 x
   // 128: 59 -> 48; from K = 512 the large tiles are ahead again).
   if (p.K <= 256) return launch_dma<BF16, TRANS_B, 2, 2, 32, 4>(p, batch, stream);
-  auto fill = [](int n, int tile) { return (double)n / ((double)ceil_div(n, tile) * tile); };
-  const long long huge_tiles = (long long)ceil_div(p.M, 256) * ceil_div(p.N, 256) * batch;
-  if (huge_tiles >= 512 && fill(p.M, 256) * fill(p.N, 256) >= 0.8) return launch_dma<BF16, TRANS_B, 4, 4, 32, 4>(p, batch, stream);
-  const long long wide_tiles = (long long)ceil_div(p.M, 128) * ceil_div(p.N, 256) * batch;
-  if (wide_tiles >= 256 && fill(p.N, 256) >= 0.8) return launch_dma<BF16, TRANS_B, 2, 4, 32, 4>(p, batch, stream);
+  const long long small_tiles = (long long)ceil_div(p.M, 128) * ceil_div(p.N, 128) * batch;
+  if (small_tiles > 256) {
+    // More 128 x 128 tiles than CUs: the tile shape that finishes first, counting whole rounds of workgroups (a
+    // workgroup of the last round takes as long as any other) at the rate each shape reaches with every CU busy.
+    // TFLOP/s measured: 256 x 256 (one workgroup per CU) 1200; 128 x 256 by eight waves (64 x 64 each, two per
+    // SIMD that cover for each other at the barrier and the waits of every K step; one workgroup per CU) 930,
+    // by four waves (64 x 128 each) 790; 128 x 128 (two workgroups per CU) 750.
+    //   4096 x 2048 x 4096 (config 4): 627 / 907 / 788 / 750      4096 x 4096 x 4096: 1080 / 985 / 903
+    //   11008 x 4096 x 4096: 1093 / 952 / 914                      8192^3: 1208 / 1065 / 1055
+    // (128 x 256 by eight waves with five or six stages instead of four: 860 and 850 on config 4's shape.)
+    auto cost = [&](int bm, int bn, int slots, double rate) {
+      const long long tiles = (long long)ceil_div(p.M, bm) * ceil_div(p.N, bn) * batch;
+      return (double)ceil_div(tiles, slots) * slots * bm * bn / rate;
+    };
+    const double huge = cost(256, 256, 256, 1200.0), wide = cost(128, 256, 256, 930.0), small = cost(128, 128, 512, 750.0);
+    if (huge <= wide && huge <= small) return launch_dma<BF16, TRANS_B, 4, 4, 32, 4>(p, batch, stream);
+    if (wide <= small) return launch_dma<BF16, TRANS_B, 2, 2, 32, 4, 4>(p, batch, stream);
+    return launch_dma<BF16, TRANS_B, 2, 2, 32, 4>(p, batch, stream);
+  }
   // One round of at most one 128 x 128 tile per CU and a long K: eight waves (64 x 32 each) and K steps of 64
   // (4096 x 512 x 4096: 44 -> 34.5 us; eight waves with steps of 32 and eight stages 38.6; 64 x 128 tiles 36.8).
   // Such a product runs on the few CUs that have a tile (128 x 128 x 4096 is 16 us of one CU's matrix cores at
@@ -126,8 +140,7 @@ int launch_shape(const GemmParams& p, int batch, int force, hipStream_t stream) 
   // (4096 x 256 x 4096: 35 -> 27.5 us, 4096 x 512 x 4096: 35 -> 30, 1024 x 2048 x 1024: 13.9 -> 12.4).
   const long long half_tiles = (long long)ceil_div(p.M, 64) * ceil_div(p.N, 128) * batch;
   if (half_tiles <= 256 && p.K >= 512) return launch_dma<BF16, TRANS_B, 1, 1, 64, 4, 4>(p, batch, stream);
-  const long long small_tiles = (long long)ceil_div(p.M, 128) * ceil_div(p.N, 128) * batch;
-  if (small_tiles <= 256 && p.K >= 2048) return launch_dma<BF16, TRANS_B, 2, 1, 64, 4, 4>(p, batch, stream);
+  if (p.K >= 2048) return launch_dma<BF16, TRANS_B, 2, 1, 64, 4, 4>(p, batch, stream);
   return launch_dma<BF16, TRANS_B, 2, 2, 32, 4>(p, batch, stream);
 }
 
@@ -136,7 +149,8 @@ int launch_shape(const GemmParams& p, int batch, int force, hipStream_t stream) 
 
 // trans_b: bit 0 = B is (N, K); bits 4..7 force the kernel for tuning.  Register-staged operands:
 // 1 = 128x128 tiles, 2 = 128x256, 3 = 256x256, 4 = 128x128 with K steps of 64.  Operands loaded
-// straight into LDS: 5 = 128x128, 6 = 128x256, 7 = 256x256, 8 = 128x128, 9 = 64x128 by eight waves with K steps of 64.  0 = choose (one of 5..9).
+// straight into LDS: 5 = 128x128, 6 = 128x256, 7 = 256x256, 8 = 128x128, 9 = 64x128 by eight waves with K steps of 64,
+// 10 = 128x256 by eight waves, 11 = the same with K steps of 64.  0 = choose (one of 5..10).
 extern "C" int iex_gemm(int dtype, int trans_b_and_shape, int M, int N, int K, const void* A, const void* B, void* C, int batch,
                         long long stride_a, long long stride_b, long long stride_c, void* stream) {
   return iex::gemm_dispatch(dtype, trans_b_and_shape, M, N, K, A, B, C, batch, stride_a, stride_b, stride_c, stream, nullptr, 0, 0);

@@ -73,6 +73,13 @@ def main():
     ap.add_argument("--pmc-probe", action="store_true",
                     help="for `rocprofv3 --pmc ...`: 3 plain copies of 256 MiB (iex_copy_bytes), then 3 launches of each "
                          "fp32 cell, and exit")
+    ap.add_argument("--gemm-probe", action="store_true",
+                    help="bf16 GEMM (B as (K, N)): every tile shape on a few products, one line per product on stdout; with "
+                         "--gemm-probe-tile T only that shape on config 4's product, 3 launches (for rocprofv3 --pmc)")
+    ap.add_argument("--gemm-probe-tile", type=int, default=-1)
+    ap.add_argument("--sddmm-probe", action="store_true",
+                    help="config 3's SDDMM (fp16, 16 heads), 3 launches of what the operator picks and 3 of the gather kernel "
+                         "(for rocprofv3 --kernel-trace / --pmc)")
     ap.add_argument("--overlap-probe", action="store_true",
                     help="for `rocprofv3 --kernel-trace`: 3 replays of config 4's two-branch graph, and exit")
     ap.add_argument("--summarize-pmc", nargs=3, metavar=("FETCH_CSV", "WRITE_CSV", "CELLS_JSON"),
@@ -148,6 +155,46 @@ def main():
         os.makedirs(os.path.join(ROOT, "gpurun_out"), exist_ok=True)
         json.dump({"copy_bytes": nbytes, "cells": names}, open(os.path.join(ROOT, "gpurun_out", "pmc_probe_cells.json"), "w"))
         log("[bench] pmc probe done: copy of %d bytes x3 (copy_kernel), then every fp32 cell x3" % nbytes)
+        return
+
+    if args.gemm_probe:
+        from intrasm_engine_amd.pytorch import ops as pyops_g
+        if args.gemm_probe_tile >= 0:
+            a_ = torch.randn(4096, 4096, device=dev).bfloat16()
+            b_ = torch.randn(4096, 2048, device=dev).bfloat16()
+            with pyops_g.kernel_params(gemm={"tile": args.gemm_probe_tile} if args.gemm_probe_tile else None):
+                for _ in range(3):
+                    ops.gemm_mfma(a_, b_, False)
+            torch.cuda.synchronize()
+            return
+        names = {0: "chosen", 5: "128x128", 6: "128x256/4 waves", 10: "128x256/8 waves", 11: "128x256/8 waves, K steps of 64", 7: "256x256"}
+        for (gm, gn, gk) in ((4096, 2048, 4096), (4096, 4096, 4096), (11008, 4096, 4096), (4096, 8192, 4096), (8192, 8192, 8192), (2048, 2048, 2048)):
+            a_ = torch.randn(gm, gk, device=dev).bfloat16()
+            b_ = torch.randn(gk, gn, device=dev).bfloat16()
+            cells_ = []
+            for tile_ in (0, 0, 5, 6, 10, 11, 7):       # (the first pass warms the clocks up and is dropped)
+                with pyops_g.kernel_params(gemm={"tile": tile_} if tile_ else None):
+                    f_ = lambda: ops.gemm_mfma(a_, b_, False)
+                    f_()
+                    ms_ = IL.time_execs([f_] * 10, repeats=3) / 10
+                cells_.append(f"{names[tile_]} {IL.gemm_tflops(gm, gn, gk, ms_):.0f}")
+            print(f"{gm} x {gn} x {gk} (TFLOP/s): " + " | ".join(cells_[1:]), flush=True)
+            del a_, b_
+        return
+
+    if args.sddmm_probe:
+        from intrasm_engine_amd.pytorch import ops as pyops_s
+        pat_, q_, k_, _ = W.config3()
+        ri_, _, ro_, ci_ = csr_dev(pat_)
+        qt_, kt_ = (torch.from_numpy(x).to(dev).half() for x in (q_, k_))
+        for _ in range(3):
+            ops.sddmm_sputnik_half(qt_, kt_, ri_, ro_, ci_)
+        log("[sddmm-probe] operator:", _lib.last_kernels())
+        with pyops_s.kernel_params(sddmm={"force_variant": 1}):
+            for _ in range(3):
+                ops.sddmm_sputnik_half(qt_, kt_, ri_, ro_, ci_)
+        log("[sddmm-probe] gather kernel:", _lib.last_kernels())
+        torch.cuda.synchronize()
         return
 
     if args.overlap_probe:
@@ -472,6 +519,33 @@ def run_extras(torch, ops, dev, W, IL, mats, dens, csr_dev, time_cell, time_cold
                                     "kernel": kernel_of(lambda: ops.sddmm_sputnik_half(qt, kt, ri3, ro3, ci3)),
                                     "GBps": round(by / us / 1e3, 1), "hbm_frac": round(by / us / 1e3 / HBM_PEAK_GBPS, 4),
                                     "GFLOPs": round(W.sddmm_flops(pat.nnz, 64, 16) / us / 1e3, 1)}
+    from intrasm_engine_amd.pytorch import ops as pyops_k
+    with pyops_k.kernel_params(sddmm={"force_variant": 1}):
+        out["sddmm_c3_fp16_16heads"]["gather_kernel_us"] = round(time_cell(lambda: ops.sddmm_sputnik_half(qt, kt, ri3, ro3, ci3), repeats=10), 2)
+    # the same operator on other masks (16 heads x 4096 x 4096, k = 64): what it picks by itself against the gather kernel
+    import numpy as np_
+    rng_ = np_.random.default_rng(0)
+    idx_ = np_.arange(4096)
+    masks_ = {"band_512_plus_32_scattered": W.config3(band=512, extra=32)[0],
+              "band_128_plus_16_scattered": W.config3(band=128, extra=16)[0]}
+    for label_, m_ in (("block_diagonal_256", (idx_[:, None] // 256) == (idx_[None, :] // 256)),
+                       ("causal_window_512", (idx_[:, None] >= idx_[None, :]) & (idx_[:, None] - idx_[None, :] < 512))):
+        ro_, ci_, _ = W.csr_from_mask(m_)
+        masks_[label_] = W.CSR(4096, 4096, np_.ones(ci_.shape[0], np_.float32), W.swizzle_from_offsets(ro_), ro_, ci_)
+    for d_ in (0.01, 0.05, 0.10, 0.20):
+        ro_, ci_ = W.csr_from_row_lengths(rng_, 4096, 4096, np_.full(4096, int(4096 * d_)))
+        masks_[f"equal_rows_random_columns_{d_:.2f}"] = W.CSR(4096, 4096, np_.ones(ci_.shape[0], np_.float32), W.swizzle_from_offsets(ro_), ro_, ci_)
+    rows_m = []
+    for label_, c_ in masks_.items():
+        rim, _, rom, cim = csr_dev(c_)
+        f_ = lambda: ops.sddmm_sputnik_half(qt, kt, rim, rom, cim)
+        us_op = time_cell(f_, repeats=5, samples=3)
+        with pyops_k.kernel_params(sddmm={"force_variant": 1}):
+            us_ga = time_cell(f_, repeats=5, samples=3)
+        rows_m.append({"mask": label_, "density": round(c_.nnz / 4096 / 4096, 4), "operator_us": round(us_op, 1), "gather_kernel_us": round(us_ga, 1),
+                       "operator_kernel": kernel_of(f_)})
+        del rim, rom, cim
+    out["sddmm_fp16_16heads_by_mask"] = rows_m
     scores = ops.sddmm_sputnik_half(qt, kt, ri3, ro3, ci3)
     us = time_cell(lambda: ops.spmm_sputnik_batched_values(vt, ri3, scores, ro3, ci3, pat.m), repeats=10)
     by = W.spmm_bytes(pat.m, pat.k, 64, pat.nnz, 16, 2, 4, True)

@@ -55,6 +55,8 @@ int launch(GemmParams p, int batch, hipStream_t stream) {
       raised = true;
     }
   }
+  note_kernel("gemm_kernel<%s, %s, %d, %d, %d> (%d x %d tiles, operands staged through registers)", BF16 ? "bf16" : "f16",
+              TRANS_B ? "B(N,K)" : "B(K,N)", WM, WN, BK, BM, BN);
   hipLaunchKernelGGL(kern, dim3(per_xcd * kXcds, batch), dim3(256), lds, stream, p);
   return check_hip(hipGetLastError(), "gemm launch");
 }
@@ -86,6 +88,8 @@ int launch_dma(GemmParams p, int batch, hipStream_t stream) {
       raised = true;
     }
   }
+  note_kernel("gemm_dma_kernel<%s, %s, %d, %d, %d, %d, %d> (%d x %d tiles, %d waves)", BF16 ? "bf16" : "f16", TRANS_B ? "B(N,K)" : "B(K,N)", WM, WN,
+              BK, STAGES, WCN, BM, BN, 2 * WCN);
   hipLaunchKernelGGL(kern, dim3(per_xcd * kXcds, batch), dim3(WCN * 128), lds, stream, p);
   return check_hip(hipGetLastError(), "gemm launch");
 }
@@ -153,6 +157,7 @@ int launch_shape(const GemmParams& p, int batch, int force, hipStream_t stream) 
 // 10 = 128x256 by eight waves, 11 = the same with K steps of 64.  0 = choose (one of 5..10).
 extern "C" int iex_gemm(int dtype, int trans_b_and_shape, int M, int N, int K, const void* A, const void* B, void* C, int batch,
                         long long stride_a, long long stride_b, long long stride_c, void* stream) {
+  iex::trail_reset();
   return iex::gemm_dispatch(dtype, trans_b_and_shape, M, N, K, A, B, C, batch, stride_a, stride_b, stride_c, stream, nullptr, 0, 0);
 }
 

@@ -165,6 +165,10 @@ int iex_CudaSpmm5(int m, int k, int n, int nonzeros, const int* row_indices,
 /* ----------------------------------------------------------------- SDDMM ---- */
 #define IEX_SDDMM_SUM_OVER_BATCH 0x1 /* one (nnz) output summed over the batch            */
 #define IEX_SDDMM_ACCUMULATE 0x2     /* out += ... instead of out = ...                   */
+/* iex_sddmm_ws, variant 3 only (ignored elsewhere): the workspace still holds the tables that an
+ * earlier call with the same m, n, nonzeros and index arrays (and a kind-3 workspace) wrote there;
+ * the setup kernel is skipped.  For callers whose mask does not change from call to call.        */
+#define IEX_SDDMM_TABLES_READY 0x4
 /* bits 8..15: force wavefronts per row (1 or 4); 0 = choose from nnz/m.  For tuning.
  * With variant 3 the same bits set the number of nonzeros from which a 128 x 128 block of the
  * mask counts as dense: 0 = built in, 1 = every block, 255 = none, else 64 * value.       */
@@ -208,6 +212,9 @@ int iex_sddmm_ws(int dtype, int flags, int m, int k, int n, int nonzeros,
                  const void* lhs_matrix, const void* rhs_matrix, void* output_values,
                  void* stream, int batch, void* workspace, size_t workspace_bytes);
 size_t iex_sddmm_workspace_bytes(int dtype, int flags, int m, int k, int n, int nonzeros, int batch);
+/* What the workspace would hold: 0 = nothing (not used), 3 = the tables of variant 3 (a function of m, n
+ * and the index arrays only: see IEX_SDDMM_TABLES_READY), 7 = the dense product. */
+int iex_sddmm_workspace_kind(int dtype, int flags, int m, int k, int n, int nonzeros, int batch);
 
 /* Drop-in for CudaSddmm2 (csrc/extensions.h:31; sddmm_sputnik_atomic_upd_weight,
  * sputnik_kernels.cpp:182-184): fp32, output (nnz) = sum over the batch, written

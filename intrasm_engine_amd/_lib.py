@@ -19,6 +19,7 @@ SPMM_ACCUMULATE = 0x2
 SPMM_RELU = 0x4
 SDDMM_SUM_OVER_BATCH = 0x1
 SDDMM_ACCUMULATE = 0x2
+SDDMM_TABLES_READY = 0x4
 
 _c = ctypes
 _vp, _i, _ll, _f = _c.c_void_p, _c.c_int, _c.c_longlong, _c.c_float
@@ -42,6 +43,7 @@ SIGNATURES = {
     "iex_sddmm_ex": (_i, [_i, _i, _i, _i, _i, _i, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i]),
     "iex_sddmm_ws": (_i, [_i, _i, _i, _i, _i, _i, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _vp, _c.c_size_t]),
     "iex_sddmm_workspace_bytes": (_c.c_size_t, [_i, _i, _i, _i, _i, _i, _i]),
+    "iex_sddmm_workspace_kind": (_i, [_i, _i, _i, _i, _i, _i, _i]),
     "iex_CudaSddmm2": (_i, [_i, _i, _i, _i, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i]),
     "iex_csr_softmax": (_i, [_i, _i, _i, _vp, _vp, _vp, _f, _vp, _i]),
     "iex_gemm": (_i, [_i, _i, _i, _i, _i, _vp, _vp, _vp, _i, _ll, _ll, _ll, _vp]),

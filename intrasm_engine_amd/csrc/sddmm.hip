@@ -329,14 +329,16 @@ int launch_sddmm_mfma_ks(const SddmmMfmaParams& q, int batch, hipStream_t stream
   return check_hip(hipGetLastError(), "sddmm (matrix-core) launch");
 }
 
-int launch_sddmm_mfma(int dtype, const SddmmParams& p, void* ws, int dense_code, hipStream_t stream) {
+int launch_sddmm_mfma(int dtype, const SddmmParams& p, void* ws, int dense_code, bool tables_ready, hipStream_t stream) {
   const int tiles_n = ceil_div(p.n, kSdBN);
   u32x4* mask = static_cast<u32x4*>(ws);
   int* tile_ptr = reinterpret_cast<int*>(mask + (size_t)tiles_n * p.m);
   int* brief = tile_ptr + (size_t)(tiles_n + 1) * p.m;
-  note_kernel("sddmm_tile_ptr_kernel");
-  hipLaunchKernelGGL(sddmm_tile_ptr_kernel, dim3(ceil_div(p.m, 4)), dim3(256), 0, stream, p.m, tiles_n, p.row_offsets, p.cols, tile_ptr, brief, mask);
-  if (int rc = check_hip(hipGetLastError(), "sddmm row-cursor launch")) return rc;
+  if (!tables_ready) {   // (else: the caller vouches that an earlier call on this pattern left them in the workspace)
+    note_kernel("sddmm_tile_ptr_kernel");
+    hipLaunchKernelGGL(sddmm_tile_ptr_kernel, dim3(ceil_div(p.m, 4)), dim3(256), 0, stream, p.m, tiles_n, p.row_offsets, p.cols, tile_ptr, brief, mask);
+    if (int rc = check_hip(hipGetLastError(), "sddmm row-cursor launch")) return rc;
+  }
   // dense_code (for tests and tuning): 0 = the built-in threshold, 1 = every tile on the matrix cores, 255 = none,
   // else 64 * code nonzeros per 128 x 128 block
   const int dense_min = dense_code == 0 ? kSdDenseMin : dense_code == 1 ? 0 : dense_code == 255 ? kSdBM * kSdBN + 1 : 64 * dense_code;
@@ -353,6 +355,20 @@ int launch_sddmm_mfma(int dtype, const SddmmParams& p, void* ws, int dense_code,
 
 // Bytes of workspace with which iex_sddmm_ws would compute the dense product and sample it (0: it
 // would not, whatever the workspace).  Pointers are taken to be 16-byte aligned.
+// What iex_sddmm_ws would do with a workspace of the size that sddmm_workspace_bytes names: 0 = not use it, 3 = keep the
+// tables of the kernel for masks with structure in it, 7 = the dense product.
+int sddmm_workspace_kind(int dtype, int flags, int m, int k, int n, int nonzeros, int batch) {
+  if (m <= 0 || k <= 0 || n <= 0 || nonzeros <= 0 || batch <= 0) return 0;
+  const int variant = (flags >> 16) & 0xf;
+  if (variant != 0 && variant != 7 && variant != 3) return 0;
+  void* const some_aligned = reinterpret_cast<void*>(size_t(256));
+  SddmmParams p{m, k, n, nonzeros, batch, nullptr, nullptr, nullptr, some_aligned, some_aligned, nullptr,
+                (flags & IEX_SDDMM_SUM_OVER_BATCH) != 0, (flags & IEX_SDDMM_ACCUMULATE) != 0};
+  if (variant != 7 && sddmm_mfma_fits(dtype, p) && (variant == 3 || sddmm_mfma_wins(p))) return 3;
+  if (variant == 3 || !sddmm_dense_fits(dtype, p)) return 0;
+  return (variant == 7 || sddmm_dense_wins(p)) ? 7 : 0;
+}
+
 size_t sddmm_workspace_bytes(int dtype, int flags, int m, int k, int n, int nonzeros, int batch) {
   if (m <= 0 || k <= 0 || n <= 0 || nonzeros <= 0 || batch <= 0) return 0;
   const int variant = (flags >> 16) & 0xf;
@@ -393,7 +409,7 @@ int sddmm_dispatch(int dtype, int flags, int m, int k, int n, int nonzeros, cons
       IEX_REQUIRE(fits, IEX_ERR_UNSUPPORTED, "sddmm: the matrix-core kernel needs fp16 / bf16, k = 32, 64 or 128, plain store, one output per batch entry and 16-byte aligned operands");
       IEX_REQUIRE(room, IEX_ERR_BAD_ARGUMENT, "sddmm: the matrix-core kernel needs a 16-byte aligned workspace of %zu bytes (iex_sddmm_ws)", sddmm_mfma_bytes(p));
     }
-    if (fits && room && (variant == 3 || sddmm_mfma_wins(p))) return launch_sddmm_mfma(dtype, p, workspace, variant == 3 ? (flags >> 8) & 0xff : 0, s);
+    if (fits && room && (variant == 3 || sddmm_mfma_wins(p))) return launch_sddmm_mfma(dtype, p, workspace, variant == 3 ? (flags >> 8) & 0xff : 0, (flags & IEX_SDDMM_TABLES_READY) != 0, s);
   }
   if (variant == 0 || variant == 7) {
     const bool fits = sddmm_dense_fits(dtype, p);
@@ -433,6 +449,10 @@ int iex_sddmm_ws(int dtype, int flags, int m, int k, int n, int nonzeros, const 
 
 size_t iex_sddmm_workspace_bytes(int dtype, int flags, int m, int k, int n, int nonzeros, int batch) {
   return iex::sddmm_workspace_bytes(dtype, flags, m, k, n, nonzeros, batch);
+}
+
+int iex_sddmm_workspace_kind(int dtype, int flags, int m, int k, int n, int nonzeros, int batch) {
+  return iex::sddmm_workspace_kind(dtype, flags, m, k, n, nonzeros, batch);
 }
 
 int iex_CudaSddmm2(int m, int k, int n, int nonzeros, const int* row_indices, const int* row_offsets,

@@ -157,8 +157,32 @@ def _spmm(b, row_indices, values, row_offsets, column_indices, m, *, per_batch_v
     return out
 
 
+class SddmmPlan:
+    """Memory that per-entry SDDMM calls on one CSR pattern keep between calls.
+
+    The kernel for masks with structure (``iex_sddmm_ws``, variant 3) works from tables that a setup kernel derives
+    from the pattern alone (m, n, row_offsets, column_indices).  A caller whose mask does not change passes the same
+    plan to every call: the first call writes the tables into the plan's workspace, later calls skip the setup kernel
+    (``IEX_SDDMM_TABLES_READY``).  The plan notices other index tensors, other shapes and in-place changes of the index
+    tensors (their version counters) and then lets the tables be written again.  Calls that share a plan must be
+    ordered on one stream (the workspace is theirs for the duration of the work)."""
+
+    def __init__(self):
+        self.workspace = None
+        self.key = None
+
+    def _ready(self, key, nbytes, device):
+        """Workspace of nbytes for this key; True when it already holds the key's tables."""
+        if self.workspace is None or self.workspace.numel() < nbytes or self.workspace.device != device:
+            self.workspace = torch.empty(nbytes, dtype=torch.uint8, device=device)
+            self.key = None
+        ready = self.key == key
+        self.key = key
+        return ready
+
+
 def _sddmm(a, b, row_indices, row_offsets, column_indices, *, sum_over_batch, dtypes,
-           out=None, accumulate=False, force_wpr=0, force_variant=0, no_workspace=False):
+           out=None, accumulate=False, force_wpr=0, force_variant=0, no_workspace=False, plan=None):
     tuned = getattr(_TUNING, "sddmm", None)
     if tuned and not (force_wpr or force_variant):
         force_wpr, force_variant = tuned.get("force_wpr", 0), tuned.get("force_variant", 0)
@@ -193,7 +217,14 @@ def _sddmm(a, b, row_indices, row_offsets, column_indices, *, sum_over_batch, dt
         # room for the dense product where the library would rather compute all of it on the matrix
         # cores and pick the nonzeros (16-bit, long k): from torch's allocator, on the current stream
         ws_bytes = 0 if no_workspace else lib.iex_sddmm_workspace_bytes(_DT[a.dtype], flags, m, k, n, nonzeros, batch)
-        ws = torch.empty(ws_bytes, dtype=torch.uint8, device=a.device) if ws_bytes else None
+        if plan is not None and ws_bytes and lib.iex_sddmm_workspace_kind(_DT[a.dtype], flags, m, k, n, nonzeros, batch) == 3:
+            key = (row_offsets.data_ptr(), column_indices.data_ptr(), row_offsets._version, column_indices._version,
+                   m, n, nonzeros)
+            if plan._ready(key, ws_bytes, a.device):
+                flags |= _lib.SDDMM_TABLES_READY
+            ws = plan.workspace
+        else:
+            ws = torch.empty(ws_bytes, dtype=torch.uint8, device=a.device) if ws_bytes else None
         rc = lib.iex_sddmm_ws(
             _DT[a.dtype], flags, m, k, n, nonzeros, row_indices.data_ptr(), row_offsets.data_ptr(),
             column_indices.data_ptr(), a.data_ptr(), b.data_ptr(), out.data_ptr(),
@@ -232,6 +263,13 @@ def sddmm_sputnik_atomic_upd_weight(a, b, row_indices, row_offsets, column_indic
 def sddmm_sputnik_half(a, b, row_indices, row_offsets, column_indices):
     return _sddmm(a, b, row_indices, row_offsets, column_indices, sum_over_batch=False,
                   dtypes=(torch.float32, torch.float16, torch.bfloat16))
+
+
+def sddmm_half_planned(a, b, row_indices, row_offsets, column_indices, plan: SddmmPlan):
+    """``sddmm_sputnik_half`` for a caller that keeps an :class:`SddmmPlan` for the pattern (not a registered operator:
+    the plan is a Python object)."""
+    return _sddmm(a, b, row_indices, row_offsets, column_indices, sum_over_batch=False,
+                  dtypes=(torch.float32, torch.float16, torch.bfloat16), plan=plan)
 
 
 def csr_softmax_(values, row_indices, row_offsets, scale):

@@ -23,11 +23,13 @@ ops = torch.ops.iex_ops
 
 def sparse_attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, row_indices: torch.Tensor,
                      row_offsets: torch.Tensor, column_indices: torch.Tensor, scale: float | None = None,
-                     return_probs: bool = False):
+                     return_probs: bool = False, plan=None):
     """q, k: (heads, tokens, d); v: (heads, tokens, dv); mask pattern tokens x tokens as int32 CSR
     arrays (``row_indices`` = rows by decreasing length).  fp16, bf16 or fp32.  Returns
     (heads, tokens, dv), and the (heads, nnz) probabilities when ``return_probs``.
-    Rows of the mask without entries give zero output rows."""
+    Rows of the mask without entries give zero output rows.
+    ``plan``: an ``ops.SddmmPlan`` that the caller keeps for this mask; with it the tables that the score kernel derives
+    from the mask are written by the first call only (16-bit inputs; ignored where that kernel is not the one that runs)."""
     if q.dim() != 3 or k.shape != q.shape or v.dim() != 3 or v.shape[:2] != q.shape[:2]:
         raise RuntimeError("q, k must be (heads, tokens, d) and v (heads, tokens, dv)")
     tokens = q.shape[1]
@@ -35,7 +37,11 @@ def sparse_attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, row_indi
         raise RuntimeError("the mask must be tokens x tokens")
     if scale is None:
         scale = 1.0 / math.sqrt(q.shape[2])
-    scores = ops.sddmm_sputnik_half(q, k, row_indices, row_offsets, column_indices)     # (heads, nnz)
+    if plan is not None:
+        from . import ops as _pyops
+        scores = _pyops.sddmm_half_planned(q, k, row_indices, row_offsets, column_indices, plan)
+    else:
+        scores = ops.sddmm_sputnik_half(q, k, row_indices, row_offsets, column_indices)     # (heads, nnz)
     probs = ops.csr_softmax_(scores, row_indices, row_offsets, float(scale))
     out = ops.spmm_sputnik_batched_values(v, row_indices, probs, row_offsets, column_indices, tokens)
     return (out, probs) if return_probs else out

@@ -104,6 +104,45 @@ def test_config3_four_heads_against_the_oracle_and_sixteen_against_the_gather_ke
     assert torch.allclose(auto.float(), gather, rtol=1e-2, atol=1e-2 * 8.0 * 0.1)
 
 
+def test_tables_kept_between_calls_of_one_mask(oracle, dev):
+    """A caller with a fixed mask keeps a plan: the second call skips the setup kernel and gives the same bits; another
+    mask (or the same index tensor changed in place) makes the plan write the tables again; the attention block takes
+    a plan too."""
+    from intrasm_engine_amd import _lib
+    from intrasm_engine_amd.pytorch import ops as pyops
+    from intrasm_engine_amd.pytorch.sparse_attention import sparse_attention
+    pattern, q, k, v = W.config3(heads=8)
+    ri, _, ro, ci = to_dev(pattern, dev)
+    qt, kt, vt = (torch.from_numpy(x).to(dev).half() for x in (q, k, v))
+    want = ops.sddmm_sputnik_half(qt, kt, ri, ro, ci)
+    assert "sddmm_tile_ptr_kernel" in _lib.last_kernels()
+    plan = pyops.SddmmPlan()
+    first = pyops.sddmm_half_planned(qt, kt, ri, ro, ci, plan)
+    assert "sddmm_tile_ptr_kernel" in _lib.last_kernels() and torch.equal(first, want)
+    second = pyops.sddmm_half_planned(qt, kt, ri, ro, ci, plan)
+    assert _lib.last_kernels().startswith("sddmm_mfma_kernel") and torch.equal(second, want)
+    # other operands, same mask: still no setup
+    third = pyops.sddmm_half_planned(kt, qt, ri, ro, ci, plan)
+    assert _lib.last_kernels().startswith("sddmm_mfma_kernel") and torch.equal(third, ops.sddmm_sputnik_half(kt, qt, ri, ro, ci))
+    # another mask through the same plan: tables written again, results those of the new mask
+    p2, *_ = W.config3(seed=11, heads=1, band=128, extra=16)
+    ri2, _, ro2, ci2 = to_dev(p2, dev)
+    other = pyops.sddmm_half_planned(qt, kt, ri2, ro2, ci2, plan)
+    assert "sddmm_tile_ptr_kernel" in _lib.last_kernels()
+    assert torch.equal(other, ops.sddmm_sputnik_half(qt, kt, ri2, ro2, ci2))
+    # the first mask again, then changed in place (one scattered column moved): noticed through the version counter
+    assert torch.equal(pyops.sddmm_half_planned(qt, kt, ri, ro, ci, plan), want)
+    ci.add_(0)
+    pyops.sddmm_half_planned(qt, kt, ri, ro, ci, plan)
+    assert "sddmm_tile_ptr_kernel" in _lib.last_kernels()
+    # the attention block
+    plan2 = pyops.SddmmPlan()
+    a0 = sparse_attention(qt, kt, vt, ri, ro, ci)
+    a1 = sparse_attention(qt, kt, vt, ri, ro, ci, plan=plan2)
+    a2 = sparse_attention(qt, kt, vt, ri, ro, ci, plan=plan2)
+    assert torch.equal(a0, a1) and torch.equal(a0, a2)
+
+
 def test_refusals(dev):
     from intrasm_engine_amd import _lib
     rng = np.random.default_rng(1)
@@ -115,3 +154,7 @@ def test_refusals(dev):
     lib = _lib.load()
     assert lib.iex_sddmm_workspace_bytes(_lib.F16, 3 << 16, 4096, 64, 4096, 1000, 16) == (6 * 32 + 1) * 4096 * 4
     assert lib.iex_sddmm_workspace_bytes(_lib.F32, 3 << 16, 4096, 64, 4096, 1000, 16) == 0
+    assert lib.iex_sddmm_workspace_kind(_lib.F16, 3 << 16, 4096, 64, 4096, 1000, 16) == 3
+    assert lib.iex_sddmm_workspace_kind(_lib.F16, 0, 4096, 64, 4096, 1150000, 16) == 3
+    assert lib.iex_sddmm_workspace_kind(_lib.F16, 0, 1024, 4096, 1024, 300000, 1) == 7
+    assert lib.iex_sddmm_workspace_kind(_lib.F32, 0, 4096, 64, 4096, 1150000, 16) == 0

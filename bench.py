@@ -167,12 +167,13 @@ def main():
                     ops.gemm_mfma(a_, b_, False)
             torch.cuda.synchronize()
             return
-        names = {0: "chosen", 5: "128x128", 6: "128x256/4 waves", 10: "128x256/8 waves", 11: "128x256/8 waves, K steps of 64", 7: "256x256"}
+        names = {0: "chosen", 5: "128x128", 6: "128x256/4 waves", 10: "128x256/8 waves", 11: "128x256/8 waves, K steps of 64", 7: "256x256",
+                 12: "256x256, K split over 2 workgroups"}
         for (gm, gn, gk) in ((4096, 2048, 4096), (4096, 4096, 4096), (11008, 4096, 4096), (4096, 8192, 4096), (8192, 8192, 8192), (2048, 2048, 2048)):
             a_ = torch.randn(gm, gk, device=dev).bfloat16()
             b_ = torch.randn(gk, gn, device=dev).bfloat16()
             cells_ = []
-            for tile_ in (0, 0, 5, 6, 10, 11, 7):       # (the first pass warms the clocks up and is dropped)
+            for tile_ in (0, 0, 5, 6, 10, 11, 7, 12):       # (the first pass warms the clocks up and is dropped)
                 with pyops_g.kernel_params(gemm={"tile": tile_} if tile_ else None):
                     f_ = lambda: ops.gemm_mfma(a_, b_, False)
                     f_()

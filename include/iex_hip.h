@@ -239,14 +239,29 @@ int iex_csr_softmax(int dtype, int m, int nonzeros, const int* row_indices,
  * stride_* are element strides between batch entries (0 = operand shared by the batch).
  * Bits 4..7 of trans_b force the kernel for tuning: 5 = 128x128, 6 = 128x256, 7 = 256x256 tiles,
  * 8 = 128x128 and 9 = 64x128 by eight waves with K steps of 64 (few tiles, long K), 10 = 128x256 by eight waves
- * (11: with K steps of 64), all with the operands loaded from global memory straight into LDS (0 = choose picks
- * among 5 and 7..10);
+ * (11: with K steps of 64), 12 = 256x256 with K split over two workgroups per tile (iex_gemm_ws only), all with the
+ * operands loaded from global memory straight into LDS (0 = choose picks among 5 and 7..10);
  * 1 = 128x128, 2 = 128x256, 3 = 256x256, 4 = 128x128 with K steps of 64, operands staged through
  * registers.  K % 8 == 0, N % 8 == 0 for a (K,N) B, 16-byte aligned operands.
  * Replaces the cuBLAS / CUTLASS / Triton companions of tests/test_interleaving.py:26-345. */
 int iex_gemm(int dtype, int trans_b, int M, int N, int K, const void* A, const void* B,
              void* C, int batch, long long stride_a, long long stride_b,
              long long stride_c, void* stream);
+
+/* iex_gemm with a workspace in device memory that the call may use (and overwrite) until the work it
+ * puts on `stream` has run.  Used by one kernel, which runs on request only: shape code 12 (bits 4..7
+ * of trans_b) = 256 x 256 tiles with K split over two workgroups per tile; the first of the two to
+ * finish leaves its fp32 partial sums in the workspace (M * N * 4 bytes rounded up to whole tiles, plus
+ * two words per tile; 256-byte aligned), the other adds them to its own and stores the tile; the result
+ * does not depend on which was first.  K >= 64, plain store.  Code 12 fails without the workspace;
+ * every other code ignores it and runs exactly as iex_gemm.  iex_gemm_workspace_bytes returns 0 where
+ * the workspace would not be used.  Neither call allocates.  (Measured on the product it was built
+ * for, 4096 x 2048 x 4096: slower than what iex_gemm picks by itself, so it is never picked.)
+ * No counterpart in the reference (its dense companions are library calls). */
+int iex_gemm_ws(int dtype, int trans_b, int M, int N, int K, const void* A, const void* B,
+                void* C, int batch, long long stride_a, long long stride_b,
+                long long stride_c, void* stream, void* workspace, size_t workspace_bytes);
+size_t iex_gemm_workspace_bytes(int dtype, int trans_b, int M, int N, int K, int batch);
 
 /* ----------------------------------------------- horizontally fused launch ---- */
 /* One launch whose workgroups are split between tiles of the dense GEMM C[z] = A[z]*B[z]

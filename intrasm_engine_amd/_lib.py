@@ -47,6 +47,8 @@ SIGNATURES = {
     "iex_CudaSddmm2": (_i, [_i, _i, _i, _i, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i]),
     "iex_csr_softmax": (_i, [_i, _i, _i, _vp, _vp, _vp, _f, _vp, _i]),
     "iex_gemm": (_i, [_i, _i, _i, _i, _i, _vp, _vp, _vp, _i, _ll, _ll, _ll, _vp]),
+    "iex_gemm_ws": (_i, [_i, _i, _i, _i, _i, _vp, _vp, _vp, _i, _ll, _ll, _ll, _vp, _vp, _c.c_size_t]),
+    "iex_gemm_workspace_bytes": (_c.c_size_t, [_i, _i, _i, _i, _i, _i]),
     "iex_fused_spmm_gemm": (_i, [_i, _i, _i, _i, _i, _vp, _vp, _vp, _vp, _vp, _vp,
                                  _i, _i, _i, _i, _i, _vp, _vp, _vp, _i, _ll, _ll, _ll, _i, _vp]),
     "iex_fused_role": (_i, [_i, _i, _i, _i, _c.POINTER(_i), _c.POINTER(_i)]),

@@ -94,8 +94,76 @@ int launch_dma(GemmParams p, int batch, hipStream_t stream) {
   return check_hip(hipGetLastError(), "gemm launch");
 }
 
+// K split over two workgroups per 256 x 256 tile, for products with so few tiles that half the CUs would idle
+// and a long K.  Workgroups b and b + 8 (same XCD, dispatched one after the other) take the two halves of one tile.
+// On request only (shape code 12): built for config 4's 4096 x 2048 x 4096 (128 tiles of 256 x 256), where it takes
+// 92 us against 71 for 128 x 256 tiles by eight waves and 107 for the unsplit 256 x 256 tiles: the K loop of half the
+// length runs 74 us, not half of 107 (prologue and epilogue of a 256 x 256 tile are 10 us whatever K is), and handing
+// 32 MB of fp32 partial sums from one workgroup to the other costs another 18.
+__global__ void fill_zero_kernel(int* p, int n) {
+  const int i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < n) p[i] = 0;
+}
+
 template <bool BF16, bool TRANS_B>
-int launch_shape(const GemmParams& p, int batch, int force, hipStream_t stream) {
+__global__ __launch_bounds__(256, 1) void gemm_dma_splitk_kernel(GemmParams p) {
+  extern __shared__ __align__(16) unsigned char smem[];
+  const int b = blockIdx.x;
+  const int part = (b >> 3) & 1, slot = (b >> 4) * kXcds + (b & 7);
+  int tile_m, tile_n;
+  if (!xcd_tile(slot, p.tiles_m, p.tiles_n, tile_m, tile_n)) return;  // uniform per block
+  const int first = ((p.K + 31) / 32 / 2) * 32;   // K entries of the first half: whole steps
+  GemmParams q = p;
+  q.ldk = p.K;
+  if (part == 0) {
+    q.K = first;
+  } else {
+    q.K = p.K - first;
+    q.A = static_cast<const unsigned short*>(p.A) + first;
+    q.B = static_cast<const unsigned short*>(p.B) + (TRANS_B ? (size_t)first : (size_t)first * p.N);
+  }
+  gemm_tile_dma<BF16, TRANS_B, 4, 4, 2, 32, 4, true>(q, tile_m, tile_n, blockIdx.y, smem);
+}
+
+inline size_t gemm_splitk_bytes(int M, int N, int batch) {
+  const size_t tiles = (size_t)ceil_div(M, 256) * ceil_div(N, 256) * batch;
+  return tiles * 256 * 256 * sizeof(float) + ((tiles * 2 * sizeof(int) + 255) / 256) * 256;
+}
+
+template <bool BF16, bool TRANS_B>
+int launch_dma_splitk(GemmParams p, int batch, void* ws, hipStream_t stream) {
+  p.tiles_m = ceil_div(p.M, 256);
+  p.tiles_n = ceil_div(p.N, 256);
+  const int total = p.tiles_m * p.tiles_n;
+  const int per_xcd = (total + kXcds - 1) / kXcds;
+  p.split_ws = static_cast<float*>(ws);
+  p.split_flags = reinterpret_cast<int*>(static_cast<unsigned char*>(ws) + (size_t)total * batch * 256 * 256 * sizeof(float));
+  constexpr int lds = gemm_dma_lds_bytes<4, 4, 2, 32, 4>();
+  auto kern = gemm_dma_splitk_kernel<BF16, TRANS_B>;
+  static thread_local bool raised = false;  // per instantiation
+  if (!raised) {
+    if (int rc = check_hip(hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, lds),
+                           "hipFuncSetAttribute(LDS size)"))
+      return rc;
+    raised = true;
+  }
+  const int flags = 2 * total * batch;
+  note_kernel("fill_zero_kernel");
+  hipLaunchKernelGGL(fill_zero_kernel, dim3(ceil_div(flags, 256)), dim3(256), 0, stream, p.split_flags, flags);
+  note_kernel("gemm_dma_splitk_kernel<%s, %s> (256 x 256 tiles, K in two halves)", BF16 ? "bf16" : "f16", TRANS_B ? "B(N,K)" : "B(K,N)");
+  hipLaunchKernelGGL(kern, dim3(per_xcd * kXcds * 2, batch), dim3(256), lds, stream, p);
+  return check_hip(hipGetLastError(), "gemm (split K) launch");
+}
+
+template <bool BF16, bool TRANS_B>
+int launch_shape(const GemmParams& p, int batch, int force, hipStream_t stream, void* ws, size_t ws_bytes) {
+  const bool ws_fits = ws && aligned(ws, 256) && ws_bytes >= gemm_splitk_bytes(p.M, p.N, batch);
+  if (force == 12) {
+    IEX_REQUIRE(p.K >= 64, IEX_ERR_UNSUPPORTED, "gemm: the K-split kernel needs K >= 64 (K=%d)", p.K);
+    IEX_REQUIRE(ws_fits && !p.accumulate, IEX_ERR_BAD_ARGUMENT, "gemm: the K-split kernel needs a 256-byte aligned workspace of %zu bytes (iex_gemm_ws) and a plain store",
+                gemm_splitk_bytes(p.M, p.N, batch));
+    return launch_dma_splitk<BF16, TRANS_B>(p, batch, ws, stream);
+  }
   if (force == 1) return launch<BF16, TRANS_B, 2, 2>(p, batch, stream);
   if (force == 2) return launch<BF16, TRANS_B, 2, 4>(p, batch, stream);
   if (force == 3) return launch<BF16, TRANS_B, 4, 4>(p, batch, stream);
@@ -154,16 +222,31 @@ int launch_shape(const GemmParams& p, int batch, int force, hipStream_t stream) 
 // trans_b: bit 0 = B is (N, K); bits 4..7 force the kernel for tuning.  Register-staged operands:
 // 1 = 128x128 tiles, 2 = 128x256, 3 = 256x256, 4 = 128x128 with K steps of 64.  Operands loaded
 // straight into LDS: 5 = 128x128, 6 = 128x256, 7 = 256x256, 8 = 128x128, 9 = 64x128 by eight waves with K steps of 64,
-// 10 = 128x256 by eight waves, 11 = the same with K steps of 64.  0 = choose (one of 5..10).
+// 10 = 128x256 by eight waves, 11 = the same with K steps of 64, 12 = 256x256 with K split over two workgroups per tile
+// (iex_gemm_ws only; never chosen).  0 = choose (one of 5..10).
 extern "C" int iex_gemm(int dtype, int trans_b_and_shape, int M, int N, int K, const void* A, const void* B, void* C, int batch,
                         long long stride_a, long long stride_b, long long stride_c, void* stream) {
   iex::trail_reset();
   return iex::gemm_dispatch(dtype, trans_b_and_shape, M, N, K, A, B, C, batch, stride_a, stride_b, stride_c, stream, nullptr, 0, 0);
 }
 
+extern "C" int iex_gemm_ws(int dtype, int trans_b_and_shape, int M, int N, int K, const void* A, const void* B, void* C, int batch,
+                           long long stride_a, long long stride_b, long long stride_c, void* stream, void* workspace, size_t workspace_bytes) {
+  iex::trail_reset();
+  return iex::gemm_dispatch(dtype, trans_b_and_shape, M, N, K, A, B, C, batch, stride_a, stride_b, stride_c, stream, nullptr, 0, 0, workspace,
+                            workspace_bytes);
+}
+
+extern "C" size_t iex_gemm_workspace_bytes(int dtype, int trans_b_and_shape, int M, int N, int K, int batch) {
+  if (M <= 0 || N <= 0 || K <= 0 || batch <= 0 || (dtype != IEX_F16 && dtype != IEX_BF16)) return 0;
+  const int force = (trans_b_and_shape >> 4) & 0xf;
+  if (force == 12) return iex::gemm_splitk_bytes(M, N, batch);
+  return 0;
+}
+
 int iex::gemm_dispatch(int dtype, int trans_b_and_shape, int M, int N, int K, const void* A, const void* B, void* C, int batch,
                        long long stride_a, long long stride_b, long long stride_c, void* stream, const float* row_bias, int relu,
-                       int accumulate) {
+                       int accumulate, void* workspace, size_t workspace_bytes) {
   const int trans_b = trans_b_and_shape & 1, force = (trans_b_and_shape >> 4) & 0xf;
   IEX_REQUIRE(M >= 0 && N >= 0 && K >= 0 && batch >= 0, IEX_ERR_BAD_ARGUMENT, "gemm: negative dimension");
   if (M == 0 || N == 0 || batch == 0) return 0;
@@ -180,8 +263,8 @@ int iex::gemm_dispatch(int dtype, int trans_b_and_shape, int M, int N, int K, co
   p.stream_out = (double)M * N * batch * 2 >= 128e6;
   hipStream_t s = static_cast<hipStream_t>(stream);
   const bool bf = dtype == IEX_BF16;
-  if (bf && trans_b) return launch_shape<true, true>(p, batch, force, s);
-  if (bf && !trans_b) return launch_shape<true, false>(p, batch, force, s);
-  if (!bf && trans_b) return launch_shape<false, true>(p, batch, force, s);
-  return launch_shape<false, false>(p, batch, force, s);
+  if (bf && trans_b) return launch_shape<true, true>(p, batch, force, s, workspace, workspace_bytes);
+  if (bf && !trans_b) return launch_shape<true, false>(p, batch, force, s, workspace, workspace_bytes);
+  if (!bf && trans_b) return launch_shape<false, true>(p, batch, force, s, workspace, workspace_bytes);
+  return launch_shape<false, false>(p, batch, force, s, workspace, workspace_bytes);
 }

@@ -36,16 +36,23 @@ struct GemmParams {
   const float* row_bias = nullptr;
   int relu = 0, accumulate = 0;
   int stream_out = 0;  // C is far larger than the caches: store it with the streaming hint
+  // K split over two workgroups per tile (gemm.hip): the row stride of A and of an (N, K) B when K above is only a
+  // part of it (0: K is the stride), where the first workgroup to finish a tile leaves its fp32 partial sums, and
+  // per tile a ticket counter and a "partial sums written" flag (both zero at launch)
+  int ldk = 0;
+  float* split_ws = nullptr;
+  int* split_flags = nullptr;
 };
 
 // iex_gemm with the epilogue options above (gemm.hip).
 int gemm_dispatch(int dtype, int trans_b_and_shape, int M, int N, int K, const void* A, const void* B, void* C, int batch,
                   long long stride_a, long long stride_b, long long stride_c, void* stream, const float* row_bias, int relu,
-                  int accumulate);
+                  int accumulate, void* workspace = nullptr, size_t workspace_bytes = 0);
 
 typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef float f32x16 __attribute__((ext_vector_type(16)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
 typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
 typedef unsigned int u32x2 __attribute__((ext_vector_type(2)));
 
@@ -173,7 +180,7 @@ struct GemmStage {
 // Writes the WM x WN accumulator blocks of one wavefront to C (rounded to the 16-bit type).
 template <bool BF16, int WM, int WN>
 __device__ __forceinline__ void gemm_store_tile(const GemmParams& p, const f32x16 (&acc)[WM][WN], unsigned short* __restrict__ C,
-                                                int m0, int n0, int wm, int wn, int lane) {
+                                                int m0, int n0, int wm, int wn, int lane, const float* partial = nullptr) {
   typedef unsigned short u16;
   // Swapped-operand result layout: lane holds row (lane % 32) of the 32x32 block and, in
   // accumulator quad q, columns q*8 + (lane / 32)*4 .. +3.
@@ -193,6 +200,10 @@ __device__ __forceinline__ void gemm_store_tile(const GemmParams& p, const f32x1
         float x[4];
 #pragma unroll
         for (int e = 0; e < 4; ++e) x[e] = acc[i][j][q * 4 + e];
+        if (partial) {   // the other half of K: this lane's sums in the same order, 256 floats per (block, quad)
+          const f32x4 o = *reinterpret_cast<const f32x4*>(partial + ((i * WN + j) * 4 + q) * 256);
+          x[0] += o.x, x[1] += o.y, x[2] += o.z, x[3] += o.w;
+        }
         if (p.accumulate) {
           if (vec_ok) {
             const u32x2 w = *reinterpret_cast<const u32x2*>(dst);
@@ -241,7 +252,8 @@ constexpr int gemm_store_lds_bytes() { return 32 * (WN * 64 + 16); }
 
 template <bool BF16, int WM, int WN>
 __device__ __forceinline__ void gemm_store_tile_lds(const GemmParams& p, const f32x16 (&acc)[WM][WN], unsigned short* __restrict__ C,
-                                                    int m0, int n0, int wm, int wn, int lane, unsigned char* lds, bool stream) {
+                                                    int m0, int n0, int wm, int wn, int lane, unsigned char* lds, bool stream,
+                                                    const float* partial = nullptr) {
   typedef unsigned short u16;
   constexpr int ROWB = WN * 64 + 16;   // bytes of a padded row
   constexpr int CPR = WN * 4;          // 16-byte chunks per row
@@ -258,9 +270,11 @@ __device__ __forceinline__ void gemm_store_tile_lds(const GemmParams& p, const f
 #pragma unroll
       for (int q = 0; q < 4; ++q) {
         u16 h[4];
+        f32x4 o = {0.f, 0.f, 0.f, 0.f};
+        if (partial) o = *reinterpret_cast<const f32x4*>(partial + ((i * WN + j) * 4 + q) * 256);   // the other half of K
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
-          float y = acc[i][j][q * 4 + e] + bias;
+          float y = acc[i][j][q * 4 + e] + o[e] + bias;
           if (p.relu) y = fmaxf(y, 0.f);
           h[e] = f32_to_16(y, BF16);
         }

@@ -44,7 +44,7 @@ constexpr int gemm_dma_lds_bytes() {
   return STAGES * (2 * WM * 32 + WCN * WN * 32) * BK * 2;
 }
 
-template <bool BF16, bool TRANS_B, int WM, int WN, int WCN, int BK, int STAGES>
+template <bool BF16, bool TRANS_B, int WM, int WN, int WCN, int BK, int STAGES, bool SPLIT = false>
 __device__ __forceinline__ void gemm_tile_dma(const GemmParams& p, int tile_m, int tile_n, int z, unsigned char* smem) {
   constexpr int BM = 2 * WM * 32, BN = WCN * WN * 32, WAVES = 2 * WCN;
   constexpr int CPR = BK / 8;          // 16-byte chunks per K-contiguous row
@@ -72,6 +72,7 @@ __device__ __forceinline__ void gemm_tile_dma(const GemmParams& p, int tile_m, i
   const u16* __restrict__ B = static_cast<const u16*>(p.B) + (size_t)z * p.stride_b;
   u16* __restrict__ C = static_cast<u16*>(p.C) + (size_t)z * p.stride_c;
   const unsigned lds0 = (unsigned)(size_t)(lds_u8*)smem;  // LDS byte address of stage 0
+  const int ld = p.ldk ? p.ldk : p.K;  // row stride of the K-contiguous operands
 
   // ---- what this lane fetches: per instruction a row pointer (or a column offset) and a chunk
   const u16* a_row[A_INSTR];
@@ -80,7 +81,7 @@ __device__ __forceinline__ void gemm_tile_dma(const GemmParams& p, int tile_m, i
   for (int q = 0; q < A_INSTR; ++q) {
     const int row = (wave * A_INSTR + q) * RPI + lane / CPR;
     const int sw = CPR == 4 ? (row >> 2) & 3 : (row >> 1) & 7;
-    a_row[q] = A + (size_t)min(m0 + row, p.M - 1) * p.K;
+    a_row[q] = A + (size_t)min(m0 + row, p.M - 1) * ld;
     a_k8[q] = ((lane % CPR) ^ sw) * 8;
   }
   const u16* b_row[B_INSTR];  // (N,K): row pointer; (K,N): B + clamped column
@@ -90,7 +91,7 @@ __device__ __forceinline__ void gemm_tile_dma(const GemmParams& p, int tile_m, i
     if constexpr (TRANS_B) {
       const int row = (wave * B_INSTR + q) * RPI + lane / CPR;
       const int sw = CPR == 4 ? (row >> 2) & 3 : (row >> 1) & 7;
-      b_row[q] = B + (size_t)min(n0 + row, p.N - 1) * p.K;
+      b_row[q] = B + (size_t)min(n0 + row, p.N - 1) * ld;
       b_k8[q] = ((lane % CPR) ^ sw) * 8;
     } else {
       const int kr = (wave * B_INSTR + q) * RPIB + lane / CPRB;
@@ -233,13 +234,54 @@ __device__ __forceinline__ void gemm_tile_dma(const GemmParams& p, int tile_m, i
   }
   wait_vmcnt<0>();  // the re-fetched last tiles: nothing may still be writing LDS when the workgroup ends
 
+  const float* partial = nullptr;
+  if constexpr (SPLIT) {
+    // Two workgroups hold partial sums of this tile (one half of K each).  Whichever finishes first leaves its sums in
+    // the workspace and is done; the other adds them to its own and stores the tile (a + b = b + a: the result does
+    // not depend on who was first).  The second only ever waits for a workgroup that is past its K loop and waits for
+    // nothing itself.
+    constexpr int NMT = WM * WN;
+    const int tile_id = (z * p.tiles_m + tile_m) * p.tiles_n + tile_n;
+    int* tickets = p.split_flags;
+    int* written = p.split_flags + (size_t)gridDim.y * p.tiles_m * p.tiles_n;
+    float* mine = p.split_ws + (size_t)tile_id * (BM * BN) + (size_t)wave * (NMT * 16 * 64) + lane * 4;
+    __syncthreads();  // everybody has read its last fragments: the stages are free
+    if (tid == 0) *reinterpret_cast<int*>(smem) = atomicAdd(&tickets[tile_id], 1);
+    __syncthreads();
+    const int ticket = *reinterpret_cast<volatile int*>(smem);
+    if (ticket == 0) {
+#pragma unroll
+      for (int i = 0; i < WM; ++i)
+#pragma unroll
+        for (int j = 0; j < WN; ++j)
+#pragma unroll
+          for (int q = 0; q < 4; ++q) {
+            const f32x4 v = {acc[i][j][q * 4], acc[i][j][q * 4 + 1], acc[i][j][q * 4 + 2], acc[i][j][q * 4 + 3]};
+            *reinterpret_cast<f32x4*>(mine + ((i * WN + j) * 4 + q) * 256) = v;
+            if (q == 3) __builtin_amdgcn_sched_barrier(0);
+          }
+      // The two workgroups of a tile run on one XCD (the launcher's numbering), whose L2 both see: once my stores
+      // have left the CU (the workgroup-scope fence waits for that) the flag may go up.  Device-scope fences here
+      // would write back and invalidate that L2 under every workgroup still multiplying (measured: 2.5 x slower).
+      __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+      __syncthreads();
+      if (tid == 0) __hip_atomic_store(&written[tile_id], 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      return;
+    }
+    if (tid == 0)   // (bounded: about a tenth of a second, far beyond any epilogue; a kernel must end whatever happens)
+      for (int spins = 0; spins < (1 << 20) && __hip_atomic_load(&written[tile_id], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == 0; ++spins)
+        __builtin_amdgcn_s_sleep(4);
+    __syncthreads();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");   // (this CU has never read these lines: they come from L2)
+    partial = mine;   // added where the sums are rounded and stored (adding them here would need all 256 sums in VGPRs at once)
+  }
   // the stages are free now: row-contiguous stores through LDS where the shape allows
   static_assert(WAVES * gemm_store_lds_bytes<WN>() <= gemm_dma_lds_bytes<WM, WN, WCN, BK, STAGES>(), "the epilogue fits the stages");
   if (!p.accumulate && p.N % 8 == 0 && (reinterpret_cast<uintptr_t>(C) & 15) == 0) {
     __syncthreads();  // everybody has read its last fragments
-    gemm_store_tile_lds<BF16, WM, WN>(p, acc, C, m0, n0, wm, wn, lane, smem + wave * gemm_store_lds_bytes<WN>(), p.stream_out != 0);
+    gemm_store_tile_lds<BF16, WM, WN>(p, acc, C, m0, n0, wm, wn, lane, smem + wave * gemm_store_lds_bytes<WN>(), p.stream_out != 0, partial);
   } else {
-    gemm_store_tile<BF16, WM, WN>(p, acc, C, m0, n0, wm, wn, lane);
+    gemm_store_tile<BF16, WM, WN>(p, acc, C, m0, n0, wm, wn, lane, partial);
   }
 }
 

@@ -40,7 +40,7 @@ def kernel_params(*, spmm: dict | None = None, sddmm: dict | None = None, gemm: 
     """Kernel choices for the operators called inside the block (this thread only), for tuning:
     ``spmm`` = any of force_variant / force_rpw / force_nt / force_lpg / force_wpr (the tuning
     bits of ``iex_spmm_ex``), ``sddmm`` = force_wpr / force_variant, ``gemm`` = tile (the shape code of
-    ``iex_gemm``: 5 = 128x128, 6 = 128x256, 7 = 256x256 tiles, 8 = 128x128 and 9 = 64x128 by eight waves with K steps of 64, 10 = 128x256 by eight waves; 1..4 = the
+    ``iex_gemm``: 5 = 128x128, 6 = 128x256, 7 = 256x256 tiles, 8 = 128x128 and 9 = 64x128 by eight waves with K steps of 64, 10 = 128x256 by eight waves, 12 = 256x256 with K split over two workgroups per tile; 1..4 = the
     register-staged kernels).
     Without a block, or for a key left out, the library chooses; a category left out (None) keeps
     what an enclosing block set for it.  A kernel family that cannot
@@ -316,8 +316,13 @@ def gemm_mfma(a, b, trans_b=False, out=None):
              and out.device == a.device, "out has the wrong shape, dtype, layout or device")
     with torch.cuda.device(a.device):
         tile = (getattr(_TUNING, "gemm", None) or {}).get("tile", 0)
-        rc = _lib.load().iex_gemm(_DT[a.dtype], int(bool(trans_b)) | ((int(tile) & 0xf) << 4), M, N, K, a.data_ptr(), b.data_ptr(),
-                                  out.data_ptr(), batch, sa, sb, M * N, _stream_ptr(a.device))
+        lib = _lib.load()
+        code = int(bool(trans_b)) | ((int(tile) & 0xf) << 4)
+        # room for the partial sums where the library would split K over two workgroups per tile (few tiles, long K)
+        ws_bytes = lib.iex_gemm_workspace_bytes(_DT[a.dtype], code, M, N, K, batch)
+        ws = torch.empty(ws_bytes, dtype=torch.uint8, device=a.device) if ws_bytes else None
+        rc = lib.iex_gemm_ws(_DT[a.dtype], code, M, N, K, a.data_ptr(), b.data_ptr(), out.data_ptr(), batch, sa, sb, M * N,
+                             _stream_ptr(a.device), ws.data_ptr() if ws is not None else None, ws_bytes)
     _lib.check(rc, "gemm")
     return out
 

@@ -38,13 +38,13 @@ def test_gemm_ragged_n_with_transposed_b(oracle, dev, shape):
         ops.gemm_mfma(torch.zeros(8, 8, device=dev).half(), torch.zeros(8, shape[1] | 1, device=dev).half(), False)
 
 
-@pytest.mark.parametrize("shape_code", [1, 2, 3, 4, 5, 6, 7, 8, 9])
+@pytest.mark.parametrize("shape_code", [1, 2, 3, 4, 5, 6, 7, 8, 9, 10, 11])
 @pytest.mark.parametrize("trans_b", [False, True])
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
 @pytest.mark.parametrize("mnk", [(300, 520, 200), (129, 136, 8), (260, 264, 1000)])
 def test_every_tile_shape(oracle, dev, shape_code, trans_b, dtype, mnk):
     """Every kernel of the GEMM entry point forced through the C ABI (register-staged 128x128, 128x256, 256x256 tiles
-    and 128x128 with K steps of 64; 128x128, 128x256, 256x256, and 128x128 and 64x128 by eight waves with K steps of 64, operands loaded straight
+    and 128x128 with K steps of 64; 128x128, 128x256, 256x256, 128x128 and 64x128 by eight waves with K steps of 64, and 128x256 by eight waves with K steps of 32 and 64, operands loaded straight
     into LDS) on ragged
     problems: m, n and k leave partial tiles and a partial last K step; k = 8 is a single, mostly empty step;
     k = 1000 runs the load pipeline through many steps and ends on a partial one."""
@@ -139,3 +139,65 @@ def test_argument_checks(dev):
         ops.gemm_mfma(a.float(), a.float(), True)
     with pytest.raises(RuntimeError, match="inner dimensions"):
         ops.gemm_mfma(torch.randn(16, 16, device=dev).half(), torch.randn(8, 16, device=dev).half(), False)
+
+
+@pytest.mark.parametrize("trans_b", [False, True])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("mnk,batch", [((300, 520, 200), 1), ((260, 264, 1000), 3), ((512, 256, 64), 2), ((129, 136, 2048), 1)])
+def test_k_split_over_two_workgroups(oracle, dev, trans_b, dtype, mnk, batch):
+    """256 x 256 tiles with K split over two workgroups per tile (partial sums meet in a workspace, the second
+    workgroup to arrive adds and stores), on request: ragged m, n, a K whose halves are 96 + 104, 512 + 488 (a partial
+    last step), 32 + 32; batches; against the oracle, twice with the same bits, and on integer operands exactly equal
+    to the unsplit kernel."""
+    from intrasm_engine_amd.pytorch import ops as pyops
+    rng = np.random.default_rng(batch)
+    M, N, K = mnk
+    a_np = rng.standard_normal((batch, M, K)).astype(np.float32)
+    b_np = rng.standard_normal((batch, N, K) if trans_b else (batch, K, N)).astype(np.float32)
+    a, b = torch.from_numpy(a_np).to(dev).to(dtype), torch.from_numpy(b_np).to(dev).to(dtype)
+    with pyops.kernel_params(gemm={"tile": 12}):
+        out = ops.gemm_mfma(a, b, trans_b)
+        again = ops.gemm_mfma(a, b, trans_b)
+    assert torch.equal(out, again)
+    for z in range(batch):
+        a_r, b_r = rounded(a_np[z], dtype), rounded(b_np[z], dtype)
+        want = oracle.gemm(a_r, b_r, trans_b=trans_b)
+        scale = oracle.gemm(np.abs(a_r), np.abs(b_r), trans_b=trans_b)
+        assert_close(out[z].float().cpu().numpy(), want, scale, 1e-2, f"split-K gemm {M}x{N}x{K} {dtype} trans_b={trans_b} entry {z}")
+    ai = torch.from_numpy(rng.integers(-3, 4, a_np.shape).astype(np.float32)).to(dev).to(dtype)
+    bi = torch.from_numpy(rng.integers(-3, 4, b_np.shape).astype(np.float32)).to(dev).to(dtype)
+    with pyops.kernel_params(gemm={"tile": 12}):
+        split = ops.gemm_mfma(ai, bi, trans_b)
+    with pyops.kernel_params(gemm={"tile": 7}):
+        whole = ops.gemm_mfma(ai, bi, trans_b)
+    assert torch.equal(split, whole)
+
+
+def test_k_split_on_config4s_product_and_refused_without_workspace(oracle, dev):
+    """The product the kernel was built for (4096 x 2048 x 4096: 128 tiles of 256 x 256), on request; the library never
+    picks it by itself (it measured slower than 128 x 256 tiles by eight waves)."""
+    from intrasm_engine_amd import _lib
+    from intrasm_engine_amd.pytorch import ops as pyops
+    lib = _lib.load()
+    assert lib.iex_gemm_workspace_bytes(_lib.BF16, 12 << 4, 4096, 2048, 4096, 1) == 128 * 256 * 256 * 4 + 1024
+    assert lib.iex_gemm_workspace_bytes(_lib.BF16, 0, 4096, 2048, 4096, 1) == 0
+    rng = np.random.default_rng(4)
+    a_np = rng.standard_normal((4096, 4096)).astype(np.float32)
+    b_np = rng.standard_normal((4096, 2048)).astype(np.float32)
+    a, b = torch.from_numpy(a_np).to(dev).bfloat16(), torch.from_numpy(b_np).to(dev).bfloat16()
+    plain = ops.gemm_mfma(a, b, False)
+    assert "splitk" not in _lib.last_kernels()
+    with pyops.kernel_params(gemm={"tile": 12}):
+        out = ops.gemm_mfma(a, b, False)
+    assert "gemm_dma_splitk_kernel" in _lib.last_kernels()
+    rows = np.arange(0, 4096, 67)
+    a_r, b_r = rounded(a_np[rows], torch.bfloat16), rounded(b_np, torch.bfloat16)
+    want = oracle.gemm(a_r, b_r)
+    scale = np.abs(a_r).astype(np.float64) @ np.abs(b_r).astype(np.float64)
+    assert_close(out[torch.from_numpy(rows).to(dev)].float().cpu().numpy(), want, scale, 1e-2, "config 4's product, K split")
+    assert torch.allclose(plain.float(), out.float(), rtol=2e-2, atol=1.0)
+    c = torch.empty_like(out)
+    rc = lib.iex_gemm(_lib.BF16, 12 << 4, 4096, 2048, 4096, a.data_ptr(), b.data_ptr(), c.data_ptr(), 1, 0, 0, 0,
+                      torch.cuda.current_stream().cuda_stream)
+    assert rc != 0 and "workspace" in _lib.last_error()
+    torch.cuda.synchronize()

@@ -170,6 +170,24 @@ class SddmmPlan:
     def __init__(self):
         self.workspace = None
         self.key = None
+        self.variant = 0        # 0: the library's rule (by density); 1 / 3 after analyze()
+        self.dense_share = None
+
+    def analyze(self, row_offsets, column_indices, n, dense_min=2048):
+        """Look at the pattern once (copies the index arrays to the host: a synchronisation, so not under capture and
+        not per call) and settle which kernel the plan's calls use: the one for masks with structure when at least
+        half of the nonzeros sit in 128 x 128 blocks that hold ``dense_min`` or more of them, else the gather kernel.
+        The library's own rule only knows the overall density, which a band and a random mask can share."""
+        import numpy as np
+        ro = row_offsets.detach().cpu().numpy().astype(np.int64)
+        ci = column_indices.detach().cpu().numpy().astype(np.int64)
+        m = ro.shape[0] - 1
+        rows = np.repeat(np.arange(m, dtype=np.int64), np.diff(ro))
+        tiles_n = (int(n) + 127) // 128
+        counts = np.bincount((rows // 128) * tiles_n + np.minimum(ci // 128, tiles_n - 1), minlength=((m + 127) // 128) * tiles_n)
+        self.dense_share = float(counts[counts >= dense_min].sum()) / max(1, ci.shape[0])
+        self.variant = 3 if self.dense_share >= 0.5 else 1
+        return self.variant
 
     def _ready(self, key, nbytes, device):
         """Workspace of nbytes for this key; True when it already holds the key's tables."""
@@ -186,6 +204,8 @@ def _sddmm(a, b, row_indices, row_offsets, column_indices, *, sum_over_batch, dt
     tuned = getattr(_TUNING, "sddmm", None)
     if tuned and not (force_wpr or force_variant):
         force_wpr, force_variant = tuned.get("force_wpr", 0), tuned.get("force_variant", 0)
+    if plan is not None and plan.variant and not force_variant:
+        force_variant = plan.variant      # settled by SddmmPlan.analyze(); variant 3 still has to fit (dtype, k): checked below
     _chk(a.dim() == b.dim())
     _chk(a.dim() == 3)
     _chk(a.size(0) == b.size(0))
@@ -213,6 +233,9 @@ def _sddmm(a, b, row_indices, row_offsets, column_indices, *, sum_over_batch, dt
             (_lib.SDDMM_ACCUMULATE if accumulate else 0) | ((int(force_wpr) & 0xff) << 8) | \
             ((int(force_variant) & 0xf) << 16)
     lib = _lib.load()
+    if plan is not None and plan.variant == 3 and force_variant == 3 and \
+            lib.iex_sddmm_workspace_kind(_DT[a.dtype], flags, m, k, n, nonzeros, batch) != 3:
+        flags &= ~(0xf << 16)            # the planned kernel does not serve this call (fp32, another k): the library's rule
     with torch.cuda.device(a.device):
         # room for the dense product where the library would rather compute all of it on the matrix
         # cores and pick the nonzeros (16-bit, long k): from torch's allocator, on the current stream

@@ -143,6 +143,35 @@ def test_tables_kept_between_calls_of_one_mask(oracle, dev):
     assert torch.equal(a0, a1) and torch.equal(a0, a2)
 
 
+def test_plan_settles_the_kernel_by_the_masks_structure(dev):
+    """Two masks of the same density: a band (its nonzeros sit in dense 128 x 128 blocks) and columns at random.  The
+    library's rule (by density) takes the kernel for masks with structure for both; a plan that has looked at the
+    pattern keeps it for the band and takes the gather kernel for the random one.  Same results either way."""
+    from intrasm_engine_amd import _lib
+    from intrasm_engine_amd.pytorch import ops as pyops
+    rng = np.random.default_rng(5)
+    tokens, heads = 2048, 16
+    q = rng.standard_normal((heads, tokens, 64)).astype(np.float32)
+    k = rng.standard_normal((heads, tokens, 64)).astype(np.float32)
+    qt, kt = torch.from_numpy(q).to(dev).half(), torch.from_numpy(k).to(dev).half()
+    band, *_ = W.config3(tokens=tokens, heads=1, band=160, extra=4)
+    per_row = band.nnz // tokens
+    ro, ci = W.csr_from_row_lengths(rng, tokens, tokens, np.full(tokens, per_row))
+    rand = W.CSR(tokens, tokens, np.ones(ci.shape[0], np.float32), W.swizzle_from_offsets(ro), ro, ci)
+    for csr, variant, kernel in ((band, 3, "sddmm_mfma_kernel"), (rand, 1, "sddmm_kernel")):
+        ri, _, ro_t, ci_t = to_dev(csr, dev)
+        auto = ops.sddmm_sputnik_half(qt, kt, ri, ro_t, ci_t)
+        assert "sddmm_mfma_kernel" in _lib.last_kernels()
+        plan = pyops.SddmmPlan()
+        assert plan.analyze(ro_t, ci_t, tokens) == variant, plan.dense_share
+        planned = pyops.sddmm_half_planned(qt, kt, ri, ro_t, ci_t, plan)
+        assert kernel in _lib.last_kernels()
+        assert torch.allclose(planned.float(), auto.float(), rtol=1e-2, atol=1e-2 * 8.0 * 0.1)
+        # fp32 operands through the same plan: the planned kernel does not serve them, the call runs all the same
+        f32 = pyops.sddmm_half_planned(qt.float(), kt.float(), ri, ro_t, ci_t, plan)
+        assert torch.allclose(f32, auto.float(), rtol=1e-2, atol=1e-2 * 8.0 * 0.1)
+
+
 def test_refusals(dev):
     from intrasm_engine_amd import _lib
     rng = np.random.default_rng(1)

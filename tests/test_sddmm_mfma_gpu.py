@@ -104,6 +104,35 @@ def test_config3_four_heads_against_the_oracle_and_sixteen_against_the_gather_ke
     assert torch.allclose(auto.float(), gather, rtol=1e-2, atol=1e-2 * 8.0 * 0.1)
 
 
+@pytest.mark.parametrize("n", [9000, 20100, 65536])
+@pytest.mark.parametrize("blocks", [0, 1, 255])
+def test_many_column_blocks(oracle, dev, n, blocks):
+    """More than 64 (and more than 128) blocks of 128 columns per row: the setup kernel, the workgroup's list of dense
+    and thin blocks and the runs of thin blocks between dense ones all work in pieces of 64 blocks.  A band that
+    wanders through the columns plus scattered entries, 260 rows, two batch entries; n = 65536 is the largest the
+    kernel takes (one more column is refused)."""
+    rng = np.random.default_rng(n)
+    m, k = 260, 64
+    idx = np.arange(m)
+    centre = (idx * (n - 200) // m) + 100
+    cols = [np.unique(np.concatenate([np.arange(c - 40, c + 40), rng.integers(0, n, 12)])) for c in centre]
+    cols[7] = np.array([], dtype=np.int64)
+    cols[100] = np.arange(0, n, 97)                       # a long row that touches every block
+    lens = np.array([len(c) for c in cols])
+    ro = np.zeros(m + 1, dtype=np.int32)
+    np.cumsum(lens, out=ro[1:])
+    ci = np.concatenate(cols).astype(np.int32)
+    csr = W.CSR(m, n, np.ones(ci.shape[0], np.float32), W.swizzle_from_offsets(ro), ro, ci)
+    lhs = rng.standard_normal((2, m, k)).astype(np.float32)
+    rhs = rng.standard_normal((2, n, k)).astype(np.float32)
+    out = _run(dev, csr, lhs, rhs, torch.float16, force_variant=3, force_wpr=blocks)
+    want, scale = _want(oracle, csr, lhs, rhs, torch.float16)
+    assert_close(out.float().cpu().numpy(), want, scale, RTOL[torch.float16], f"n={n} blocks={blocks}", atol=FP16_SUBNORMAL_HALF_STEP)
+    if n == 65536 and blocks == 0:
+        with pytest.raises(RuntimeError, match="matrix-core kernel needs"):
+            _run(dev, csr, lhs, np.concatenate([rhs, rhs[:, :1]], axis=1), torch.float16, force_variant=3)
+
+
 def test_tables_kept_between_calls_of_one_mask(oracle, dev):
     """A caller with a fixed mask keeps a plan: the second call skips the setup kernel and gives the same bits; another
     mask (or the same index tensor changed in place) makes the plan write the tables again; the attention block takes

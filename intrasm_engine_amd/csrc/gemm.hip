@@ -5,28 +5,6 @@
 namespace iex {
 namespace {
 
-constexpr int kXcds = 8;
-constexpr int kGroupM = 4;
-
-// Workgroup ids are dealt round-robin to the 8 XCDs (each with its own L2).  Give every
-// XCD a contiguous band of C tiles (row-major over tiles) so that the A row panels a
-// band needs are fetched into one L2 instead of eight.
-__device__ __forceinline__ bool xcd_tile(int block, int tiles_m, int tiles_n, int& tile_m, int& tile_n) {
-  const int total = tiles_m * tiles_n;
-  const int per_xcd = (total + kXcds - 1) / kXcds;
-  const int linear = (block % kXcds) * per_xcd + block / kXcds;
-  if (linear >= total) return false;
-  // inside the band, walk kGroupM tile rows column by column: the 32 tiles an XCD works on at one
-  // time then share kGroupM row panels of A and 32 / kGroupM column panels of B in its L2
-  const int per_group = kGroupM * tiles_n;
-  const int first_row = (linear / per_group) * kGroupM;
-  const int rows = min(tiles_m - first_row, kGroupM);
-  const int in_group = linear % per_group;
-  tile_m = first_row + in_group % rows;
-  tile_n = in_group / rows;
-  return true;
-}
-
 template <bool BF16, bool TRANS_B, int WM, int WN, int BK>
 __global__ __launch_bounds__(256, (WM * WN <= 8 ? 2 : 1)) void gemm_kernel(GemmParams p) {
   extern __shared__ __align__(16) unsigned char smem[];

@@ -137,7 +137,7 @@ def main():
 
     if args.pmc_probe:
         # for `rocprofv3 --pmc ...`: 3 plain copies of 256 MiB (the calibration of FETCH_SIZE / WRITE_SIZE), then every
-        # fp32 cell 3 times in cell order; the kernel names go to stderr and to gpurun_out/pmc_probe_cells.json
+        # fp32 cell 3 times in cell order; the kernel names go to stderr and to pmc_probe_cells.json in the output folder
         nbytes = 256 << 20
         src = torch.zeros(nbytes // 4, dtype=torch.float32, device=dev)
         dst = torch.empty_like(src)

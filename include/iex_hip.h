@@ -253,7 +253,9 @@ int iex_gemm(int dtype, int trans_b, int M, int N, int K, const void* A, const v
  * of trans_b) = 256 x 256 tiles with K split over two workgroups per tile; the first of the two to
  * finish leaves its fp32 partial sums in the workspace (M * N * 4 bytes rounded up to whole tiles, plus
  * two words per tile; 256-byte aligned), the other adds them to its own and stores the tile; the result
- * does not depend on which was first.  K >= 64, plain store.  Code 12 fails without the workspace;
+ * does not depend on which was first.  The exchange goes through the L2 of the XCD that both workgroups
+ * run on (workgroup ids b and b + 8: ids are dealt round-robin to the 8 XCDs in the mode this library is
+ * built for, one partition spanning the whole GPU).  K >= 64, plain store.  Code 12 fails without the workspace;
  * every other code ignores it and runs exactly as iex_gemm.  iex_gemm_workspace_bytes returns 0 where
  * the workspace would not be used.  Neither call allocates.  (Measured on the product it was built
  * for, 4096 x 2048 x 4096: slower than what iex_gemm picks by itself, so it is never picked.)

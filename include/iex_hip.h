@@ -61,6 +61,14 @@ int iex_copy_bytes(void* dst, const void* src, size_t nbytes, void* stream);
 #define IEX_SPMM_PER_BATCH_VALUES 0x1 /* values is (batch, nnz) instead of (nnz)            */
 #define IEX_SPMM_ACCUMULATE 0x2       /* out += A*b (reference "atomic" store mode)         */
 #define IEX_SPMM_RELU 0x4             /* out = max(0, A*b + bias)                           */
+/* iex_spmm_ws, family 10 only (ignored elsewhere): the workspace still holds the tables that an earlier
+ * call with the same m, k, nonzeros and index arrays wrote there -- a family-10 SpMM, or an SDDMM of
+ * variant 3 on the same pattern (iex_sddmm_ws with n = this call's k): the tables are the same.   */
+#define IEX_SPMM_TABLES_READY 0x8
+/* ... and the lists that family 10 itself derives from the tables (which blocks count as dense, the nonzeros
+ * outside them) are still there too, from a family-10 call with the same bits 8..15.  Only with
+ * IEX_SPMM_TABLES_READY.                                                                              */
+#define IEX_SPMM_LISTS_READY 0x10
 /* bits 8..15: force waves-per-row (1, 4 or 8); 0 = choose from nnz/m.  For tuning.    */
 #define IEX_SPMM_FORCE_WPR(w) (((w) & 0xff) << 8)
 /* bits 16..19: force the kernel family: 1 = row kernel gathering from L2, 2 = LDS-staged
@@ -76,10 +84,18 @@ int iex_copy_bytes(void* dst, const void* src, size_t nbytes, void* stream);
  * kernel in slice order (deterministic); needs n a multiple of 4, 16-byte aligned dense operands, k <= 262144 and,
  * for more than one slice, iex_spmm_ws with the workspace iex_spmm_workspace_bytes reports (bits 20..23: slices,
  * 0 = choose; bits 24..27 = 2: workgroups of 16 wavefronts and 128 rows instead of 8 and 64); fails on other
- * shapes.  0 = choose.
- * Families 2-6 and 9 rely on strictly ascending column indices inside a row (canonical CSR, what
+ * shapes, 10 = sparse operands with structure (attention probabilities: bands, blocks, windows) times a dense
+ * operand of 64 columns, on request only: per 128 rows, the dense 128 x 128 blocks of A are laid out in LDS and
+ * multiplied on the matrix cores, the nonzeros elsewhere are gathered row by row (fp16 / bf16, int32 indices,
+ * n = 64, k <= 65536, plain store without bias or ReLU, values shared or per batch entry; iex_spmm_ws only, with
+ * the workspace iex_spmm_workspace_bytes reports: the tables of SDDMM variant 3 for the pattern, which a small
+ * kernel writes first, and behind them lists that two more small kernels derive from the tables -- see
+ * IEX_SPMM_TABLES_READY / IEX_SPMM_LISTS_READY; bits 8..15 set the number of nonzeros from which a block counts
+ * as dense: 0 = built in (2048), 1 = every block, 255 = none, else 64 * value); fails on other shapes.
+ * 0 = choose.
+ * Families 2-6, 9 and 10 rely on strictly ascending column indices inside a row (canonical CSR, what
  * dense_to_sparse produces); family 1 accepts any order and duplicates -- force it for such
- * input.  Families 3-6 multiply explicit zeros with the dense operand, so a non-finite entry
+ * input.  Families 3-6 and 10 multiply explicit zeros with the dense operand, so a non-finite entry
  * in a row of `dense` that no nonzero references still reaches the output (0 * inf = NaN).
  * bits 20..23: rows per wavefront of family 2 (2, 4 or 8); windows of nonzeros held in
  * registers per row of family 4 (1, 2, 4 or 5 windows of 16), 5 (2, 4 or 8 windows of 8) and

@@ -17,6 +17,8 @@ I32, I16 = 0, 1
 SPMM_PER_BATCH_VALUES = 0x1
 SPMM_ACCUMULATE = 0x2
 SPMM_RELU = 0x4
+SPMM_TABLES_READY = 0x8
+SPMM_LISTS_READY = 0x10
 SDDMM_SUM_OVER_BATCH = 0x1
 SDDMM_ACCUMULATE = 0x2
 SDDMM_TABLES_READY = 0x4

@@ -331,18 +331,14 @@ int launch_sddmm_mfma_ks(const SddmmMfmaParams& q, int batch, hipStream_t stream
 
 int launch_sddmm_mfma(int dtype, const SddmmParams& p, void* ws, int dense_code, bool tables_ready, hipStream_t stream) {
   const int tiles_n = ceil_div(p.n, kSdBN);
-  u32x4* mask = static_cast<u32x4*>(ws);
-  int* tile_ptr = reinterpret_cast<int*>(mask + (size_t)tiles_n * p.m);
-  int* brief = tile_ptr + (size_t)(tiles_n + 1) * p.m;
+  const SdTables t = sd_tables(ws, p.m, tiles_n);
   if (!tables_ready) {   // (else: the caller vouches that an earlier call on this pattern left them in the workspace)
-    note_kernel("sddmm_tile_ptr_kernel");
-    hipLaunchKernelGGL(sddmm_tile_ptr_kernel, dim3(ceil_div(p.m, 4)), dim3(256), 0, stream, p.m, tiles_n, p.row_offsets, p.cols, tile_ptr, brief, mask);
-    if (int rc = check_hip(hipGetLastError(), "sddmm row-cursor launch")) return rc;
+    if (int rc = sd_write_tables(t, p.m, tiles_n, p.row_offsets, p.cols, stream)) return rc;
   }
   // dense_code (for tests and tuning): 0 = the built-in threshold, 1 = every tile on the matrix cores, 255 = none,
   // else 64 * code nonzeros per 128 x 128 block
   const int dense_min = dense_code == 0 ? kSdDenseMin : dense_code == 1 ? 0 : dense_code == 255 ? kSdBM * kSdBN + 1 : 64 * dense_code;
-  SddmmMfmaParams q{p.m, p.k, p.n, p.nnz, p.cols, p.lhs, p.rhs, p.out, mask, tile_ptr, brief, tiles_n, dense_min};
+  SddmmMfmaParams q{p.m, p.k, p.n, p.nnz, p.cols, p.lhs, p.rhs, p.out, t.mask, t.tile_ptr, t.brief, tiles_n, dense_min};
   const bool bf16 = dtype == IEX_BF16;
   switch (p.k) {
     case 32: return bf16 ? launch_sddmm_mfma_ks<true, 2>(q, p.batch, stream) : launch_sddmm_mfma_ks<false, 2>(q, p.batch, stream);

@@ -91,7 +91,7 @@ inline size_t sddmm_mfma_words(int m, int tiles_n) { return (size_t)m * (4 * (si
 // column of nonzero u inside the tile.  The mask of a pair with more has bit c set when column 128 t + c is present.
 // The row's columns are first marked in a bit map in LDS (n bits); counts, cursors and packed words come from the
 // map, 64 tiles at a time, one tile per lane.
-__global__ __launch_bounds__(256) void sddmm_tile_ptr_kernel(int m, int tiles_n, const int* __restrict__ row_offsets,
+static __global__ __launch_bounds__(256) void sddmm_tile_ptr_kernel(int m, int tiles_n, const int* __restrict__ row_offsets,
                                                              const int* __restrict__ cols, int* __restrict__ tile_ptr,
                                                              int* __restrict__ brief, u32x4* __restrict__ mask) {
   __shared__ unsigned bits[4][kSdMaxTiles * 4];
@@ -159,6 +159,68 @@ __global__ __launch_bounds__(256) void sddmm_tile_ptr_kernel(int m, int tiles_n,
   if (lane == 0) tile_ptr[(size_t)tiles_n * m + r] = e;
 }
 
+// Where the three tables sit in a workspace of sddmm_mfma_words(m, tiles_n) words, and the launch that fills them.
+struct SdTables {
+  u32x4* mask;
+  int* tile_ptr;
+  int* brief;
+};
+inline SdTables sd_tables(void* workspace, int m, int tiles_n) {
+  SdTables t;
+  t.mask = static_cast<u32x4*>(workspace);
+  t.tile_ptr = reinterpret_cast<int*>(t.mask + (size_t)tiles_n * m);
+  t.brief = t.tile_ptr + (size_t)(tiles_n + 1) * m;
+  return t;
+}
+inline int sd_write_tables(const SdTables& t, int m, int tiles_n, const int* row_offsets, const int* cols, hipStream_t stream) {
+  note_kernel("sddmm_tile_ptr_kernel");
+  hipLaunchKernelGGL(sddmm_tile_ptr_kernel, dim3(ceil_div(m, 4)), dim3(256), 0, stream, m, tiles_n, row_offsets, cols, t.tile_ptr, t.brief, t.mask);
+  return check_hip(hipGetLastError(), "row-cursor launch");
+}
+
+// Which column tiles of the workgroup's 128 rows (row0 ..) are dense: nonzeros of the rows in tile t = sum over the
+// rows of tile_ptr[t + 1] - tile_ptr[t].  Leaves the dense tiles, ascending, at the front of list[0 .. tiles_n) and
+// the others, descending, at its back, and their number in *n_dense.  colsum: tiles_n + 1 words of LDS that the
+// caller may reuse afterwards.  All 256 threads call it (it holds two workgroup barriers, the last one at its end).
+__device__ __forceinline__ void sd_sort_tiles(const int* __restrict__ tile_ptr, int m, int tiles_n, int row0, int dense_min,
+                                              unsigned* colsum, unsigned short* list, int* n_dense) {
+  typedef unsigned short u16;
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int ra = min(row0 + lane, m - 1), rb = min(row0 + kWave + lane, m - 1);
+  for (int t0 = wave; t0 <= tiles_n; t0 += 32) {   // 8 tiles per step: 16 loads in flight
+    unsigned v[8];
+#pragma unroll
+    for (int u = 0; u < 8; ++u) {
+      const int t = min(t0 + 4 * u, tiles_n);
+      v[u] = (unsigned)tile_ptr[(size_t)t * m + ra] + (unsigned)tile_ptr[(size_t)t * m + rb];
+    }
+#pragma unroll
+    for (int u = 0; u < 8; ++u) {
+      const unsigned sum = wave_sum_u(v[u]);
+      if (lane == 0 && t0 + 4 * u <= tiles_n) colsum[t0 + 4 * u] = sum;
+    }
+  }
+  __syncthreads();
+  if (wave == 0) {
+    int nd = 0, ns = 0;
+    for (int base = 0; base < tiles_n; base += kWave) {
+      const int t = base + lane;
+      const bool in = t < tiles_n;
+      const int tc = min(t, tiles_n - 1);
+      const bool dense = in && (int)(colsum[tc + 1] - colsum[tc]) >= dense_min;
+      const unsigned long long dm = __ballot(dense), sm = __ballot(in && !dense);
+      const unsigned long long below = (1ull << lane) - 1;
+      if (dense) list[nd + __popcll(dm & below)] = (u16)t;
+      if (in && !dense) list[tiles_n - 1 - ns - __popcll(sm & below)] = (u16)t;
+      nd += __popcll(dm);
+      ns += __popcll(sm);
+    }
+    if (lane == 0) *n_dense = nd;
+  }
+  __syncthreads();
+}
+
 // acc + <a, b> over 8 elements of 16 bits, products and sums in fp32
 template <bool BF16>
 __device__ __forceinline__ float dot8(u32x4 a, u32x4 b, float acc) {
@@ -215,42 +277,7 @@ __global__ __launch_bounds__(kSdThreads, KS == 8 ? 1 : 2) void sddmm_mfma_kernel
   u16* __restrict__ out = static_cast<u16*>(p.out) + (size_t)z * p.nnz;
   const int tiles_n = p.tiles_n;
 
-  // ---- which tiles are dense: nonzeros of the 128 rows in tile t = sum over rows of tile_ptr[t + 1] - tile_ptr[t]
-  {
-    unsigned* colsum = reinterpret_cast<unsigned*>(S);
-    const int ra = min(row0 + lane, p.m - 1), rb = min(row0 + kWave + lane, p.m - 1);
-    for (int t0 = wave; t0 <= tiles_n; t0 += 32) {   // 8 tiles per step: 16 loads in flight
-      unsigned v[8];
-#pragma unroll
-      for (int u = 0; u < 8; ++u) {
-        const int t = min(t0 + 4 * u, tiles_n);
-        v[u] = (unsigned)p.tile_ptr[(size_t)t * p.m + ra] + (unsigned)p.tile_ptr[(size_t)t * p.m + rb];
-      }
-#pragma unroll
-      for (int u = 0; u < 8; ++u) {
-        const unsigned sum = wave_sum_u(v[u]);
-        if (lane == 0 && t0 + 4 * u <= tiles_n) colsum[t0 + 4 * u] = sum;
-      }
-    }
-    __syncthreads();
-    if (wave == 0) {
-      int nd = 0, ns = 0;
-      for (int base = 0; base < tiles_n; base += kWave) {
-        const int t = base + lane;
-        const bool in = t < tiles_n;
-        const int tc = min(t, tiles_n - 1);
-        const bool dense = in && (int)(colsum[tc + 1] - colsum[tc]) >= p.dense_min;
-        const unsigned long long dm = __ballot(dense), sm = __ballot(in && !dense);
-        const unsigned long long below = (1ull << lane) - 1;
-        if (dense) list[nd + __popcll(dm & below)] = (u16)t;
-        if (in && !dense) list[tiles_n - 1 - ns - __popcll(sm & below)] = (u16)t;
-        nd += __popcll(dm);
-        ns += __popcll(sm);
-      }
-      if (lane == 0) *n_dense = nd;
-    }
-    __syncthreads();
-  }
+  sd_sort_tiles(p.tile_ptr, p.m, tiles_n, row0, p.dense_min, reinterpret_cast<unsigned*>(S), list, n_dense);
   const int nd = __builtin_amdgcn_readfirstlane(*n_dense);
 
   for (int phase = 0; phase < 2; ++phase) {

@@ -712,6 +712,15 @@ int spmm_dispatch(int dtype, int itype, int flags, int m, int k, int n, int nonz
   // beyond the 256 MB last-level cache an output can only stream; the hint is worth 15-25 % of the write rate
   p.stream_out = (double)m * n * batch * (dtype == IEX_F32 ? 4 : 2) >= 128e6;
   hipStream_t s = static_cast<hipStream_t>(stream);
+  if (ch.variant == 10 && nonzeros == 0) ch.variant = 1;   // nothing to lay out: the row kernel writes the zeros
+  if (ch.variant == 10) {
+    IEX_REQUIRE(spmm_blocks_fits(dtype, itype, p), IEX_ERR_UNSUPPORTED,
+                "spmm: the dense-blocks kernel needs fp16 / bf16, int32 indices, n = 64, plain store without bias or ReLU, k <= 65536 and 16-byte aligned dense operands");
+    IEX_REQUIRE(ch.ws && aligned(ch.ws, 16) && ch.ws_bytes >= spmm_blocks_bytes(p), IEX_ERR_BAD_ARGUMENT,
+                "spmm: the dense-blocks kernel needs a 16-byte aligned workspace of %zu bytes (iex_spmm_ws)", spmm_blocks_bytes(p));
+    return launch_spmm_blocks(dtype, p, batch, ch.ws, (flags >> 8) & 0xff,
+                              ((flags & IEX_SPMM_TABLES_READY) ? 1 : 0) | ((flags & IEX_SPMM_LISTS_READY) ? 2 : 0), s);
+  }
   if (dtype == IEX_F32 && itype == IEX_I32) return launch_typed<float, int>(p, batch, ch, s);
   if (dtype == IEX_F16 && itype == IEX_I32) return launch_typed<__half, int>(p, batch, ch, s);
   if (dtype == IEX_F16 && itype == IEX_I16) return launch_typed<__half, short>(p, batch, ch, s);
@@ -731,8 +740,10 @@ size_t spmm_workspace_bytes(int dtype, int itype, int flags, int m, int k, int n
     return 0;
   }
   if (!(dtype == IEX_F16 || dtype == IEX_BF16) || !(itype == IEX_I32 || itype == IEX_I16)) return 0;
-  if (variant != 0 && variant != 7) return 0;
-  SpmmParams p{m, k, n, nonzeros, nullptr, nullptr, nullptr, nullptr, some_aligned, nullptr, some_aligned, 0, 0, 0};
+  if (variant != 0 && variant != 7 && variant != 10) return 0;
+  SpmmParams p{m, k, n, nonzeros, nullptr, nullptr, nullptr, nullptr, some_aligned, nullptr, some_aligned,
+               (flags & IEX_SPMM_PER_BATCH_VALUES) != 0, (flags & IEX_SPMM_ACCUMULATE) != 0, (flags & IEX_SPMM_RELU) != 0};
+  if (variant == 10) return spmm_blocks_fits(dtype, itype, p) ? spmm_blocks_bytes(p) : 0;
   if (!dense_path_fits(2, p, (flags & IEX_SPMM_PER_BATCH_VALUES) != 0)) return 0;
   if (variant == 0) {
     Choice ch;

@@ -1,0 +1,59 @@
+// Host side of the SpMM for attention-like sparse operands (spmm_blocks_device.cuh): what it serves, how much
+// workspace it needs, the launch.
+#include "spmm_blocks_device.cuh"
+#include "spmm_device.cuh"
+
+namespace iex {
+
+// fp16 / bf16, int32 indices, 64 output columns, plain store without bias or ReLU.
+bool spmm_blocks_fits(int dtype, int itype, const SpmmParams& p) {
+  return (dtype == IEX_F16 || dtype == IEX_BF16) && itype == IEX_I32 && p.n == kSbN && !p.accumulate && !p.relu && !p.bias &&
+         aligned(p.dense, 16) && aligned(p.out, 16) && ceil_div(p.k, kSdBN) <= kSdMaxTiles &&
+         (long long)(ceil_div(p.k, kSdBN) + 1) * p.m < (1ll << 28);
+}
+
+size_t spmm_blocks_bytes(const SpmmParams& p) { return sb_words(p.m, ceil_div(p.k, kSdBN), p.nnz) * sizeof(int); }
+
+template <bool BF16>
+static int launch_blocks(const SpmmBlocksParams& q, int batch, hipStream_t stream) {
+  constexpr int lds = spmm_blocks_lds_bytes();
+  auto kernel = spmm_blocks_kernel<BF16>;
+  static thread_local bool raised = false;   // per instantiation: more than 64 KB of dynamic LDS
+  if (!raised) {
+    if (int rc = check_hip(hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, lds),
+                           "hipFuncSetAttribute(LDS size)"))
+      return rc;
+    raised = true;
+  }
+  note_kernel("spmm_blocks_kernel<%s>", BF16 ? "true" : "false");
+  hipLaunchKernelGGL(kernel, dim3(ceil_div(q.m, kSdBM), batch), dim3(kSdThreads), lds, stream, q);
+  return check_hip(hipGetLastError(), "spmm (dense blocks) launch");
+}
+
+// dense_code (for tests and tuning): 0 = the built-in threshold, 1 = every tile on the matrix cores, 255 = none,
+// else 64 * code nonzeros per 128 x 128 block.  ready: bit 0 = the caller vouches that an earlier call on this
+// pattern (this kernel's or the SDDMM's for masks with structure: same tables) left the tables in the workspace,
+// bit 1 = that an earlier call of this kernel with the same dense_code left its lists there too.
+int launch_spmm_blocks(int dtype, const SpmmParams& p, int batch, void* ws, int dense_code, int ready, hipStream_t stream) {
+  const int tiles_k = ceil_div(p.k, kSdBN);
+  const SdTables t = sd_tables(ws, p.m, tiles_k);
+  const SbLists l = sb_lists(ws, p.m, tiles_k, p.nnz);
+  const int* cols = static_cast<const int*>(p.cols);
+  if (!(ready & 1)) {
+    if (int rc = sd_write_tables(t, p.m, tiles_k, p.row_offsets, cols, stream)) return rc;
+  }
+  if ((ready & 3) != 3) {
+    const int dense_min = dense_code == 0 ? kSdDenseMin : dense_code == 1 ? 0 : dense_code == 255 ? kSdBM * kSdBN + 1 : 64 * dense_code;
+    note_kernel("sb_dense_list_kernel");
+    hipLaunchKernelGGL(sb_dense_list_kernel, dim3(ceil_div(p.m, kSdBM)), dim3(kSdThreads), 0, stream, p.m, tiles_k, dense_min, t.tile_ptr, l.dense_list, l.zeros);
+    if (int rc = check_hip(hipGetLastError(), "spmm (dense tile list) launch")) return rc;
+    note_kernel("sb_thin_list_kernel");
+    hipLaunchKernelGGL(sb_thin_list_kernel, dim3(ceil_div(p.m, 4)), dim3(256), 0, stream, p.m, tiles_k, p.row_offsets, cols, l.dense_list, l.thin_cnt, l.thin_ent);
+    if (int rc = check_hip(hipGetLastError(), "spmm (list of the other nonzeros) launch")) return rc;
+  }
+  SpmmBlocksParams q{p.m, p.k, p.nnz, p.row_offsets, p.values, p.per_batch_values ? (size_t)p.nnz : 0, p.dense, p.out,
+                     t.mask, t.tile_ptr, t.brief, tiles_k, l.zeros, l.thin_ent, l.thin_cnt, l.dense_list};
+  return dtype == IEX_BF16 ? launch_blocks<true>(q, batch, stream) : launch_blocks<false>(q, batch, stream);
+}
+
+}  // namespace iex

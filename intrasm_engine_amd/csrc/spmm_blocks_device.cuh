@@ -1,0 +1,419 @@
+// CSR SpMM for attention-like sparse operands (gfx950, fp16 / bf16, 64 output columns): out = A * dense with A a
+// mask with structure (a dense band plus scattered entries) whose values differ per batch entry -- the second
+// product of sparse attention, probabilities times V.
+//
+// The row kernel (spmm_device.cuh) reads n * 2 bytes of the dense operand per nonzero through the L2 -> CU path;
+// for 16 heads of a 4096 x 4096 mask with 7 % of its entries that is 2.4 GB and that path bounds it.  This kernel
+// is the mirror image of the SDDMM for such masks (sddmm_mfma_device.cuh) and works from the same tables, written
+// by the same setup kernel into the caller's workspace (tile_ptr, brief, mask: per row and 128-column tile of A the
+// position of the row's first nonzero there, and which of the tile's columns the row holds), plus two lists that
+// two more small kernels derive from the tables (they depend on the pattern and on the threshold below, not on
+// values: a caller whose pattern stays keeps them): per block of 128 rows the column tiles that hold dense_min
+// nonzeros or more ("dense"), and per row its nonzeros outside those tiles, compacted.
+// A workgroup (4 wavefronts) owns 128 consecutive rows of one batch entry, a wavefront 32 of them:
+//   * dense tiles: the block of A is laid out as a dense 32 x 128 tile per wavefront in LDS -- zeros, then the
+//     values: up to 4 per (row, tile) by the row's own lane from the packed word, more by the whole wavefront from
+//     the row's 128-bit mask (lane i owns columns i and 64 + i; a population count of the bits below gives the
+//     position of each in the row's values, so the loads of a row are contiguous and no column index is read; all
+//     loads of a tile are issued before the first is used) -- and multiplied on the matrix cores with the 128 rows
+//     of the dense operand that the tile names: they go through registers into LDS once per workgroup,
+//     double-buffered, 16-byte chunks permuted so that the transposing operand reads (ds_read_tr16_b64) are
+//     conflict-free.  Operands swapped (out^T = dense^T * A^T) so that a lane ends up with 4 adjacent output
+//     columns of one row.
+//   * everything else: 8 lanes per row walk the row's list, two rows at a time, 8 nonzeros of each per step: 16
+//     bytes of the dense operand's row per lane and nonzero, fp32 FMAs, no reduction across lanes.
+// Both parts meet in LDS: the matrix-core sums of a wavefront's 32 rows are written there as fp32, each lane adds
+// its own sums of the second kind to the 8 of them it owns, rounds once and stores 16 bytes.  The order of the
+// additions is fixed: results are bit-stable from call to call.
+// The tile of A holds explicit zeros: a non-finite entry in a row of the dense operand that a dense tile covers
+// reaches the output rows of that tile's 128-row block whether or not they reference it (0 * inf = NaN).
+#pragma once
+#include "sddmm_mfma_device.cuh"
+
+namespace iex {
+
+constexpr int kSbN = 64;                       // output columns
+constexpr int kSbTileBytes = 32 * kSdLd * 2;   // a wavefront's 32 x 128 tile of A (rows padded to 272 bytes); later its 32 x 64 fp32 sums
+constexpr int kSbStage = kSdBN * kSbN * 2;     // 128 rows of the dense operand
+constexpr int kSbZeroWords = 32;               // 128 bytes of zeros: what the lanes of an absent nonzero read
+
+struct SbEntry {
+  int col, pos;   // column of a nonzero outside the dense tiles and its position in the CSR arrays
+};
+
+// What the kernel reads besides the operands: the SDDMM's tables and, behind them in the same workspace, the lists
+// that depend on which tiles count as dense.
+struct SbLists {
+  unsigned* zeros;                  // [kSbZeroWords]
+  SbEntry* thin_ent;                // [nnz]: row r's entries outside dense tiles, in row order, from thin_ent[row_offsets[r]]
+  int* thin_cnt;                    // [m]: how many
+  unsigned short* dense_list;       // [row blocks][tiles_k + 2]: number of dense tiles of the 128 rows, then the tiles, ascending
+};
+inline size_t sb_lists_offset_words(int m, int tiles_k) { return (sddmm_mfma_words(m, tiles_k) + 3) & ~size_t(3); }
+inline size_t sb_words(int m, int tiles_k, int nnz) {
+  return sb_lists_offset_words(m, tiles_k) + kSbZeroWords + 2 * (size_t)nnz + m + ((size_t)ceil_div(m, kSdBM) * (tiles_k + 2) + 1) / 2;
+}
+inline SbLists sb_lists(void* workspace, int m, int tiles_k, int nnz) {
+  SbLists l;
+  l.zeros = static_cast<unsigned*>(workspace) + sb_lists_offset_words(m, tiles_k);
+  l.thin_ent = reinterpret_cast<SbEntry*>(l.zeros + kSbZeroWords);
+  l.thin_cnt = reinterpret_cast<int*>(l.thin_ent + nnz);
+  l.dense_list = reinterpret_cast<unsigned short*>(l.thin_cnt + m);
+  return l;
+}
+
+struct SpmmBlocksParams {
+  int m, k, nnz;
+  const int* row_offsets;
+  const void* values;
+  size_t values_stride;   // elements between batch entries (0: shared)
+  const void* dense;      // (batch, k, 64)
+  void* out;              // (batch, m, 64)
+  const u32x4* mask;      // [tiles_k][m]
+  const int* tile_ptr;    // [(tiles_k + 1)][m]
+  const int* brief;       // [tiles_k][m]
+  int tiles_k;
+  const unsigned* zeros;
+  const SbEntry* thin_ent;
+  const int* thin_cnt;
+  const unsigned short* dense_list;
+};
+
+constexpr int spmm_blocks_lds_bytes() { return 4 * kSbTileBytes + 2 * kSbStage; }
+
+// The dense tiles of every block of 128 rows (one workgroup each): dense_list[block][0] = their number, then the tiles.
+static __global__ __launch_bounds__(kSdThreads) void sb_dense_list_kernel(int m, int tiles_k, int dense_min, const int* __restrict__ tile_ptr,
+                                                                          unsigned short* __restrict__ dense_list, unsigned* __restrict__ zeros) {
+  __shared__ unsigned colsum[kSdMaxTiles + 1];
+  __shared__ unsigned short list[kSdMaxTiles];
+  __shared__ int n_dense;
+  sd_sort_tiles(tile_ptr, m, tiles_k, blockIdx.x * kSdBM, dense_min, colsum, list, &n_dense);
+  unsigned short* mine = dense_list + (size_t)blockIdx.x * (tiles_k + 2);
+  const int nd = n_dense;
+  if (threadIdx.x == 0) mine[0] = (unsigned short)nd;
+  for (int i = threadIdx.x; i < nd; i += kSdThreads) mine[1 + i] = list[i];
+  if (blockIdx.x == 0 && threadIdx.x < kSbZeroWords) zeros[threadIdx.x] = 0u;
+}
+
+// The nonzeros of every row that lie outside the dense tiles of the row's block, compacted in row order (one wavefront
+// per row): column and position in the CSR arrays.
+static __global__ __launch_bounds__(256) void sb_thin_list_kernel(int m, int tiles_k, const int* __restrict__ row_offsets, const int* __restrict__ cols,
+                                                                  const unsigned short* __restrict__ dense_list, int* __restrict__ thin_cnt,
+                                                                  SbEntry* __restrict__ thin_ent) {
+  __shared__ unsigned is_dense[4][kSdMaxTiles / 32];
+  const int lane = lane_id();
+  const int wave = threadIdx.x >> 6;
+  const int r = blockIdx.x * 4 + wave;
+  if (r >= m) return;   // (no workgroup barrier below: every wavefront works alone)
+  const unsigned short* mine = dense_list + (size_t)(r / kSdBM) * (tiles_k + 2);
+  const int nd = uniform((int)mine[0]);
+  if (lane < kSdMaxTiles / 32) is_dense[wave][lane] = 0;
+  __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+  __builtin_amdgcn_wave_barrier();
+  for (int i = lane; i < nd; i += kWave) {
+    const int t = mine[1 + i];
+    atomicOr(&is_dense[wave][t >> 5], 1u << (t & 31));
+  }
+  __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+  __builtin_amdgcn_wave_barrier();
+  const int s = uniform(row_offsets[r]), e = uniform(row_offsets[r + 1]);
+  int count = 0;
+  for (int base = s; base < e; base += 4 * kWave) {   // four loads in flight
+    int c[4];
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      const int j = base + u * kWave + lane;
+      c[u] = j < e ? cols[j] : -1;
+    }
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      const int t = min(max(c[u], 0) >> 7, tiles_k - 1);
+      const bool thin = c[u] >= 0 && !((is_dense[wave][t >> 5] >> (t & 31)) & 1);
+      const unsigned long long b = __ballot(thin);
+      if (thin) {
+        SbEntry en;
+        en.col = c[u];
+        en.pos = base + u * kWave + lane;
+        thin_ent[s + count + __popcll(b & ((1ull << lane) - 1))] = en;
+      }
+      count += __popcll(b);
+    }
+  }
+  if (lane == 0) thin_cnt[r] = count;
+}
+
+template <bool BF16>
+__global__ __launch_bounds__(kSdThreads, 2) void spmm_blocks_kernel(SpmmBlocksParams p) {
+  typedef unsigned short u16;
+  typedef __attribute__((address_space(3))) s16x4 lds_s16x4;
+  constexpr int NT = kSbN / 32;
+  extern __shared__ __align__(16) unsigned char smem[];
+  unsigned char* sV = smem + 4 * kSbTileBytes;                               // [2][128][128 bytes]
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  // Workgroups go to the 8 XCDs round-robin by their linear id; renumbered so that an XCD gets all row blocks of a
+  // batch entry (and then of the next): the dense operand of that entry stays in that XCD's L2.
+  const int row_blocks = gridDim.x, total = row_blocks * gridDim.y;
+  int id = blockIdx.x + row_blocks * blockIdx.y;
+  // the two workgroups that share a CU take the two parts in opposite order (matrix cores and LDS beside gathers)
+  const int launch_slot = id / 8;
+  const bool thin_first = ((launch_slot ^ (launch_slot >> 5)) & 1) != 0;
+  if (total % 8 == 0) id = (id % 8) * (total / 8) + id / 8;
+  const int z = id / row_blocks;
+  const int row_block = id % row_blocks;
+  const int row0 = row_block * kSdBM;
+  const u16* __restrict__ vals = static_cast<const u16*>(p.values) + (size_t)z * p.values_stride;
+  const u16* __restrict__ V = static_cast<const u16*>(p.dense) + (size_t)z * p.k * kSbN;
+  u16* __restrict__ out = static_cast<u16*>(p.out) + (size_t)z * p.m * kSbN;
+  const int m = p.m;
+  const int last = p.nnz - 1;   // (the host does not launch this kernel without nonzeros)
+  const u16* __restrict__ list = p.dense_list + (size_t)row_block * (p.tiles_k + 2);
+  const int nd = __builtin_amdgcn_readfirstlane((int)list[0]);
+  ++list;
+
+  unsigned char* Pw = smem + wave * kSbTileBytes;   // this wavefront's tile of A
+  u16* P16 = reinterpret_cast<u16*>(Pw);
+  const int wrow0 = row0 + wave * 32;               // first of this wavefront's rows
+
+  f32x16 acc[NT];
+#pragma unroll
+  for (int t = 0; t < NT; ++t)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) acc[t][r] = 0.f;
+  float tacc[4][8];   // sums over the nonzeros outside dense tiles: row it * 8 + lane / 8, columns (lane % 8) * 8 .. + 7
+#pragma unroll
+  for (int it = 0; it < 4; ++it)
+#pragma unroll
+    for (int c = 0; c < 8; ++c) tacc[it][c] = 0.f;
+
+  for (int phase = 0; phase < 2; ++phase) {
+    if ((phase == 0) != thin_first) {
+      // ---- dense tiles
+      if (nd > 0) {
+        // 128 rows x 128 bytes of the dense operand: chunk L = q * 256 + tid sits at LDS byte 16 L and holds global
+        // chunk (L % 8) ^ 4 * ((row / 2) % 2) of row L / 8
+        auto load_rows = [&](int i, u32x4 (&rv)[4]) {
+          const int ct = __builtin_amdgcn_readfirstlane((int)list[min(i, nd - 1)]);
+#pragma unroll
+          for (int q = 0; q < 4; ++q) {
+            const int L = q * kSdThreads + tid;
+            const int row = L >> 3, pos = L & 7;
+            const int g = pos ^ (((row >> 1) & 1) << 2);
+            const int krow = ct * kSdBN + row;
+            const u32x4 got = *reinterpret_cast<const u32x4*>(V + (size_t)min(krow, p.k - 1) * kSbN + g * 8);
+            const u32x4 zero = {0u, 0u, 0u, 0u};
+            rv[q] = krow < p.k ? got : zero;
+          }
+        };
+        auto store_rows = [&](int i, const u32x4 (&rv)[4]) {
+          unsigned char* base = sV + (i & 1) * kSbStage;
+#pragma unroll
+          for (int q = 0; q < 4; ++q) *reinterpret_cast<u32x4*>(base + (q * kSdThreads + tid) * 16) = rv[q];
+        };
+        // what lanes 0..31 know of their row in a tile: cursor, packed word, mask
+        const int meta_row = min(wrow0 + (lane & 31), m - 1);
+        const bool meta_valid = lane < 32 && wrow0 + lane < m;
+        auto load_meta = [&](int i, int& tp, int& bf, u32x4& mk) {
+          const int ct = __builtin_amdgcn_readfirstlane((int)list[min(i, nd - 1)]);
+          tp = p.tile_ptr[(size_t)ct * m + meta_row];
+          bf = p.brief[(size_t)ct * m + meta_row];
+          mk = p.mask[(size_t)ct * m + meta_row];
+        };
+
+        // transposing operand reads of the dense operand's tile: lane group lane / 16 covers column half (group % 2)
+        // and k half (group / 2) of a 16-wide k step; lane r of a group points at k row r / 4, columns 4 (r % 4) .. + 3
+        const int fkh = lane >> 5;
+        const int tr_k = fkh * 8 + ((lane & 15) >> 2);
+        const int tr_sw = ((tr_k >> 1) & 1) << 2;
+        int v_off[NT];
+#pragma unroll
+        for (int t = 0; t < NT; ++t) {
+          const int chunk = (t * 4 + ((lane >> 4) & 1) * 2 + ((lane & 3) >> 1)) ^ tr_sw;
+          v_off[t] = tr_k * (kSbN * 2) + chunk * 16 + (lane & 1) * 8;
+        }
+        const int p_off = (lane & 31) * (kSdLd * 2) + fkh * 16;
+
+        u32x4 rv[4];
+        int tp, bf;
+        u32x4 mk;
+        load_rows(0, rv);
+        load_meta(0, tp, bf, mk);
+        store_rows(0, rv);
+        __syncthreads();
+
+        for (int i = 0; i < nd; ++i) {
+          int tp_n, bf_n;
+          u32x4 mk_n;
+          const bool more = i + 1 < nd;
+          if (more) load_rows(i + 1, rv);
+          load_meta(i + 1, tp_n, bf_n, mk_n);
+
+          // ---- this wavefront's 32 x 128 tile of A: zeros ...
+          {
+            const u32x4 zero = {0u, 0u, 0u, 0u};
+#pragma unroll
+            for (int q = 0; q < 8; ++q) {
+              const int c = q * kWave + lane;
+              *reinterpret_cast<u32x4*>(Pw + (c >> 4) * (kSdLd * 2) + (c & 15) * 16) = zero;
+            }
+          }
+          const int count = meta_valid ? (bf >> 28) & 7 : 0;
+          // ... up to 4 values of a row by the row's lane (loads from clamped positions: no branch around a load) ...
+          u16 sv[kSdShort];
+#pragma unroll
+          for (int u = 0; u < kSdShort; ++u) sv[u] = vals[min(max(tp, 0) + u, last)];
+          // ... longer runs by the wavefront: lane i owns columns i and 64 + i of the row; all loads first
+          const unsigned longs = (unsigned)__ballot(count == 7);
+          u16 lo[32], hi[32];   // (as loaded: which of them exist is looked at when they are written)
+#pragma unroll
+          for (int r = 0; r < 32; ++r) {
+            lo[r] = 0;
+            hi[r] = 0;
+            if ((longs >> r) & 1) {   // (uniform)
+              const unsigned mx = (unsigned)__builtin_amdgcn_readlane((int)mk.x, r), my = (unsigned)__builtin_amdgcn_readlane((int)mk.y, r);
+              const unsigned mz = (unsigned)__builtin_amdgcn_readlane((int)mk.z, r), mw = (unsigned)__builtin_amdgcn_readlane((int)mk.w, r);
+              const int start = max(__builtin_amdgcn_readlane(tp, r), 0);
+              const int rank_lo = __builtin_amdgcn_mbcnt_hi(my, __builtin_amdgcn_mbcnt_lo(mx, 0));
+              const int rank_hi = __builtin_amdgcn_mbcnt_hi(mw, __builtin_amdgcn_mbcnt_lo(mz, 0)) + __popc(mx) + __popc(my);
+              lo[r] = vals[min(start + rank_lo, last)];
+              hi[r] = vals[min(start + rank_hi, last)];
+            }
+          }
+          if (count >= 1 && count <= kSdShort) {
+#pragma unroll
+            for (int u = 0; u < kSdShort; ++u)
+              if (u < count) P16[lane * kSdLd + ((bf >> (7 * u)) & 127)] = sv[u];
+          }
+#pragma unroll
+          for (int r = 0; r < 32; ++r) {
+            if ((longs >> r) & 1) {
+              const unsigned mx = (unsigned)__builtin_amdgcn_readlane((int)mk.x, r), my = (unsigned)__builtin_amdgcn_readlane((int)mk.y, r);
+              const unsigned mz = (unsigned)__builtin_amdgcn_readlane((int)mk.z, r), mw = (unsigned)__builtin_amdgcn_readlane((int)mk.w, r);
+              const unsigned word_lo = lane < 32 ? mx : my, word_hi = lane < 32 ? mz : mw;
+              P16[r * kSdLd + lane] = ((word_lo >> (lane & 31)) & 1) ? lo[r] : (u16)0;
+              P16[r * kSdLd + kWave + lane] = ((word_hi >> (lane & 31)) & 1) ? hi[r] : (u16)0;
+            }
+          }
+          __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+          __builtin_amdgcn_wave_barrier();
+
+          // ---- out^T (64 x 32 per wavefront) += dense^T (64 x 128) * A^T (128 x 32)
+          const unsigned char* stage = sV + (i & 1) * kSbStage;
+#pragma unroll
+          for (int ks = 0; ks < kSdBN / 16; ++ks) {
+            const u32x4 pf = *reinterpret_cast<const u32x4*>(Pw + p_off + ks * 32);
+#pragma unroll
+            for (int t = 0; t < NT; ++t) {
+              const unsigned char* q0 = stage + ks * 16 * (kSbN * 2) + v_off[t];
+              const s16x4 l4 = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)(q0));
+              const s16x4 h4 = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)(q0 + 4 * (kSbN * 2)));
+              const u32x2 l2 = __builtin_bit_cast(u32x2, l4), h2 = __builtin_bit_cast(u32x2, h4);
+              acc[t] = mfma_32x32x16<BF16>(u32x4{l2.x, l2.y, h2.x, h2.y}, pf, acc[t]);
+            }
+          }
+          __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+          __builtin_amdgcn_wave_barrier();
+
+          if (more) store_rows(i + 1, rv);   // into the stage that everybody left before the last barrier
+          tp = tp_n, bf = bf_n, mk = mk_n;
+          __syncthreads();
+        }
+      }
+    } else {
+      // ---- nonzeros outside dense tiles: lane group g = lane / 8 takes rows g, 8 + g, 16 + g, 24 + g of the
+      // wavefront's 32, two at a time, 8 nonzeros of each per step: lane sl of the group reads entry sl of the step
+      // (column, position) and its value, the group's lanes exchange them, and every lane reads its 16 bytes of the
+      // 8 rows of the dense operand.  The lanes of an absent nonzero read zeros instead (never a row of the dense
+      // operand that the row does not reference).  The entries of the next step are fetched before this step's sums.
+      const int g = lane >> 3, sl = lane & 7, gl = lane & ~7;
+      const u16* __restrict__ zeros = reinterpret_cast<const u16*>(p.zeros);
+      int base[4], cnt[4];
+#pragma unroll
+      for (int it = 0; it < 4; ++it) {
+        const int r = wrow0 + it * 8 + g;
+        const int rc = min(r, m - 1);
+        base[it] = p.row_offsets[rc];
+        cnt[it] = r < m ? p.thin_cnt[rc] : 0;
+      }
+#pragma unroll
+      for (int h = 0; h < 4; h += 2) {
+        const int nmax = max(cnt[h], cnt[h + 1]);
+        SbEntry en[2];
+#pragma unroll
+        for (int w = 0; w < 2; ++w) en[w] = p.thin_ent[min(base[h + w] + min(sl, max(cnt[h + w] - 1, 0)), last)];
+        for (int st = 0; __ballot(st * 8 < nmax); ++st) {
+          u16 pv[2];
+          u32x4 v[2][8];
+          int colw[2];
+#pragma unroll
+          for (int w = 0; w < 2; ++w) {
+            pv[w] = vals[min((unsigned)en[w].pos, (unsigned)last)];
+            colw[w] = en[w].col;
+          }
+#pragma unroll
+          for (int w = 0; w < 2; ++w)
+#pragma unroll
+            for (int u = 0; u < 8; ++u) {
+              const int cu = __shfl(colw[w], gl + u, kWave);
+              const u16* src = st * 8 + u < cnt[h + w] ? V + (size_t)cu * kSbN + sl * 8 : zeros + sl * 8;
+              v[w][u] = *reinterpret_cast<const u32x4*>(src);
+            }
+#pragma unroll
+          for (int w = 0; w < 2; ++w) {
+            if (st * 8 + sl >= cnt[h + w]) pv[w] = 0;
+            en[w] = p.thin_ent[min(base[h + w] + min((st + 1) * 8 + sl, max(cnt[h + w] - 1, 0)), last)];
+          }
+#pragma unroll
+          for (int w = 0; w < 2; ++w)
+#pragma unroll
+            for (int u = 0; u < 8; ++u) {
+              const float pf = f16_to_32((u16)__shfl((int)pv[w], gl + u, kWave), BF16);
+              const unsigned x[4] = {v[w][u].x, v[w][u].y, v[w][u].z, v[w][u].w};
+#pragma unroll
+              for (int c = 0; c < 4; ++c) {
+                tacc[h + w][2 * c] = fmaf(pf, f16_to_32((u16)(x[c] & 0xffffu), BF16), tacc[h + w][2 * c]);
+                tacc[h + w][2 * c + 1] = fmaf(pf, f16_to_32((u16)(x[c] >> 16), BF16), tacc[h + w][2 * c + 1]);
+              }
+            }
+        }
+      }
+    }
+  }
+
+  // ---- both parts meet: the matrix-core sums as fp32 in this wavefront's tile (rows of 68 floats), then every lane
+  // adds its own sums to the 8 entries it owns, rounds and stores 16 bytes
+  __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+  __builtin_amdgcn_wave_barrier();
+  float* T = reinterpret_cast<float*>(Pw);
+  constexpr int TLD = kSdLd / 2;   // 68 floats = the 272 bytes of a row of the tile
+#pragma unroll
+  for (int t = 0; t < NT; ++t)
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      const f32x4 x = {acc[t][q * 4], acc[t][q * 4 + 1], acc[t][q * 4 + 2], acc[t][q * 4 + 3]};
+      *reinterpret_cast<f32x4*>(T + (lane & 31) * TLD + t * 32 + q * 8 + (lane >> 5) * 4) = x;
+    }
+  __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+  __builtin_amdgcn_wave_barrier();
+  {
+    const int g = lane >> 3, sl = lane & 7;
+#pragma unroll
+    for (int it = 0; it < 4; ++it) {
+      const int row = it * 8 + g;
+      const f32x4 x0 = *reinterpret_cast<const f32x4*>(T + row * TLD + sl * 8);
+      const f32x4 x1 = *reinterpret_cast<const f32x4*>(T + row * TLD + sl * 8 + 4);
+      const float y[8] = {x0[0] + tacc[it][0], x0[1] + tacc[it][1], x0[2] + tacc[it][2], x0[3] + tacc[it][3],
+                          x1[0] + tacc[it][4], x1[1] + tacc[it][5], x1[2] + tacc[it][6], x1[3] + tacc[it][7]};
+      u32x4 w;
+      w.x = (unsigned)f32_to_16(y[0], BF16) | ((unsigned)f32_to_16(y[1], BF16) << 16);
+      w.y = (unsigned)f32_to_16(y[2], BF16) | ((unsigned)f32_to_16(y[3], BF16) << 16);
+      w.z = (unsigned)f32_to_16(y[4], BF16) | ((unsigned)f32_to_16(y[5], BF16) << 16);
+      w.w = (unsigned)f32_to_16(y[6], BF16) | ((unsigned)f32_to_16(y[7], BF16) << 16);
+      if (wrow0 + row < m) *reinterpret_cast<u32x4*>(out + (size_t)(wrow0 + row) * kSbN + sl * 8) = w;
+    }
+  }
+}
+
+}  // namespace iex

@@ -36,6 +36,11 @@ struct SpmmParams {
   int stream_out = 0;  // the output is far larger than the caches: store it with the streaming hint
 };
 
+// The kernel for 16-bit sparse operands with structure and 64 output columns (spmm_blocks.hip)
+bool spmm_blocks_fits(int dtype, int itype, const SpmmParams& p);
+size_t spmm_blocks_bytes(const SpmmParams& p);
+int launch_spmm_blocks(int dtype, const SpmmParams& p, int batch, void* ws, int dense_code, int ready, hipStream_t stream);
+
 constexpr int kSpmmUnroll = 8;
 
 template <int VEC, int WPR, int NT = 1>

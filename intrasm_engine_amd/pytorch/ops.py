@@ -97,7 +97,7 @@ def _check_index_dtypes(row_indices, row_offsets, column_indices, allow_i16=Fals
 
 def _spmm(b, row_indices, values, row_offsets, column_indices, m, *, per_batch_values,
           accumulate, dtypes, allow_i16, out=None, bias=None, relu=False, force_wpr=0, force_variant=0, force_rpw=0,
-          force_nt=0, force_lpg=0, no_workspace=False):
+          force_nt=0, force_lpg=0, no_workspace=False, plan=None):
     tuned = getattr(_TUNING, "spmm", None)
     if tuned and not (force_wpr or force_variant or force_rpw or force_nt or force_lpg):
         force_wpr, force_variant, force_rpw, force_nt, force_lpg = (tuned.get(key, 0) for key in _SPMM_KEYS)
@@ -147,7 +147,19 @@ def _spmm(b, row_indices, values, row_offsets, column_indices, m, *, per_batch_v
         # stream, released (stream-ordered) when this call returns
         ws_bytes = 0 if no_workspace else lib.iex_spmm_workspace_bytes(
             _DT[b.dtype], _IT[column_indices.dtype], flags, m, k, n, nonzeros, batch)
-        ws = torch.empty(ws_bytes, dtype=torch.uint8, device=b.device) if ws_bytes else None
+        if plan is not None and ws_bytes and ((flags >> 16) & 0xf) == 10:
+            # the tables of the dense-blocks kernel depend on the pattern only and are those of the SDDMM for masks
+            # with structure: a plan shared with that operator's calls on the pattern serves both
+            key = (row_offsets.data_ptr(), column_indices.data_ptr(), row_offsets._version, column_indices._version,
+                   m, k, nonzeros)
+            if plan._ready(key, ws_bytes, b.device):
+                flags |= _lib.SPMM_TABLES_READY
+                if plan.lists_key == (key, int(force_wpr)):
+                    flags |= _lib.SPMM_LISTS_READY
+            plan.lists_key = (key, int(force_wpr))
+            ws = plan.workspace
+        else:
+            ws = torch.empty(ws_bytes, dtype=torch.uint8, device=b.device) if ws_bytes else None
         rc = lib.iex_spmm_ws(
             _DT[b.dtype], _IT[column_indices.dtype], flags, m, k, n, nonzeros,
             row_indices.data_ptr(), values.data_ptr(), row_offsets.data_ptr(),
@@ -170,6 +182,7 @@ class SddmmPlan:
     def __init__(self):
         self.workspace = None
         self.key = None
+        self.lists_key = None   # the SpMM for the same patterns keeps lists of its own behind the tables
         self.variant = 0        # 0: the library's rule (by density); 1 / 3 after analyze()
         self.dense_share = None
 
@@ -194,6 +207,7 @@ class SddmmPlan:
         if self.workspace is None or self.workspace.numel() < nbytes or self.workspace.device != device:
             self.workspace = torch.empty(nbytes, dtype=torch.uint8, device=device)
             self.key = None
+            self.lists_key = None
         ready = self.key == key
         self.key = key
         return ready

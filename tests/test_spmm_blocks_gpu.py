@@ -1,0 +1,160 @@
+"""The SpMM kernel for attention-like sparse operands (family 10: the dense 128 x 128 blocks of A laid out in LDS and
+multiplied on the matrix cores, the nonzeros elsewhere gathered row by row): parity with the CPU oracle on ragged
+shapes and on config 3's product with V, with every block treated as dense, every block as thin, and with the
+built-in threshold; values per batch entry and shared; tables kept between calls and shared with the SDDMM."""
+import numpy as np
+import pytest
+import torch
+
+from intrasm_engine_amd import workloads as W
+from _util import FP16_SUBNORMAL_HALF_STEP, RTOL, assert_close, rounded, to_dev
+
+pytestmark = pytest.mark.gpu
+ops = torch.ops.iex_ops
+
+
+def _run(dev, csr, values, dense, dtype, **force):
+    from intrasm_engine_amd.pytorch import ops as pyops
+    ri, _, ro, ci = to_dev(csr, dev)
+    vt, dt = torch.from_numpy(values).to(dev).to(dtype), torch.from_numpy(dense).to(dev).to(dtype)
+    return pyops._spmm(dt, ri, vt, ro, ci, csr.m, per_batch_values=values.ndim == 2, accumulate=False, dtypes=(dtype,),
+                       allow_i16=False, **force)
+
+
+def _want(oracle, csr, values, dense, dtype):
+    v16, d16 = rounded(values, dtype), rounded(dense, dtype)
+    want = oracle.spmm(d16, csr.row_indices, v16, csr.row_offsets, csr.column_indices, csr.m)
+    scale = oracle.spmm_abs_scale(d16, csr.row_indices, v16, csr.row_offsets, csr.column_indices, csr.m)
+    return want, scale
+
+
+def _pattern(rng, m, k, lens):
+    ro, ci = W.csr_from_row_lengths(rng, m, k, lens)
+    return W.CSR(m, k, np.ones(ci.shape[0], np.float32), W.swizzle_from_offsets(ro), ro, ci)
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("m,k", [(131, 97), (300, 517), (128, 128), (64, 1000)])
+@pytest.mark.parametrize("blocks", [0, 1, 255, 2])      # threshold: built-in, all dense, all thin, 128 nonzeros
+def test_ragged_shapes_forced(oracle, dev, dtype, m, k, blocks):
+    """m and k that are no multiples of the 128 x 128 tile, empty rows, a completely dense row, rows of 1 to 4
+    nonzeros per tile (the row's own lane) and of 5 and more (the wavefront), two batch entries with values of
+    their own."""
+    rng = np.random.default_rng(k + m)
+    lens = rng.integers(0, min(k, 40), m)
+    lens[[0, 9, m - 1]] = 0
+    lens[5] = k
+    lens[6] = min(k, 70)
+    csr = _pattern(rng, m, k, lens)
+    values = rng.standard_normal((2, csr.nnz)).astype(np.float32)
+    dense = rng.standard_normal((2, k, 64)).astype(np.float32)
+    out = _run(dev, csr, values, dense, dtype, force_variant=10, force_wpr=blocks)
+    want, scale = _want(oracle, csr, values, dense, dtype)
+    assert_close(out.float().cpu().numpy(), want, scale, RTOL[dtype], f"dense-blocks SpMM {m}x{k} {dtype} blocks={blocks}",
+                 atol=FP16_SUBNORMAL_HALF_STEP if dtype == torch.float16 else 0.0)
+    assert torch.equal(out, _run(dev, csr, values, dense, dtype, force_variant=10, force_wpr=blocks))   # same call, same bits
+
+
+def test_integer_operands_agree_with_the_row_kernel_exactly(dev):
+    rng = np.random.default_rng(8)
+    m, k = 260, 390
+    csr = _pattern(rng, m, k, rng.integers(0, 200, m))
+    values = rng.integers(-3, 4, (3, csr.nnz)).astype(np.float32)
+    dense = rng.integers(-3, 4, (3, k, 64)).astype(np.float32)
+    want = _run(dev, csr, values, dense, torch.float16, force_variant=1)
+    for blocks in (0, 1, 255, 3):
+        assert torch.equal(_run(dev, csr, values, dense, torch.float16, force_variant=10, force_wpr=blocks), want), blocks
+    shared = values[0]
+    want = _run(dev, csr, shared, dense, torch.float16, force_variant=1)
+    assert torch.equal(_run(dev, csr, shared, dense, torch.float16, force_variant=10), want)
+
+
+def test_band_plus_scattered_mask_mixes_both_kinds_of_block(oracle, dev):
+    rng = np.random.default_rng(77)
+    m, k = 640, 1100
+    idx = np.arange(m)
+    mask = np.abs(idx[:, None] * k // m - np.arange(k)[None, :]) < 48
+    mask[np.repeat(idx, 3), rng.integers(0, k, (m, 3)).ravel()] = True
+    ro, ci, _ = W.csr_from_mask(mask)
+    csr = W.CSR(m, k, np.ones(ci.shape[0], np.float32), W.swizzle_from_offsets(ro), ro, ci)
+    values = rng.standard_normal((3, csr.nnz)).astype(np.float32)
+    dense = rng.standard_normal((3, k, 64)).astype(np.float32)
+    for dtype in (torch.float16, torch.bfloat16):
+        out = _run(dev, csr, values, dense, dtype, force_variant=10)
+        want, scale = _want(oracle, csr, values, dense, dtype)
+        assert_close(out.float().cpu().numpy(), want, scale, RTOL[dtype], f"band + scattered {dtype}",
+                     atol=FP16_SUBNORMAL_HALF_STEP if dtype == torch.float16 else 0.0)
+
+
+def test_config3_probabilities_times_v(oracle, dev):
+    """Config 3's second product at full size: 4 heads against the oracle, 16 heads against the row kernel head by
+    head (same fp32 sums up to their order: compared at the 16-bit tolerance)."""
+    pat, _, _, v = W.config3()
+    rng = np.random.default_rng(3)
+    probs = (rng.random((16, pat.nnz)) / 280.0).astype(np.float32)
+    out = _run(dev, pat, probs[:4], v[:4], torch.float16, force_variant=10)
+    want, scale = _want(oracle, pat, probs[:4], v[:4], torch.float16)
+    assert_close(out.float().cpu().numpy(), want, scale, RTOL[torch.float16], "config 3, 4 heads", atol=FP16_SUBNORMAL_HALF_STEP)
+    full = _run(dev, pat, probs, v, torch.float16, force_variant=10)
+    assert torch.equal(full[:4], out)
+    rows = _run(dev, pat, probs, v, torch.float16, force_variant=1)
+    assert torch.allclose(full.float(), rows.float(), rtol=1e-2, atol=2e-3)
+
+
+def test_tables_kept_between_calls_and_shared_with_the_sddmm(dev):
+    """One plan serves the SDDMM for masks with structure and this kernel on the same pattern: whichever runs first
+    writes the tables, the other finds them; another pattern makes them be written again."""
+    from intrasm_engine_amd import _lib
+    from intrasm_engine_amd.pytorch import ops as pyops
+    rng = np.random.default_rng(5)
+    m = 512
+    idx = np.arange(m)
+    mask = np.abs(idx[:, None] - idx[None, :]) < 40
+    mask[np.repeat(idx, 2), rng.integers(0, m, (m, 2)).ravel()] = True
+    ro, ci, _ = W.csr_from_mask(mask)
+    csr = W.CSR(m, m, np.ones(ci.shape[0], np.float32), W.swizzle_from_offsets(ro), ro, ci)
+    ri, _, rot, cit = to_dev(csr, dev)
+    q = torch.randn(2, m, 64, device=dev, dtype=torch.float16)
+    kk = torch.randn(2, m, 64, device=dev, dtype=torch.float16)
+    v = torch.randn(2, m, 64, device=dev, dtype=torch.float16)
+    plan = pyops.SddmmPlan()
+    plan.variant = 3
+    scores = pyops.sddmm_half_planned(q, kk, ri, rot, cit, plan)
+    assert plan.key is not None
+    kw = dict(per_batch_values=True, accumulate=False, dtypes=(torch.float16,), allow_i16=False, force_variant=10)
+    fresh = pyops._spmm(v, ri, scores, rot, cit, m, **kw)
+    assert _lib.last_kernels().split(" + ") == ["sddmm_tile_ptr_kernel", "sb_dense_list_kernel", "sb_thin_list_kernel", "spmm_blocks_kernel<false>"]
+    first = pyops._spmm(v, ri, scores, rot, cit, m, plan=plan, **kw)      # needs more room than the SDDMM: everything is written again
+    kept = pyops._spmm(v, ri, scores, rot, cit, m, plan=plan, **kw)
+    assert _lib.last_kernels() == "spmm_blocks_kernel<false>"
+    assert torch.equal(kept, fresh) and torch.equal(first, fresh)
+    again_scores = pyops.sddmm_half_planned(q, kk, ri, rot, cit, plan)    # the SDDMM finds its tables in the larger workspace
+    assert "sddmm_tile_ptr_kernel" not in _lib.last_kernels() and torch.equal(again_scores, scores)
+    other_threshold = pyops._spmm(v, ri, scores, rot, cit, m, plan=plan, force_wpr=1, **kw)    # tables kept, lists not
+    assert _lib.last_kernels().split(" + ") == ["sb_dense_list_kernel", "sb_thin_list_kernel", "spmm_blocks_kernel<false>"]
+    assert torch.allclose(other_threshold.float(), fresh.float(), rtol=1e-2, atol=1e-2)
+    mask2 = np.abs(idx[:, None] - idx[None, :]) < 90
+    ro2, ci2, _ = W.csr_from_mask(mask2)
+    csr2 = W.CSR(m, m, np.ones(ci2.shape[0], np.float32), W.swizzle_from_offsets(ro2), ro2, ci2)
+    ri2, _, rot2, cit2 = to_dev(csr2, dev)
+    vals2 = torch.randn(2, csr2.nnz, device=dev, dtype=torch.float16)
+    again = pyops._spmm(v, ri2, vals2, rot2, cit2, m, plan=plan, **kw)
+    assert _lib.last_kernels().split(" + ")[0] == "sddmm_tile_ptr_kernel" and "spmm_blocks_kernel" in _lib.last_kernels()
+    assert torch.equal(again, pyops._spmm(v, ri2, vals2, rot2, cit2, m, **kw))
+
+
+def test_refusals_and_workspace_size(dev):
+    from intrasm_engine_amd import _lib
+    lib = _lib.load()
+    flags = (10 << 16) | _lib.SPMM_PER_BATCH_VALUES
+    assert lib.iex_spmm_workspace_bytes(_lib.F16, _lib.I32, flags, 4096, 4096, 64, 1000, 16) == ((6 * 32 + 1) * 4096 + 32 + 2 * 1000 + 4096 + 32 * (32 + 2) // 2) * 4
+    assert lib.iex_spmm_workspace_bytes(_lib.F16, _lib.I32, flags, 4096, 4096, 128, 1000, 16) == 0      # n != 64
+    assert lib.iex_spmm_workspace_bytes(_lib.F32, _lib.I32, flags, 4096, 4096, 64, 1000, 16) == 0
+    assert lib.iex_spmm_workspace_bytes(_lib.F16, _lib.I16, flags, 4096, 4096, 64, 1000, 16) == 0
+    rng = np.random.default_rng(1)
+    csr = _pattern(rng, 64, 64, rng.integers(0, 20, 64))
+    values = rng.standard_normal((1, csr.nnz)).astype(np.float32)
+    with pytest.raises(RuntimeError, match="dense-blocks kernel needs fp16"):
+        _run(dev, csr, values, rng.standard_normal((1, 64, 32)).astype(np.float32), torch.float16, force_variant=10)
+    with pytest.raises(RuntimeError, match="workspace"):
+        _run(dev, csr, values, rng.standard_normal((1, 64, 64)).astype(np.float32), torch.float16, force_variant=10, no_workspace=True)

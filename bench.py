@@ -559,6 +559,13 @@ def run_extras(torch, ops, dev, W, IL, mats, dens, csr_dev, time_cell, time_cold
                                    "kernel": kernel_of(lambda: ops.spmm_sputnik_batched_values(vt, ri3, scores, ro3, ci3, pat.m)),
                                    "hbm_frac": round(by / us / 1e3 / HBM_PEAK_GBPS, 4),
                                    "GFLOPs": round(W.spmm_flops(pat.nnz, 64, 16) / us / 1e3, 1)}
+    # the same plan as the SDDMM's: the tables are shared, the SpMM keeps two lists of its own behind them
+    f_planned = lambda: pyops_k.spmm_batched_values_planned(vt, ri3, scores, ro3, ci3, pat.m, plan_)
+    f_planned()
+    out["spmm_c3_fp16_16heads"]["tables_kept_us"] = round(time_cell(f_planned, repeats=10), 2)
+    out["spmm_c3_fp16_16heads"]["tables_kept_kernel"] = kernel_of(f_planned)
+    with pyops_k.kernel_params(spmm={"force_variant": 1}):
+        out["spmm_c3_fp16_16heads"]["row_kernel_us"] = round(time_cell(lambda: ops.spmm_sputnik_batched_values(vt, ri3, scores, ro3, ci3, pat.m), repeats=10), 2)
     from intrasm_engine_amd.pytorch.sparse_attention import sparse_attention
     us_block = time_cell(lambda: sparse_attention(qt, kt, vt, ri3, ro3, ci3), repeats=10)
     us_block_planned = time_cell(lambda: sparse_attention(qt, kt, vt, ri3, ro3, ci3, plan=plan_), repeats=10)

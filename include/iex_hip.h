@@ -140,6 +140,10 @@ int iex_spmm_ws(int dtype, int itype, int flags, int m, int k, int n, int nonzer
                 void* out, void* stream, int batch, void* workspace, size_t workspace_bytes);
 size_t iex_spmm_workspace_bytes(int dtype, int itype, int flags, int m, int k, int n,
                                 int nonzeros, int batch);
+/* What that workspace would hold: 0 = nothing (not used), 7 = the dense form of A, 9 = the partial sums of family 9,
+ * 10 = the tables and lists of family 10 (functions of the pattern only: a caller that keeps the workspace for a
+ * pattern may say so with IEX_SPMM_TABLES_READY / IEX_SPMM_LISTS_READY on later calls). */
+int iex_spmm_workspace_kind(int dtype, int itype, int flags, int m, int k, int n, int nonzeros, int batch);
 
 /* iex_spmm_ws for callers that cannot allocate device memory (code under hipGraph capture, tight serving
  * loops, harnesses that forbid hipMalloc): same arguments as iex_spmm_ex, same results as iex_spmm_ws with a

@@ -37,6 +37,7 @@ SIGNATURES = {
     "iex_spmm_ex": (_i, [_i, _i, _i, _i, _i, _i, _i, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i]),
     "iex_spmm_ws": (_i, [_i, _i, _i, _i, _i, _i, _i, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _vp, _c.c_size_t]),
     "iex_spmm_workspace_bytes": (_c.c_size_t, [_i, _i, _i, _i, _i, _i, _i, _i]),
+    "iex_spmm_workspace_kind": (_i, [_i, _i, _i, _i, _i, _i, _i, _i]),
     "iex_spmm_static": (_i, [_i, _i, _i, _i, _i, _i, _i, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i]),
     "iex_spmm_static_scratch_bytes": (_c.c_size_t, []),
     "iex_CudaSpmm2": (_i, [_i, _i, _i, _i, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i]),

@@ -712,14 +712,17 @@ int spmm_dispatch(int dtype, int itype, int flags, int m, int k, int n, int nonz
   // beyond the 256 MB last-level cache an output can only stream; the hint is worth 15-25 % of the write rate
   p.stream_out = (double)m * n * batch * (dtype == IEX_F32 ? 4 : 2) >= 128e6;
   hipStream_t s = static_cast<hipStream_t>(stream);
-  if (ch.variant == 10 && nonzeros == 0) ch.variant = 1;   // nothing to lay out: the row kernel writes the zeros
+  if (ch.variant == 10 && nonzeros < 4) ch.variant = 1;   // (its loads of four values at a time need four to exist)
+  const int blocks_ready = ((flags & IEX_SPMM_TABLES_READY) ? 1 : 0) | ((flags & IEX_SPMM_LISTS_READY) ? 2 : 0);
+  if (ch.variant == 0 && ch.ws && aligned(ch.ws, 16) && spmm_blocks_fits(dtype, itype, p) && spmm_blocks_wins(p, batch) &&
+      ch.ws_bytes >= spmm_blocks_bytes(p))
+    return launch_spmm_blocks(dtype, p, batch, ch.ws, 0, blocks_ready, s);
   if (ch.variant == 10) {
     IEX_REQUIRE(spmm_blocks_fits(dtype, itype, p), IEX_ERR_UNSUPPORTED,
                 "spmm: the dense-blocks kernel needs fp16 / bf16, int32 indices, n = 64, plain store without bias or ReLU, k <= 65536 and 16-byte aligned dense operands");
     IEX_REQUIRE(ch.ws && aligned(ch.ws, 16) && ch.ws_bytes >= spmm_blocks_bytes(p), IEX_ERR_BAD_ARGUMENT,
                 "spmm: the dense-blocks kernel needs a 16-byte aligned workspace of %zu bytes (iex_spmm_ws)", spmm_blocks_bytes(p));
-    return launch_spmm_blocks(dtype, p, batch, ch.ws, (flags >> 8) & 0xff,
-                              ((flags & IEX_SPMM_TABLES_READY) ? 1 : 0) | ((flags & IEX_SPMM_LISTS_READY) ? 2 : 0), s);
+    return launch_spmm_blocks(dtype, p, batch, ch.ws, (flags >> 8) & 0xff, blocks_ready, s);
   }
   if (dtype == IEX_F32 && itype == IEX_I32) return launch_typed<float, int>(p, batch, ch, s);
   if (dtype == IEX_F16 && itype == IEX_I32) return launch_typed<__half, int>(p, batch, ch, s);
@@ -730,20 +733,29 @@ int spmm_dispatch(int dtype, int itype, int flags, int m, int k, int n, int nonz
 
 // Bytes of workspace with which iex_spmm_ws would take the dense-form path for this call (0: it
 // would not, whatever the workspace).  Pointers are taken to be 16-byte aligned.
-size_t spmm_workspace_bytes(int dtype, int itype, int flags, int m, int k, int n, int nonzeros, int batch) {
+// kind: which family the workspace would serve (0 = none, 7 = dense form, 9 = partial sums of the k split, 10 = the
+// tables and lists of the dense-blocks kernel).
+static size_t workspace_plan(int dtype, int itype, int flags, int m, int k, int n, int nonzeros, int batch, int* kind) {
+  *kind = 0;
   if (m <= 0 || k <= 0 || n <= 0 || nonzeros <= 0 || batch <= 0) return 0;
   const int variant = (flags >> 16) & 0xf;
   void* const some_aligned = reinterpret_cast<void*>(size_t(256));
   if (dtype == IEX_F32 && itype == IEX_I32) {
     SpmmParams p{m, k, n, nonzeros, nullptr, nullptr, nullptr, nullptr, some_aligned, nullptr, some_aligned, 0, 0, 0};
-    if (variant == 9) return ksplit_plan<float>(p, batch, (flags >> 20) & 0xf, ((flags >> 24) & 0xf) == 2 ? 16 : 8).partial_bytes;
-    return 0;
+    if (variant != 9) return 0;
+    const size_t bytes = ksplit_plan<float>(p, batch, (flags >> 20) & 0xf, ((flags >> 24) & 0xf) == 2 ? 16 : 8).partial_bytes;
+    if (bytes) *kind = 9;
+    return bytes;
   }
   if (!(dtype == IEX_F16 || dtype == IEX_BF16) || !(itype == IEX_I32 || itype == IEX_I16)) return 0;
   if (variant != 0 && variant != 7 && variant != 10) return 0;
   SpmmParams p{m, k, n, nonzeros, nullptr, nullptr, nullptr, nullptr, some_aligned, nullptr, some_aligned,
                (flags & IEX_SPMM_PER_BATCH_VALUES) != 0, (flags & IEX_SPMM_ACCUMULATE) != 0, (flags & IEX_SPMM_RELU) != 0};
-  if (variant == 10) return spmm_blocks_fits(dtype, itype, p) ? spmm_blocks_bytes(p) : 0;
+  if (variant != 7 && nonzeros >= 4 && spmm_blocks_fits(dtype, itype, p) && (variant == 10 || spmm_blocks_wins(p, batch))) {
+    *kind = 10;
+    return spmm_blocks_bytes(p);
+  }
+  if (variant == 10) return 0;
   if (!dense_path_fits(2, p, (flags & IEX_SPMM_PER_BATCH_VALUES) != 0)) return 0;
   if (variant == 0) {
     Choice ch;
@@ -752,7 +764,19 @@ size_t spmm_workspace_bytes(int dtype, int itype, int flags, int m, int k, int n
     const bool few = smallk_wanted<__half>(p, batch);
     if (!dense_path_wins(p, batch, few ? 0 : mfma_variant<__half>(p, batch, ch).kind, few)) return 0;
   }
+  *kind = 7;
   return dense_path_bytes(p);
+}
+
+size_t spmm_workspace_bytes(int dtype, int itype, int flags, int m, int k, int n, int nonzeros, int batch) {
+  int kind;
+  return workspace_plan(dtype, itype, flags, m, k, n, nonzeros, batch, &kind);
+}
+
+int spmm_workspace_kind(int dtype, int itype, int flags, int m, int k, int n, int nonzeros, int batch) {
+  int kind;
+  workspace_plan(dtype, itype, flags, m, k, n, nonzeros, batch, &kind);
+  return kind;
 }
 
 // ---- the library's own scratch memory, for callers that cannot allocate ---------------------------------
@@ -826,6 +850,10 @@ int iex_spmm_ws(int dtype, int itype, int flags, int m, int k, int n, int nonzer
 
 size_t iex_spmm_workspace_bytes(int dtype, int itype, int flags, int m, int k, int n, int nonzeros, int batch) {
   return iex::spmm_workspace_bytes(dtype, itype, flags, m, k, n, nonzeros, batch);
+}
+
+int iex_spmm_workspace_kind(int dtype, int itype, int flags, int m, int k, int n, int nonzeros, int batch) {
+  return iex::spmm_workspace_kind(dtype, itype, flags, m, k, n, nonzeros, batch);
 }
 
 int iex_CudaSpmm2(int m, int k, int n, int nonzeros, const int* row_indices, const float* values,

@@ -12,6 +12,22 @@ bool spmm_blocks_fits(int dtype, int itype, const SpmmParams& p) {
          (long long)(ceil_div(p.k, kSdBN) + 1) * p.m < (1ll << 28);
 }
 
+// The host does not look at the pattern, so where nothing is forced the choice goes by the overall density, and only
+// for values per batch entry (attention probabilities: masks with structure).  Measured on MI355X (fp16, 16 batch
+// entries of 4096 x 4096, n = 64, microseconds, row kernel / this kernel with its three setup kernels / with tables
+// and lists kept):
+//   band of 256 + 32 scattered per row (7 %)   99 /  55 /  38     band of 512 + 32 (13 %)        184 /  75 /  51
+//   band of 128 + 16 scattered (3.5 %)          60 /  48 /  31     block diagonal 256 (6 %)        83 /  37 /  21
+//   causal window of 512 (12 %)                161 /  62 /  38     band 256 + 128 scattered (9 %) 134 / 101 /  77
+//   equal rows, columns at random:  1 %  37 / 35 / 22     3 %  62 / 77 / 59     5 %  80 / 114 / 90
+//                                  10 % 152 / 195 / 171   15 % 222 / 212 / 198  20 % 298 / 215 / 192
+// Masks with structure gain 1.3x to 4x from 3 % up; a mask without any loses 1.1x to 1.4x between 3 and 10 %.
+// IEX_SPMM_FORCE_VARIANT(1) keeps the row kernel.
+bool spmm_blocks_wins(const SpmmParams& p, int batch) {
+  const double density = (double)p.nnz / ((double)p.m * p.k);
+  return p.per_batch_values && p.nnz >= 4 && density >= 0.03 && (double)batch * p.m * p.k >= 32.0 * 1024 * 1024;
+}
+
 size_t spmm_blocks_bytes(const SpmmParams& p) { return sb_words(p.m, ceil_div(p.k, kSdBN), p.nnz) * sizeof(int); }
 
 template <bool BF16>

@@ -35,6 +35,7 @@ namespace iex {
 constexpr int kSbN = 64;                       // output columns
 constexpr int kSbTileBytes = 32 * kSdLd * 2;   // a wavefront's 32 x 128 tile of A (rows padded to 272 bytes); later its 32 x 64 fp32 sums
 constexpr int kSbStage = kSdBN * kSbN * 2;     // 128 rows of the dense operand
+constexpr int kSbRows = 2;                     // rows whose nonzeros outside dense tiles a lane group gathers side by side (1, 2 or 4)
 constexpr int kSbZeroWords = 32;               // 128 bytes of zeros: what the lanes of an absent nonzero read
 
 struct SbEntry {
@@ -79,7 +80,7 @@ struct SpmmBlocksParams {
   const unsigned short* dense_list;
 };
 
-constexpr int spmm_blocks_lds_bytes() { return 4 * kSbTileBytes + 2 * kSbStage; }
+constexpr int spmm_blocks_lds_bytes() { return 4 * kSbTileBytes + 2 * kSbStage + 32 + 4 * 32 * 32; }
 
 // The dense tiles of every block of 128 rows (one workgroup each): dense_list[block][0] = their number, then the tiles.
 static __global__ __launch_bounds__(kSdThreads) void sb_dense_list_kernel(int m, int tiles_k, int dense_min, const int* __restrict__ tile_ptr,
@@ -146,13 +147,17 @@ template <bool BF16>
 __global__ __launch_bounds__(kSdThreads, 2) void spmm_blocks_kernel(SpmmBlocksParams p) {
   typedef unsigned short u16;
   typedef __attribute__((address_space(3))) s16x4 lds_s16x4;
+  typedef unsigned u32_a2 __attribute__((aligned(2)));             // loads of two and four values at the alignment of one
+  typedef unsigned long long u64_a2 __attribute__((aligned(2)));
   constexpr int NT = kSbN / 32;
   extern __shared__ __align__(16) unsigned char smem[];
   unsigned char* sV = smem + 4 * kSbTileBytes;                               // [2][128][128 bytes]
+  unsigned* lut = reinterpret_cast<unsigned*>(sV + 2 * kSbStage);           // [8]
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  unsigned* rec = lut + 8 + wave * (32 * 8);                                 // [32][8]: what a wavefront's rows know of the current tile
   // Workgroups go to the 8 XCDs round-robin by their linear id; renumbered so that an XCD gets all row blocks of a
   // batch entry (and then of the next): the dense operand of that entry stays in that XCD's L2.
   const int row_blocks = gridDim.x, total = row_blocks * gridDim.y;
@@ -177,11 +182,8 @@ __global__ __launch_bounds__(kSdThreads, 2) void spmm_blocks_kernel(SpmmBlocksPa
   u16* P16 = reinterpret_cast<u16*>(Pw);
   const int wrow0 = row0 + wave * 32;               // first of this wavefront's rows
 
-  f32x16 acc[NT];
-#pragma unroll
-  for (int t = 0; t < NT; ++t)
-#pragma unroll
-    for (int r = 0; r < 16; ++r) acc[t][r] = 0.f;
+  float* T = reinterpret_cast<float*>(Pw);           // after the dense tiles: the matrix-core sums of the 32 rows, fp32
+  constexpr int TLD = kSdLd / 2;                     // 68 floats = the 272 bytes of a row of the tile
   float tacc[4][8];   // sums over the nonzeros outside dense tiles: row it * 8 + lane / 8, columns (lane % 8) * 8 .. + 7
 #pragma unroll
   for (int it = 0; it < 4; ++it)
@@ -191,6 +193,11 @@ __global__ __launch_bounds__(kSdThreads, 2) void spmm_blocks_kernel(SpmmBlocksPa
   for (int phase = 0; phase < 2; ++phase) {
     if ((phase == 0) != thin_first) {
       // ---- dense tiles
+      f32x16 acc[NT];
+#pragma unroll
+      for (int t = 0; t < NT; ++t)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) acc[t][r] = 0.f;
       if (nd > 0) {
         // 128 rows x 128 bytes of the dense operand: chunk L = q * 256 + tid sits at LDS byte 16 L and holds global
         // chunk (L % 8) ^ 4 * ((row / 2) % 2) of row L / 8
@@ -234,7 +241,16 @@ __global__ __launch_bounds__(kSdThreads, 2) void spmm_blocks_kernel(SpmmBlocksPa
           v_off[t] = tr_k * (kSbN * 2) + chunk * 16 + (lane & 1) * 8;
         }
         const int p_off = (lane & 31) * (kSdLd * 2) + fkh * 16;
+        // the mask word and the bits in it of the two columns that this lane owns in a long row
+        const int own_word = lane >> 4, own_bit = (2 * lane) & 31;
+        const unsigned own_below = (1u << own_bit) - 1u;
 
+        // byte selectors for v_perm(0, loaded, selector), by (column 2 i present) + 2 (column 2 i + 1 present) + 4 (the
+        // load was moved back by one value: the wanted value is in the upper half)
+        if (tid < 8) {
+          const unsigned none = 0x0c0c0c0cu;
+          lut[tid] = tid == 1 ? 0x0c0c0100u : tid == 2 ? 0x01000c0cu : tid == 3 || tid == 7 ? 0x03020100u : tid == 5 ? 0x0c0c0302u : tid == 6 ? 0x03020c0cu : none;
+        }
         u32x4 rv[4];
         int tp, bf;
         u32x4 mk;
@@ -260,41 +276,48 @@ __global__ __launch_bounds__(kSdThreads, 2) void spmm_blocks_kernel(SpmmBlocksPa
             }
           }
           const int count = meta_valid ? (bf >> 28) & 7 : 0;
-          // ... up to 4 values of a row by the row's lane (loads from clamped positions: no branch around a load) ...
-          u16 sv[kSdShort];
-#pragma unroll
-          for (int u = 0; u < kSdShort; ++u) sv[u] = vals[min(max(tp, 0) + u, last)];
-          // ... longer runs by the wavefront: lane i owns columns i and 64 + i of the row; all loads first
+          // ... up to 4 values of a row by the row's lane: the 8 bytes from the row's first value in the tile (a load
+          // at 2-byte alignment; moved back where it would pass the end of the values, and shifted to make up) ...
+          const int s_at = min(max(tp, 0), last - 3);
+          const int s_shift = min(max(tp, 0) - s_at, 3) * 16;   // (more than 3 only for rows without values here)
+          const unsigned long long sv = *reinterpret_cast<const u64_a2*>(vals + s_at);
+          // ... longer runs by the wavefront: lane i owns columns 2 i and 2 i + 1 of the row.  The number of the row's
+          // nonzeros below column 2 i gives the position of the pair's first value among the row's values in the
+          // tile; its 4 bytes hold both values when both columns are present.  Lanes 0..31 publish what they know of
+          // their rows in LDS (mask, nonzeros below each mask word, cursor), every lane picks from there what concerns
+          // its two columns; how the loaded bytes map to the pair (byte selectors for v_perm) comes from a table of 8.
+          // All loads first.
           const unsigned longs = (unsigned)__ballot(count == 7);
-          u16 lo[32], hi[32];   // (as loaded: which of them exist is looked at when they are written)
+          if (lane < 32) {
+            const unsigned cx = __popc(mk.x), cy = cx + __popc(mk.y), cz = cy + __popc(mk.z);
+            *reinterpret_cast<u32x4*>(rec + lane * 8) = mk;
+            *reinterpret_cast<u32x2*>(rec + lane * 8 + 4) = u32x2{(cx << 8) | (cy << 16) | (cz << 24), (unsigned)max(tp, 0)};
+          }
+          __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+          __builtin_amdgcn_wave_barrier();
+          unsigned pair[32], sel[32];
 #pragma unroll
           for (int r = 0; r < 32; ++r) {
-            lo[r] = 0;
-            hi[r] = 0;
+            pair[r] = 0;
+            sel[r] = 0;
             if ((longs >> r) & 1) {   // (uniform)
-              const unsigned mx = (unsigned)__builtin_amdgcn_readlane((int)mk.x, r), my = (unsigned)__builtin_amdgcn_readlane((int)mk.y, r);
-              const unsigned mz = (unsigned)__builtin_amdgcn_readlane((int)mk.z, r), mw = (unsigned)__builtin_amdgcn_readlane((int)mk.w, r);
-              const int start = max(__builtin_amdgcn_readlane(tp, r), 0);
-              const int rank_lo = __builtin_amdgcn_mbcnt_hi(my, __builtin_amdgcn_mbcnt_lo(mx, 0));
-              const int rank_hi = __builtin_amdgcn_mbcnt_hi(mw, __builtin_amdgcn_mbcnt_lo(mz, 0)) + __popc(mx) + __popc(my);
-              lo[r] = vals[min(start + rank_lo, last)];
-              hi[r] = vals[min(start + rank_hi, last)];
+              const unsigned word = rec[r * 8 + own_word];
+              const u32x2 pt = *reinterpret_cast<const u32x2*>(rec + r * 8 + 4);
+              const int at = (int)(pt.y + ((pt.x >> (own_word * 8)) & 0xffu)) + __popc(word & own_below);
+              const int at_c = min(at, last - 1);
+              sel[r] = lut[((word >> own_bit) & 3u) | (at > at_c ? 4u : 0u)];   // (lanes past the row's last value own no column: entry 0 or 4, all zeros)
+              pair[r] = *reinterpret_cast<const u32_a2*>(vals + at_c);
             }
           }
           if (count >= 1 && count <= kSdShort) {
 #pragma unroll
             for (int u = 0; u < kSdShort; ++u)
-              if (u < count) P16[lane * kSdLd + ((bf >> (7 * u)) & 127)] = sv[u];
+              if (u < count) P16[lane * kSdLd + ((bf >> (7 * u)) & 127)] = (u16)(sv >> ((s_shift + 16 * u) & 63));
           }
 #pragma unroll
           for (int r = 0; r < 32; ++r) {
-            if ((longs >> r) & 1) {
-              const unsigned mx = (unsigned)__builtin_amdgcn_readlane((int)mk.x, r), my = (unsigned)__builtin_amdgcn_readlane((int)mk.y, r);
-              const unsigned mz = (unsigned)__builtin_amdgcn_readlane((int)mk.z, r), mw = (unsigned)__builtin_amdgcn_readlane((int)mk.w, r);
-              const unsigned word_lo = lane < 32 ? mx : my, word_hi = lane < 32 ? mz : mw;
-              P16[r * kSdLd + lane] = ((word_lo >> (lane & 31)) & 1) ? lo[r] : (u16)0;
-              P16[r * kSdLd + kWave + lane] = ((word_hi >> (lane & 31)) & 1) ? hi[r] : (u16)0;
-            }
+            if ((longs >> r) & 1)
+              *reinterpret_cast<unsigned*>(P16 + r * kSdLd + 2 * lane) = __builtin_amdgcn_perm(0u, pair[r], sel[r]);
           }
           __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
           __builtin_amdgcn_wave_barrier();
@@ -321,6 +344,17 @@ __global__ __launch_bounds__(kSdThreads, 2) void spmm_blocks_kernel(SpmmBlocksPa
           __syncthreads();
         }
       }
+      // the sums leave the registers here (the other part needs them for loads in flight): this wavefront's tile, no
+      // longer read by anybody, takes them as fp32
+      __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+      __builtin_amdgcn_wave_barrier();
+#pragma unroll
+      for (int t = 0; t < NT; ++t)
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+          const f32x4 x = {acc[t][q * 4], acc[t][q * 4 + 1], acc[t][q * 4 + 2], acc[t][q * 4 + 3]};
+          *reinterpret_cast<f32x4*>(T + (lane & 31) * TLD + t * 32 + q * 8 + (lane >> 5) * 4) = x;
+        }
     } else {
       // ---- nonzeros outside dense tiles: lane group g = lane / 8 takes rows g, 8 + g, 16 + g, 24 + g of the
       // wavefront's 32, two at a time, 8 nonzeros of each per step: lane sl of the group reads entry sl of the step
@@ -338,22 +372,25 @@ __global__ __launch_bounds__(kSdThreads, 2) void spmm_blocks_kernel(SpmmBlocksPa
         cnt[it] = r < m ? p.thin_cnt[rc] : 0;
       }
 #pragma unroll
-      for (int h = 0; h < 4; h += 2) {
-        const int nmax = max(cnt[h], cnt[h + 1]);
-        SbEntry en[2];
+      for (int h = 0; h < 4; h += kSbRows) {
+        int nmax = 0;
+        SbEntry en[kSbRows];
 #pragma unroll
-        for (int w = 0; w < 2; ++w) en[w] = p.thin_ent[min(base[h + w] + min(sl, max(cnt[h + w] - 1, 0)), last)];
+        for (int w = 0; w < kSbRows; ++w) {
+          nmax = max(nmax, cnt[h + w]);
+          en[w] = p.thin_ent[min(base[h + w] + min(sl, max(cnt[h + w] - 1, 0)), last)];
+        }
         for (int st = 0; __ballot(st * 8 < nmax); ++st) {
-          u16 pv[2];
-          u32x4 v[2][8];
-          int colw[2];
+          u16 pv[kSbRows];
+          u32x4 v[kSbRows][8];
+          int colw[kSbRows];
 #pragma unroll
-          for (int w = 0; w < 2; ++w) {
+          for (int w = 0; w < kSbRows; ++w) {
             pv[w] = vals[min((unsigned)en[w].pos, (unsigned)last)];
             colw[w] = en[w].col;
           }
 #pragma unroll
-          for (int w = 0; w < 2; ++w)
+          for (int w = 0; w < kSbRows; ++w)
 #pragma unroll
             for (int u = 0; u < 8; ++u) {
               const int cu = __shfl(colw[w], gl + u, kWave);
@@ -361,12 +398,12 @@ __global__ __launch_bounds__(kSdThreads, 2) void spmm_blocks_kernel(SpmmBlocksPa
               v[w][u] = *reinterpret_cast<const u32x4*>(src);
             }
 #pragma unroll
-          for (int w = 0; w < 2; ++w) {
+          for (int w = 0; w < kSbRows; ++w) {
             if (st * 8 + sl >= cnt[h + w]) pv[w] = 0;
             en[w] = p.thin_ent[min(base[h + w] + min((st + 1) * 8 + sl, max(cnt[h + w] - 1, 0)), last)];
           }
 #pragma unroll
-          for (int w = 0; w < 2; ++w)
+          for (int w = 0; w < kSbRows; ++w)
 #pragma unroll
             for (int u = 0; u < 8; ++u) {
               const float pf = f16_to_32((u16)__shfl((int)pv[w], gl + u, kWave), BF16);
@@ -382,19 +419,7 @@ __global__ __launch_bounds__(kSdThreads, 2) void spmm_blocks_kernel(SpmmBlocksPa
     }
   }
 
-  // ---- both parts meet: the matrix-core sums as fp32 in this wavefront's tile (rows of 68 floats), then every lane
-  // adds its own sums to the 8 entries it owns, rounds and stores 16 bytes
-  __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
-  __builtin_amdgcn_wave_barrier();
-  float* T = reinterpret_cast<float*>(Pw);
-  constexpr int TLD = kSdLd / 2;   // 68 floats = the 272 bytes of a row of the tile
-#pragma unroll
-  for (int t = 0; t < NT; ++t)
-#pragma unroll
-    for (int q = 0; q < 4; ++q) {
-      const f32x4 x = {acc[t][q * 4], acc[t][q * 4 + 1], acc[t][q * 4 + 2], acc[t][q * 4 + 3]};
-      *reinterpret_cast<f32x4*>(T + (lane & 31) * TLD + t * 32 + q * 8 + (lane >> 5) * 4) = x;
-    }
+  // ---- both parts meet: every lane adds its own sums to the 8 matrix-core sums it owns, rounds and stores 16 bytes
   __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
   __builtin_amdgcn_wave_barrier();
   {

@@ -38,6 +38,7 @@ struct SpmmParams {
 
 // The kernel for 16-bit sparse operands with structure and 64 output columns (spmm_blocks.hip)
 bool spmm_blocks_fits(int dtype, int itype, const SpmmParams& p);
+bool spmm_blocks_wins(const SpmmParams& p, int batch);
 size_t spmm_blocks_bytes(const SpmmParams& p);
 int launch_spmm_blocks(int dtype, const SpmmParams& p, int batch, void* ws, int dense_code, int ready, hipStream_t stream);
 

@@ -101,6 +101,10 @@ def _spmm(b, row_indices, values, row_offsets, column_indices, m, *, per_batch_v
     tuned = getattr(_TUNING, "spmm", None)
     if tuned and not (force_wpr or force_variant or force_rpw or force_nt or force_lpg):
         force_wpr, force_variant, force_rpw, force_nt, force_lpg = (tuned.get(key, 0) for key in _SPMM_KEYS)
+    if plan is not None and plan.variant and not force_variant:
+        # settled by SddmmPlan.analyze(): the dense-blocks kernel for masks with structure (it still has to fit dtype and
+        # shape: checked below), else the row kernel
+        force_variant = 10 if plan.variant == 3 else 1
     _chk(b.dim() == 3)
     if per_batch_values:
         _chk(values.dim() == 2)
@@ -145,18 +149,21 @@ def _spmm(b, row_indices, values, row_offsets, column_indices, m, *, per_batch_v
         # room for the dense form of the sparse operand where the library would rather hand the
         # product to its dense GEMM (large 16-bit products): from torch's allocator, on the current
         # stream, released (stream-ordered) when this call returns
-        ws_bytes = 0 if no_workspace else lib.iex_spmm_workspace_bytes(
-            _DT[b.dtype], _IT[column_indices.dtype], flags, m, k, n, nonzeros, batch)
-        if plan is not None and ws_bytes and ((flags >> 16) & 0xf) == 10:
+        shape = (_DT[b.dtype], _IT[column_indices.dtype], flags, m, k, n, nonzeros, batch)
+        if plan is not None and plan.variant == 3 and ((flags >> 16) & 0xf) == 10 and lib.iex_spmm_workspace_kind(*shape) != 10:
+            flags &= ~((0xf << 16) | (0xff << 8))      # the planned kernel does not serve this call (fp32, another n): the library's rule
+            shape = shape[:2] + (flags,) + shape[3:]
+        ws_bytes = 0 if no_workspace else lib.iex_spmm_workspace_bytes(*shape)
+        if plan is not None and ws_bytes and lib.iex_spmm_workspace_kind(*shape) == 10:
             # the tables of the dense-blocks kernel depend on the pattern only and are those of the SDDMM for masks
             # with structure: a plan shared with that operator's calls on the pattern serves both
             key = (row_offsets.data_ptr(), column_indices.data_ptr(), row_offsets._version, column_indices._version,
                    m, k, nonzeros)
             if plan._ready(key, ws_bytes, b.device):
                 flags |= _lib.SPMM_TABLES_READY
-                if plan.lists_key == (key, int(force_wpr)):
+                if plan.lists_key == (key, (flags >> 8) & 0xff):
                     flags |= _lib.SPMM_LISTS_READY
-            plan.lists_key = (key, int(force_wpr))
+            plan.lists_key = (key, (flags >> 8) & 0xff)
             ws = plan.workspace
         else:
             ws = torch.empty(ws_bytes, dtype=torch.uint8, device=b.device) if ws_bytes else None
@@ -170,7 +177,8 @@ def _spmm(b, row_indices, values, row_offsets, column_indices, m, *, per_batch_v
 
 
 class SddmmPlan:
-    """Memory that per-entry SDDMM calls on one CSR pattern keep between calls.
+    """Memory that per-entry SDDMM calls on one CSR pattern (and the SpMM calls with per-entry values on the same pattern:
+    the two products of sparse attention) keep between calls.
 
     The kernel for masks with structure (``iex_sddmm_ws``, variant 3) works from tables that a setup kernel derives
     from the pattern alone (m, n, row_offsets, column_indices).  A caller whose mask does not change passes the same
@@ -290,6 +298,15 @@ def spmm_sputnik_batched_values(b, row_indices, values, row_offsets, column_indi
     return _spmm(b, row_indices, values, row_offsets, column_indices, m, per_batch_values=True,
                  accumulate=False, dtypes=(torch.float32, torch.float16, torch.bfloat16),
                  allow_i16=True)
+
+
+def spmm_batched_values_planned(b, row_indices, values, row_offsets, column_indices, m, plan: "SddmmPlan"):
+    """``spmm_sputnik_batched_values`` for a caller that keeps an :class:`SddmmPlan` for the pattern (not a registered
+    operator: the plan is a Python object).  The plan may be the one that the pattern's SDDMM calls use: the tables are
+    the same, the SpMM keeps two lists of its own behind them."""
+    return _spmm(b, row_indices, values, row_offsets, column_indices, m, per_batch_values=True,
+                 accumulate=False, dtypes=(torch.float32, torch.float16, torch.bfloat16),
+                 allow_i16=True, plan=plan)
 
 
 def sddmm_sputnik_atomic_upd_weight(a, b, row_indices, row_offsets, column_indices):

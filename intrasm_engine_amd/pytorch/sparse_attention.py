@@ -28,8 +28,9 @@ def sparse_attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, row_indi
     arrays (``row_indices`` = rows by decreasing length).  fp16, bf16 or fp32.  Returns
     (heads, tokens, dv), and the (heads, nnz) probabilities when ``return_probs``.
     Rows of the mask without entries give zero output rows.
-    ``plan``: an ``ops.SddmmPlan`` that the caller keeps for this mask; with it the tables that the score kernel derives
-    from the mask are written by the first call only (16-bit inputs; ignored where that kernel is not the one that runs)."""
+    ``plan``: an ``ops.SddmmPlan`` that the caller keeps for this mask; with it the tables and lists that the two sparse
+    products derive from the mask are written by the first call only (16-bit inputs; ignored where those kernels are not
+    the ones that run)."""
     if q.dim() != 3 or k.shape != q.shape or v.dim() != 3 or v.shape[:2] != q.shape[:2]:
         raise RuntimeError("q, k must be (heads, tokens, d) and v (heads, tokens, dv)")
     tokens = q.shape[1]
@@ -43,5 +44,8 @@ def sparse_attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, row_indi
     else:
         scores = ops.sddmm_sputnik_half(q, k, row_indices, row_offsets, column_indices)     # (heads, nnz)
     probs = ops.csr_softmax_(scores, row_indices, row_offsets, float(scale))
-    out = ops.spmm_sputnik_batched_values(v, row_indices, probs, row_offsets, column_indices, tokens)
+    if plan is not None:
+        out = _pyops.spmm_batched_values_planned(v, row_indices, probs, row_offsets, column_indices, tokens, plan)
+    else:
+        out = ops.spmm_sputnik_batched_values(v, row_indices, probs, row_offsets, column_indices, tokens)
     return (out, probs) if return_probs else out

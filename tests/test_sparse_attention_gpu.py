@@ -68,3 +68,29 @@ def test_rows_without_entries_and_default_scale(oracle, dev):
     assert np.abs(out - dense).max() <= 2e-5 * np.abs(v).max()
     with pytest.raises(RuntimeError, match="tokens x tokens"):
         sparse_attention(t(q), t(k), t(v), t(ri[:-1]), t(ro[:-1]), t(ci))
+
+
+def test_block_with_a_plan_runs_both_structured_kernels_and_keeps_their_tables(oracle, dev):
+    """A caller that keeps a plan for its mask: both sparse products take their kernels for masks with structure, the
+    second call launches nothing but the three kernels of the block, and the result is that of the block without a
+    plan (whose products, at this size, the library gives to the gather and row kernels) up to fp16 rounding, and
+    the oracle's."""
+    from intrasm_engine_amd import _lib
+    from intrasm_engine_amd.pytorch import ops as pyops
+    pattern, q, k, v = W.config3(seed=21, tokens=640, heads=2, head_dim=64, band=160, extra=4)
+    ri, _, ro, ci = to_dev(pattern, dev)
+    t = lambda a: torch.from_numpy(a).to(dev).half()
+    plan = pyops.SddmmPlan()
+    assert plan.analyze(ro, ci, pattern.k) == 3
+    first = sparse_attention(t(q), t(k), t(v), ri, ro, ci, plan=plan)
+    assert "spmm_blocks_kernel" in _lib.last_kernels()
+    again = sparse_attention(t(q), t(k), t(v), ri, ro, ci, plan=plan)
+    assert _lib.last_kernels() == "spmm_blocks_kernel<false>" and torch.equal(again, first)
+    plain = sparse_attention(t(q), t(k), t(v), ri, ro, ci)
+    assert "spmm_blocks_kernel" not in _lib.last_kernels()
+    assert torch.allclose(first.float(), plain.float(), rtol=1e-2, atol=5e-3)
+    qr, kr, vr = (rounded(x, torch.float16) for x in (q, k, v))
+    scores = oracle.sddmm(qr, kr, pattern.row_indices, pattern.row_offsets, pattern.column_indices, sum_over_batch=False)
+    want = oracle.spmm(vr, pattern.row_indices, oracle.csr_softmax(scores * 0.125, pattern.row_offsets), pattern.row_offsets,
+                       pattern.column_indices, pattern.m)
+    assert np.abs(first.float().cpu().numpy() - want).max() <= 1e-2 * np.abs(vr).max()

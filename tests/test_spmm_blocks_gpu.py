@@ -143,11 +143,48 @@ def test_tables_kept_between_calls_and_shared_with_the_sddmm(dev):
     assert torch.equal(again, pyops._spmm(v, ri2, vals2, rot2, cit2, m, **kw))
 
 
+def test_picked_for_attention_sized_products_with_values_per_head(dev):
+    """Nothing forced: 16 heads of config 3's mask take this kernel when the values differ per head, the row kernel
+    when they are shared or the product is small; a plan whose analysis found no structure keeps the row kernel."""
+    from intrasm_engine_amd import _lib
+    from intrasm_engine_amd.pytorch import ops as pyops
+    pat, _, _, v = W.config3()
+    ri, _, ro, ci = to_dev(pat, dev)
+    vt = torch.from_numpy(v).to(dev).half()
+    probs = (torch.rand(16, pat.nnz, device=dev) / 280).half()
+    got = ops.spmm_sputnik_batched_values(vt, ri, probs, ro, ci, pat.m)
+    assert "spmm_blocks_kernel" in _lib.last_kernels()
+    with pyops.kernel_params(spmm={"force_variant": 1}):
+        rows = ops.spmm_sputnik_batched_values(vt, ri, probs, ro, ci, pat.m)
+    assert "spmm_blocks_kernel" not in _lib.last_kernels()
+    assert torch.allclose(got.float(), rows.float(), rtol=1e-2, atol=2e-3)
+    ops.spmm_sputnik_reuse_weight_half(vt, ri, probs[0].contiguous(), ro, ci, pat.m)
+    assert "spmm_blocks_kernel" not in _lib.last_kernels()
+    ops.spmm_sputnik_batched_values(vt[:1], ri, probs[:1], ro, ci, pat.m)
+    assert "spmm_blocks_kernel" not in _lib.last_kernels()
+    plan = pyops.SddmmPlan()
+    assert plan.analyze(ro, ci, pat.k) == 3
+    planned = pyops.spmm_batched_values_planned(vt, ri, probs, ro, ci, pat.m, plan)
+    assert "spmm_blocks_kernel" in _lib.last_kernels() and torch.equal(planned, got)
+    pyops.spmm_batched_values_planned(vt, ri, probs, ro, ci, pat.m, plan)
+    assert _lib.last_kernels() == "spmm_blocks_kernel<false>"
+    fp32 = pyops.spmm_batched_values_planned(vt.float(), ri, probs.float(), ro, ci, pat.m, plan)     # the planned kernel does not serve fp32
+    assert "spmm_blocks_kernel" not in _lib.last_kernels() and torch.allclose(fp32, rows.float(), rtol=1e-2, atol=2e-3)
+    flat = pyops.SddmmPlan()
+    flat.variant = 1
+    pyops.spmm_batched_values_planned(vt, ri, probs, ro, ci, pat.m, flat)
+    assert "spmm_blocks_kernel" not in _lib.last_kernels()
+
+
 def test_refusals_and_workspace_size(dev):
     from intrasm_engine_amd import _lib
     lib = _lib.load()
     flags = (10 << 16) | _lib.SPMM_PER_BATCH_VALUES
     assert lib.iex_spmm_workspace_bytes(_lib.F16, _lib.I32, flags, 4096, 4096, 64, 1000, 16) == ((6 * 32 + 1) * 4096 + 32 + 2 * 1000 + 4096 + 32 * (32 + 2) // 2) * 4
+    assert lib.iex_spmm_workspace_kind(_lib.F16, _lib.I32, flags, 4096, 4096, 64, 1000, 16) == 10
+    assert lib.iex_spmm_workspace_kind(_lib.F16, _lib.I32, _lib.SPMM_PER_BATCH_VALUES, 4096, 4096, 64, 1000, 16) == 0        # too sparse for the rule
+    assert lib.iex_spmm_workspace_kind(_lib.F16, _lib.I32, _lib.SPMM_PER_BATCH_VALUES, 4096, 4096, 64, 1 << 20, 16) == 10
+    assert lib.iex_spmm_workspace_kind(_lib.F16, _lib.I32, 0, 4096, 4096, 64, 1 << 20, 16) != 10                              # shared values
     assert lib.iex_spmm_workspace_bytes(_lib.F16, _lib.I32, flags, 4096, 4096, 128, 1000, 16) == 0      # n != 64
     assert lib.iex_spmm_workspace_bytes(_lib.F32, _lib.I32, flags, 4096, 4096, 64, 1000, 16) == 0
     assert lib.iex_spmm_workspace_bytes(_lib.F16, _lib.I16, flags, 4096, 4096, 64, 1000, 16) == 0

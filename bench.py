@@ -77,6 +77,9 @@ def main():
                     help="bf16 GEMM (B as (K, N)): every tile shape on a few products, one line per product on stdout; with "
                          "--gemm-probe-tile T only that shape on config 4's product, 3 launches (for rocprofv3 --pmc)")
     ap.add_argument("--gemm-probe-tile", type=int, default=-1)
+    ap.add_argument("--spmm-probe", action="store_true",
+                    help="config 3's SpMM against V (fp16, 16 heads), 3 launches of what the operator picks and 3 of the row kernel "
+                         "(for rocprofv3; no JSON line)")
     ap.add_argument("--sddmm-probe", action="store_true",
                     help="config 3's SDDMM (fp16, 16 heads), 3 launches of what the operator picks and 3 of the gather kernel "
                          "(for rocprofv3 --kernel-trace / --pmc)")
@@ -195,6 +198,22 @@ def main():
             for _ in range(3):
                 ops.sddmm_sputnik_half(qt_, kt_, ri_, ro_, ci_)
         log("[sddmm-probe] gather kernel:", _lib.last_kernels())
+        torch.cuda.synchronize()
+        return
+
+    if args.spmm_probe:
+        from intrasm_engine_amd.pytorch import ops as pyops_s
+        pat_, _, _, v_ = W.config3()
+        ri_, _, ro_, ci_ = csr_dev(pat_)
+        vt_ = torch.from_numpy(v_).to(dev).half()
+        probs_ = (torch.rand(16, pat_.nnz, device=dev, generator=torch.Generator(dev).manual_seed(4)) / 280).half()
+        for _ in range(3):
+            ops.spmm_sputnik_batched_values(vt_, ri_, probs_, ro_, ci_, pat_.m)
+        log("[spmm-probe] operator:", _lib.last_kernels())
+        with pyops_s.kernel_params(spmm={"force_variant": 1}):
+            for _ in range(3):
+                ops.spmm_sputnik_batched_values(vt_, ri_, probs_, ro_, ci_, pat_.m)
+        log("[spmm-probe] row kernel:", _lib.last_kernels())
         torch.cuda.synchronize()
         return
 

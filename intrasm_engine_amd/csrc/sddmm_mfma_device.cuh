@@ -88,7 +88,9 @@ inline size_t sddmm_mfma_words(int m, int tiles_n) { return (size_t)m * (4 * (si
 // tile_ptr[t][row] for t = 0 .. tiles_n, brief[t][row] and (where needed) mask[t][row] for t < tiles_n: one
 // wavefront per row.  brief packs what a lane needs to sample a (row, tile) pair without touching the column indices
 // again: bits 28..30 = number of nonzeros of the row in the tile (0..4, or 7 for "more"), bits 7u .. 7u + 6 =
-// column of nonzero u inside the tile.  The mask of a pair with more has bit c set when column 128 t + c is present.
+// column of nonzero u inside the tile.  The mask of a pair with more has bit c set when column 128 t + c is present,
+// and its packed word then holds the number of nonzeros in the first 32, 64 and 96 columns of the tile (bits 0..5,
+// 6..12, 13..19).
 // The row's columns are first marked in a bit map in LDS (n bits); counts, cursors and packed words come from the
 // map, 64 tiles at a time, one tile per lane.
 static __global__ __launch_bounds__(256) void sddmm_tile_ptr_kernel(int m, int tiles_n, const int* __restrict__ row_offsets,
@@ -135,6 +137,8 @@ static __global__ __launch_bounds__(256) void sddmm_tile_ptr_kernel(int m, int t
       int word = (count <= kSdShort ? count : 7) << 28;
       if (count > kSdShort) {
         mask[(size_t)t * m + r] = w;
+        const int cx = __popc(w.x), cy = cx + __popc(w.y), cz = cy + __popc(w.z);
+        word |= cx | (cy << 6) | (cz << 13);
       } else {
         unsigned left[4] = {w.x, w.y, w.z, w.w};
 #pragma unroll
@@ -245,6 +249,7 @@ __global__ __launch_bounds__(kSdThreads, KS == 8 ? 1 : 2) void sddmm_mfma_kernel
   constexpr int STAGE = kSdBN * RB;
   static_assert(KS == 2 || KS == 4 || KS == 8, "k = 32, 64 or 128");
   typedef unsigned short u16;
+  typedef unsigned u32_a2 __attribute__((aligned(2)));   // two neighbouring scores stored at once
   typedef __attribute__((address_space(3))) unsigned char lds_u8;
   extern __shared__ __align__(16) unsigned char smem[];
   u16* S = reinterpret_cast<u16*>(smem);                                      // [128][kSdLd]; before the loop: column sums
@@ -325,6 +330,12 @@ __global__ __launch_bounds__(kSdThreads, KS == 8 ? 1 : 2) void sddmm_mfma_kernel
       for (int ks = 0; ks < KS; ++ks) fl[i][ks] = *reinterpret_cast<const u32x4*>(lhs + (size_t)row * p.k + ks * 16 + frag_k);
     }
     const bool owner = tid < kSdBM && row0 + tid < p.m;   // threads 0..127: one row each
+    // what a lane needs to find its two columns (2 lane, 2 lane + 1) in a long row's words: the mask word with their
+    // bits, the bits below them in it, and the field of the packed word that counts the nonzeros of the words before
+    const int own_word = lane >> 4, own_bit = (2 * lane) & 31;
+    const unsigned own_below = (1u << own_bit) - 1u;
+    const int own_shift = own_word == 2 ? 6 : own_word == 3 ? 13 : 0;
+    const unsigned own_field = own_word == 0 ? 0u : own_word == 1 ? 0x3fu : 0x7fu;
 
     wait_vmcnt<0>();        // the first tile's rhs rows, the first words and the lhs fragments have landed
 #pragma unroll
@@ -393,8 +404,13 @@ __global__ __launch_bounds__(kSdThreads, KS == 8 ? 1 : 2) void sddmm_mfma_kernel
         for (int u = 0; u < kSdShort; ++u)
           if (u < count) out[tp + u] = S[tid * kSdLd + ((pk >> (7 * u)) & 127)];
       }
-      // long runs: this wavefront takes rows 32 * wave .. + 31, four at a time; every lane reads the row's mask and
-      // cursor itself (the same LDS address for all lanes: a broadcast)
+      // long runs: this wavefront takes rows 32 * wave .. + 31, four at a time.  Lane i owns columns 2 i and 2 i + 1
+      // of a row: it reads the mask word that holds their bits and the row's packed word and cursor (LDS broadcasts);
+      // the nonzeros below column 2 i (those of the mask words before its own, from the packed word, plus the bits
+      // below in its own) give the position of its first score in the row's output.  With both columns present the
+      // two scores are neighbours there: one 4-byte store (at 2-byte alignment); with one, a 2-byte store.  A row
+      // that holds all its columns is one store instruction, and the CU's rate of store instructions is what bounds
+      // this step.
       unsigned todo = (unsigned)(long_rows[wave >> 1] >> ((wave & 1) * 32));
       todo = __builtin_amdgcn_readfirstlane(todo);
       while (todo) {
@@ -406,25 +422,22 @@ __global__ __launch_bounds__(kSdThreads, KS == 8 ? 1 : 2) void sddmm_mfma_kernel
           rr[u] = wave * 32 + (todo ? __builtin_ctz(todo) : 0);
           todo &= todo - 1;
         }
-        u32x4 mk[4];
-        int start[4];
-        u16 lo[4], hi[4];
+        unsigned word[4], both[4];
+        int start[4], packed[4];
 #pragma unroll
         for (int u = 0; u < 4; ++u) {
-          mk[u] = *reinterpret_cast<const u32x4*>(slot + 1024 + rr[u] * 16);
+          word[u] = *reinterpret_cast<const unsigned*>(slot + 1024 + rr[u] * 16 + own_word * 4);
           start[u] = reinterpret_cast<const int*>(slot)[rr[u]];
-          lo[u] = S[rr[u] * kSdLd + lane];
-          hi[u] = S[rr[u] * kSdLd + kWave + lane];
+          packed[u] = reinterpret_cast<const int*>(slot + 512)[rr[u]];
+          both[u] = *reinterpret_cast<const unsigned*>(S + rr[u] * kSdLd + 2 * lane);
         }
 #pragma unroll
         for (int u = 0; u < 4; ++u) {
           if (!on[u]) continue;
-          const int half = __popc(mk[u].x) + __popc(mk[u].y);
-          const int rank_lo = __builtin_amdgcn_mbcnt_hi(mk[u].y, __builtin_amdgcn_mbcnt_lo(mk[u].x, 0));
-          const int rank_hi = __builtin_amdgcn_mbcnt_hi(mk[u].w, __builtin_amdgcn_mbcnt_lo(mk[u].z, 0)) + half;
-          const unsigned word_lo = lane < 32 ? mk[u].x : mk[u].y, word_hi = lane < 32 ? mk[u].z : mk[u].w;
-          if ((word_lo >> (lane & 31)) & 1) out[min(start[u] + rank_lo, p.nnz - 1)] = lo[u];
-          if ((word_hi >> (lane & 31)) & 1) out[min(start[u] + rank_hi, p.nnz - 1)] = hi[u];
+          const int at = min(start[u] + (int)(((unsigned)packed[u] >> own_shift) & own_field) + __popc(word[u] & own_below), p.nnz - 1);
+          const unsigned have = (word[u] >> own_bit) & 3u;
+          if (have == 3u) *reinterpret_cast<u32_a2*>(out + min(at, max(p.nnz - 2, 0))) = both[u];   // (never clamped when the tables fit the arrays)
+          if (have == 1u || have == 2u) out[at] = (u16)(have == 1u ? both[u] : both[u] >> 16);
         }
       }
     }

@@ -167,6 +167,25 @@ def test_csr_softmax_long_short_and_empty_rows(oracle, dev, dtype):
         assert np.allclose(got[:, ro[r]:ro[r + 1]].sum(axis=1), 1.0, atol=1e-5 if dtype == torch.float32 else 2e-2), r
 
 
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("tail", [1, 2, 129, 385])
+def test_csr_softmax_pairs_of_16_bit_entries(oracle, dev, dtype, tail):
+    """16-bit entries are read and written two at a time: row lengths on both sides of every slot boundary of that
+    path (128, 384, 512 entries), rows that start at odd positions, and a last row of `tail` entries whose final
+    pair ends exactly at (or one entry before) the end of the tensor; one and three batch entries."""
+    lens = np.array([2, 3, 127, 128, 129, 0, 383, 384, 385, 511, 512, 5, tail])
+    ro = np.concatenate([[0], np.cumsum(lens)]).astype(np.int32)
+    rng = np.random.default_rng(tail)
+    ri = torch.from_numpy(W.swizzle_from_offsets(ro)).to(dev)
+    for batch in (1, 3):
+        vals = rng.standard_normal((batch, int(ro[-1]))).astype(np.float32) * 4
+        v = torch.from_numpy(vals).to(dev).to(dtype)
+        ops.csr_softmax_(v, ri, torch.from_numpy(ro).to(dev), 0.5)
+        want = oracle.csr_softmax(rounded(vals, dtype).astype(np.float64) * 0.5, ro)
+        got = v.float().cpu().numpy()
+        assert np.abs(got - want).max() <= (2e-3 if dtype == torch.float16 else 8e-3), batch
+
+
 def test_operator_argument_checks(dev):
     a, _, lhs_np, rhs_np = W.config1()
     ri, _, ro, ci = to_dev(a, dev)

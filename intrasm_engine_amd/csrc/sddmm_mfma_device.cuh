@@ -249,7 +249,7 @@ __global__ __launch_bounds__(kSdThreads, KS == 8 ? 1 : 2) void sddmm_mfma_kernel
   constexpr int STAGE = kSdBN * RB;
   static_assert(KS == 2 || KS == 4 || KS == 8, "k = 32, 64 or 128");
   typedef unsigned short u16;
-  typedef unsigned u32_a2 __attribute__((aligned(2)));   // two neighbouring scores stored at once
+  typedef u32x4 u128_a2 __attribute__((aligned(2)));   // eight neighbouring scores stored at once
   typedef __attribute__((address_space(3))) unsigned char lds_u8;
   extern __shared__ __align__(16) unsigned char smem[];
   u16* S = reinterpret_cast<u16*>(smem);                                      // [128][kSdLd]; before the loop: column sums
@@ -330,9 +330,11 @@ __global__ __launch_bounds__(kSdThreads, KS == 8 ? 1 : 2) void sddmm_mfma_kernel
       for (int ks = 0; ks < KS; ++ks) fl[i][ks] = *reinterpret_cast<const u32x4*>(lhs + (size_t)row * p.k + ks * 16 + frag_k);
     }
     const bool owner = tid < kSdBM && row0 + tid < p.m;   // threads 0..127: one row each
-    // what a lane needs to find its two columns (2 lane, 2 lane + 1) in a long row's words: the mask word with their
-    // bits, the bits below them in it, and the field of the packed word that counts the nonzeros of the words before
-    const int own_word = lane >> 4, own_bit = (2 * lane) & 31;
+    // what a lane needs to find its 8 columns in a long row's words (sampling below): which of the step's four rows,
+    // which group of 8 columns, the mask word with their bits, the bits below them in it, and the field of the packed
+    // word that counts the nonzeros of the mask words before
+    const int own_row = lane >> 4, own_col8 = lane & 15;
+    const int own_word = own_col8 >> 2, own_bit = (own_col8 & 3) * 8;
     const unsigned own_below = (1u << own_bit) - 1u;
     const int own_shift = own_word == 2 ? 6 : own_word == 3 ? 13 : 0;
     const unsigned own_field = own_word == 0 ? 0u : own_word == 1 ? 0x3fu : 0x7fu;
@@ -404,40 +406,52 @@ __global__ __launch_bounds__(kSdThreads, KS == 8 ? 1 : 2) void sddmm_mfma_kernel
         for (int u = 0; u < kSdShort; ++u)
           if (u < count) out[tp + u] = S[tid * kSdLd + ((pk >> (7 * u)) & 127)];
       }
-      // long runs: this wavefront takes rows 32 * wave .. + 31, four at a time.  Lane i owns columns 2 i and 2 i + 1
-      // of a row: it reads the mask word that holds their bits and the row's packed word and cursor (LDS broadcasts);
-      // the nonzeros below column 2 i (those of the mask words before its own, from the packed word, plus the bits
-      // below in its own) give the position of its first score in the row's output.  With both columns present the
-      // two scores are neighbours there: one 4-byte store (at 2-byte alignment); with one, a 2-byte store.  A row
-      // that holds all its columns is one store instruction, and the CU's rate of store instructions is what bounds
-      // this step.
+      // long runs: this wavefront takes rows 32 * wave .. + 31, four consecutive rows per step, 16 lanes per row: a
+      // lane owns 8 neighbouring columns.  It reads the mask word that holds their bits, the row's packed word and
+      // cursor and its 8 scores from LDS; the nonzeros below its first column (those of the mask words before its
+      // own, from the packed word, plus the bits below in its own) give the position of its first score in the row's
+      // output.  All 8 present (the inside of a band): one 16-byte store at 2-byte alignment, four rows per
+      // instruction.  Else (the edge of a run): a 2-byte store per score present.  What this step costs is
+      // instructions and LDS round trips per row, which is why it works on as many rows per instruction as it can.
       unsigned todo = (unsigned)(long_rows[wave >> 1] >> ((wave & 1) * 32));
       todo = __builtin_amdgcn_readfirstlane(todo);
-      while (todo) {
-        int rr[4];
-        bool on[4];
+      struct Words {
+        unsigned word, packed;
+        int start;
+        u32x4 sc;
+      };
+      auto read_words = [&](int g) {   // (every group is read, also one without long rows: no branch around LDS reads)
+        const int r = wave * 32 + 4 * g + own_row;
+        Words w;
+        w.word = *reinterpret_cast<const unsigned*>(slot + 1024 + r * 16 + own_word * 4);
+        w.start = reinterpret_cast<const int*>(slot)[r];
+        w.packed = reinterpret_cast<const unsigned*>(slot + 512)[r];
+        w.sc = *reinterpret_cast<const u32x4*>(S + r * kSdLd + 8 * own_col8);
+        return w;
+      };
+      if (todo) {
+        Words next = read_words(0);
 #pragma unroll
-        for (int u = 0; u < 4; ++u) {
-          on[u] = todo != 0;
-          rr[u] = wave * 32 + (todo ? __builtin_ctz(todo) : 0);
-          todo &= todo - 1;
-        }
-        unsigned word[4], both[4];
-        int start[4], packed[4];
+        for (int g = 0; g < 8; ++g) {
+          const Words cur = next;
+          if (g + 1 < 8) next = read_words(g + 1);   // in flight while this group is stored
+          const unsigned four = (todo >> (4 * g)) & 0xfu;
+          if (!four) continue;   // (uniform)
+          const unsigned have = ((four >> own_row) & 1u) ? (cur.word >> own_bit) & 0xffu : 0u;
+          const int at = cur.start + (int)((cur.packed >> own_shift) & own_field) + __popc(cur.word & own_below);
+          if (have == 0xffu) *reinterpret_cast<u128_a2*>(out + min(at, max(p.nnz - 8, 0))) = cur.sc;   // (never clamped when the tables fit the arrays)
+          const unsigned some = have == 0xffu ? 0u : have;
+          if (__ballot(some != 0)) {
+            const unsigned w[4] = {cur.sc.x, cur.sc.y, cur.sc.z, cur.sc.w};
+            int k = min(at, p.nnz - 1);
 #pragma unroll
-        for (int u = 0; u < 4; ++u) {
-          word[u] = *reinterpret_cast<const unsigned*>(slot + 1024 + rr[u] * 16 + own_word * 4);
-          start[u] = reinterpret_cast<const int*>(slot)[rr[u]];
-          packed[u] = reinterpret_cast<const int*>(slot + 512)[rr[u]];
-          both[u] = *reinterpret_cast<const unsigned*>(S + rr[u] * kSdLd + 2 * lane);
-        }
-#pragma unroll
-        for (int u = 0; u < 4; ++u) {
-          if (!on[u]) continue;
-          const int at = min(start[u] + (int)(((unsigned)packed[u] >> own_shift) & own_field) + __popc(word[u] & own_below), p.nnz - 1);
-          const unsigned have = (word[u] >> own_bit) & 3u;
-          if (have == 3u) *reinterpret_cast<u32_a2*>(out + min(at, max(p.nnz - 2, 0))) = both[u];   // (never clamped when the tables fit the arrays)
-          if (have == 1u || have == 2u) out[at] = (u16)(have == 1u ? both[u] : both[u] >> 16);
+            for (int b = 0; b < 8; ++b) {
+              if ((some >> b) & 1u) {
+                out[min(k, p.nnz - 1)] = (u16)((b & 1) ? w[b >> 1] >> 16 : w[b >> 1]);
+                ++k;
+              }
+            }
+          }
         }
       }
     }

@@ -712,7 +712,7 @@ int spmm_dispatch(int dtype, int itype, int flags, int m, int k, int n, int nonz
   // beyond the 256 MB last-level cache an output can only stream; the hint is worth 15-25 % of the write rate
   p.stream_out = (double)m * n * batch * (dtype == IEX_F32 ? 4 : 2) >= 128e6;
   hipStream_t s = static_cast<hipStream_t>(stream);
-  if (ch.variant == 10 && nonzeros < 4) ch.variant = 1;   // (its loads of four values at a time need four to exist)
+  if (ch.variant == 10 && nonzeros < 8) ch.variant = 1;   // (its loads of eight values at a time need eight to exist)
   const int blocks_ready = ((flags & IEX_SPMM_TABLES_READY) ? 1 : 0) | ((flags & IEX_SPMM_LISTS_READY) ? 2 : 0);
   if (ch.variant == 0 && ch.ws && aligned(ch.ws, 16) && spmm_blocks_fits(dtype, itype, p) && spmm_blocks_wins(p, batch) &&
       ch.ws_bytes >= spmm_blocks_bytes(p))
@@ -751,7 +751,7 @@ static size_t workspace_plan(int dtype, int itype, int flags, int m, int k, int 
   if (variant != 0 && variant != 7 && variant != 10) return 0;
   SpmmParams p{m, k, n, nonzeros, nullptr, nullptr, nullptr, nullptr, some_aligned, nullptr, some_aligned,
                (flags & IEX_SPMM_PER_BATCH_VALUES) != 0, (flags & IEX_SPMM_ACCUMULATE) != 0, (flags & IEX_SPMM_RELU) != 0};
-  if (variant != 7 && nonzeros >= 4 && spmm_blocks_fits(dtype, itype, p) && (variant == 10 || spmm_blocks_wins(p, batch))) {
+  if (variant != 7 && nonzeros >= 8 && spmm_blocks_fits(dtype, itype, p) && (variant == 10 || spmm_blocks_wins(p, batch))) {
     *kind = 10;
     return spmm_blocks_bytes(p);
   }

@@ -25,7 +25,7 @@ bool spmm_blocks_fits(int dtype, int itype, const SpmmParams& p) {
 // IEX_SPMM_FORCE_VARIANT(1) keeps the row kernel.
 bool spmm_blocks_wins(const SpmmParams& p, int batch) {
   const double density = (double)p.nnz / ((double)p.m * p.k);
-  return p.per_batch_values && p.nnz >= 4 && density >= 0.03 && (double)batch * p.m * p.k >= 32.0 * 1024 * 1024;
+  return p.per_batch_values && p.nnz >= 8 && density >= 0.03 && (double)batch * p.m * p.k >= 32.0 * 1024 * 1024;
 }
 
 size_t spmm_blocks_bytes(const SpmmParams& p) { return sb_words(p.m, ceil_div(p.k, kSdBN), p.nnz) * sizeof(int); }

@@ -12,13 +12,15 @@
 // nonzeros or more ("dense"), and per row its nonzeros outside those tiles, compacted.
 // A workgroup (4 wavefronts) owns 128 consecutive rows of one batch entry, a wavefront 32 of them:
 //   * dense tiles: the block of A is laid out as a dense 32 x 128 tile per wavefront in LDS -- zeros, then the
-//     values: up to 4 per (row, tile) by the row's own lane from the packed word, more by the whole wavefront from
-//     the row's 128-bit mask (lane i owns columns i and 64 + i; a population count of the bits below gives the
-//     position of each in the row's values, so the loads of a row are contiguous and no column index is read; all
-//     loads of a tile are issued before the first is used) -- and multiplied on the matrix cores with the 128 rows
-//     of the dense operand that the tile names: they go through registers into LDS once per workgroup,
-//     double-buffered, 16-byte chunks permuted so that the transposing operand reads (ds_read_tr16_b64) are
-//     conflict-free.  Operands swapped (out^T = dense^T * A^T) so that a lane ends up with 4 adjacent output
+//     values: up to 4 per (row, tile) by the row's own lane from the packed word, more by the whole wavefront, four
+//     rows per step and 16 lanes per row, from the row's 128-bit mask: a lane owns 8 neighbouring columns, a
+//     population count of the mask bits below them gives the position of its first value in the row's values, one
+//     16-byte load from there holds all it owns (no column index is read), and they go to the tile as loaded when
+//     all 8 columns are present, shifted and masked when the present ones are neighbours (the edge of a band), one
+//     by one otherwise; all loads of a tile are issued before the first is used -- and multiplied on the matrix
+//     cores with the 128 rows of the dense operand that the tile names: they go through registers into LDS once per
+//     workgroup, double-buffered, 16-byte chunks permuted so that the transposing operand reads (ds_read_tr16_b64)
+//     are conflict-free.  Operands swapped (out^T = dense^T * A^T) so that a lane ends up with 4 adjacent output
 //     columns of one row.
 //   * everything else: 8 lanes per row walk the row's list, two rows at a time, 8 nonzeros of each per step: 16
 //     bytes of the dense operand's row per lane and nonzero, fp32 FMAs, no reduction across lanes.
@@ -80,7 +82,7 @@ struct SpmmBlocksParams {
   const unsigned short* dense_list;
 };
 
-constexpr int spmm_blocks_lds_bytes() { return 4 * kSbTileBytes + 2 * kSbStage + 32 + 4 * 32 * 32; }
+constexpr int spmm_blocks_lds_bytes() { return 4 * kSbTileBytes + 2 * kSbStage + 4 * 32 * 32; }
 
 // The dense tiles of every block of 128 rows (one workgroup each): dense_list[block][0] = their number, then the tiles.
 static __global__ __launch_bounds__(kSdThreads) void sb_dense_list_kernel(int m, int tiles_k, int dense_min, const int* __restrict__ tile_ptr,
@@ -147,17 +149,16 @@ template <bool BF16>
 __global__ __launch_bounds__(kSdThreads, 2) void spmm_blocks_kernel(SpmmBlocksParams p) {
   typedef unsigned short u16;
   typedef __attribute__((address_space(3))) s16x4 lds_s16x4;
-  typedef unsigned u32_a2 __attribute__((aligned(2)));             // loads of two and four values at the alignment of one
+  typedef u32x4 u128_a2 __attribute__((aligned(2)));               // loads of eight and four values at the alignment of one
   typedef unsigned long long u64_a2 __attribute__((aligned(2)));
   constexpr int NT = kSbN / 32;
   extern __shared__ __align__(16) unsigned char smem[];
   unsigned char* sV = smem + 4 * kSbTileBytes;                               // [2][128][128 bytes]
-  unsigned* lut = reinterpret_cast<unsigned*>(sV + 2 * kSbStage);           // [8]
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-  unsigned* rec = lut + 8 + wave * (32 * 8);                                 // [32][8]: what a wavefront's rows know of the current tile
+  unsigned* rec = reinterpret_cast<unsigned*>(sV + 2 * kSbStage) + wave * (32 * 8);                                 // [32][8]: what a wavefront's rows know of the current tile
   // Workgroups go to the 8 XCDs round-robin by their linear id; renumbered so that an XCD gets all row blocks of a
   // batch entry (and then of the next): the dense operand of that entry stays in that XCD's L2.
   const int row_blocks = gridDim.x, total = row_blocks * gridDim.y;
@@ -241,16 +242,11 @@ __global__ __launch_bounds__(kSdThreads, 2) void spmm_blocks_kernel(SpmmBlocksPa
           v_off[t] = tr_k * (kSbN * 2) + chunk * 16 + (lane & 1) * 8;
         }
         const int p_off = (lane & 31) * (kSdLd * 2) + fkh * 16;
-        // the mask word and the bits in it of the two columns that this lane owns in a long row
-        const int own_word = lane >> 4, own_bit = (2 * lane) & 31;
+        // what a lane needs to find the 8 columns that it owns in a long row: which of a step's four rows, which group
+        // of 8 columns, the mask word that holds their bits and the bits below them in it
+        const int own_row = lane >> 4, own_col8 = lane & 15;
+        const int own_word = own_col8 >> 2, own_bit = (own_col8 & 3) * 8;
         const unsigned own_below = (1u << own_bit) - 1u;
-
-        // byte selectors for v_perm(0, loaded, selector), by (column 2 i present) + 2 (column 2 i + 1 present) + 4 (the
-        // load was moved back by one value: the wanted value is in the upper half)
-        if (tid < 8) {
-          const unsigned none = 0x0c0c0c0cu;
-          lut[tid] = tid == 1 ? 0x0c0c0100u : tid == 2 ? 0x01000c0cu : tid == 3 || tid == 7 ? 0x03020100u : tid == 5 ? 0x0c0c0302u : tid == 6 ? 0x03020c0cu : none;
-        }
         u32x4 rv[4];
         int tp, bf;
         u32x4 mk;
@@ -281,12 +277,14 @@ __global__ __launch_bounds__(kSdThreads, 2) void spmm_blocks_kernel(SpmmBlocksPa
           const int s_at = min(max(tp, 0), last - 3);
           const int s_shift = min(max(tp, 0) - s_at, 3) * 16;   // (more than 3 only for rows without values here)
           const unsigned long long sv = *reinterpret_cast<const u64_a2*>(vals + s_at);
-          // ... longer runs by the wavefront: lane i owns columns 2 i and 2 i + 1 of the row.  The number of the row's
-          // nonzeros below column 2 i gives the position of the pair's first value among the row's values in the
-          // tile; its 4 bytes hold both values when both columns are present.  Lanes 0..31 publish what they know of
-          // their rows in LDS (mask, nonzeros below each mask word, cursor), every lane picks from there what concerns
-          // its two columns; how the loaded bytes map to the pair (byte selectors for v_perm) comes from a table of 8.
-          // All loads first.
+          // ... longer runs by the wavefront, four consecutive rows per step, 16 lanes per row: a lane owns 8
+          // neighbouring columns.  Lanes 0..31 publish what they know of their rows in LDS (mask, nonzeros below each
+          // mask word, cursor); every lane picks from there what concerns its 8 columns: the number of the row's
+          // nonzeros below its first column is the position of its first value among the row's values in the tile,
+          // and the 16 bytes from there (one load at 2-byte alignment, moved back where it would pass the end of the
+          // values) hold all the values it owns.  All 8 columns present (the inside of a band): the 16 bytes go to the
+          // tile as they are.  Else they are spread over the columns present: by a shift and a mask when those are
+          // neighbours (the edge of a run), one by one otherwise.  All loads of the tile first.
           const unsigned longs = (unsigned)__ballot(count == 7);
           if (lane < 32) {
             const unsigned cx = __popc(mk.x), cy = cx + __popc(mk.y), cz = cy + __popc(mk.z);
@@ -295,18 +293,23 @@ __global__ __launch_bounds__(kSdThreads, 2) void spmm_blocks_kernel(SpmmBlocksPa
           }
           __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
           __builtin_amdgcn_wave_barrier();
-          unsigned pair[32], sel[32];
+          u32x4 got[8];
+          unsigned have[8], back[8];
 #pragma unroll
-          for (int r = 0; r < 32; ++r) {
-            pair[r] = 0;
-            sel[r] = 0;
-            if ((longs >> r) & 1) {   // (uniform)
+          for (int g = 0; g < 8; ++g) {
+            got[g] = u32x4{0u, 0u, 0u, 0u};
+            have[g] = 0;
+            back[g] = 0;
+            const unsigned four = (longs >> (4 * g)) & 0xfu;
+            if (four) {   // (uniform)
+              const int r = 4 * g + own_row;
               const unsigned word = rec[r * 8 + own_word];
               const u32x2 pt = *reinterpret_cast<const u32x2*>(rec + r * 8 + 4);
               const int at = (int)(pt.y + ((pt.x >> (own_word * 8)) & 0xffu)) + __popc(word & own_below);
-              const int at_c = min(at, last - 1);
-              sel[r] = lut[((word >> own_bit) & 3u) | (at > at_c ? 4u : 0u)];   // (lanes past the row's last value own no column: entry 0 or 4, all zeros)
-              pair[r] = *reinterpret_cast<const u32_a2*>(vals + at_c);
+              const int at_c = max(min(at, last - 7), 0);
+              have[g] = ((four >> own_row) & 1u) ? (word >> own_bit) & 0xffu : 0u;
+              back[g] = (unsigned)min(at - at_c, 7);   // (values that the load was moved back by: only at the end of the values)
+              got[g] = *reinterpret_cast<const u128_a2*>(vals + at_c);
             }
           }
           if (count >= 1 && count <= kSdShort) {
@@ -315,9 +318,42 @@ __global__ __launch_bounds__(kSdThreads, 2) void spmm_blocks_kernel(SpmmBlocksPa
               if (u < count) P16[lane * kSdLd + ((bf >> (7 * u)) & 127)] = (u16)(sv >> ((s_shift + 16 * u) & 63));
           }
 #pragma unroll
-          for (int r = 0; r < 32; ++r) {
-            if ((longs >> r) & 1)
-              *reinterpret_cast<unsigned*>(P16 + r * kSdLd + 2 * lane) = __builtin_amdgcn_perm(0u, pair[r], sel[r]);
+          for (int g = 0; g < 8; ++g) {
+            const unsigned four = (longs >> (4 * g)) & 0xfu;
+            if (!four) continue;   // (uniform)
+            u32x4 put = got[g];
+            const unsigned h = have[g];
+            const bool plain = h == 0xffu;               // all 8 present: as loaded (never moved back: 8 values exist from `at`)
+            if (__ballot(h != 0 && !plain)) {
+              typedef unsigned long long u64;
+              u64 lo = (u64)got[g].x | ((u64)got[g].y << 32), hi = (u64)got[g].z | ((u64)got[g].w << 32);
+              const unsigned low_bit = h & (0u - h);
+              const bool run = ((h + low_bit) & h) == 0 && back[g] == 0;   // the columns present are neighbours
+              if (__ballot(h != 0 && !plain && !run)) {
+                // any pattern: value k of the 16 bytes (counted from `back`) goes to the k-th column present
+                u64 rlo = 0, rhi = 0;
+                unsigned k = back[g];
+#pragma unroll
+                for (int c = 0; c < 8; ++c) {
+                  const u64 src = k < 4 ? lo : hi;
+                  const u64 v = ((h >> c) & 1u) ? (src >> ((k & 3) * 16)) & 0xffffull : 0ull;
+                  if (c < 4) rlo |= v << (c * 16); else rhi |= v << ((c - 4) * 16);
+                  k += (h >> c) & 1u;
+                }
+                if (!plain && !run) lo = rlo, hi = rhi;
+              }
+              if (run && !plain) {
+                // n neighbours from column s on: keep the first n values, move them up by s columns
+                const int n = __popc(h), sh = (h ? __builtin_ctz(h) : 0) * 16;
+                const u64 keep_lo = n >= 4 ? ~0ull : (1ull << (n * 16)) - 1ull;
+                const u64 keep_hi = n <= 4 ? 0ull : n >= 8 ? ~0ull : (1ull << ((n - 4) * 16)) - 1ull;
+                const u64 a = lo & keep_lo, b = hi & keep_hi;
+                lo = sh >= 64 ? 0ull : a << (sh & 63);
+                hi = sh >= 64 ? a << ((sh - 64) & 63) : (b << (sh & 63)) | (sh ? a >> ((64 - sh) & 63) : 0ull);
+              }
+              if (!plain) put = u32x4{(unsigned)lo, (unsigned)(lo >> 32), (unsigned)hi, (unsigned)(hi >> 32)};
+            }
+            if (h) *reinterpret_cast<u32x4*>(Pw + (4 * g + own_row) * (kSdLd * 2) + own_col8 * 16) = put;
           }
           __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
           __builtin_amdgcn_wave_barrier();

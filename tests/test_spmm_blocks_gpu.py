@@ -55,6 +55,29 @@ def test_ragged_shapes_forced(oracle, dev, dtype, m, k, blocks):
     assert torch.equal(out, _run(dev, csr, values, dense, dtype, force_variant=10, force_wpr=blocks))   # same call, same bits
 
 
+@pytest.mark.parametrize("last_row", [[3, 4, 5, 6, 7, 8], [1, 2, 9, 17, 18, 40, 41], [120, 121, 122, 123, 124, 125, 126, 127],
+                                      [0, 1, 2, 3, 4, 5, 6, 7, 8]])
+def test_rows_at_the_end_of_the_values(oracle, dev, last_row):
+    """The kernel reads a long row's values 16 bytes at a time; the reads of the last rows are moved back so that none
+    passes the end of the values: last rows of neighbouring columns, of scattered columns, of exactly 8 and of 9, with
+    a few rows before them, every block on the matrix cores, two batch entries."""
+    rng = np.random.default_rng(len(last_row))
+    m, k = 40, 128
+    mask = np.zeros((m, k), bool)
+    for r in range(m - 3):
+        mask[r, rng.choice(k, int(rng.integers(0, 12)), replace=False)] = True
+    mask[m - 3, 5:11] = True
+    mask[m - 2, [0, 64, 65, 66, 100, 127]] = True
+    mask[m - 1, last_row] = True
+    ro, ci, _ = W.csr_from_mask(mask)
+    csr = W.CSR(m, k, np.ones(ci.shape[0], np.float32), W.swizzle_from_offsets(ro), ro, ci)
+    values = rng.integers(-4, 5, (2, csr.nnz)).astype(np.float32)
+    dense = rng.integers(-4, 5, (2, k, 64)).astype(np.float32)
+    out = _run(dev, csr, values, dense, torch.float16, force_variant=10, force_wpr=1)
+    want, _ = _want(oracle, csr, values, dense, torch.float16)
+    assert np.array_equal(out.float().cpu().numpy(), want)          # small integers: exact
+
+
 def test_integer_operands_agree_with_the_row_kernel_exactly(dev):
     rng = np.random.default_rng(8)
     m, k = 260, 390

@@ -515,16 +515,21 @@ __global__ __launch_bounds__(kSdThreads, KS == 8 ? 1 : 2) void sddmm_mfma_kernel
       if (T > 0) {
         __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
         __builtin_amdgcn_wave_barrier();
-        unsigned wa, wb;
-        u32x4 rva[LPN], rvb[LPN];
+        // three steps' loads in flight (a step is fetched only while its entries are still entries: results replace them)
+        unsigned wa, wb, wc;
+        u32x4 rva[LPN], rvb[LPN], rvc[LPN];
         fetch(0, wa, rva);
-        for (int base = 0; base < T; base += 2 * kWave) {
-          const bool second = base + kWave < T;
-          if (second) fetch(base + kWave, wb, rvb);
+        if (kWave < T) fetch(kWave, wb, rvb);
+        for (int base = 0; base < T; base += 3 * kWave) {
+          if (base + 2 * kWave < T) fetch(base + 2 * kWave, wc, rvc);
           finish(base, wa, rva);
-          if (second) {
-            if (base + 2 * kWave < T) fetch(base + 2 * kWave, wa, rva);
+          if (base + kWave < T) {
+            if (base + 3 * kWave < T) fetch(base + 3 * kWave, wa, rva);
             finish(base + kWave, wb, rvb);
+          }
+          if (base + 2 * kWave < T) {
+            if (base + 4 * kWave < T) fetch(base + 4 * kWave, wb, rvb);
+            finish(base + 2 * kWave, wc, rvc);
           }
         }
         __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");

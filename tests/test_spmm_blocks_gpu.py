@@ -78,6 +78,35 @@ def test_rows_at_the_end_of_the_values(oracle, dev, last_row):
     assert np.array_equal(out.float().cpu().numpy(), want)          # small integers: exact
 
 
+@pytest.mark.parametrize("k", [9000, 20100, 65536])
+@pytest.mark.parametrize("blocks", [0, 2])
+def test_many_column_blocks(oracle, dev, k, blocks):
+    """More than 64 (and more than 128) blocks of 128 columns per row: the setup kernels and the kernel's walk over
+    the dense blocks all work on lists of up to 512 blocks.  A band that wanders through the columns plus scattered
+    entries, 260 rows, two batch entries; k = 65536 is the largest the kernel takes (one more column is refused)."""
+    rng = np.random.default_rng(k)
+    m = 260
+    idx = np.arange(m)
+    centre = (idx * (k - 200) // m) + 100
+    cols = [np.unique(np.concatenate([np.arange(c - 40, c + 40), rng.integers(0, k, 12)])) for c in centre]
+    cols[7] = np.array([], dtype=np.int64)
+    cols[100] = np.arange(0, k, 97)                       # a long row that touches every block
+    lens = np.array([len(c) for c in cols])
+    ro = np.zeros(m + 1, dtype=np.int32)
+    np.cumsum(lens, out=ro[1:])
+    ci = np.concatenate(cols).astype(np.int32)
+    csr = W.CSR(m, k, np.ones(ci.shape[0], np.float32), W.swizzle_from_offsets(ro), ro, ci)
+    values = rng.standard_normal((2, csr.nnz)).astype(np.float32)
+    dense = rng.standard_normal((2, k, 64)).astype(np.float32)
+    out = _run(dev, csr, values, dense, torch.float16, force_variant=10, force_wpr=blocks)
+    want, scale = _want(oracle, csr, values, dense, torch.float16)
+    assert_close(out.float().cpu().numpy(), want, scale, RTOL[torch.float16], f"k={k} blocks={blocks}", atol=FP16_SUBNORMAL_HALF_STEP)
+    if k == 65536 and blocks == 0:
+        with pytest.raises(RuntimeError, match="dense-blocks kernel needs fp16"):
+            wide = W.CSR(m, k + 1, csr.values, csr.row_indices, csr.row_offsets, csr.column_indices)
+            _run(dev, wide, values, rng.standard_normal((2, k + 1, 64)).astype(np.float32), torch.float16, force_variant=10)
+
+
 def test_integer_operands_agree_with_the_row_kernel_exactly(dev):
     rng = np.random.default_rng(8)
     m, k = 260, 390

@@ -85,9 +85,11 @@ int iex_copy_bytes(void* dst, const void* src, size_t nbytes, void* stream);
  * for more than one slice, iex_spmm_ws with the workspace iex_spmm_workspace_bytes reports (bits 20..23: slices,
  * 0 = choose; bits 24..27 = 2: workgroups of 16 wavefronts and 128 rows instead of 8 and 64); fails on other
  * shapes, 10 = sparse operands with structure (attention probabilities: bands, blocks, windows) times a dense
- * operand of 64 columns, on request only: per 128 rows, the dense 128 x 128 blocks of A are laid out in LDS and
+ * operand of 64, 128, ... columns (served 64 at a time): per 128 rows, the dense 128 x 128 blocks of A are laid out in LDS and
  * multiplied on the matrix cores, the nonzeros elsewhere are gathered row by row (fp16 / bf16, int32 indices,
- * n = 64, k <= 65536, plain store without bias or ReLU, values shared or per batch entry; iex_spmm_ws only, with
+ * n a multiple of 64 up to 1024, k <= 65536, plain store without bias or ReLU, values shared or per batch entry;
+ * chosen by itself for values per batch entry on patterns at least 3 % dense with batch * m * k >= 2^25, on request
+ * elsewhere; iex_spmm_ws only, with
  * the workspace iex_spmm_workspace_bytes reports: the tables of SDDMM variant 3 for the pattern, which a small
  * kernel writes first, and behind them lists that two more small kernels derive from the tables -- see
  * IEX_SPMM_TABLES_READY / IEX_SPMM_LISTS_READY; bits 8..15 set the number of nonzeros from which a block counts

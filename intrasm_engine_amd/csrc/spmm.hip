@@ -719,7 +719,7 @@ int spmm_dispatch(int dtype, int itype, int flags, int m, int k, int n, int nonz
     return launch_spmm_blocks(dtype, p, batch, ch.ws, 0, blocks_ready, s);
   if (ch.variant == 10) {
     IEX_REQUIRE(spmm_blocks_fits(dtype, itype, p), IEX_ERR_UNSUPPORTED,
-                "spmm: the dense-blocks kernel needs fp16 / bf16, int32 indices, n = 64, plain store without bias or ReLU, k <= 65536 and 16-byte aligned dense operands");
+                "spmm: the dense-blocks kernel needs fp16 / bf16, int32 indices, n a multiple of 64 up to 1024, plain store without bias or ReLU, k <= 65536 and 16-byte aligned dense operands");
     IEX_REQUIRE(ch.ws && aligned(ch.ws, 16) && ch.ws_bytes >= spmm_blocks_bytes(p), IEX_ERR_BAD_ARGUMENT,
                 "spmm: the dense-blocks kernel needs a 16-byte aligned workspace of %zu bytes (iex_spmm_ws)", spmm_blocks_bytes(p));
     return launch_spmm_blocks(dtype, p, batch, ch.ws, (flags >> 8) & 0xff, blocks_ready, s);

@@ -5,9 +5,9 @@
 
 namespace iex {
 
-// fp16 / bf16, int32 indices, 64 output columns, plain store without bias or ReLU.
+// fp16 / bf16, int32 indices, output columns a multiple of 64 (served in slices of 64), plain store without bias or ReLU.
 bool spmm_blocks_fits(int dtype, int itype, const SpmmParams& p) {
-  return (dtype == IEX_F16 || dtype == IEX_BF16) && itype == IEX_I32 && p.n == kSbN && !p.accumulate && !p.relu && !p.bias &&
+  return (dtype == IEX_F16 || dtype == IEX_BF16) && itype == IEX_I32 && p.n >= kSbN && p.n % kSbN == 0 && p.n <= 1024 && !p.accumulate && !p.relu && !p.bias &&
          aligned(p.dense, 16) && aligned(p.out, 16) && ceil_div(p.k, kSdBN) <= kSdMaxTiles &&
          (long long)(ceil_div(p.k, kSdBN) + 1) * p.m < (1ll << 28);
 }
@@ -42,7 +42,7 @@ static int launch_blocks(const SpmmBlocksParams& q, int batch, hipStream_t strea
     raised = true;
   }
   note_kernel("spmm_blocks_kernel<%s>", BF16 ? "true" : "false");
-  hipLaunchKernelGGL(kernel, dim3(ceil_div(q.m, kSdBM), batch), dim3(kSdThreads), lds, stream, q);
+  hipLaunchKernelGGL(kernel, dim3(ceil_div(q.m, kSdBM), batch * (q.n / kSbN)), dim3(kSdThreads), lds, stream, q);
   return check_hip(hipGetLastError(), "spmm (dense blocks) launch");
 }
 
@@ -51,6 +51,7 @@ static int launch_blocks(const SpmmBlocksParams& q, int batch, hipStream_t strea
 // pattern (this kernel's or the SDDMM's for masks with structure: same tables) left the tables in the workspace,
 // bit 1 = that an earlier call of this kernel with the same dense_code left its lists there too.
 int launch_spmm_blocks(int dtype, const SpmmParams& p, int batch, void* ws, int dense_code, int ready, hipStream_t stream) {
+  IEX_REQUIRE((long long)batch * (p.n / kSbN) <= 65535, IEX_ERR_TOO_LARGE, "spmm: batch %d x %d column slices exceed 65535", batch, p.n / kSbN);
   const int tiles_k = ceil_div(p.k, kSdBN);
   const SdTables t = sd_tables(ws, p.m, tiles_k);
   const SbLists l = sb_lists(ws, p.m, tiles_k, p.nnz);
@@ -67,7 +68,7 @@ int launch_spmm_blocks(int dtype, const SpmmParams& p, int batch, void* ws, int 
     hipLaunchKernelGGL(sb_thin_list_kernel, dim3(ceil_div(p.m, 4)), dim3(256), 0, stream, p.m, tiles_k, p.row_offsets, cols, l.dense_list, l.thin_cnt, l.thin_ent);
     if (int rc = check_hip(hipGetLastError(), "spmm (list of the other nonzeros) launch")) return rc;
   }
-  SpmmBlocksParams q{p.m, p.k, p.nnz, p.row_offsets, p.values, p.per_batch_values ? (size_t)p.nnz : 0, p.dense, p.out,
+  SpmmBlocksParams q{p.m, p.k, p.nnz, p.row_offsets, p.values, p.per_batch_values ? (size_t)p.nnz : 0, p.dense, p.out, p.n,
                      t.mask, t.tile_ptr, t.brief, tiles_k, l.zeros, l.thin_ent, l.thin_cnt, l.dense_list};
   return dtype == IEX_BF16 ? launch_blocks<true>(q, batch, stream) : launch_blocks<false>(q, batch, stream);
 }

@@ -1,4 +1,5 @@
-// CSR SpMM for attention-like sparse operands (gfx950, fp16 / bf16, 64 output columns): out = A * dense with A a
+// CSR SpMM for attention-like sparse operands (gfx950, fp16 / bf16, 64 output columns per workgroup, wider outputs in
+// slices of 64): out = A * dense with A a
 // mask with structure (a dense band plus scattered entries) whose values differ per batch entry -- the second
 // product of sparse attention, probabilities times V.
 //
@@ -34,7 +35,7 @@
 
 namespace iex {
 
-constexpr int kSbN = 64;                       // output columns
+constexpr int kSbN = 64;                       // output columns per workgroup (a wider output is served in slices of 64)
 constexpr int kSbTileBytes = 32 * kSdLd * 2;   // a wavefront's 32 x 128 tile of A (rows padded to 272 bytes); later its 32 x 64 fp32 sums
 constexpr int kSbStage = kSdBN * kSbN * 2;     // 128 rows of the dense operand
 constexpr int kSbRows = 2;                     // rows whose nonzeros outside dense tiles a lane group gathers side by side (1, 2 or 4)
@@ -70,8 +71,9 @@ struct SpmmBlocksParams {
   const int* row_offsets;
   const void* values;
   size_t values_stride;   // elements between batch entries (0: shared)
-  const void* dense;      // (batch, k, 64)
-  void* out;              // (batch, m, 64)
+  const void* dense;      // (batch, k, n)
+  void* out;              // (batch, m, n)
+  int n;                  // a multiple of 64: gridDim.y = batch * n / 64, a workgroup serves 64 columns
   const u32x4* mask;      // [tiles_k][m]
   const int* tile_ptr;    // [(tiles_k + 1)][m]
   const int* brief;       // [tiles_k][m]
@@ -167,12 +169,14 @@ __global__ __launch_bounds__(kSdThreads, 2) void spmm_blocks_kernel(SpmmBlocksPa
   const int launch_slot = id / 8;
   const bool thin_first = ((launch_slot ^ (launch_slot >> 5)) & 1) != 0;
   if (total % 8 == 0) id = (id % 8) * (total / 8) + id / 8;
-  const int z = id / row_blocks;
+  const int slices = p.n / kSbN;                     // (the slices of a batch entry are neighbours in this order: same XCD)
+  const int z = (id / row_blocks) / slices, slice = (id / row_blocks) % slices;
+  const int ld = p.n;                                // elements between rows of the dense operand and of the output
   const int row_block = id % row_blocks;
   const int row0 = row_block * kSdBM;
   const u16* __restrict__ vals = static_cast<const u16*>(p.values) + (size_t)z * p.values_stride;
-  const u16* __restrict__ V = static_cast<const u16*>(p.dense) + (size_t)z * p.k * kSbN;
-  u16* __restrict__ out = static_cast<u16*>(p.out) + (size_t)z * p.m * kSbN;
+  const u16* __restrict__ V = static_cast<const u16*>(p.dense) + (size_t)z * p.k * ld + slice * kSbN;
+  u16* __restrict__ out = static_cast<u16*>(p.out) + (size_t)z * p.m * ld + slice * kSbN;
   const int m = p.m;
   const int last = p.nnz - 1;   // (the host does not launch this kernel without nonzeros)
   const u16* __restrict__ list = p.dense_list + (size_t)row_block * (p.tiles_k + 2);
@@ -210,7 +214,7 @@ __global__ __launch_bounds__(kSdThreads, 2) void spmm_blocks_kernel(SpmmBlocksPa
             const int row = L >> 3, pos = L & 7;
             const int g = pos ^ (((row >> 1) & 1) << 2);
             const int krow = ct * kSdBN + row;
-            const u32x4 got = *reinterpret_cast<const u32x4*>(V + (size_t)min(krow, p.k - 1) * kSbN + g * 8);
+            const u32x4 got = *reinterpret_cast<const u32x4*>(V + (size_t)min(krow, p.k - 1) * ld + g * 8);
             const u32x4 zero = {0u, 0u, 0u, 0u};
             rv[q] = krow < p.k ? got : zero;
           }
@@ -430,7 +434,7 @@ __global__ __launch_bounds__(kSdThreads, 2) void spmm_blocks_kernel(SpmmBlocksPa
 #pragma unroll
             for (int u = 0; u < 8; ++u) {
               const int cu = __shfl(colw[w], gl + u, kWave);
-              const u16* src = st * 8 + u < cnt[h + w] ? V + (size_t)cu * kSbN + sl * 8 : zeros + sl * 8;
+              const u16* src = st * 8 + u < cnt[h + w] ? V + (size_t)cu * ld + sl * 8 : zeros + sl * 8;
               v[w][u] = *reinterpret_cast<const u32x4*>(src);
             }
 #pragma unroll
@@ -472,7 +476,7 @@ __global__ __launch_bounds__(kSdThreads, 2) void spmm_blocks_kernel(SpmmBlocksPa
       w.y = (unsigned)f32_to_16(y[2], BF16) | ((unsigned)f32_to_16(y[3], BF16) << 16);
       w.z = (unsigned)f32_to_16(y[4], BF16) | ((unsigned)f32_to_16(y[5], BF16) << 16);
       w.w = (unsigned)f32_to_16(y[6], BF16) | ((unsigned)f32_to_16(y[7], BF16) << 16);
-      if (wrow0 + row < m) *reinterpret_cast<u32x4*>(out + (size_t)(wrow0 + row) * kSbN + sl * 8) = w;
+      if (wrow0 + row < m) *reinterpret_cast<u32x4*>(out + (size_t)(wrow0 + row) * ld + sl * 8) = w;
     }
   }
 }

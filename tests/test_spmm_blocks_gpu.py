@@ -107,6 +107,21 @@ def test_many_column_blocks(oracle, dev, k, blocks):
             _run(dev, wide, values, rng.standard_normal((2, k + 1, 64)).astype(np.float32), torch.float16, force_variant=10)
 
 
+@pytest.mark.parametrize("n", [128, 192])
+def test_wider_outputs_in_slices_of_64_columns(oracle, dev, n):
+    rng = np.random.default_rng(n)
+    m, k = 300, 517
+    lens = rng.integers(0, 60, m)
+    lens[5] = k
+    csr = _pattern(rng, m, k, lens)
+    values = rng.standard_normal((3, csr.nnz)).astype(np.float32)
+    dense = rng.standard_normal((3, k, n)).astype(np.float32)
+    for blocks in (0, 1):
+        out = _run(dev, csr, values, dense, torch.bfloat16, force_variant=10, force_wpr=blocks)
+        want, scale = _want(oracle, csr, values, dense, torch.bfloat16)
+        assert_close(out.float().cpu().numpy(), want, scale, RTOL[torch.bfloat16], f"n={n} blocks={blocks}")
+
+
 def test_integer_operands_agree_with_the_row_kernel_exactly(dev):
     rng = np.random.default_rng(8)
     m, k = 260, 390
@@ -237,7 +252,8 @@ def test_refusals_and_workspace_size(dev):
     assert lib.iex_spmm_workspace_kind(_lib.F16, _lib.I32, _lib.SPMM_PER_BATCH_VALUES, 4096, 4096, 64, 1000, 16) == 0        # too sparse for the rule
     assert lib.iex_spmm_workspace_kind(_lib.F16, _lib.I32, _lib.SPMM_PER_BATCH_VALUES, 4096, 4096, 64, 1 << 20, 16) == 10
     assert lib.iex_spmm_workspace_kind(_lib.F16, _lib.I32, 0, 4096, 4096, 64, 1 << 20, 16) != 10                              # shared values
-    assert lib.iex_spmm_workspace_bytes(_lib.F16, _lib.I32, flags, 4096, 4096, 128, 1000, 16) == 0      # n != 64
+    assert lib.iex_spmm_workspace_bytes(_lib.F16, _lib.I32, flags, 4096, 4096, 128, 1000, 16) != 0      # two slices of 64 columns
+    assert lib.iex_spmm_workspace_bytes(_lib.F16, _lib.I32, flags, 4096, 4096, 96, 1000, 16) == 0       # n no multiple of 64
     assert lib.iex_spmm_workspace_bytes(_lib.F32, _lib.I32, flags, 4096, 4096, 64, 1000, 16) == 0
     assert lib.iex_spmm_workspace_bytes(_lib.F16, _lib.I16, flags, 4096, 4096, 64, 1000, 16) == 0
     rng = np.random.default_rng(1)

@@ -91,7 +91,7 @@ int iex_copy_bytes(void* dst, const void* src, size_t nbytes, void* stream);
  * chosen by itself for values per batch entry on patterns at least 3 % dense with batch * m * k >= 2^25, on request
  * elsewhere; iex_spmm_ws only, with
  * the workspace iex_spmm_workspace_bytes reports: the tables of SDDMM variant 3 for the pattern, which a small
- * kernel writes first, and behind them lists that two more small kernels derive from the tables -- see
+ * kernel writes first, and behind them lists that one more small kernel derives from the tables -- see
  * IEX_SPMM_TABLES_READY / IEX_SPMM_LISTS_READY; bits 8..15 set the number of nonzeros from which a block counts
  * as dense: 0 = built in (2048), 1 = every block, 255 = none, else 64 * value); fails on other shapes.
  * 0 = choose.

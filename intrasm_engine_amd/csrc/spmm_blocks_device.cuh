@@ -8,7 +8,7 @@
 // is the mirror image of the SDDMM for such masks (sddmm_mfma_device.cuh) and works from the same tables, written
 // by the same setup kernel into the caller's workspace (tile_ptr, brief, mask: per row and 128-column tile of A the
 // position of the row's first nonzero there, and which of the tile's columns the row holds), plus two lists that
-// two more small kernels derive from the tables (they depend on the pattern and on the threshold below, not on
+// one more small kernel derives from the tables (they depend on the pattern and on the threshold below, not on
 // values: a caller whose pattern stays keeps them): per block of 128 rows the column tiles that hold dense_min
 // nonzeros or more ("dense"), and per row its nonzeros outside those tiles, compacted.
 // A workgroup (4 wavefronts) owns 128 consecutive rows of one batch entry, a wavefront 32 of them:
@@ -86,41 +86,38 @@ struct SpmmBlocksParams {
 
 constexpr int spmm_blocks_lds_bytes() { return 4 * kSbTileBytes + 2 * kSbStage + 4 * 32 * 32; }
 
-// The dense tiles of every block of 128 rows (one workgroup each): dense_list[block][0] = their number, then the tiles.
-static __global__ __launch_bounds__(kSdThreads) void sb_dense_list_kernel(int m, int tiles_k, int dense_min, const int* __restrict__ tile_ptr,
-                                                                          unsigned short* __restrict__ dense_list, unsigned* __restrict__ zeros) {
+// The lists, one wavefront per row (4 rows per workgroup, all in one block of 128 rows).  Every workgroup first sorts the
+// column tiles of its block of rows into dense and other (33 x 128 cursors out of L2: cheaper than a launch of its own
+// for the 32 blocks); the workgroup with the block's first rows also writes that list: dense_list[block][0] = number of
+// dense tiles, then the tiles.  Then each wavefront compacts the nonzeros of its row that lie outside the dense tiles,
+// in row order: column and position in the CSR arrays.
+static __global__ __launch_bounds__(kSdThreads) void sb_lists_kernel(int m, int tiles_k, int dense_min, const int* __restrict__ tile_ptr,
+                                                                     const int* __restrict__ row_offsets, const int* __restrict__ cols,
+                                                                     unsigned short* __restrict__ dense_list, unsigned* __restrict__ zeros,
+                                                                     int* __restrict__ thin_cnt, SbEntry* __restrict__ thin_ent) {
   __shared__ unsigned colsum[kSdMaxTiles + 1];
   __shared__ unsigned short list[kSdMaxTiles];
   __shared__ int n_dense;
-  sd_sort_tiles(tile_ptr, m, tiles_k, blockIdx.x * kSdBM, dense_min, colsum, list, &n_dense);
-  unsigned short* mine = dense_list + (size_t)blockIdx.x * (tiles_k + 2);
-  const int nd = n_dense;
-  if (threadIdx.x == 0) mine[0] = (unsigned short)nd;
-  for (int i = threadIdx.x; i < nd; i += kSdThreads) mine[1 + i] = list[i];
-  if (blockIdx.x == 0 && threadIdx.x < kSbZeroWords) zeros[threadIdx.x] = 0u;
-}
-
-// The nonzeros of every row that lie outside the dense tiles of the row's block, compacted in row order (one wavefront
-// per row): column and position in the CSR arrays.
-static __global__ __launch_bounds__(256) void sb_thin_list_kernel(int m, int tiles_k, const int* __restrict__ row_offsets, const int* __restrict__ cols,
-                                                                  const unsigned short* __restrict__ dense_list, int* __restrict__ thin_cnt,
-                                                                  SbEntry* __restrict__ thin_ent) {
-  __shared__ unsigned is_dense[4][kSdMaxTiles / 32];
+  __shared__ unsigned is_dense[kSdMaxTiles / 32];
   const int lane = lane_id();
   const int wave = threadIdx.x >> 6;
   const int r = blockIdx.x * 4 + wave;
-  if (r >= m) return;   // (no workgroup barrier below: every wavefront works alone)
-  const unsigned short* mine = dense_list + (size_t)(r / kSdBM) * (tiles_k + 2);
-  const int nd = uniform((int)mine[0]);
-  if (lane < kSdMaxTiles / 32) is_dense[wave][lane] = 0;
-  __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
-  __builtin_amdgcn_wave_barrier();
-  for (int i = lane; i < nd; i += kWave) {
-    const int t = mine[1 + i];
-    atomicOr(&is_dense[wave][t >> 5], 1u << (t & 31));
+  const int block = (blockIdx.x * 4) / kSdBM;
+  if (threadIdx.x < kSdMaxTiles / 32) is_dense[threadIdx.x] = 0;
+  sd_sort_tiles(tile_ptr, m, tiles_k, block * kSdBM, dense_min, colsum, list, &n_dense);
+  const int nd = n_dense;
+  if ((blockIdx.x * 4) % kSdBM == 0) {
+    unsigned short* mine = dense_list + (size_t)block * (tiles_k + 2);
+    if (threadIdx.x == 0) mine[0] = (unsigned short)nd;
+    for (int i = threadIdx.x; i < nd; i += kSdThreads) mine[1 + i] = list[i];
   }
-  __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
-  __builtin_amdgcn_wave_barrier();
+  if (blockIdx.x == 0 && threadIdx.x < kSbZeroWords) zeros[threadIdx.x] = 0u;
+  for (int i = threadIdx.x; i < nd; i += kSdThreads) {
+    const int t = list[i];
+    atomicOr(&is_dense[t >> 5], 1u << (t & 31));
+  }
+  __syncthreads();
+  if (r >= m) return;   // (no workgroup barrier below: every wavefront works alone)
   const int s = uniform(row_offsets[r]), e = uniform(row_offsets[r + 1]);
   int count = 0;
   for (int base = s; base < e; base += 4 * kWave) {   // four loads in flight
@@ -133,7 +130,7 @@ static __global__ __launch_bounds__(256) void sb_thin_list_kernel(int m, int til
 #pragma unroll
     for (int u = 0; u < 4; ++u) {
       const int t = min(max(c[u], 0) >> 7, tiles_k - 1);
-      const bool thin = c[u] >= 0 && !((is_dense[wave][t >> 5] >> (t & 31)) & 1);
+      const bool thin = c[u] >= 0 && !((is_dense[t >> 5] >> (t & 31)) & 1);
       const unsigned long long b = __ballot(thin);
       if (thin) {
         SbEntry en;

@@ -190,7 +190,7 @@ def test_tables_kept_between_calls_and_shared_with_the_sddmm(dev):
     assert plan.key is not None
     kw = dict(per_batch_values=True, accumulate=False, dtypes=(torch.float16,), allow_i16=False, force_variant=10)
     fresh = pyops._spmm(v, ri, scores, rot, cit, m, **kw)
-    assert _lib.last_kernels().split(" + ") == ["sddmm_tile_ptr_kernel", "sb_dense_list_kernel", "sb_thin_list_kernel", "spmm_blocks_kernel<false>"]
+    assert _lib.last_kernels().split(" + ") == ["sddmm_tile_ptr_kernel", "sb_lists_kernel", "spmm_blocks_kernel<false>"]
     first = pyops._spmm(v, ri, scores, rot, cit, m, plan=plan, **kw)      # needs more room than the SDDMM: everything is written again
     kept = pyops._spmm(v, ri, scores, rot, cit, m, plan=plan, **kw)
     assert _lib.last_kernels() == "spmm_blocks_kernel<false>"
@@ -198,7 +198,7 @@ def test_tables_kept_between_calls_and_shared_with_the_sddmm(dev):
     again_scores = pyops.sddmm_half_planned(q, kk, ri, rot, cit, plan)    # the SDDMM finds its tables in the larger workspace
     assert "sddmm_tile_ptr_kernel" not in _lib.last_kernels() and torch.equal(again_scores, scores)
     other_threshold = pyops._spmm(v, ri, scores, rot, cit, m, plan=plan, force_wpr=1, **kw)    # tables kept, lists not
-    assert _lib.last_kernels().split(" + ") == ["sb_dense_list_kernel", "sb_thin_list_kernel", "spmm_blocks_kernel<false>"]
+    assert _lib.last_kernels().split(" + ") == ["sb_lists_kernel", "spmm_blocks_kernel<false>"]
     assert torch.allclose(other_threshold.float(), fresh.float(), rtol=1e-2, atol=1e-2)
     mask2 = np.abs(idx[:, None] - idx[None, :]) < 90
     ro2, ci2, _ = W.csr_from_mask(mask2)

@@ -189,8 +189,12 @@ int iex_CudaSpmm5(int m, int k, int n, int nonzeros, const int* row_indices,
 #define IEX_SDDMM_ACCUMULATE 0x2     /* out += ... instead of out = ...                   */
 /* iex_sddmm_ws, variant 3 only (ignored elsewhere): the workspace still holds the tables that an
  * earlier call with the same m, n, nonzeros and index arrays (and a kind-3 workspace) wrote there;
- * the setup kernel is skipped.  For callers whose mask does not change from call to call.        */
+ * the kernel that writes them is skipped.  For callers whose mask does not change from call to call. */
 #define IEX_SDDMM_TABLES_READY 0x4
+/* ... and the lists that variant 3 derives from the tables (which blocks count as dense, the nonzeros outside them)
+ * are still there too, from a call with the same bits 8..15 -- of iex_sddmm_ws, or of iex_spmm_ws family 10 on the same
+ * pattern: the lists are the same.  Only with IEX_SDDMM_TABLES_READY.                                              */
+#define IEX_SDDMM_LISTS_READY 0x8
 /* bits 8..15: force wavefronts per row (1 or 4); 0 = choose from nnz/m.  For tuning.
  * With variant 3 the same bits set the number of nonzeros from which a 128 x 128 block of the
  * mask counts as dense: 0 = built in, 1 = every block, 255 = none, else 64 * value.       */
@@ -200,8 +204,10 @@ int iex_CudaSpmm5(int m, int k, int n, int nonzeros, const int* row_indices,
  * matrix cores, sampled inside the workgroup and never stored, the nonzeros elsewhere one dot
  * product each (fp16 / bf16, k = 32, 64 or 128, n <= 65536, plain store, one output per batch
  * entry, strictly ascending columns inside a row; iex_sddmm_ws only: the workspace holds
- * (6 ceil(n / 128) + 1) * m words -- per row and block of columns a cursor, a packed word and a
- * 128-bit mask -- that a small kernel writes first, once for all batch entries); 7 = dense
+ * (6 ceil(n / 128) + 1) * m words of tables -- per row and block of columns a cursor, a packed word and a
+ * 128-bit mask -- and behind them 2 * nonzeros + m words and a few more of lists -- the dense blocks
+ * of every 128 rows, the nonzeros outside them row by row -- that two small kernels write first, once
+ * for all batch entries: iex_sddmm_workspace_bytes gives the total); 7 = dense
  * product in the caller's workspace, then sampling (iex_sddmm_ws only).
  * 3 and 7 fail where they cannot run.  0 = choose: 3 when the mask is at least 3 % dense and
  * batch * m * n is at least 2^25, else 7 or 1 by a time model.                              */

@@ -22,6 +22,7 @@ SPMM_LISTS_READY = 0x10
 SDDMM_SUM_OVER_BATCH = 0x1
 SDDMM_ACCUMULATE = 0x2
 SDDMM_TABLES_READY = 0x4
+SDDMM_LISTS_READY = 0x8
 
 _c = ctypes
 _vp, _i, _ll, _f = _c.c_void_p, _c.c_int, _c.c_longlong, _c.c_float

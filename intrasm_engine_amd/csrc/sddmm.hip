@@ -297,7 +297,7 @@ inline bool sddmm_mfma_fits(int dtype, const SddmmParams& p) {
          ceil_div(p.n, kSdBN) <= kSdMaxTiles && (long long)(ceil_div(p.n, kSdBN) + 1) * p.m < (1ll << 28);
 }
 
-inline size_t sddmm_mfma_bytes(const SddmmParams& p) { return sddmm_mfma_words(p.m, ceil_div(p.n, kSdBN)) * sizeof(int); }
+inline size_t sddmm_mfma_bytes(const SddmmParams& p) { return sb_words(p.m, ceil_div(p.n, kSdBN), p.nnz) * sizeof(int); }
 
 // The host does not look at the pattern, so the choice goes by the mask's overall density.  Measured on MI355X
 // (fp16, 16 heads of 4096 x 4096, k = 64, microseconds, gather kernel / this kernel):
@@ -329,16 +329,23 @@ int launch_sddmm_mfma_ks(const SddmmMfmaParams& q, int batch, hipStream_t stream
   return check_hip(hipGetLastError(), "sddmm (matrix-core) launch");
 }
 
-int launch_sddmm_mfma(int dtype, const SddmmParams& p, void* ws, int dense_code, bool tables_ready, hipStream_t stream) {
+// ready: bit 0 = the caller vouches that an earlier call on this pattern left the tables in the workspace, bit 1 = that the
+// lists are there too, from a call with the same dense_code (this kernel's, or the SpMM's for such patterns: same lists).
+int launch_sddmm_mfma(int dtype, const SddmmParams& p, void* ws, int dense_code, int ready, hipStream_t stream) {
   const int tiles_n = ceil_div(p.n, kSdBN);
   const SdTables t = sd_tables(ws, p.m, tiles_n);
-  if (!tables_ready) {   // (else: the caller vouches that an earlier call on this pattern left them in the workspace)
+  const SbLists l = sb_lists(ws, p.m, tiles_n, p.nnz);
+  if (!(ready & 1)) {
     if (int rc = sd_write_tables(t, p.m, tiles_n, p.row_offsets, p.cols, stream)) return rc;
   }
-  // dense_code (for tests and tuning): 0 = the built-in threshold, 1 = every tile on the matrix cores, 255 = none,
-  // else 64 * code nonzeros per 128 x 128 block
-  const int dense_min = dense_code == 0 ? kSdDenseMin : dense_code == 1 ? 0 : dense_code == 255 ? kSdBM * kSdBN + 1 : 64 * dense_code;
-  SddmmMfmaParams q{p.m, p.k, p.n, p.nnz, p.cols, p.lhs, p.rhs, p.out, t.mask, t.tile_ptr, t.brief, tiles_n, dense_min};
+  if ((ready & 3) != 3) {
+    // dense_code (for tests and tuning): 0 = the built-in threshold, 1 = every tile on the matrix cores, 255 = none,
+    // else 64 * code nonzeros per 128 x 128 block
+    const int dense_min = dense_code == 0 ? kSdDenseMin : dense_code == 1 ? 0 : dense_code == 255 ? kSdBM * kSdBN + 1 : 64 * dense_code;
+    if (int rc = sb_write_lists(t, l, p.m, tiles_n, dense_min, p.row_offsets, p.cols, stream)) return rc;
+  }
+  SddmmMfmaParams q{p.m, p.k, p.n, p.nnz, p.cols, p.lhs, p.rhs, p.out, t.mask, t.tile_ptr, t.brief, tiles_n,
+                    p.row_offsets, l.zeros, l.thin_ent, l.thin_cnt, l.dense_list};
   const bool bf16 = dtype == IEX_BF16;
   switch (p.k) {
     case 32: return bf16 ? launch_sddmm_mfma_ks<true, 2>(q, p.batch, stream) : launch_sddmm_mfma_ks<false, 2>(q, p.batch, stream);
@@ -405,7 +412,8 @@ int sddmm_dispatch(int dtype, int flags, int m, int k, int n, int nonzeros, cons
       IEX_REQUIRE(fits, IEX_ERR_UNSUPPORTED, "sddmm: the matrix-core kernel needs fp16 / bf16, k = 32, 64 or 128, plain store, one output per batch entry and 16-byte aligned operands");
       IEX_REQUIRE(room, IEX_ERR_BAD_ARGUMENT, "sddmm: the matrix-core kernel needs a 16-byte aligned workspace of %zu bytes (iex_sddmm_ws)", sddmm_mfma_bytes(p));
     }
-    if (fits && room && (variant == 3 || sddmm_mfma_wins(p))) return launch_sddmm_mfma(dtype, p, workspace, variant == 3 ? (flags >> 8) & 0xff : 0, (flags & IEX_SDDMM_TABLES_READY) != 0, s);
+    if (fits && room && (variant == 3 || sddmm_mfma_wins(p))) return launch_sddmm_mfma(dtype, p, workspace, variant == 3 ? (flags >> 8) & 0xff : 0,
+                                                                                 ((flags & IEX_SDDMM_TABLES_READY) ? 1 : 0) | ((flags & IEX_SDDMM_LISTS_READY) ? 2 : 0), s);
   }
   if (variant == 0 || variant == 7) {
     const bool fits = sddmm_dense_fits(dtype, p);

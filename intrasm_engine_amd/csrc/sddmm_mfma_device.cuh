@@ -6,25 +6,26 @@
 // mask (a dense band plus scattered entries, 5-10 % dense) that is 2.4 GB per 16 heads and that path is what bounds
 // it.  A dense product of everything (34 GFLOP) is cheap on the matrix cores but wasted on the nine tenths of the
 // 128 x 128 tiles that hold one entry per row.  So a workgroup (4 wavefronts) owns 128 consecutive rows of one batch
-// entry and sorts the column tiles (128 columns each) of its rows by how many nonzeros they hold:
+// entry, and the column tiles (128 columns each) of its rows are sorted by how many nonzeros they hold:
 //   * dense tiles (dense_min nonzeros or more in the 128 x 128 block): the rhs rows of the tile come from global
 //     memory straight into LDS (global_load_lds_dwordx4, double-buffered, 16-byte chunks permuted so that the
 //     operand reads are conflict-free), 2 x 2 x k/16 MFMAs of 32 x 32 x 16 per wavefront (each owns 64 x 64 of the
 //     tile; the lhs fragments stay in registers for the whole phase), operands swapped so that a lane ends up with
 //     4 adjacent columns of one row and writes them to the score tile in LDS with one 64-bit store, already rounded
 //     to the element type.  Sampling, two ways per (row, tile): up to 4 nonzeros -> the row's own lane (threads
-//     0..127) copies the scores named by a packed word; more -> a wavefront takes the row: a 128-bit mask of the
-//     row's columns in the tile tells each lane whether its two columns are present and, by a population count
-//     of the bits below, where in the row's output they go; the stores of a row are contiguous.  No column index
-//     is read from memory in this phase.
-//   * thin tiles: a wavefront lays the nonzeros that its 32 rows have there end to end (a list in LDS, so that rows
-//     of different lengths cost no idle lanes) and takes them 64 at a time, k/8 lanes per nonzero: 16 bytes of
-//     the rhs row per lane from memory, of the lhs row from LDS, v_dot2 in fp32, summed across the lanes, rounded
-//     once; the results are stored 64 at a time.
-// What the kernel needs to know about the mask comes from a small kernel that runs first, once per call for all
-// batch entries, into the caller's workspace: tile_ptr[t][row] = position of the row's first nonzero with column
-// >= 128 t (columns ascend inside a row), brief[t][row] = count and in-tile columns of up to 4 nonzeros, packed in
-// one word, and mask[t][row] for the pairs with more.
+//     0..127) copies the scores named by a packed word; more -> a wavefront takes four rows at a time, 16 lanes per
+//     row: a 128-bit mask of the row's columns in the tile tells each lane which of its 8 columns are present and, by
+//     a population count of the bits below, where in the row's output they go; all 8 present is one 16-byte store.
+//     No column index is read from memory in this phase.
+//   * the nonzeros elsewhere: k / 8 lanes per row walk the row's list of them (column, position in the output), the
+//     row's lhs in registers: 16 bytes of the rhs row per lane from memory, v_dot2 in fp32, summed across the lanes,
+//     rounded once, stored at the position.
+// What the kernel needs to know about the mask comes from two small kernels that run first, once per call for all
+// batch entries, into the caller's workspace (functions of the index arrays only: a caller whose mask stays keeps
+// them): the tables -- tile_ptr[t][row] = position of the row's first nonzero with column >= 128 t (columns ascend
+// inside a row), brief[t][row] = count and in-tile columns of up to 4 nonzeros, packed in one word, and
+// mask[t][row] for the pairs with more -- and, from the tables, the lists: per block of 128 rows its dense tiles,
+// per row its nonzeros outside them, compacted.  The SpMM for the same patterns (spmm_blocks_device.cuh) reads both.
 // The dense phase runs on a hand-counted pipeline: all its global reads (rhs rows for the next dense tile, the
 // per-row words two dense tiles ahead) are direct-to-LDS loads in inline assembly, invisible to the compiler's
 // wait-count pass; each wavefront issues a fixed number of them per tile and waits with s_waitcnt vmcnt(N), N =
@@ -53,7 +54,11 @@ struct SddmmMfmaParams {
   const int* tile_ptr;   // [(tiles_n + 1)][m]
   const int* brief;      // [tiles_n][m]
   int tiles_n;
-  int dense_min;
+  const int* row_offsets;
+  const unsigned* zeros;              // lists (see SbLists below)
+  const struct SbEntry* thin_ent;
+  const int* thin_cnt;
+  const unsigned short* dense_list;
 };
 
 // Workgroup barrier for LDS traffic only.  __syncthreads() also waits until the thread's global stores have
@@ -79,7 +84,7 @@ __device__ __forceinline__ unsigned wave_sum_u(unsigned v) {
 
 template <int KS>
 constexpr int sddmm_mfma_lds_bytes() {
-  return kSdBM * kSdLd * 2 + 2 * kSdBN * KS * 32 + 3 * kSdSlot + 16 + kSdMaxTiles * 2 + 16;
+  return kSdBM * kSdLd * 2 + 2 * kSdBN * KS * 32 + 3 * kSdSlot + 16;
 }
 
 // Words of workspace per call: masks first (16-byte entries), then the cursors, then the packed words.
@@ -225,6 +230,99 @@ __device__ __forceinline__ void sd_sort_tiles(const int* __restrict__ tile_ptr, 
   __syncthreads();
 }
 
+constexpr int kSbZeroWords = 64;               // 256 bytes of zeros: what the lanes of an absent nonzero read
+
+struct SbEntry {
+  int col, pos;   // column of a nonzero outside the dense tiles and its position in the CSR arrays
+};
+
+// Behind the tables in the same workspace: the lists that depend on which tiles count as dense (read by the SDDMM
+// below and by the SpMM for the same patterns, spmm_blocks_device.cuh).
+struct SbLists {
+  unsigned* zeros;                  // [kSbZeroWords]
+  SbEntry* thin_ent;                // [nnz]: row r's entries outside dense tiles, in row order, from thin_ent[row_offsets[r]]
+  int* thin_cnt;                    // [m]: how many
+  unsigned short* dense_list;       // [row blocks][tiles_k + 2]: number of dense tiles of the 128 rows, then the tiles, ascending
+};
+inline size_t sb_lists_offset_words(int m, int tiles_k) { return (sddmm_mfma_words(m, tiles_k) + 3) & ~size_t(3); }
+inline size_t sb_words(int m, int tiles_k, int nnz) {
+  return sb_lists_offset_words(m, tiles_k) + kSbZeroWords + 2 * (size_t)nnz + m + ((size_t)ceil_div(m, kSdBM) * (tiles_k + 2) + 1) / 2;
+}
+inline SbLists sb_lists(void* workspace, int m, int tiles_k, int nnz) {
+  SbLists l;
+  l.zeros = static_cast<unsigned*>(workspace) + sb_lists_offset_words(m, tiles_k);
+  l.thin_ent = reinterpret_cast<SbEntry*>(l.zeros + kSbZeroWords);
+  l.thin_cnt = reinterpret_cast<int*>(l.thin_ent + nnz);
+  l.dense_list = reinterpret_cast<unsigned short*>(l.thin_cnt + m);
+  return l;
+}
+
+
+// The lists, one wavefront per row (4 rows per workgroup, all in one block of 128 rows).  Every workgroup first sorts the
+// column tiles of its block of rows into dense and other (33 x 128 cursors out of L2: cheaper than a launch of its own
+// for the 32 blocks); the workgroup with the block's first rows also writes that list: dense_list[block][0] = number of
+// dense tiles, then the tiles.  Then each wavefront compacts the nonzeros of its row that lie outside the dense tiles,
+// in row order: column and position in the CSR arrays.
+static __global__ __launch_bounds__(kSdThreads) void sb_lists_kernel(int m, int tiles_k, int dense_min, const int* __restrict__ tile_ptr,
+                                                                     const int* __restrict__ row_offsets, const int* __restrict__ cols,
+                                                                     unsigned short* __restrict__ dense_list, unsigned* __restrict__ zeros,
+                                                                     int* __restrict__ thin_cnt, SbEntry* __restrict__ thin_ent) {
+  __shared__ unsigned colsum[kSdMaxTiles + 1];
+  __shared__ unsigned short list[kSdMaxTiles];
+  __shared__ int n_dense;
+  __shared__ unsigned is_dense[kSdMaxTiles / 32];
+  const int lane = lane_id();
+  const int wave = threadIdx.x >> 6;
+  const int r = blockIdx.x * 4 + wave;
+  const int block = (blockIdx.x * 4) / kSdBM;
+  if (threadIdx.x < kSdMaxTiles / 32) is_dense[threadIdx.x] = 0;
+  sd_sort_tiles(tile_ptr, m, tiles_k, block * kSdBM, dense_min, colsum, list, &n_dense);
+  const int nd = n_dense;
+  if ((blockIdx.x * 4) % kSdBM == 0) {
+    unsigned short* mine = dense_list + (size_t)block * (tiles_k + 2);
+    if (threadIdx.x == 0) mine[0] = (unsigned short)nd;
+    for (int i = threadIdx.x; i < nd; i += kSdThreads) mine[1 + i] = list[i];
+  }
+  if (blockIdx.x == 0 && threadIdx.x < kSbZeroWords) zeros[threadIdx.x] = 0u;
+  for (int i = threadIdx.x; i < nd; i += kSdThreads) {
+    const int t = list[i];
+    atomicOr(&is_dense[t >> 5], 1u << (t & 31));
+  }
+  __syncthreads();
+  if (r >= m) return;   // (no workgroup barrier below: every wavefront works alone)
+  const int s = uniform(row_offsets[r]), e = uniform(row_offsets[r + 1]);
+  int count = 0;
+  for (int base = s; base < e; base += 4 * kWave) {   // four loads in flight
+    int c[4];
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      const int j = base + u * kWave + lane;
+      c[u] = j < e ? cols[j] : -1;
+    }
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      const int t = min(max(c[u], 0) >> 7, tiles_k - 1);
+      const bool thin = c[u] >= 0 && !((is_dense[t >> 5] >> (t & 31)) & 1);
+      const unsigned long long b = __ballot(thin);
+      if (thin) {
+        SbEntry en;
+        en.col = c[u];
+        en.pos = base + u * kWave + lane;
+        thin_ent[s + count + __popcll(b & ((1ull << lane) - 1))] = en;
+      }
+      count += __popcll(b);
+    }
+  }
+  if (lane == 0) thin_cnt[r] = count;
+}
+
+inline int sb_write_lists(const SdTables& t, const SbLists& l, int m, int tiles_n, int dense_min, const int* row_offsets, const int* cols, hipStream_t stream) {
+  note_kernel("sb_lists_kernel");
+  hipLaunchKernelGGL(sb_lists_kernel, dim3(ceil_div(m, 4)), dim3(kSdThreads), 0, stream, m, tiles_n, dense_min, t.tile_ptr, row_offsets, cols, l.dense_list,
+                     l.zeros, l.thin_cnt, l.thin_ent);
+  return check_hip(hipGetLastError(), "list kernel launch");
+}
+
 // acc + <a, b> over 8 elements of 16 bits, products and sums in fp32
 template <bool BF16>
 __device__ __forceinline__ float dot8(u32x4 a, u32x4 b, float acc) {
@@ -256,8 +354,6 @@ __global__ __launch_bounds__(kSdThreads, KS == 8 ? 1 : 2) void sddmm_mfma_kernel
   unsigned char* sR = smem + kSdBM * kSdLd * 2;                               // [2][128][RB]
   unsigned char* sM = sR + 2 * STAGE;                                         // [3] slots of per-row words
   unsigned long long* long_rows = reinterpret_cast<unsigned long long*>(sM + 3 * kSdSlot);   // [2] rows with more than kSdShort
-  u16* list = reinterpret_cast<u16*>(long_rows + 2);                          // [tiles_n] dense tiles from the front, thin from the back
-  int* n_dense = reinterpret_cast<int*>(list + kSdMaxTiles);
   const unsigned ldsR = (unsigned)(size_t)(lds_u8*)sR;
   const unsigned ldsM = (unsigned)(size_t)(lds_u8*)sM;
 
@@ -282,8 +378,10 @@ __global__ __launch_bounds__(kSdThreads, KS == 8 ? 1 : 2) void sddmm_mfma_kernel
   u16* __restrict__ out = static_cast<u16*>(p.out) + (size_t)z * p.nnz;
   const int tiles_n = p.tiles_n;
 
-  sd_sort_tiles(p.tile_ptr, p.m, tiles_n, row0, p.dense_min, reinterpret_cast<unsigned*>(S), list, n_dense);
-  const int nd = __builtin_amdgcn_readfirstlane(*n_dense);
+  // the dense tiles of this block of rows (sorted out by the list kernel)
+  const u16* __restrict__ list = p.dense_list + (size_t)(row0 / kSdBM) * (tiles_n + 2);
+  const int nd = __builtin_amdgcn_readfirstlane((int)list[0]);
+  ++list;
 
   for (int phase = 0; phase < 2; ++phase) {
   // ---- dense tiles
@@ -459,127 +557,68 @@ __global__ __launch_bounds__(kSdThreads, KS == 8 ? 1 : 2) void sddmm_mfma_kernel
    }
   } else {
 
-  // ---- thin tiles.  A wavefront serves its 32 rows.  The nonzeros of a row between two dense tiles are
-  // consecutive in the row (columns ascend): one stretch of the CSR arrays per row and run of thin tiles.  The
-  // stretches of the 32 rows and of as many runs as fit (at most 32 nonzeros per row and run at a time) are laid
-  // end to end as a list of (column, row) entries in LDS, with the position of each in the output beside it, so
-  // that the work is the same for every lane whatever the rows' lengths; then, 64 entries per step, LPN lanes per
-  // entry: each lane reads 16 bytes of the entry's rhs row from memory (a load instruction covers whole rows) and
-  // of its lhs row from LDS, v_dot2 in fp32, summed over the LPN lanes, and lane i keeps the result of entry i of
-  // the step.  Results replace their entries and go to memory 64 at a time at the end: the loop holds no global
-  // store (its waits for loads never sit out a store's round trip) and the loads of the next step are in flight
-  // while this one computes.
+  // ---- the nonzeros outside dense tiles, from the per-row lists (column, position in the output) that the list
+  // kernel compacted.  A group of LPN = k / 8 lanes takes a row: lane j of the group keeps elements 8 j .. 8 j + 7 of the
+  // row's lhs in registers for the whole row.  Two rows of a group side by side, LPN entries of each per step: lane j
+  // reads entry j of the step, the group's lanes exchange the columns, every lane reads its 16 bytes of the LPN rhs
+  // rows (the lanes of an absent entry read zeros instead), v_dot2 in fp32, summed over the group's lanes; lane j
+  // keeps the result of entry j and stores it at the entry's position.  The entries of the next step are fetched
+  // before this step's dot products.
   {
-    constexpr int LPN = CH;              // lanes per nonzero
-    constexpr int LROW = RB + 16;        // bytes per lhs row in LDS (padded: rows start 4 banks apart)
-    constexpr int CAP = 1024;            // entries of a wavefront's list
-    constexpr int CAPR = 32;             // nonzeros a row contributes per run and round
-    const int sl = lane % LPN, g = lane / LPN;
-    unsigned* ent = reinterpret_cast<unsigned*>(smem) + wave * (2 * CAP);          // in the score tile: [CAP] entries,
-    int* pos = reinterpret_cast<int*>(ent + CAP);                                  // [CAP] output positions
-    unsigned char* lrows = sR + wave * (32 * LROW);
-    for (int i = lane; i < 32 * CH; i += kWave) {
-      const int r = i / CH, ch = i % CH;
-      const int gr = min(row0 + wave * 32 + r, p.m - 1);
-      *reinterpret_cast<u32x4*>(lrows + r * LROW + ch * 16) = *reinterpret_cast<const u32x4*>(lhs + (size_t)gr * p.k + ch * 8);
-    }
-    const int* __restrict__ cols = p.cols;
-    // lanes 0..31 hold the bounds of the wavefront's rows; when the list is built, lanes 0..31 serve an even row
-    // and lanes 32..63 the odd row after it
-    const int hl = lane & 31, hsel = lane >> 5;
-    const int my_row = row0 + wave * 32 + hl;
-    const bool valid = lane < 32 && my_row < p.m;
-    const int grow = min(my_row, p.m - 1);
-    int T = 0;   // entries in the list
-
-    auto fetch = [&](int base, unsigned& w, u32x4 (&rv)[LPN]) {
-      w = ent[min(base + lane, T - 1)];
+    constexpr int LPN = CH;              // lanes per row
+    constexpr int G = kWave / LPN;       // rows side by side in a wavefront
+    constexpr int ROUNDS = 32 / G;       // rounds of G rows over the wavefront's 32
+    constexpr int RS = 2;                // rows of a group side by side (4 for k = 64 filled the register file for 2 % of the time)
+    static_assert(ROUNDS % RS == 0, "rows side by side");
+    const int g = lane / LPN, sl = lane % LPN, gl = lane - sl;
+    const u16* __restrict__ zeros = reinterpret_cast<const u16*>(p.zeros);
+    const int last = p.nnz - 1;
+    for (int h = 0; h < ROUNDS; h += RS) {
+      int base[RS], cnt[RS], nmax = 0;
+      u32x4 lf[RS];
+      SbEntry en[RS];
 #pragma unroll
-      for (int u = 0; u < LPN; ++u) {
-        const unsigned wu = (unsigned)__shfl((int)w, g * LPN + u, kWave);
-        rv[u] = *reinterpret_cast<const u32x4*>(rhs + (size_t)(wu >> 5) * RB + sl * 16);
+      for (int w = 0; w < RS; ++w) {
+        const int r = row0 + wave * 32 + (h + w) * G + g;
+        const int rc = min(r, p.m - 1);
+        base[w] = p.row_offsets[rc];
+        cnt[w] = r < p.m ? p.thin_cnt[rc] : 0;
+        lf[w] = *reinterpret_cast<const u32x4*>(lhs + (size_t)rc * p.k + sl * 8);
       }
-    };
-    auto finish = [&](int base, unsigned w, u32x4 (&rv)[LPN]) {
-      float res = 0.f;
 #pragma unroll
-      for (int u = 0; u < LPN; ++u) {
-        const unsigned wu = (unsigned)__shfl((int)w, g * LPN + u, kWave);
-        const u32x4 lf = *reinterpret_cast<const u32x4*>(lrows + (wu & 31) * LROW + sl * 16);
-        const float acc = group_sum<LPN>(dot8<BF16>(lf, rv[u], 0.f));
-        res = sl == u ? acc : res;
+      for (int w = 0; w < RS; ++w) {
+        nmax = max(nmax, cnt[w]);
+        en[w] = p.thin_ent[min(base[w] + min(sl, max(cnt[w] - 1, 0)), last)];
       }
-      if (base + lane < T) ent[base + lane] = (unsigned)f32_to_16(res, BF16);
-    };
-    auto work_off = [&]() {   // the list: compute, store, empty
-      if (T > 0) {
-        __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
-        __builtin_amdgcn_wave_barrier();
-        // three steps' loads in flight (a step is fetched only while its entries are still entries: results replace them)
-        unsigned wa, wb, wc;
-        u32x4 rva[LPN], rvb[LPN], rvc[LPN];
-        fetch(0, wa, rva);
-        if (kWave < T) fetch(kWave, wb, rvb);
-        for (int base = 0; base < T; base += 3 * kWave) {
-          if (base + 2 * kWave < T) fetch(base + 2 * kWave, wc, rvc);
-          finish(base, wa, rva);
-          if (base + kWave < T) {
-            if (base + 3 * kWave < T) fetch(base + 3 * kWave, wa, rva);
-            finish(base + kWave, wb, rvb);
-          }
-          if (base + 2 * kWave < T) {
-            if (base + 4 * kWave < T) fetch(base + 4 * kWave, wb, rvb);
-            finish(base + 2 * kWave, wc, rvc);
+      for (int st = 0; __ballot(st * LPN < nmax); ++st) {
+        u32x4 rv[RS][LPN];
+        int at[RS];
+#pragma unroll
+        for (int w = 0; w < RS; ++w) {
+          at[w] = en[w].pos;
+#pragma unroll
+          for (int u = 0; u < LPN; ++u) {
+            const int cu = __shfl(en[w].col, gl + u, kWave);
+            const unsigned char* src = st * LPN + u < cnt[w] ? rhs + (size_t)cu * RB + sl * 16 : reinterpret_cast<const unsigned char*>(zeros) + sl * 16;
+            rv[w][u] = *reinterpret_cast<const u32x4*>(src);
           }
         }
-        __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
-        __builtin_amdgcn_wave_barrier();
-        for (int i = lane; i < T; i += kWave) out[pos[i]] = (u16)ent[i];
-        __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
-        __builtin_amdgcn_wave_barrier();
-      }
-      T = 0;
-    };
-
-    for (int run = 0; run <= nd; ++run) {
-      const int a = run == 0 ? 0 : __builtin_amdgcn_readfirstlane((int)list[run - 1]) + 1;
-      const int b = run == nd ? tiles_n : __builtin_amdgcn_readfirstlane((int)list[run]);
-      if (a >= b) continue;   // two dense tiles side by side
-      int s = p.tile_ptr[(size_t)a * p.m + grow];
-      const int e = valid ? p.tile_ptr[(size_t)b * p.m + grow] : s;
-      while (__ballot(s < e)) {
-        const int len = min(max(e - s, 0), CAPR);
-        int upto = len;   // inclusive prefix sum over lanes 0..31
 #pragma unroll
-        for (int d = 1; d < 32; d <<= 1) {
-          const int t = __shfl_up(upto, d, kWave);
-          if (lane >= d) upto += t;
-        }
-        const int before = upto - len;
-        const int round_total = __builtin_amdgcn_readlane(upto, 31);
-        if (T + round_total > CAP) work_off();
-        int sr[16], cv[16];
+        for (int w = 0; w < RS; ++w) en[w] = p.thin_ent[min(base[w] + min((st + 1) * LPN + sl, max(cnt[w] - 1, 0)), last)];
 #pragma unroll
-        for (int i = 0; i < 16; ++i) {
-          sr[i] = __shfl(s, 2 * i + hsel, kWave);
-          cv[i] = cols[min(sr[i] + hl, p.nnz - 1)];
-        }
+        for (int w = 0; w < RS; ++w) {
+          float res = 0.f;
 #pragma unroll
-        for (int i = 0; i < 16; ++i) {
-          const int lr = __shfl(len, 2 * i + hsel, kWave), pr = __shfl(before, 2 * i + hsel, kWave);
-          if (hl < lr) {
-            ent[T + pr + hl] = ((unsigned)cv[i] << 5) | (unsigned)(2 * i + hsel);
-            pos[T + pr + hl] = sr[i] + hl;
+          for (int u = 0; u < LPN; ++u) {
+            const float acc = group_sum<LPN>(dot8<BF16>(lf[w], rv[w][u], 0.f));
+            res = sl == u ? acc : res;
           }
+          if (st * LPN + sl < cnt[w]) out[min((unsigned)at[w], (unsigned)last)] = f32_to_16(res, BF16);
         }
-        T += round_total;
-        s += len;
       }
     }
-    work_off();
   }
   }
-  __syncthreads();   // the score tile changes hands: sampled by one phase, collecting results in the other
   }
 }
 

@@ -61,10 +61,7 @@ int launch_spmm_blocks(int dtype, const SpmmParams& p, int batch, void* ws, int 
   }
   if ((ready & 3) != 3) {
     const int dense_min = dense_code == 0 ? kSdDenseMin : dense_code == 1 ? 0 : dense_code == 255 ? kSdBM * kSdBN + 1 : 64 * dense_code;
-    note_kernel("sb_lists_kernel");
-    hipLaunchKernelGGL(sb_lists_kernel, dim3(ceil_div(p.m, 4)), dim3(kSdThreads), 0, stream, p.m, tiles_k, dense_min, t.tile_ptr, p.row_offsets, cols,
-                       l.dense_list, l.zeros, l.thin_cnt, l.thin_ent);
-    if (int rc = check_hip(hipGetLastError(), "spmm (lists) launch")) return rc;
+    if (int rc = sb_write_lists(t, l, p.m, tiles_k, dense_min, p.row_offsets, cols, stream)) return rc;
   }
   SpmmBlocksParams q{p.m, p.k, p.nnz, p.row_offsets, p.values, p.per_batch_values ? (size_t)p.nnz : 0, p.dense, p.out, p.n,
                      t.mask, t.tile_ptr, t.brief, tiles_k, l.zeros, l.thin_ent, l.thin_cnt, l.dense_list};

@@ -39,33 +39,6 @@ constexpr int kSbN = 64;                       // output columns per workgroup (
 constexpr int kSbTileBytes = 32 * kSdLd * 2;   // a wavefront's 32 x 128 tile of A (rows padded to 272 bytes); later its 32 x 64 fp32 sums
 constexpr int kSbStage = kSdBN * kSbN * 2;     // 128 rows of the dense operand
 constexpr int kSbRows = 2;                     // rows whose nonzeros outside dense tiles a lane group gathers side by side (1, 2 or 4)
-constexpr int kSbZeroWords = 32;               // 128 bytes of zeros: what the lanes of an absent nonzero read
-
-struct SbEntry {
-  int col, pos;   // column of a nonzero outside the dense tiles and its position in the CSR arrays
-};
-
-// What the kernel reads besides the operands: the SDDMM's tables and, behind them in the same workspace, the lists
-// that depend on which tiles count as dense.
-struct SbLists {
-  unsigned* zeros;                  // [kSbZeroWords]
-  SbEntry* thin_ent;                // [nnz]: row r's entries outside dense tiles, in row order, from thin_ent[row_offsets[r]]
-  int* thin_cnt;                    // [m]: how many
-  unsigned short* dense_list;       // [row blocks][tiles_k + 2]: number of dense tiles of the 128 rows, then the tiles, ascending
-};
-inline size_t sb_lists_offset_words(int m, int tiles_k) { return (sddmm_mfma_words(m, tiles_k) + 3) & ~size_t(3); }
-inline size_t sb_words(int m, int tiles_k, int nnz) {
-  return sb_lists_offset_words(m, tiles_k) + kSbZeroWords + 2 * (size_t)nnz + m + ((size_t)ceil_div(m, kSdBM) * (tiles_k + 2) + 1) / 2;
-}
-inline SbLists sb_lists(void* workspace, int m, int tiles_k, int nnz) {
-  SbLists l;
-  l.zeros = static_cast<unsigned*>(workspace) + sb_lists_offset_words(m, tiles_k);
-  l.thin_ent = reinterpret_cast<SbEntry*>(l.zeros + kSbZeroWords);
-  l.thin_cnt = reinterpret_cast<int*>(l.thin_ent + nnz);
-  l.dense_list = reinterpret_cast<unsigned short*>(l.thin_cnt + m);
-  return l;
-}
-
 struct SpmmBlocksParams {
   int m, k, nnz;
   const int* row_offsets;
@@ -85,64 +58,6 @@ struct SpmmBlocksParams {
 };
 
 constexpr int spmm_blocks_lds_bytes() { return 4 * kSbTileBytes + 2 * kSbStage + 4 * 32 * 32; }
-
-// The lists, one wavefront per row (4 rows per workgroup, all in one block of 128 rows).  Every workgroup first sorts the
-// column tiles of its block of rows into dense and other (33 x 128 cursors out of L2: cheaper than a launch of its own
-// for the 32 blocks); the workgroup with the block's first rows also writes that list: dense_list[block][0] = number of
-// dense tiles, then the tiles.  Then each wavefront compacts the nonzeros of its row that lie outside the dense tiles,
-// in row order: column and position in the CSR arrays.
-static __global__ __launch_bounds__(kSdThreads) void sb_lists_kernel(int m, int tiles_k, int dense_min, const int* __restrict__ tile_ptr,
-                                                                     const int* __restrict__ row_offsets, const int* __restrict__ cols,
-                                                                     unsigned short* __restrict__ dense_list, unsigned* __restrict__ zeros,
-                                                                     int* __restrict__ thin_cnt, SbEntry* __restrict__ thin_ent) {
-  __shared__ unsigned colsum[kSdMaxTiles + 1];
-  __shared__ unsigned short list[kSdMaxTiles];
-  __shared__ int n_dense;
-  __shared__ unsigned is_dense[kSdMaxTiles / 32];
-  const int lane = lane_id();
-  const int wave = threadIdx.x >> 6;
-  const int r = blockIdx.x * 4 + wave;
-  const int block = (blockIdx.x * 4) / kSdBM;
-  if (threadIdx.x < kSdMaxTiles / 32) is_dense[threadIdx.x] = 0;
-  sd_sort_tiles(tile_ptr, m, tiles_k, block * kSdBM, dense_min, colsum, list, &n_dense);
-  const int nd = n_dense;
-  if ((blockIdx.x * 4) % kSdBM == 0) {
-    unsigned short* mine = dense_list + (size_t)block * (tiles_k + 2);
-    if (threadIdx.x == 0) mine[0] = (unsigned short)nd;
-    for (int i = threadIdx.x; i < nd; i += kSdThreads) mine[1 + i] = list[i];
-  }
-  if (blockIdx.x == 0 && threadIdx.x < kSbZeroWords) zeros[threadIdx.x] = 0u;
-  for (int i = threadIdx.x; i < nd; i += kSdThreads) {
-    const int t = list[i];
-    atomicOr(&is_dense[t >> 5], 1u << (t & 31));
-  }
-  __syncthreads();
-  if (r >= m) return;   // (no workgroup barrier below: every wavefront works alone)
-  const int s = uniform(row_offsets[r]), e = uniform(row_offsets[r + 1]);
-  int count = 0;
-  for (int base = s; base < e; base += 4 * kWave) {   // four loads in flight
-    int c[4];
-#pragma unroll
-    for (int u = 0; u < 4; ++u) {
-      const int j = base + u * kWave + lane;
-      c[u] = j < e ? cols[j] : -1;
-    }
-#pragma unroll
-    for (int u = 0; u < 4; ++u) {
-      const int t = min(max(c[u], 0) >> 7, tiles_k - 1);
-      const bool thin = c[u] >= 0 && !((is_dense[t >> 5] >> (t & 31)) & 1);
-      const unsigned long long b = __ballot(thin);
-      if (thin) {
-        SbEntry en;
-        en.col = c[u];
-        en.pos = base + u * kWave + lane;
-        thin_ent[s + count + __popcll(b & ((1ull << lane) - 1))] = en;
-      }
-      count += __popcll(b);
-    }
-  }
-  if (lane == 0) thin_cnt[r] = count;
-}
 
 template <bool BF16>
 __global__ __launch_bounds__(kSdThreads, 2) void spmm_blocks_kernel(SpmmBlocksParams p) {

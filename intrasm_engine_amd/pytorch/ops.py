@@ -161,9 +161,10 @@ def _spmm(b, row_indices, values, row_offsets, column_indices, m, *, per_batch_v
                    m, k, nonzeros)
             if plan._ready(key, ws_bytes, b.device):
                 flags |= _lib.SPMM_TABLES_READY
-                if plan.lists_key == (key, (flags >> 8) & 0xff):
+                code = (flags >> 8) & 0xff if ((flags >> 16) & 0xf) == 10 else 0    # (what counts as a dense block: the lists depend on it)
+                if plan.lists_key == (key, code):
                     flags |= _lib.SPMM_LISTS_READY
-            plan.lists_key = (key, (flags >> 8) & 0xff)
+            plan.lists_key = (key, (flags >> 8) & 0xff if ((flags >> 16) & 0xf) == 10 else 0)
             ws = plan.workspace
         else:
             ws = torch.empty(ws_bytes, dtype=torch.uint8, device=b.device) if ws_bytes else None
@@ -182,15 +183,15 @@ class SddmmPlan:
 
     The kernel for masks with structure (``iex_sddmm_ws``, variant 3) works from tables that a setup kernel derives
     from the pattern alone (m, n, row_offsets, column_indices).  A caller whose mask does not change passes the same
-    plan to every call: the first call writes the tables into the plan's workspace, later calls skip the setup kernel
-    (``IEX_SDDMM_TABLES_READY``).  The plan notices other index tensors, other shapes and in-place changes of the index
+    plan to every call: the first call writes the tables and lists into the plan's workspace, later calls skip the setup
+    kernels (``IEX_SDDMM_TABLES_READY``, ``IEX_SDDMM_LISTS_READY``).  The plan notices other index tensors, other shapes and in-place changes of the index
     tensors (their version counters) and then lets the tables be written again.  Calls that share a plan must be
     ordered on one stream (the workspace is theirs for the duration of the work)."""
 
     def __init__(self):
         self.workspace = None
         self.key = None
-        self.lists_key = None   # the SpMM for the same patterns keeps lists of its own behind the tables
+        self.lists_key = None   # (the lists behind the tables also depend on what counts as a dense block)
         self.variant = 0        # 0: the library's rule (by density); 1 / 3 after analyze()
         self.dense_share = None
 
@@ -265,8 +266,12 @@ def _sddmm(a, b, row_indices, row_offsets, column_indices, *, sum_over_batch, dt
         if plan is not None and ws_bytes and lib.iex_sddmm_workspace_kind(_DT[a.dtype], flags, m, k, n, nonzeros, batch) == 3:
             key = (row_offsets.data_ptr(), column_indices.data_ptr(), row_offsets._version, column_indices._version,
                    m, n, nonzeros)
+            code = (flags >> 8) & 0xff if ((flags >> 16) & 0xf) == 3 else 0     # (what counts as a dense block: the lists depend on it)
             if plan._ready(key, ws_bytes, a.device):
                 flags |= _lib.SDDMM_TABLES_READY
+                if plan.lists_key == (key, code):
+                    flags |= _lib.SDDMM_LISTS_READY
+            plan.lists_key = (key, code)
             ws = plan.workspace
         else:
             ws = torch.empty(ws_bytes, dtype=torch.uint8, device=a.device) if ws_bytes else None

@@ -38,8 +38,10 @@ def sparse_attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, row_indi
         raise RuntimeError("the mask must be tokens x tokens")
     if scale is None:
         scale = 1.0 / math.sqrt(q.shape[2])
+    from . import ops as _pyops
+    if plan is None and q.dtype in (torch.float16, torch.bfloat16):
+        plan = _pyops.SddmmPlan()     # for this call only: what the first product derives from the mask serves the second too
     if plan is not None:
-        from . import ops as _pyops
         scores = _pyops.sddmm_half_planned(q, k, row_indices, row_offsets, column_indices, plan)
     else:
         scores = ops.sddmm_sputnik_half(q, k, row_indices, row_offsets, column_indices)     # (heads, nnz)

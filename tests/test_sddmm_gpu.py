@@ -245,7 +245,7 @@ def test_dense_product_path_is_chosen_with_a_workspace_and_only_then(oracle, dev
     assert lib.iex_sddmm_workspace_bytes(_lib.F16, _lib.SDDMM_SUM_OVER_BATCH, m, k, n, nnz, 1) == need
     assert lib.iex_sddmm_workspace_bytes(_lib.F16, _lib.SDDMM_ACCUMULATE, m, k, n, nnz, 1) == 0
     # config 3: not the dense product; the tables of the kernel that samples score tiles inside the workgroup
-    assert lib.iex_sddmm_workspace_bytes(_lib.F16, 0, 4096, 64, 4096, 1150000, 16) == (6 * 32 + 1) * 4096 * 4
+    assert lib.iex_sddmm_workspace_bytes(_lib.F16, 0, 4096, 64, 4096, 1150000, 16) == ((6 * 32 + 1) * 4096 + 64 + 2 * 1150000 + 4096 + 32 * (32 + 2) // 2) * 4   # tables + lists
     assert lib.iex_sddmm_workspace_bytes(_lib.F16, 0, 4096, 64, 4096, 1150000 // 4, 16) == 0   # a mask this thin: the gather kernel
     assert lib.iex_sddmm_workspace_bytes(_lib.F16, 7 << 16, 4096, 64, 4096, 1150000, 16) == 4096 * 4096 * 2  # on request
     kw = dict(sum_over_batch=False, dtypes=(dtype,))

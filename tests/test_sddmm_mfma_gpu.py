@@ -210,7 +210,7 @@ def test_refusals(dev):
         _run(dev, csr, rng.standard_normal((1, 64, 48)).astype(np.float32), rng.standard_normal((1, 64, 48)).astype(np.float32),
              torch.float16, force_variant=3)
     lib = _lib.load()
-    assert lib.iex_sddmm_workspace_bytes(_lib.F16, 3 << 16, 4096, 64, 4096, 1000, 16) == (6 * 32 + 1) * 4096 * 4
+    assert lib.iex_sddmm_workspace_bytes(_lib.F16, 3 << 16, 4096, 64, 4096, 1000, 16) == ((6 * 32 + 1) * 4096 + 64 + 2 * 1000 + 4096 + 32 * (32 + 2) // 2) * 4   # tables + lists
     assert lib.iex_sddmm_workspace_bytes(_lib.F32, 3 << 16, 4096, 64, 4096, 1000, 16) == 0
     assert lib.iex_sddmm_workspace_kind(_lib.F16, 3 << 16, 4096, 64, 4096, 1000, 16) == 3
     assert lib.iex_sddmm_workspace_kind(_lib.F16, 0, 4096, 64, 4096, 1150000, 16) == 3

@@ -170,7 +170,8 @@ def test_config3_probabilities_times_v(oracle, dev):
 
 def test_tables_kept_between_calls_and_shared_with_the_sddmm(dev):
     """One plan serves the SDDMM for masks with structure and this kernel on the same pattern: whichever runs first
-    writes the tables, the other finds them; another pattern makes them be written again."""
+    writes the tables and lists, the other finds them; another threshold for dense blocks makes the lists, another
+    pattern makes everything be written again."""
     from intrasm_engine_amd import _lib
     from intrasm_engine_amd.pytorch import ops as pyops
     rng = np.random.default_rng(5)
@@ -191,12 +192,13 @@ def test_tables_kept_between_calls_and_shared_with_the_sddmm(dev):
     kw = dict(per_batch_values=True, accumulate=False, dtypes=(torch.float16,), allow_i16=False, force_variant=10)
     fresh = pyops._spmm(v, ri, scores, rot, cit, m, **kw)
     assert _lib.last_kernels().split(" + ") == ["sddmm_tile_ptr_kernel", "sb_lists_kernel", "spmm_blocks_kernel<false>"]
-    first = pyops._spmm(v, ri, scores, rot, cit, m, plan=plan, **kw)      # needs more room than the SDDMM: everything is written again
+    first = pyops._spmm(v, ri, scores, rot, cit, m, plan=plan, **kw)      # tables and lists are the SDDMM's: nothing to write
+    assert _lib.last_kernels() == "spmm_blocks_kernel<false>"
     kept = pyops._spmm(v, ri, scores, rot, cit, m, plan=plan, **kw)
     assert _lib.last_kernels() == "spmm_blocks_kernel<false>"
     assert torch.equal(kept, fresh) and torch.equal(first, fresh)
-    again_scores = pyops.sddmm_half_planned(q, kk, ri, rot, cit, plan)    # the SDDMM finds its tables in the larger workspace
-    assert "sddmm_tile_ptr_kernel" not in _lib.last_kernels() and torch.equal(again_scores, scores)
+    again_scores = pyops.sddmm_half_planned(q, kk, ri, rot, cit, plan)
+    assert _lib.last_kernels() == "sddmm_mfma_kernel<false, 4>" and torch.equal(again_scores, scores)
     other_threshold = pyops._spmm(v, ri, scores, rot, cit, m, plan=plan, force_wpr=1, **kw)    # tables kept, lists not
     assert _lib.last_kernels().split(" + ") == ["sb_lists_kernel", "spmm_blocks_kernel<false>"]
     assert torch.allclose(other_threshold.float(), fresh.float(), rtol=1e-2, atol=1e-2)
@@ -247,7 +249,7 @@ def test_refusals_and_workspace_size(dev):
     from intrasm_engine_amd import _lib
     lib = _lib.load()
     flags = (10 << 16) | _lib.SPMM_PER_BATCH_VALUES
-    assert lib.iex_spmm_workspace_bytes(_lib.F16, _lib.I32, flags, 4096, 4096, 64, 1000, 16) == ((6 * 32 + 1) * 4096 + 32 + 2 * 1000 + 4096 + 32 * (32 + 2) // 2) * 4
+    assert lib.iex_spmm_workspace_bytes(_lib.F16, _lib.I32, flags, 4096, 4096, 64, 1000, 16) == ((6 * 32 + 1) * 4096 + 64 + 2 * 1000 + 4096 + 32 * (32 + 2) // 2) * 4
     assert lib.iex_spmm_workspace_kind(_lib.F16, _lib.I32, flags, 4096, 4096, 64, 1000, 16) == 10
     assert lib.iex_spmm_workspace_kind(_lib.F16, _lib.I32, _lib.SPMM_PER_BATCH_VALUES, 4096, 4096, 64, 1000, 16) == 0        # too sparse for the rule
     assert lib.iex_spmm_workspace_kind(_lib.F16, _lib.I32, _lib.SPMM_PER_BATCH_VALUES, 4096, 4096, 64, 1 << 20, 16) == 10

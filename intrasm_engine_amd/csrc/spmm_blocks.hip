@@ -14,7 +14,7 @@ bool spmm_blocks_fits(int dtype, int itype, const SpmmParams& p) {
 
 // The host does not look at the pattern, so where nothing is forced the choice goes by the overall density, and only
 // for values per batch entry (attention probabilities: masks with structure).  Measured on MI355X (fp16, 16 batch
-// entries of 4096 x 4096, n = 64, microseconds, row kernel / this kernel with its three setup kernels / with tables
+// entries of 4096 x 4096, n = 64, microseconds, row kernel / this kernel with its setup kernels (three when measured, two now) / with tables
 // and lists kept):
 //   band of 256 + 32 scattered per row (7 %)   99 /  55 /  38     band of 512 + 32 (13 %)        184 /  75 /  51
 //   band of 128 + 16 scattered (3.5 %)          60 /  48 /  31     block diagonal 256 (6 %)        83 /  37 /  21

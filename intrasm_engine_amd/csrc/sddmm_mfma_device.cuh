@@ -561,7 +561,7 @@ __global__ __launch_bounds__(kSdThreads, KS == 8 ? 1 : 2) void sddmm_mfma_kernel
   // kernel compacted.  A group of LPN = k / 8 lanes takes a row: lane j of the group keeps elements 8 j .. 8 j + 7 of the
   // row's lhs in registers for the whole row.  Two rows of a group side by side, LPN entries of each per step: lane j
   // reads entry j of the step, the group's lanes exchange the columns, every lane reads its 16 bytes of the LPN rhs
-  // rows (the lanes of an absent entry read zeros instead), v_dot2 in fp32, summed over the group's lanes; lane j
+  // rows, v_dot2 in fp32, summed over the group's lanes; lane j
   // keeps the result of entry j and stores it at the entry's position.  The entries of the next step are fetched
   // before this step's dot products.
   {
@@ -571,7 +571,6 @@ __global__ __launch_bounds__(kSdThreads, KS == 8 ? 1 : 2) void sddmm_mfma_kernel
     constexpr int RS = 2;                // rows of a group side by side (4 for k = 64 filled the register file for 2 % of the time)
     static_assert(ROUNDS % RS == 0, "rows side by side");
     const int g = lane / LPN, sl = lane % LPN, gl = lane - sl;
-    const u16* __restrict__ zeros = reinterpret_cast<const u16*>(p.zeros);
     const int last = p.nnz - 1;
     for (int h = 0; h < ROUNDS; h += RS) {
       int base[RS], cnt[RS], nmax = 0;
@@ -598,9 +597,10 @@ __global__ __launch_bounds__(kSdThreads, KS == 8 ? 1 : 2) void sddmm_mfma_kernel
           at[w] = en[w].pos;
 #pragma unroll
           for (int u = 0; u < LPN; ++u) {
-            const int cu = __shfl(en[w].col, gl + u, kWave);
-            const unsigned char* src = st * LPN + u < cnt[w] ? rhs + (size_t)cu * RB + sl * 16 : reinterpret_cast<const unsigned char*>(zeros) + sl * 16;
-            rv[w][u] = *reinterpret_cast<const u32x4*>(src);
+            // (an entry past the end of the row's list is a copy of the row's last one, or -- a row without a list --
+            // whatever the slot holds: the column is clamped into the operand and the result never stored)
+            const unsigned cu = min((unsigned)__shfl(en[w].col, gl + u, kWave), (unsigned)(p.n - 1));
+            rv[w][u] = *reinterpret_cast<const u32x4*>(rhs + (size_t)cu * RB + sl * 16);
           }
         }
 #pragma unroll

@@ -345,7 +345,7 @@ int launch_sddmm_mfma(int dtype, const SddmmParams& p, void* ws, int dense_code,
     if (int rc = sb_write_lists(t, l, p.m, tiles_n, dense_min, p.row_offsets, p.cols, stream)) return rc;
   }
   SddmmMfmaParams q{p.m, p.k, p.n, p.nnz, p.cols, p.lhs, p.rhs, p.out, t.mask, t.tile_ptr, t.brief, tiles_n,
-                    p.row_offsets, l.zeros, l.thin_ent, l.thin_cnt, l.dense_list};
+                    p.row_offsets, l.thin_ent, l.thin_cnt, l.dense_list};
   const bool bf16 = dtype == IEX_BF16;
   switch (p.k) {
     case 32: return bf16 ? launch_sddmm_mfma_ks<true, 2>(q, p.batch, stream) : launch_sddmm_mfma_ks<false, 2>(q, p.batch, stream);

@@ -55,8 +55,7 @@ struct SddmmMfmaParams {
   const int* brief;      // [tiles_n][m]
   int tiles_n;
   const int* row_offsets;
-  const unsigned* zeros;              // lists (see SbLists below)
-  const struct SbEntry* thin_ent;
+  const struct SbEntry* thin_ent;     // lists (see SbLists below)
   const int* thin_cnt;
   const unsigned short* dense_list;
 };

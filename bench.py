@@ -570,6 +570,27 @@ def run_extras(torch, ops, dev, W, IL, mats, dens, csr_dev, time_cell, time_cold
                        "operator_kernel": kernel_of(f_)})
         del rim, rom, cim
     out["sddmm_fp16_16heads_by_mask"] = rows_m
+    # the second product of attention on the same masks (values per head, n = 64): what the operator picks by itself, the same
+    # with tables and lists kept in a plan, and the row kernel
+    rows_p = []
+    v16_ = torch.randn(16, 4096, 64, device=dev, generator=torch.Generator(dev).manual_seed(5)).half()
+    for label_, c_ in masks_.items():
+        rim, _, rom, cim = csr_dev(c_)
+        pr_ = (torch.rand(16, c_.nnz, device=dev, generator=torch.Generator(dev).manual_seed(6)) / 280).half()
+        f_ = lambda: ops.spmm_sputnik_batched_values(v16_, rim, pr_, rom, cim, 4096)
+        us_op = time_cell(f_, repeats=5, samples=3)
+        name_ = kernel_of(f_)
+        row_ = {"mask": label_, "density": round(c_.nnz / 4096 / 4096, 4), "operator_us": round(us_op, 1), "operator_kernel": name_}
+        if "spmm_blocks_kernel" in name_:
+            pl_ = pyops_k.SddmmPlan()
+            g_ = lambda: pyops_k.spmm_batched_values_planned(v16_, rim, pr_, rom, cim, 4096, pl_)
+            g_()
+            row_["tables_kept_us"] = round(time_cell(g_, repeats=5, samples=3), 1)
+        with pyops_k.kernel_params(spmm={"force_variant": 1}):
+            row_["row_kernel_us"] = round(time_cell(f_, repeats=5, samples=3), 1)
+        rows_p.append(row_)
+        del rim, rom, cim, pr_
+    out["spmm_fp16_16heads_by_mask"] = rows_p
     scores = ops.sddmm_sputnik_half(qt, kt, ri3, ro3, ci3)
     us = time_cell(lambda: ops.spmm_sputnik_batched_values(vt, ri3, scores, ro3, ci3, pat.m), repeats=10)
     by = W.spmm_bytes(pat.m, pat.k, 64, pat.nnz, 16, 2, 4, True)

@@ -14,14 +14,14 @@ bool spmm_blocks_fits(int dtype, int itype, const SpmmParams& p) {
 
 // The host does not look at the pattern, so where nothing is forced the choice goes by the overall density, and only
 // for values per batch entry (attention probabilities: masks with structure).  Measured on MI355X (fp16, 16 batch
-// entries of 4096 x 4096, n = 64, microseconds, row kernel / this kernel with its setup kernels (three when measured, two now) / with tables
-// and lists kept):
-//   band of 256 + 32 scattered per row (7 %)   99 /  55 /  38     band of 512 + 32 (13 %)        184 /  75 /  51
-//   band of 128 + 16 scattered (3.5 %)          60 /  48 /  31     block diagonal 256 (6 %)        83 /  37 /  21
-//   causal window of 512 (12 %)                161 /  62 /  38     band 256 + 128 scattered (9 %) 134 / 101 /  77
-//   equal rows, columns at random:  1 %  37 / 35 / 22     3 %  62 / 77 / 59     5 %  80 / 114 / 90
-//                                  10 % 152 / 195 / 171   15 % 222 / 212 / 198  20 % 298 / 215 / 192
-// Masks with structure gain 1.3x to 4x from 3 % up; a mask without any loses 1.1x to 1.4x between 3 and 10 %.
+// entries of 4096 x 4096, n = 64, microseconds, row kernel / this kernel with its two setup kernels / with tables
+// and lists kept; bench.py, extras.spmm_fp16_16heads_by_mask):
+//   band of 256 + 32 scattered per row (7 %)   96 /  50 /  36     band of 512 + 32 (13 %)        176 /  65 /  47
+//   band of 128 + 16 scattered (3.5 %)          61 /  43 /  32     block diagonal 256 (6 %)        82 /  29 /  17
+//   causal window of 512 (12 %)                151 /  46 /  30
+//   equal rows, columns at random:  1 %  38 (stays on the row kernel)    5 %  76 / 104 / 92
+//                                  10 % 135 / 185 / 168                 20 % 268 / 242 / 228
+// Masks with structure gain 1.4x to 5x from 3 % up; a mask without any loses 1.2x to 1.4x between 3 and 15 %.
 // IEX_SPMM_FORCE_VARIANT(1) keeps the row kernel.
 bool spmm_blocks_wins(const SpmmParams& p, int batch) {
   const double density = (double)p.nnz / ((double)p.m * p.k);

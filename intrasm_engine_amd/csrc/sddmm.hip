@@ -300,14 +300,16 @@ inline bool sddmm_mfma_fits(int dtype, const SddmmParams& p) {
 inline size_t sddmm_mfma_bytes(const SddmmParams& p) { return sb_words(p.m, ceil_div(p.n, kSdBN), p.nnz) * sizeof(int); }
 
 // The host does not look at the pattern, so the choice goes by the mask's overall density.  Measured on MI355X
-// (fp16, 16 heads of 4096 x 4096, k = 64, microseconds, gather kernel / this kernel):
-//   band of 256 + 32 scattered per row (7 %)  119 /  64      band of 512 + 32 (13 %)      232 /  81
-//   band of 128 + 16 scattered (3.5 %)          74 /  53      block diagonal 256 (6 %)     102 /  38
-//   causal window of 512 (12 %)                191 /  62      band 256 + 128 scattered     150 / 109
-//   equal rows, columns at random:  1 %  32 / 40    3 %  57 / 80    5 %  98 / 120    10 %  171 / 225
-//                                  15 % 252 / 237  20 % 334 / 243
-// Masks with structure (what per-entry SDDMM is used for: attention) gain 1.4x to 3x from 3 % up; a mask without
-// any loses 1.2x to 1.3x below 15 %.  IEX_SDDMM_FORCE_VARIANT(1) keeps the gather kernel.
+// (fp16, 16 heads of 4096 x 4096, k = 64, microseconds, gather kernel / this kernel with its two setup kernels;
+// bench.py, extras.sddmm_fp16_16heads_by_mask):
+//   band of 256 + 32 scattered per row (7 %)  116 /  56      band of 512 + 32 (13 %)      216 /  70
+//   band of 128 + 16 scattered (3.5 %)          71 /  44      block diagonal 256 (6 %)      95 /  33
+//   causal window of 512 (12 %)                177 /  55
+//   equal rows, columns at random:  1 %  28 (stays on the gather kernel)   5 %  90 / 100    10 %  156 / 178
+//                                  20 % 292 / 177
+// (a caller that keeps tables and lists saves 15 of these microseconds per call).  Masks with structure (what per-entry
+// SDDMM is used for: attention) gain 1.6x to 3x from 3 % up; a mask without any loses 1.1x to 1.2x below 15 %.
+// IEX_SDDMM_FORCE_VARIANT(1) keeps the gather kernel.
 inline bool sddmm_mfma_wins(const SddmmParams& p) {
   const double density = (double)p.nnz / ((double)p.m * p.n);
   return density >= 0.03 && (double)p.batch * p.m * p.n >= 32.0 * 1024 * 1024;

@@ -712,7 +712,10 @@ int spmm_dispatch(int dtype, int itype, int flags, int m, int k, int n, int nonz
   // beyond the 256 MB last-level cache an output can only stream; the hint is worth 15-25 % of the write rate
   p.stream_out = (double)m * n * batch * (dtype == IEX_F32 ? 4 : 2) >= 128e6;
   hipStream_t s = static_cast<hipStream_t>(stream);
-  if (ch.variant == 10 && nonzeros < 8) ch.variant = 1;   // (its loads of eight values at a time need eight to exist)
+  if (ch.variant == 10 && nonzeros < 8) {   // (its loads of eight values at a time need eight to exist: the row kernel instead)
+    ch.variant = 1;
+    ch.wpr = spmm_pick_wpr(m, nonzeros, dtype == IEX_F32 ? 4 : 2, n, batch);   // (bits 8..15 meant the dense-block threshold)
+  }
   const int blocks_ready = ((flags & IEX_SPMM_TABLES_READY) ? 1 : 0) | ((flags & IEX_SPMM_LISTS_READY) ? 2 : 0);
   if (ch.variant == 0 && ch.ws && aligned(ch.ws, 16) && spmm_blocks_fits(dtype, itype, p) && spmm_blocks_wins(p, batch) &&
       ch.ws_bytes >= spmm_blocks_bytes(p))

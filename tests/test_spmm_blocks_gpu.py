@@ -122,6 +122,22 @@ def test_wider_outputs_in_slices_of_64_columns(oracle, dev, n):
         assert_close(out.float().cpu().numpy(), want, scale, RTOL[torch.bfloat16], f"n={n} blocks={blocks}")
 
 
+@pytest.mark.parametrize("blocks", [0, 2, 255])
+def test_fewer_than_eight_nonzeros_go_to_the_row_kernel(oracle, dev, blocks):
+    """The kernel reads values eight at a time; a product with fewer nonzeros than that is handed to the row kernel,
+    whatever threshold for dense blocks came with the request."""
+    rng = np.random.default_rng(blocks)
+    mask = np.zeros((70, 90), bool)
+    mask[[3, 3, 40, 69, 69], [0, 89, 17, 5, 6]] = True
+    ro, ci, _ = W.csr_from_mask(mask)
+    csr = W.CSR(70, 90, np.ones(ci.shape[0], np.float32), W.swizzle_from_offsets(ro), ro, ci)
+    values = rng.standard_normal((2, csr.nnz)).astype(np.float32)
+    dense = rng.standard_normal((2, 90, 64)).astype(np.float32)
+    out = _run(dev, csr, values, dense, torch.float16, force_variant=10, force_wpr=blocks)
+    want, scale = _want(oracle, csr, values, dense, torch.float16)
+    assert_close(out.float().cpu().numpy(), want, scale, RTOL[torch.float16], f"5 nonzeros, blocks={blocks}", atol=FP16_SUBNORMAL_HALF_STEP)
+
+
 def test_integer_operands_agree_with_the_row_kernel_exactly(dev):
     rng = np.random.default_rng(8)
     m, k = 260, 390

@@ -29,7 +29,8 @@ extern "C" {
 
 /* element types of values / dense operands */
 enum { IEX_F32 = 0, IEX_F16 = 1, IEX_BF16 = 2 };
-/* element types of column_indices */
+/* element types of column_indices (IEX_I16: SpMM with IEX_F16 values only, the combination of the reference's
+ * CudaSpmm5; every other product takes IEX_I32 and fails with IEX_ERR_UNSUPPORTED otherwise) */
 enum { IEX_I32 = 0, IEX_I16 = 1 };
 
 /* negative return codes (argument errors detected on the host) */

@@ -121,6 +121,7 @@ def _spmm(b, row_indices, values, row_offsets, column_indices, m, *, per_batch_v
     _chk(b.dtype in dtypes, f"b must be one of {dtypes}")
     _chk(values.dtype == b.dtype, "values must have the dtype of b")
     _check_index_dtypes(row_indices, row_offsets, column_indices, allow_i16)
+    _chk(column_indices.dtype != torch.int16 or b.dtype == torch.float16, "int16 column_indices go with float16 values only")
     batch, k, n = b.shape
     nonzeros = column_indices.size(0)
     m = int(m)

@@ -94,7 +94,7 @@ int iex_copy_bytes(void* dst, const void* src, size_t nbytes, void* stream);
  * the workspace iex_spmm_workspace_bytes reports: the tables of SDDMM variant 3 for the pattern, which a small
  * kernel writes first, and behind them lists that one more small kernel derives from the tables -- see
  * IEX_SPMM_TABLES_READY / IEX_SPMM_LISTS_READY; bits 8..15 set the number of nonzeros from which a block counts
- * as dense: 0 = built in (2048), 1 = every block, 255 = none, else 64 * value); fails on other shapes.
+ * as dense: 0 = built in (1536), 1 = every block, 255 = none, else 64 * value); fails on other shapes.
  * 0 = choose.
  * Families 2-6, 9 and 10 rely on strictly ascending column indices inside a row (canonical CSR, what
  * dense_to_sparse produces); family 1 accepts any order and duplicates -- force it for such

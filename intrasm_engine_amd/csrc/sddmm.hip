@@ -302,11 +302,11 @@ inline size_t sddmm_mfma_bytes(const SddmmParams& p) { return sb_words(p.m, ceil
 // The host does not look at the pattern, so the choice goes by the mask's overall density.  Measured on MI355X
 // (fp16, 16 heads of 4096 x 4096, k = 64, microseconds, gather kernel / this kernel with its two setup kernels;
 // bench.py, extras.sddmm_fp16_16heads_by_mask):
-//   band of 256 + 32 scattered per row (7 %)  116 /  56      band of 512 + 32 (13 %)      216 /  70
-//   band of 128 + 16 scattered (3.5 %)          71 /  44      block diagonal 256 (6 %)      95 /  33
-//   causal window of 512 (12 %)                177 /  55
-//   equal rows, columns at random:  1 %  28 (stays on the gather kernel)   5 %  90 / 100    10 %  156 / 178
-//                                  20 % 292 / 177
+//   band of 256 + 32 scattered per row (7 %)  114 /  54      band of 512 + 32 (13 %)      213 /  70
+//   band of 128 + 16 scattered (3.5 %)          73 /  45      block diagonal 256 (6 %)      98 /  34
+//   causal window of 512 (12 %)                173 /  55
+//   equal rows, columns at random:  1 %  29 (stays on the gather kernel)   5 %  89 / 100    10 %  155 / 177
+//                                  20 % 287 / 175
 // (a caller that keeps tables and lists saves 15 of these microseconds per call).  Masks with structure (what per-entry
 // SDDMM is used for: attention) gain 1.6x to 3x from 3 % up; a mask without any loses 1.1x to 1.2x below 15 %.
 // IEX_SDDMM_FORCE_VARIANT(1) keeps the gather kernel.

@@ -41,7 +41,11 @@ constexpr int kSdBM = 128, kSdBN = 128, kSdThreads = 256;
 constexpr int kSdShort = 4;           // nonzeros of a (row, tile) pair that the row's own lane samples
 constexpr int kSdLd = kSdBN + 8;      // halves per row of the score tile (272 bytes)
 constexpr int kSdMaxTiles = 512;      // column tiles per row (n <= 65536): the tile list lives in LDS
-constexpr int kSdDenseMin = 2048;     // nonzeros in a 128 x 128 block from which its scores come from the matrix cores
+// Nonzeros in a 128 x 128 block from which it counts as dense (matrix cores).  Measured on unstructured masks (16 heads of
+// 4096 x 4096, every block alike): laying a block out / sampling it costs the same whatever it holds, the nonzeros taken one
+// by one cost per nonzero; the two meet near 1150 nonzeros per block for the SpMM and near 1650 for the SDDMM, and the lists
+// are shared by both.  On config 3 (band + scattered) 1024 .. 1792 give the same times, 2048 two microseconds more for the SpMM.
+constexpr int kSdDenseMin = 1536;
 constexpr int kSdSlot = kSdBM * (4 + 4 + 16);   // bytes of per-row words of one dense tile: cursor, packed word, mask
 
 struct SddmmMfmaParams {

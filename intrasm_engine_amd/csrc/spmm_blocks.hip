@@ -16,12 +16,12 @@ bool spmm_blocks_fits(int dtype, int itype, const SpmmParams& p) {
 // for values per batch entry (attention probabilities: masks with structure).  Measured on MI355X (fp16, 16 batch
 // entries of 4096 x 4096, n = 64, microseconds, row kernel / this kernel with its two setup kernels / with tables
 // and lists kept; bench.py, extras.spmm_fp16_16heads_by_mask):
-//   band of 256 + 32 scattered per row (7 %)   96 /  50 /  36     band of 512 + 32 (13 %)        176 /  65 /  47
-//   band of 128 + 16 scattered (3.5 %)          61 /  43 /  32     block diagonal 256 (6 %)        82 /  29 /  17
-//   causal window of 512 (12 %)                151 /  46 /  30
-//   equal rows, columns at random:  1 %  38 (stays on the row kernel)    5 %  76 / 104 / 92
-//                                  10 % 135 / 185 / 168                 20 % 268 / 242 / 228
-// Masks with structure gain 1.4x to 5x from 3 % up; a mask without any loses 1.2x to 1.4x between 3 and 15 %.
+//   band of 256 + 32 scattered per row (7 %)   94 /  48 /  35     band of 512 + 32 (13 %)        175 /  65 /  48
+//   band of 128 + 16 scattered (3.5 %)          62 /  41 /  31     block diagonal 256 (6 %)        83 /  32 /  20
+//   causal window of 512 (12 %)                149 /  47 /  32
+//   equal rows, columns at random:  1 %  40 (stays on the row kernel)    5 %  78 / 106 / 93
+//                                  10 % 142 / 154 / 141                 20 % 265 / 149 / 134
+// Masks with structure gain 1.5x to 3x from 3 % up; a mask without any loses up to 1.4x between 3 and 10 %.
 // IEX_SPMM_FORCE_VARIANT(1) keeps the row kernel.
 bool spmm_blocks_wins(const SpmmParams& p, int batch) {
   const double density = (double)p.nnz / ((double)p.m * p.k);

@@ -16,9 +16,9 @@
 //     values: up to 4 per (row, tile) by the row's own lane from the packed word, more by the whole wavefront, four
 //     rows per step and 16 lanes per row, from the row's 128-bit mask: a lane owns 8 neighbouring columns, a
 //     population count of the mask bits below them gives the position of its first value in the row's values, one
-//     16-byte load from there holds all it owns (no column index is read), and they go to the tile as loaded when
-//     all 8 columns are present, shifted and masked when the present ones are neighbours (the edge of a band), one
-//     by one otherwise; all loads of a tile are issued before the first is used -- and multiplied on the matrix
+//     16-byte load from there holds all it owns (no column index is read), and they are spread over the columns
+//     present by byte selectors (v_perm) that a table in LDS holds for each of the 256 patterns of 8 columns, one
+//     ds_write_b128 per lane; all loads of a tile are issued before the first is used -- and multiplied on the matrix
 //     cores with the 128 rows of the dense operand that the tile names: they go through registers into LDS once per
 //     workgroup, double-buffered, 16-byte chunks permuted so that the transposing operand reads (ds_read_tr16_b64)
 //     are conflict-free.  Operands swapped (out^T = dense^T * A^T) so that a lane ends up with 4 adjacent output
@@ -57,7 +57,7 @@ struct SpmmBlocksParams {
   const unsigned short* dense_list;
 };
 
-constexpr int spmm_blocks_lds_bytes() { return 4 * kSbTileBytes + 2 * kSbStage + 4 * 32 * 32; }
+constexpr int spmm_blocks_lds_bytes() { return 4 * kSbTileBytes + 2 * kSbStage + 4 * 32 * 32 + 256 * 32; }
 
 template <bool BF16>
 __global__ __launch_bounds__(kSdThreads, 2) void spmm_blocks_kernel(SpmmBlocksParams p) {
@@ -72,7 +72,8 @@ __global__ __launch_bounds__(kSdThreads, 2) void spmm_blocks_kernel(SpmmBlocksPa
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-  unsigned* rec = reinterpret_cast<unsigned*>(sV + 2 * kSbStage) + wave * (32 * 8);                                 // [32][8]: what a wavefront's rows know of the current tile
+  unsigned* rec = reinterpret_cast<unsigned*>(sV + 2 * kSbStage) + wave * (32 * 8);
+  unsigned* spread = reinterpret_cast<unsigned*>(sV + 2 * kSbStage) + 4 * (32 * 8);   // [256][8]: see the dense part                                 // [32][8]: what a wavefront's rows know of the current tile
   // Workgroups go to the 8 XCDs round-robin by their linear id; renumbered so that an XCD gets all row blocks of a
   // batch entry (and then of the next): the dense operand of that entry stays in that XCD's L2.
   const int row_blocks = gridDim.x, total = row_blocks * gridDim.y;
@@ -163,6 +164,26 @@ __global__ __launch_bounds__(kSdThreads, 2) void spmm_blocks_kernel(SpmmBlocksPa
         const int own_row = lane >> 4, own_col8 = lane & 15;
         const int own_word = own_col8 >> 2, own_bit = (own_col8 & 3) * 8;
         const unsigned own_below = (1u << own_bit) - 1u;
+        // spread[pattern]: for each of the 256 patterns of 8 columns, byte selectors (v_perm) that take value j of 16 loaded
+        // bytes to the j-th column present and zeros to the others: words 0..3 select from the first 8 bytes (one word
+        // per pair of columns), words 4..7 from the last 8
+        {
+          const unsigned pattern = (unsigned)tid;
+          unsigned lo_sel[4] = {0u, 0u, 0u, 0u}, hi_sel[4] = {0u, 0u, 0u, 0u};
+          unsigned k = 0;
+#pragma unroll
+          for (int c = 0; c < 8; ++c) {
+            const bool present = (pattern >> c) & 1u;
+            const unsigned two = 2u * (k & 3u);
+            const unsigned pick = two | ((two + 1u) << 8), none = 0x0c0cu;
+            const unsigned from_first = present && k < 4 ? pick : none, from_last = present && k >= 4 ? pick : none;
+            lo_sel[c >> 1] |= from_first << ((c & 1) * 16);
+            hi_sel[c >> 1] |= from_last << ((c & 1) * 16);
+            k += present;
+          }
+          *reinterpret_cast<u32x4*>(spread + pattern * 8) = u32x4{lo_sel[0], lo_sel[1], lo_sel[2], lo_sel[3]};
+          *reinterpret_cast<u32x4*>(spread + pattern * 8 + 4) = u32x4{hi_sel[0], hi_sel[1], hi_sel[2], hi_sel[3]};
+        }
         u32x4 rv[4];
         int tp, bf;
         u32x4 mk;
@@ -198,9 +219,8 @@ __global__ __launch_bounds__(kSdThreads, 2) void spmm_blocks_kernel(SpmmBlocksPa
           // mask word, cursor); every lane picks from there what concerns its 8 columns: the number of the row's
           // nonzeros below its first column is the position of its first value among the row's values in the tile,
           // and the 16 bytes from there (one load at 2-byte alignment, moved back where it would pass the end of the
-          // values) hold all the values it owns.  All 8 columns present (the inside of a band): the 16 bytes go to the
-          // tile as they are.  Else they are spread over the columns present: by a shift and a mask when those are
-          // neighbours (the edge of a run), one by one otherwise.  All loads of the tile first.
+          // values) hold all the values it owns; byte selectors from the table of patterns spread them over the columns
+          // present (and zeros over the others).  All loads of the tile first.
           const unsigned longs = (unsigned)__ballot(count == 7);
           if (lane < 32) {
             const unsigned cx = __popc(mk.x), cy = cx + __popc(mk.y), cz = cy + __popc(mk.z);
@@ -237,38 +257,23 @@ __global__ __launch_bounds__(kSdThreads, 2) void spmm_blocks_kernel(SpmmBlocksPa
           for (int g = 0; g < 8; ++g) {
             const unsigned four = (longs >> (4 * g)) & 0xfu;
             if (!four) continue;   // (uniform)
-            u32x4 put = got[g];
+            u32x4 in = got[g];
             const unsigned h = have[g];
-            const bool plain = h == 0xffu;               // all 8 present: as loaded (never moved back: 8 values exist from `at`)
-            if (__ballot(h != 0 && !plain)) {
+            if (__ballot(h != 0 && back[g] != 0)) {   // (only at the end of the values: the load was moved back, move its bytes forward)
               typedef unsigned long long u64;
-              u64 lo = (u64)got[g].x | ((u64)got[g].y << 32), hi = (u64)got[g].z | ((u64)got[g].w << 32);
-              const unsigned low_bit = h & (0u - h);
-              const bool run = ((h + low_bit) & h) == 0 && back[g] == 0;   // the columns present are neighbours
-              if (__ballot(h != 0 && !plain && !run)) {
-                // any pattern: value k of the 16 bytes (counted from `back`) goes to the k-th column present
-                u64 rlo = 0, rhi = 0;
-                unsigned k = back[g];
-#pragma unroll
-                for (int c = 0; c < 8; ++c) {
-                  const u64 src = k < 4 ? lo : hi;
-                  const u64 v = ((h >> c) & 1u) ? (src >> ((k & 3) * 16)) & 0xffffull : 0ull;
-                  if (c < 4) rlo |= v << (c * 16); else rhi |= v << ((c - 4) * 16);
-                  k += (h >> c) & 1u;
-                }
-                if (!plain && !run) lo = rlo, hi = rhi;
-              }
-              if (run && !plain) {
-                // n neighbours from column s on: keep the first n values, move them up by s columns
-                const int n = __popc(h), sh = (h ? __builtin_ctz(h) : 0) * 16;
-                const u64 keep_lo = n >= 4 ? ~0ull : (1ull << (n * 16)) - 1ull;
-                const u64 keep_hi = n <= 4 ? 0ull : n >= 8 ? ~0ull : (1ull << ((n - 4) * 16)) - 1ull;
-                const u64 a = lo & keep_lo, b = hi & keep_hi;
-                lo = sh >= 64 ? 0ull : a << (sh & 63);
-                hi = sh >= 64 ? a << ((sh - 64) & 63) : (b << (sh & 63)) | (sh ? a >> ((64 - sh) & 63) : 0ull);
-              }
-              if (!plain) put = u32x4{(unsigned)lo, (unsigned)(lo >> 32), (unsigned)hi, (unsigned)(hi >> 32)};
+              const u64 lo = (u64)in.x | ((u64)in.y << 32), hi = (u64)in.z | ((u64)in.w << 32);
+              const int sh = (int)back[g] * 16;
+              const u64 nlo = sh == 0 ? lo : sh >= 64 ? hi >> ((sh - 64) & 63) : (lo >> sh) | (hi << ((64 - sh) & 63));
+              const u64 nhi = sh == 0 ? hi : sh >= 64 ? 0ull : hi >> sh;
+              in = u32x4{(unsigned)nlo, (unsigned)(nlo >> 32), (unsigned)nhi, (unsigned)(nhi >> 32)};
             }
+            // value j of the 16 bytes goes to the j-th column present: byte selectors by pattern, from the table
+            const u32x4 from_lo = *reinterpret_cast<const u32x4*>(spread + h * 8), from_hi = *reinterpret_cast<const u32x4*>(spread + h * 8 + 4);
+            u32x4 put;
+            put.x = __builtin_amdgcn_perm(in.y, in.x, from_lo.x) | __builtin_amdgcn_perm(in.w, in.z, from_hi.x);
+            put.y = __builtin_amdgcn_perm(in.y, in.x, from_lo.y) | __builtin_amdgcn_perm(in.w, in.z, from_hi.y);
+            put.z = __builtin_amdgcn_perm(in.y, in.x, from_lo.z) | __builtin_amdgcn_perm(in.w, in.z, from_hi.z);
+            put.w = __builtin_amdgcn_perm(in.y, in.x, from_lo.w) | __builtin_amdgcn_perm(in.w, in.z, from_hi.w);
             if (h) *reinterpret_cast<u32x4*>(Pw + (4 * g + own_row) * (kSdLd * 2) + own_col8 * 16) = put;
           }
           __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");

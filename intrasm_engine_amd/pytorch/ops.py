@@ -196,7 +196,7 @@ class SddmmPlan:
         self.variant = 0        # 0: the library's rule (by density); 1 / 3 after analyze()
         self.dense_share = None
 
-    def analyze(self, row_offsets, column_indices, n, dense_min=2048):
+    def analyze(self, row_offsets, column_indices, n, dense_min=1536):
         """Look at the pattern once (copies the index arrays to the host: a synchronisation, so not under capture and
         not per call) and settle which kernel the plan's calls use: the one for masks with structure when at least
         half of the nonzeros sit in 128 x 128 blocks that hold ``dense_min`` or more of them, else the gather kernel.

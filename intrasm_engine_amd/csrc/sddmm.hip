@@ -337,15 +337,9 @@ int launch_sddmm_mfma(int dtype, const SddmmParams& p, void* ws, int dense_code,
   const int tiles_n = ceil_div(p.n, kSdBN);
   const SdTables t = sd_tables(ws, p.m, tiles_n);
   const SbLists l = sb_lists(ws, p.m, tiles_n, p.nnz);
-  if (!(ready & 1)) {
-    if (int rc = sd_write_tables(t, p.m, tiles_n, p.row_offsets, p.cols, stream)) return rc;
-  }
-  if ((ready & 3) != 3) {
-    // dense_code (for tests and tuning): 0 = the built-in threshold, 1 = every tile on the matrix cores, 255 = none,
-    // else 64 * code nonzeros per 128 x 128 block
-    const int dense_min = dense_code == 0 ? kSdDenseMin : dense_code == 1 ? 0 : dense_code == 255 ? kSdBM * kSdBN + 1 : 64 * dense_code;
-    if (int rc = sb_write_lists(t, l, p.m, tiles_n, dense_min, p.row_offsets, p.cols, stream)) return rc;
-  }
+  // dense_code (for tests and tuning): 0 = the built-in threshold, 1 = every tile on the matrix cores, 255 = none,
+  // else 64 * code nonzeros per 128 x 128 block
+  if (int rc = sb_setup(t, l, p.m, tiles_n, dense_code, ready, p.row_offsets, p.cols, stream)) return rc;
   SddmmMfmaParams q{p.m, p.k, p.n, p.nnz, p.cols, p.lhs, p.rhs, p.out, t.mask, t.tile_ptr, t.brief, tiles_n,
                     p.row_offsets, l.thin_ent, l.thin_cnt, l.dense_list};
   const bool bf16 = dtype == IEX_BF16;

@@ -101,32 +101,9 @@ inline size_t sddmm_mfma_words(int m, int tiles_n) { return (size_t)m * (4 * (si
 // 6..12, 13..19).
 // The row's columns are first marked in a bit map in LDS (n bits); counts, cursors and packed words come from the
 // map, 64 tiles at a time, one tile per lane.
-static __global__ __launch_bounds__(256) void sddmm_tile_ptr_kernel(int m, int tiles_n, const int* __restrict__ row_offsets,
-                                                             const int* __restrict__ cols, int* __restrict__ tile_ptr,
-                                                             int* __restrict__ brief, u32x4* __restrict__ mask) {
-  __shared__ unsigned bits[4][kSdMaxTiles * 4];
-  const int lane = lane_id();
-  const int wave = threadIdx.x >> 6;
-  const int r = blockIdx.x * 4 + wave;
-  if (r >= m) return;   // (no workgroup barrier below: every wavefront works alone)
-  unsigned* mine = bits[wave];
-  const int s = uniform(row_offsets[r]), e = uniform(row_offsets[r + 1]);
-  for (int i = lane; i < tiles_n * 4; i += kWave) mine[i] = 0;
-  __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
-  __builtin_amdgcn_wave_barrier();
-  for (int base = s; base < e; base += 4 * kWave) {   // four loads in flight
-    int c[4];
-#pragma unroll
-    for (int u = 0; u < 4; ++u) {
-      const int j = base + u * kWave + lane;
-      c[u] = j < e ? cols[j] : -1;
-    }
-#pragma unroll
-    for (int u = 0; u < 4; ++u)
-      if (c[u] >= 0) atomicOr(&mine[min(c[u] >> 5, tiles_n * 4 - 1)], 1u << (c[u] & 31));
-  }
-  __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
-  __builtin_amdgcn_wave_barrier();
+// A row's cursors, packed words and masks from its bit map (one wavefront; the map is complete and visible to it).
+__device__ __forceinline__ void sd_row_tables(const unsigned* mine, int lane, int r, int m, int tiles_n, int s, int e,
+                                              int* __restrict__ tile_ptr, int* __restrict__ brief, u32x4* __restrict__ mask) {
   int running = s;   // position of the first nonzero of tile base_t
   for (int base_t = 0; base_t < tiles_n; base_t += kWave) {
     const int t = base_t + lane;
@@ -171,6 +148,35 @@ static __global__ __launch_bounds__(256) void sddmm_tile_ptr_kernel(int m, int t
   if (lane == 0) tile_ptr[(size_t)tiles_n * m + r] = e;
 }
 
+static __global__ __launch_bounds__(256) void sddmm_tile_ptr_kernel(int m, int tiles_n, const int* __restrict__ row_offsets,
+                                                             const int* __restrict__ cols, int* __restrict__ tile_ptr,
+                                                             int* __restrict__ brief, u32x4* __restrict__ mask) {
+  __shared__ unsigned bits[4][kSdMaxTiles * 4];
+  const int lane = lane_id();
+  const int wave = threadIdx.x >> 6;
+  const int r = blockIdx.x * 4 + wave;
+  if (r >= m) return;   // (no workgroup barrier below: every wavefront works alone)
+  unsigned* mine = bits[wave];
+  const int s = uniform(row_offsets[r]), e = uniform(row_offsets[r + 1]);
+  for (int i = lane; i < tiles_n * 4; i += kWave) mine[i] = 0;
+  __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+  __builtin_amdgcn_wave_barrier();
+  for (int base = s; base < e; base += 4 * kWave) {   // four loads in flight
+    int c[4];
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      const int j = base + u * kWave + lane;
+      c[u] = j < e ? cols[j] : -1;
+    }
+#pragma unroll
+    for (int u = 0; u < 4; ++u)
+      if (c[u] >= 0) atomicOr(&mine[min(c[u] >> 5, tiles_n * 4 - 1)], 1u << (c[u] & 31));
+  }
+  __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+  __builtin_amdgcn_wave_barrier();
+  sd_row_tables(mine, lane, r, m, tiles_n, s, e, tile_ptr, brief, mask);
+}
+
 // Where the three tables sit in a workspace of sddmm_mfma_words(m, tiles_n) words, and the launch that fills them.
 struct SdTables {
   u32x4* mask;
@@ -205,7 +211,7 @@ __device__ __forceinline__ void sd_sort_tiles(const int* __restrict__ tile_ptr, 
 #pragma unroll
     for (int u = 0; u < 8; ++u) {
       const int t = min(t0 + 4 * u, tiles_n);
-      v[u] = (unsigned)tile_ptr[(size_t)t * m + ra] + (unsigned)tile_ptr[(size_t)t * m + rb];
+      v[u] = (row0 + lane < m ? (unsigned)tile_ptr[(size_t)t * m + ra] : 0u) + (row0 + kWave + lane < m ? (unsigned)tile_ptr[(size_t)t * m + rb] : 0u);
     }
 #pragma unroll
     for (int u = 0; u < 8; ++u) {
@@ -324,6 +330,26 @@ inline int sb_write_lists(const SdTables& t, const SbLists& l, int m, int tiles_
   hipLaunchKernelGGL(sb_lists_kernel, dim3(ceil_div(m, 4)), dim3(kSdThreads), 0, stream, m, tiles_n, dense_min, t.tile_ptr, row_offsets, cols, l.dense_list,
                      l.zeros, l.thin_cnt, l.thin_ent);
   return check_hip(hipGetLastError(), "list kernel launch");
+}
+
+// dense_code (for tests and tuning): 0 = the built-in threshold, 1 = every tile on the matrix cores, 255 = none, else
+// 64 * code nonzeros per 128 x 128 block.
+inline int sb_dense_min(int dense_code) {
+  return dense_code == 0 ? kSdDenseMin : dense_code == 1 ? 0 : dense_code == 255 ? kSdBM * kSdBN + 1 : 64 * dense_code;
+}
+
+// Whatever of tables and lists the caller does not vouch for (ready: bit 0 = the tables are in the workspace, bit 1 = the
+// lists too, made with this dense_code).
+inline int sb_setup(const SdTables& t, const SbLists& l, int m, int tiles, int dense_code, int ready, const int* row_offsets, const int* cols,
+                    hipStream_t stream) {
+  const int dense_min = sb_dense_min(dense_code);
+  if (!(ready & 1)) {
+    if (int rc = sd_write_tables(t, m, tiles, row_offsets, cols, stream)) return rc;
+  }
+  if ((ready & 3) != 3) {
+    if (int rc = sb_write_lists(t, l, m, tiles, dense_min, row_offsets, cols, stream)) return rc;
+  }
+  return 0;
 }
 
 // acc + <a, b> over 8 elements of 16 bits, products and sums in fp32

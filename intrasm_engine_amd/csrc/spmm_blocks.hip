@@ -56,13 +56,7 @@ int launch_spmm_blocks(int dtype, const SpmmParams& p, int batch, void* ws, int 
   const SdTables t = sd_tables(ws, p.m, tiles_k);
   const SbLists l = sb_lists(ws, p.m, tiles_k, p.nnz);
   const int* cols = static_cast<const int*>(p.cols);
-  if (!(ready & 1)) {
-    if (int rc = sd_write_tables(t, p.m, tiles_k, p.row_offsets, cols, stream)) return rc;
-  }
-  if ((ready & 3) != 3) {
-    const int dense_min = dense_code == 0 ? kSdDenseMin : dense_code == 1 ? 0 : dense_code == 255 ? kSdBM * kSdBN + 1 : 64 * dense_code;
-    if (int rc = sb_write_lists(t, l, p.m, tiles_k, dense_min, p.row_offsets, cols, stream)) return rc;
-  }
+  if (int rc = sb_setup(t, l, p.m, tiles_k, dense_code, ready, p.row_offsets, cols, stream)) return rc;
   SpmmBlocksParams q{p.m, p.k, p.nnz, p.row_offsets, p.values, p.per_batch_values ? (size_t)p.nnz : 0, p.dense, p.out, p.n,
                      t.mask, t.tile_ptr, t.brief, tiles_k, l.zeros, l.thin_ent, l.thin_cnt, l.dense_list};
   return dtype == IEX_BF16 ? launch_blocks<true>(q, batch, stream) : launch_blocks<false>(q, batch, stream);

@@ -228,6 +228,38 @@ def test_tables_kept_between_calls_and_shared_with_the_sddmm(dev):
     assert torch.equal(again, pyops._spmm(v, ri2, vals2, rot2, cit2, m, **kw))
 
 
+def test_rows_past_the_last_one_do_not_count_towards_dense_blocks(dev):
+    """The last block of 128 rows may hold fewer: its nonzeros per column block are those of the rows that exist (the
+    cursors of the last row once stood in for the missing ones, which made a long last row count up to 128 times).
+    130 rows, the last one with 43 nonzeros in each column block: none of its blocks reaches the threshold, so the
+    row's list of nonzeros outside dense blocks holds all of them and the block's list of dense blocks is empty (read
+    from the plan's workspace: the tables, 64 words of zeros, 2 words per nonzero, the rows' counts, the lists of
+    dense blocks as 16-bit entries, tiles + 2 per block of rows)."""
+    from intrasm_engine_amd.pytorch import ops as pyops
+    rng = np.random.default_rng(3)
+    m, k = 130, 700
+    rows = [np.unique(np.concatenate([np.arange(max(0, r - 60), min(k, r + 60)), rng.integers(0, k, 3)])) for r in range(m)]
+    rows[m - 1] = np.arange(0, k, 3)
+    ro = np.zeros(m + 1, dtype=np.int32)
+    np.cumsum([len(c) for c in rows], out=ro[1:])
+    ci = np.concatenate(rows).astype(np.int32)
+    csr = W.CSR(m, k, np.ones(ci.shape[0], np.float32), W.swizzle_from_offsets(ro), ro, ci)
+    ri, _, rot, cit = to_dev(csr, dev)
+    vals = torch.from_numpy(rng.integers(-3, 4, (2, csr.nnz)).astype(np.float32)).to(dev).half()
+    dense = torch.from_numpy(rng.integers(-3, 4, (2, k, 64)).astype(np.float32)).to(dev).half()
+    kw = dict(per_batch_values=True, accumulate=False, dtypes=(torch.float16,), allow_i16=False)
+    plan = pyops.SddmmPlan()
+    got = pyops._spmm(dense, ri, vals, rot, cit, m, plan=plan, force_variant=10, **kw)
+    assert torch.equal(got, pyops._spmm(dense, ri, vals, rot, cit, m, force_variant=1, **kw))
+    tiles = (k + 127) // 128
+    words = plan.workspace.view(torch.int32).cpu().numpy()
+    lists_at = (m * (6 * tiles + 1) + 3) & ~3
+    counts_at = lists_at + 64 + 2 * csr.nnz
+    assert words[counts_at + m - 1] == len(rows[m - 1])
+    dense_lists = words[counts_at + m:].view(np.uint16)
+    assert dense_lists[0] >= 1 and dense_lists[tiles + 2] == 0      # the band in the first 128 rows; nothing in the last 2
+
+
 def test_picked_for_attention_sized_products_with_values_per_head(dev):
     """Nothing forced: 16 heads of config 3's mask take this kernel when the values differ per head, the row kernel
     when they are shared or the product is small; a plan whose analysis found no structure keeps the row kernel."""

@@ -52,6 +52,19 @@ const char* iex_last_kernels(void);
 /* 1 when a gfx950 device is visible to the HIP runtime, else 0. */
 int iex_device_ok(void);
 
+/* Does a CSR pattern meet what the faster kernel families take for granted?  ORs into *status (device memory,
+ * an int that the caller has set to 0; the launch is asynchronous on `stream`):                              */
+#define IEX_CSR_BAD_OFFSETS 0x1         /* row_offsets does not start at 0, end at nonzeros or ascend            */
+#define IEX_CSR_COLUMN_OUT_OF_RANGE 0x2 /* a column index outside [0, k)                                         */
+#define IEX_CSR_NOT_ASCENDING 0x4       /* columns of a row not strictly ascending (unsorted, or a duplicate)    */
+/* Status 0 = canonical CSR: every SpMM / SDDMM family applies.  With IEX_CSR_NOT_ASCENDING alone the pattern is
+ * still valid input for the row kernel and the SDDMM gather kernel (IEX_SPMM_FORCE_VARIANT(1),
+ * IEX_SDDMM_FORCE_VARIANT(1)), as it is for the reference, whose Sputnik kernels take columns in any order; the
+ * other families would compute something else without saying so.  One pass over the index arrays (a wavefront per
+ * row).  itype = the type of column_indices (IEX_I32 or IEX_I16).  No counterpart in the reference. */
+int iex_csr_check(int itype, int m, int k, int nonzeros, const int* row_offsets, const void* column_indices,
+                  int* status, void* stream);
+
 /* dst[0:nbytes] = src[0:nbytes] with a plain 128-bit-per-lane streaming kernel (nbytes and both
  * pointers multiples of 16).  Measurement aid with no counterpart in the reference: hardware
  * traffic counters are scaled by what they read for this copy of known size. */

@@ -23,6 +23,7 @@ SDDMM_SUM_OVER_BATCH = 0x1
 SDDMM_ACCUMULATE = 0x2
 SDDMM_TABLES_READY = 0x4
 SDDMM_LISTS_READY = 0x8
+CSR_BAD_OFFSETS, CSR_COLUMN_OUT_OF_RANGE, CSR_NOT_ASCENDING = 0x1, 0x2, 0x4
 
 _c = ctypes
 _vp, _i, _ll, _f = _c.c_void_p, _c.c_int, _c.c_longlong, _c.c_float
@@ -44,6 +45,7 @@ SIGNATURES = {
     "iex_CudaSpmm2": (_i, [_i, _i, _i, _i, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i]),
     "iex_CudaSpmm3": (_i, [_i, _i, _i, _i, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i]),
     "iex_CudaSpmm5": (_i, [_i, _i, _i, _i, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i]),
+    "iex_csr_check": (_i, [_i, _i, _i, _i, _vp, _vp, _vp, _vp]),
     "iex_sddmm_ex": (_i, [_i, _i, _i, _i, _i, _i, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i]),
     "iex_sddmm_ws": (_i, [_i, _i, _i, _i, _i, _i, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _vp, _c.c_size_t]),
     "iex_sddmm_workspace_bytes": (_c.c_size_t, [_i, _i, _i, _i, _i, _i, _i]),

@@ -51,9 +51,42 @@ namespace {
 __global__ __launch_bounds__(256) void copy_kernel(uint4* __restrict__ dst, const uint4* __restrict__ src, size_t n16) {
   for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < n16; i += (size_t)gridDim.x * 256) dst[i] = src[i];
 }
+
+// What is wrong with a CSR pattern, as bits ORed into *status: one wavefront per row.
+template <typename IT>
+__global__ __launch_bounds__(256) void csr_check_kernel(int m, int k, int nnz, const int* __restrict__ row_offsets, const IT* __restrict__ cols,
+                                                        int* status) {
+  const int lane = threadIdx.x & 63;
+  const int r = blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (r >= m) return;
+  const int s = row_offsets[r], e = row_offsets[r + 1];
+  int bad = 0;
+  if (s < 0 || e < s || e > nnz || (r == 0 && s != 0) || (r == m - 1 && e != nnz)) bad |= IEX_CSR_BAD_OFFSETS;
+  if (!bad) {
+    for (int j = s + lane; j < e; j += 64) {
+      const int c = (int)cols[j];
+      if (c < 0 || c >= k) bad |= IEX_CSR_COLUMN_OUT_OF_RANGE;
+      if (j > s && (int)cols[j - 1] >= c) bad |= IEX_CSR_NOT_ASCENDING;
+    }
+  }
+  if (bad) atomicOr(status, bad);
+}
 }  // namespace
 
 extern "C" {
+
+int iex_csr_check(int itype, int m, int k, int nonzeros, const int* row_offsets, const void* column_indices, int* status, void* stream) {
+  IEX_REQUIRE(m >= 0 && k >= 0 && nonzeros >= 0, IEX_ERR_BAD_ARGUMENT, "csr_check: negative dimension");
+  IEX_REQUIRE(status && (m == 0 || row_offsets) && (nonzeros == 0 || column_indices), IEX_ERR_BAD_ARGUMENT, "csr_check: null pointer argument");
+  IEX_REQUIRE(itype == IEX_I32 || itype == IEX_I16, IEX_ERR_UNSUPPORTED, "csr_check: column indices must be int32 or int16");
+  if (m == 0) return 0;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  if (itype == IEX_I32)
+    hipLaunchKernelGGL(csr_check_kernel<int>, dim3((m + 3) / 4), dim3(256), 0, s, m, k, nonzeros, row_offsets, static_cast<const int*>(column_indices), status);
+  else
+    hipLaunchKernelGGL(csr_check_kernel<short>, dim3((m + 3) / 4), dim3(256), 0, s, m, k, nonzeros, row_offsets, static_cast<const short*>(column_indices), status);
+  return iex::check_hip(hipGetLastError(), "csr_check launch");
+}
 
 int iex_copy_bytes(void* dst, const void* src, size_t nbytes, void* stream) {
   IEX_REQUIRE(dst && src, IEX_ERR_BAD_ARGUMENT, "copy: null pointer argument");

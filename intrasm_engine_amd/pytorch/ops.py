@@ -332,6 +332,28 @@ def sddmm_half_planned(a, b, row_indices, row_offsets, column_indices, plan: Sdd
                   dtypes=(torch.float32, torch.float16, torch.bfloat16), plan=plan)
 
 
+def csr_check(row_offsets, column_indices, k):
+    """What is wrong with a CSR pattern of ``k`` columns, as the bits of ``iex_csr_check`` (0 = canonical: offsets from 0
+    to nnz ascending, columns inside [0, k) and strictly ascending inside a row -- what every kernel family but the
+    row / gather kernels takes for granted, and what ``dense_to_sparse`` produces).  One small launch and a
+    synchronising read of its result: for set-up code, not per call.  The reference's kernels take columns in any
+    order (Sputnik), so a pattern from elsewhere is worth one check."""
+    for name, t in (("row_offsets", row_offsets), ("column_indices", column_indices)):
+        _chk(t.is_cuda, f"{name} must be a CUDA tensor")
+        _chk(t.is_contiguous(), f"{name} must be a contiguous tensor")
+    _chk(row_offsets.dtype == torch.int32, "row_offsets must be int32")
+    _chk(column_indices.dtype in (torch.int32, torch.int16), "column_indices must be int32 or int16")
+    _chk(row_offsets.device == column_indices.device, "row_offsets should be in the same device as column_indices")
+    _chk(row_offsets.numel() >= 1, "row_offsets must have m + 1 entries")
+    status = torch.zeros(1, dtype=torch.int32, device=row_offsets.device)
+    with torch.cuda.device(row_offsets.device):
+        rc = _lib.load().iex_csr_check(1 if column_indices.dtype == torch.int16 else 0, row_offsets.numel() - 1, int(k),
+                                       column_indices.numel(), row_offsets.data_ptr(), column_indices.data_ptr(),
+                                       status.data_ptr(), _stream_ptr(row_offsets.device))
+    _lib.check(rc, "csr_check")
+    return int(status.item())
+
+
 def csr_softmax_(values, row_indices, row_offsets, scale):
     _chk(values.dim() == 2, "values must be (batch, nnz)")
     for name, t in (("values", values), ("row_indices", row_indices), ("row_offsets", row_offsets)):

@@ -744,3 +744,47 @@ def test_dense_form_path_is_chosen_with_a_workspace_and_only_then(oracle, dev):
     assert lib.iex_spmm_ex(*forced) != 0 and "workspace" in _lib.last_error()
     assert lib.iex_spmm_ws(*forced, short.data_ptr(), need - 16) != 0 and "workspace" in _lib.last_error()
     torch.cuda.synchronize()
+
+
+def test_csr_check_names_what_a_pattern_lacks(dev):
+    """``iex_csr_check``: 0 for what ``dense_to_sparse`` produces; unsorted or duplicated columns (valid for the row
+    kernel and for the reference, not for the other families), a column outside the matrix, offsets that do not run
+    from 0 to nnz; int16 columns; an empty pattern.  The unsorted pattern then runs on the row kernel and still
+    equals the sorted one's product."""
+    from intrasm_engine_amd import _lib
+    from intrasm_engine_amd.pytorch import ops as pyops
+    rng = np.random.default_rng(17)
+    m, k, n = 300, 500, 64
+    lens = rng.integers(0, 40, m)
+    ro, ci = W.csr_from_row_lengths(rng, m, k, lens)
+    rot, cit = torch.from_numpy(ro).to(dev), torch.from_numpy(ci).to(dev)
+    assert pyops.csr_check(rot, cit, k) == 0
+    assert pyops.csr_check(rot, cit.to(torch.int16), k) == 0
+    assert pyops.csr_check(torch.zeros(m + 1, dtype=torch.int32, device=dev), cit[:0], k) == 0
+    r = int(np.argmax(lens >= 3))
+    swapped = ci.copy()
+    swapped[ro[r]], swapped[ro[r] + 2] = ci[ro[r] + 2], ci[ro[r]]
+    assert pyops.csr_check(rot, torch.from_numpy(swapped).to(dev), k) == _lib.CSR_NOT_ASCENDING
+    twice = ci.copy()
+    twice[ro[r] + 1] = ci[ro[r]]
+    assert pyops.csr_check(rot, torch.from_numpy(twice).to(dev), k) == _lib.CSR_NOT_ASCENDING
+    assert pyops.csr_check(rot, cit, int(ci.max())) & _lib.CSR_COLUMN_OUT_OF_RANGE
+    short = ro.copy()
+    short[-1] -= 1
+    assert pyops.csr_check(torch.from_numpy(short).to(dev), cit, k) == _lib.CSR_BAD_OFFSETS
+    back = ro.copy()
+    back[5] = back[6] + 1
+    assert pyops.csr_check(torch.from_numpy(back).to(dev), cit, k) & _lib.CSR_BAD_OFFSETS
+    # any order is fine for the row kernel: same product as the sorted pattern with the values moved along
+    values = rng.standard_normal(ci.shape[0]).astype(np.float32)
+    moved = values.copy()
+    moved[ro[r]], moved[ro[r] + 2] = values[ro[r] + 2], values[ro[r]]
+    dense = torch.from_numpy(rng.standard_normal((1, k, n)).astype(np.float32)).to(dev)
+    ri = torch.from_numpy(W.swizzle_from_offsets(ro)).to(dev)
+    kw = dict(per_batch_values=False, accumulate=False, dtypes=(torch.float32,), allow_i16=False, force_variant=1, force_wpr=1)
+    a = pyops._spmm(dense, ri, torch.from_numpy(values).to(dev), rot, cit, m, **kw)
+    b = pyops._spmm(dense, ri, torch.from_numpy(moved).to(dev), rot, torch.from_numpy(swapped).to(dev), m, **kw)
+    rows = np.ones(m, bool)
+    rows[r] = False
+    assert torch.equal(a[0, torch.from_numpy(rows)], b[0, torch.from_numpy(rows)])
+    assert torch.allclose(a[0, r], b[0, r], rtol=1e-5, atol=1e-5)

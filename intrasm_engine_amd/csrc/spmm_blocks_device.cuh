@@ -267,13 +267,16 @@ __global__ __launch_bounds__(kSdThreads, 2) void spmm_blocks_kernel(SpmmBlocksPa
               const u64 nhi = sh == 0 ? hi : sh >= 64 ? 0ull : hi >> sh;
               in = u32x4{(unsigned)nlo, (unsigned)(nlo >> 32), (unsigned)nhi, (unsigned)(nhi >> 32)};
             }
-            // value j of the 16 bytes goes to the j-th column present: byte selectors by pattern, from the table
-            const u32x4 from_lo = *reinterpret_cast<const u32x4*>(spread + h * 8), from_hi = *reinterpret_cast<const u32x4*>(spread + h * 8 + 4);
-            u32x4 put;
-            put.x = __builtin_amdgcn_perm(in.y, in.x, from_lo.x) | __builtin_amdgcn_perm(in.w, in.z, from_hi.x);
-            put.y = __builtin_amdgcn_perm(in.y, in.x, from_lo.y) | __builtin_amdgcn_perm(in.w, in.z, from_hi.y);
-            put.z = __builtin_amdgcn_perm(in.y, in.x, from_lo.z) | __builtin_amdgcn_perm(in.w, in.z, from_hi.z);
-            put.w = __builtin_amdgcn_perm(in.y, in.x, from_lo.w) | __builtin_amdgcn_perm(in.w, in.z, from_hi.w);
+            // value j of the 16 bytes goes to the j-th column present: byte selectors by pattern, from the table --
+            // unless every lane that stores has all 8 of its columns (the inside of a band): as loaded
+            u32x4 put = in;
+            if (__ballot(h != 0u && h != 0xffu)) {   // (uniform)
+              const u32x4 from_lo = *reinterpret_cast<const u32x4*>(spread + h * 8), from_hi = *reinterpret_cast<const u32x4*>(spread + h * 8 + 4);
+              put.x = __builtin_amdgcn_perm(in.y, in.x, from_lo.x) | __builtin_amdgcn_perm(in.w, in.z, from_hi.x);
+              put.y = __builtin_amdgcn_perm(in.y, in.x, from_lo.y) | __builtin_amdgcn_perm(in.w, in.z, from_hi.y);
+              put.z = __builtin_amdgcn_perm(in.y, in.x, from_lo.z) | __builtin_amdgcn_perm(in.w, in.z, from_hi.z);
+              put.w = __builtin_amdgcn_perm(in.y, in.x, from_lo.w) | __builtin_amdgcn_perm(in.w, in.z, from_hi.w);
+            }
             if (h) *reinterpret_cast<u32x4*>(Pw + (4 * g + own_row) * (kSdLd * 2) + own_col8 * 16) = put;
           }
           __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");

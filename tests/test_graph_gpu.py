@@ -239,3 +239,43 @@ def test_current_stream_is_not_the_default_stream(dev):
     cs = intrasm_engine_amd.current_stream[torch.device("cuda:0")]
     assert cs.stream == torch.cuda.current_stream()
     assert cs.stream != torch.cuda.default_stream()
+
+
+@pytest.mark.parametrize("kept_plan", [False, True])
+def test_replay_sparse_attention_with_tables_in_the_captured_workspace(dev, kept_plan):
+    """The attention block on a mask with structure, captured: the workspace with the tables and lists of the two
+    kernels for such masks comes from the capture's pool (the block's own plan) or is the caller's plan, filled before
+    the capture; the second product inside the capture reuses what the first wrote.  Replays with new q, k, v (and
+    other allocations between them) equal the eager block bit for bit."""
+    from intrasm_engine_amd import _lib
+    from intrasm_engine_amd.pytorch import ops as pyops
+    from intrasm_engine_amd.pytorch.sparse_attention import sparse_attention
+    pattern, q_np, k_np, _ = W.config3(tokens=2048, heads=8, band=128, extra=8)     # (large and dense enough for the structured kernels to be picked)
+    ri, _, ro, ci = to_dev(pattern, dev)
+    heads, tokens, d = q_np.shape
+    q, k, v = (torch.randn(heads, tokens, d, device=dev).half() for _ in range(3))
+    plan = None
+    if kept_plan:
+        plan = pyops.SddmmPlan()
+        plan.variant = 3
+        sparse_attention(q, k, v, ri, ro, ci, plan=plan)           # tables and lists are in the plan before the capture
+    constructor = TorchCUDAGraphConstructor()
+    with constructor.get_primary_stream():
+        with constructor:
+            out = sparse_attention(q, k, v, ri, ro, ci, plan=plan)
+    assert "spmm_blocks_kernel" in _lib.last_kernels()
+    constructor.instantiate_graph_exec()
+    for it in range(4):
+        for t in (q, k, v):
+            t.copy_(torch.randn(heads, tokens, d, device=dev).half())
+        clutter = [torch.full((1 << 22,), float(it), device=dev, dtype=torch.float16) for _ in range(3)]
+        torch.cuda.synchronize()
+        constructor.execute_graph()
+        constructor.synchronize()
+        eager_plan = None
+        if kept_plan:                     # (the same kernels as the captured calls: the plan settles the SDDMM's)
+            eager_plan = pyops.SddmmPlan()
+            eager_plan.variant = 3
+        assert torch.equal(out, sparse_attention(q, k, v, ri, ro, ci, plan=eager_plan)), it
+        assert all(bool((t == float(it)).all()) for t in clutter), it
+    constructor.destroy_graph_exec()

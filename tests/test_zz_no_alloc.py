@@ -51,6 +51,34 @@ def test_static_scratch_equals_caller_workspace_two_calls_in_a_row(dev, oracle):
         assert_close(got.float().cpu().numpy(), want, scale, 1e-2, f"static scratch, {a.m}x{a.k}")
 
 
+def test_static_scratch_serves_the_kernel_for_patterns_with_structure_between_other_uses(dev):
+    """Family 10 keeps tables and lists in the workspace: from the library's array they are written by every call
+    (no caller can vouch for what another call left there), also right after a dense-form call has used the same
+    bytes.  Bit-equal to iex_spmm_ws with a workspace of the caller's."""
+    from intrasm_engine_amd import _lib
+    lib = _lib.load()
+    rng = np.random.default_rng(8)
+    m = 640
+    idx = np.arange(m)
+    mask = np.abs(idx[:, None] - idx[None, :]) < 70
+    mask[np.repeat(idx, 3), rng.integers(0, m, (m, 3)).ravel()] = True
+    ro, ci, _ = W.csr_from_mask(mask)
+    band = W.CSR(m, m, rng.standard_normal(ci.shape[0]).astype(np.float32), W.swizzle_from_offsets(ro), ro, ci)
+    flags = _lib.SPMM_PER_BATCH_VALUES | (10 << 16)
+    x = torch.randn(1, m, 64, device=dev).half()
+    need = lib.iex_spmm_workspace_bytes(_lib.F16, _lib.I32, flags, m, m, 64, band.nnz, 1)
+    assert lib.iex_spmm_workspace_kind(_lib.F16, _lib.I32, flags, m, m, 64, band.nnz, 1) == 10 and 0 < need < (96 << 20)
+    want = _call(lib, lib.iex_spmm_ws, dev, band, x, torch.int32, ws=torch.empty(need, dtype=torch.uint8, device=dev), flags=flags)
+    assert "spmm_blocks_kernel" in _lib.last_kernels()
+    first = _call(lib, lib.iex_spmm_static, dev, band, x, torch.int32, flags=flags)
+    other = W.pruned_weight(43, 1024, 1024, 0.70)                             # a dense-form call overwrites the array
+    _call(lib, lib.iex_spmm_static, dev, other, torch.randn(1, 1024, 1024, device=dev).half(), torch.int16)
+    assert "csr_to_dense_kernel" in _lib.last_kernels()
+    again = _call(lib, lib.iex_spmm_static, dev, band, x, torch.int32, flags=flags)
+    assert _lib.last_kernels().split(" + ") == ["sddmm_tile_ptr_kernel", "sb_lists_kernel", "spmm_blocks_kernel<false>"]
+    assert torch.equal(first, want) and torch.equal(again, want)
+
+
 def test_static_scratch_without_workspace_use_runs_as_the_plain_entry_point(dev):
     """fp32 operands never use the workspace: the call must equal iex_spmm_ex bit for bit."""
     from intrasm_engine_amd import _lib

@@ -160,7 +160,7 @@ def _spmm(b, row_indices, values, row_offsets, column_indices, m, *, per_batch_v
             # with structure: a plan shared with that operator's calls on the pattern serves both
             key = (row_offsets.data_ptr(), column_indices.data_ptr(), row_offsets._version, column_indices._version,
                    m, k, nonzeros)
-            if plan._ready(key, ws_bytes, b.device):
+            if plan._ready(key, ws_bytes, b.device, (row_offsets, column_indices)):
                 flags |= _lib.SPMM_TABLES_READY
                 code = (flags >> 8) & 0xff if ((flags >> 16) & 0xf) == 10 else 0    # (what counts as a dense block: the lists depend on it)
                 if plan.lists_key == (key, code):
@@ -194,6 +194,7 @@ class SddmmPlan:
         self.key = None
         self.lists_key = None   # (the lists behind the tables also depend on what counts as a dense block)
         self.variant = 0        # 0: the library's rule (by density); 1 / 3 after analyze()
+        self._index_tensors = ()
         self.dense_share = None
 
     def analyze(self, row_offsets, column_indices, n, dense_min=1536):
@@ -212,14 +213,17 @@ class SddmmPlan:
         self.variant = 3 if self.dense_share >= 0.5 else 1
         return self.variant
 
-    def _ready(self, key, nbytes, device):
-        """Workspace of nbytes for this key; True when it already holds the key's tables."""
+    def _ready(self, key, nbytes, device, index_tensors=()):
+        """Workspace of nbytes for this key; True when it already holds the key's tables.  The plan keeps the index
+        tensors of its key alive: the key names them by address and version, and an address that the allocator has
+        handed to another tensor since would pass for the old pattern."""
         if self.workspace is None or self.workspace.numel() < nbytes or self.workspace.device != device:
             self.workspace = torch.empty(nbytes, dtype=torch.uint8, device=device)
             self.key = None
             self.lists_key = None
         ready = self.key == key
         self.key = key
+        self._index_tensors = tuple(index_tensors)
         return ready
 
 
@@ -268,7 +272,7 @@ def _sddmm(a, b, row_indices, row_offsets, column_indices, *, sum_over_batch, dt
             key = (row_offsets.data_ptr(), column_indices.data_ptr(), row_offsets._version, column_indices._version,
                    m, n, nonzeros)
             code = (flags >> 8) & 0xff if ((flags >> 16) & 0xf) == 3 else 0     # (what counts as a dense block: the lists depend on it)
-            if plan._ready(key, ws_bytes, a.device):
+            if plan._ready(key, ws_bytes, a.device, (row_offsets, column_indices)):
                 flags |= _lib.SDDMM_TABLES_READY
                 if plan.lists_key == (key, code):
                     flags |= _lib.SDDMM_LISTS_READY

@@ -216,3 +216,35 @@ def test_refusals(dev):
     assert lib.iex_sddmm_workspace_kind(_lib.F16, 0, 4096, 64, 4096, 1150000, 16) == 3
     assert lib.iex_sddmm_workspace_kind(_lib.F16, 0, 1024, 4096, 1024, 300000, 1) == 7
     assert lib.iex_sddmm_workspace_kind(_lib.F32, 0, 4096, 64, 4096, 1150000, 16) == 0
+
+
+def test_plan_keeps_the_index_tensors_of_its_tables_alive(dev):
+    """The plan names a pattern by the addresses and versions of its index tensors.  If the caller drops them, the
+    allocator may hand the same addresses to another pattern of the same size: the plan holds the tensors, so that
+    cannot happen, and the other pattern gets tables of its own."""
+    import gc
+    from intrasm_engine_amd.pytorch import ops as pyops
+    m = 512
+    idx = np.arange(m)
+
+    def pattern(shift):
+        mask = np.abs(idx[:, None] - ((idx[None, :] + shift) % m)) < 40
+        ro, ci, _ = W.csr_from_mask(mask)
+        return W.CSR(m, m, np.ones(ci.shape[0], np.float32), W.swizzle_from_offsets(ro), ro, ci)
+
+    first, second = pattern(0), pattern(100)
+    assert first.nnz == second.nnz                                   # same sizes: the allocator would reuse the blocks
+    q = torch.randn(2, m, 64, device=dev).half()
+    k = torch.randn(2, m, 64, device=dev).half()
+    plan = pyops.SddmmPlan()
+    plan.variant = 3
+    ri, _, ro, ci = to_dev(first, dev)
+    pyops.sddmm_half_planned(q, k, ri, ro, ci, plan)
+    addresses = (ro.data_ptr(), ci.data_ptr())
+    del ro, ci
+    gc.collect()
+    ri2, _, ro2, ci2 = to_dev(second, dev)
+    assert (ro2.data_ptr(), ci2.data_ptr()) != addresses             # the plan still holds the first pattern's tensors
+    got = pyops.sddmm_half_planned(q, k, ri2, ro2, ci2, plan)
+    want = pyops._sddmm(q, k, ri2, ro2, ci2, sum_over_batch=False, dtypes=(torch.float16,), force_variant=3)
+    assert torch.equal(got, want)

@@ -83,6 +83,11 @@ int iex_copy_bytes(void* dst, const void* src, size_t nbytes, void* stream);
  * outside them) are still there too, from a family-10 call with the same bits 8..15.  Only with
  * IEX_SPMM_TABLES_READY.                                                                              */
 #define IEX_SPMM_LISTS_READY 0x10
+/* The column indices of a row may come in any order and repeat (what the reference's Sputnik kernels accept,
+ * sputnik_spmm.cu.inc:229-243): with nothing forced the call keeps to the families that take such input (1 and 8).
+ * The drop-ins iex_CudaSpmm2 / 3 / 5 below always set it: they know nothing about where their arrays come from.
+ * Ignored when bits 16..19 force a family.                                                             */
+#define IEX_SPMM_ANY_COLUMN_ORDER 0x20
 /* bits 8..15: force waves-per-row (1, 4 or 8); 0 = choose from nnz/m.  For tuning.    */
 #define IEX_SPMM_FORCE_WPR(w) (((w) & 0xff) << 8)
 /* bits 16..19: force the kernel family: 1 = row kernel gathering from L2, 2 = LDS-staged
@@ -170,7 +175,8 @@ int iex_spmm_workspace_kind(int dtype, int itype, int flags, int m, int k, int n
  * IEX_ERR_TOO_LARGE before anything is launched; a call that would not use a workspace runs as iex_spmm_ex.
  * All calls on one GPU share that GPU's array: two calls whose work may overlap in time (different streams,
  * different threads) race on it -- order them, or give one of them iex_spmm_ws with memory of its own.  The
- * array keeps the previous call's contents; every kernel that reads it writes what it reads first.
+ * array keeps the previous call's contents; every kernel that reads it writes what it reads first
+ * (IEX_SPMM_TABLES_READY / IEX_SPMM_LISTS_READY are ignored here: the array is nobody's to keep).
  * No counterpart in the reference (its launchers take no workspace, csrc/extensions.h:28-30). */
 #define IEX_SPMM_STATIC_SCRATCH_BYTES ((size_t)96 << 20)
 int iex_spmm_static(int dtype, int itype, int flags, int m, int k, int n, int nonzeros,
@@ -179,7 +185,9 @@ int iex_spmm_static(int dtype, int itype, int flags, int m, int k, int n, int no
                     void* out, void* stream, int batch);
 size_t iex_spmm_static_scratch_bytes(void);
 
-/* Drop-ins for the three launchers the reference declares in csrc/extensions.h:28-30.
+/* Drop-ins for the three launchers the reference declares in csrc/extensions.h:28-30.  Like the reference's they accept
+ * column indices in any order inside a row, and duplicates (IEX_SPMM_ANY_COLUMN_ORDER is always set: the row kernel,
+ * or the few-columns kernel); a caller that knows its CSR arrays to be canonical gets every family from iex_spmm_ex.
  * CudaSpmm2: fp32, per-batch values (batch, nnz), accumulates into `out`
  *            (spmm_sputnik_atomic, sputnik_kernels.cpp:170-172);
  * CudaSpmm3: fp32, values shared by the batch (spmm_sputnik_reuse_weight, :173-175);
@@ -209,6 +217,10 @@ int iex_CudaSpmm5(int m, int k, int n, int nonzeros, const int* row_indices,
  * are still there too, from a call with the same bits 8..15 -- of iex_sddmm_ws, or of iex_spmm_ws family 10 on the same
  * pattern: the lists are the same.  Only with IEX_SDDMM_TABLES_READY.                                              */
 #define IEX_SDDMM_LISTS_READY 0x8
+/* The column indices of a row may come in any order and repeat (sputnik_sddmm.cu.inc:137 reads them as they come):
+ * with nothing forced the call keeps to the gather kernel and the dense-product path, which take such input.
+ * Ignored when bits 16..19 force a variant.                                                            */
+#define IEX_SDDMM_ANY_COLUMN_ORDER 0x10
 /* bits 8..15: force wavefronts per row (1 or 4); 0 = choose from nnz/m.  For tuning.
  * With variant 3 the same bits set the number of nonzeros from which a 128 x 128 block of the
  * mask counts as dense: 0 = built in, 1 = every block, 255 = none, else 64 * value.       */
@@ -281,8 +293,9 @@ int iex_csr_softmax(int dtype, int m, int nonzeros, const int* row_indices,
  * stride_* are element strides between batch entries (0 = operand shared by the batch).
  * Bits 4..7 of trans_b force the kernel for tuning: 5 = 128x128, 6 = 128x256, 7 = 256x256 tiles,
  * 8 = 128x128 and 9 = 64x128 by eight waves with K steps of 64 (few tiles, long K), 10 = 128x256 by eight waves
- * (11: with K steps of 64), 12 = 256x256 with K split over two workgroups per tile (iex_gemm_ws only), all with the
- * operands loaded from global memory straight into LDS (0 = choose picks among 5 and 7..10);
+ * (11: with K steps of 64), 12 = 256x256 with K split over two workgroups per tile (iex_gemm_ws only), 13 = 256x256 by
+ * eight waves in two groups that take turns: one reads operand fragments and issues loads while the other multiplies,
+ * all with the operands loaded from global memory straight into LDS (0 = choose picks among 5, 8, 9, 10 and 13);
  * 1 = 128x128, 2 = 128x256, 3 = 256x256, 4 = 128x128 with K steps of 64, operands staged through
  * registers.  K % 8 == 0, N % 8 == 0 for a (K,N) B, 16-byte aligned operands.
  * Replaces the cuBLAS / CUTLASS / Triton companions of tests/test_interleaving.py:26-345. */
@@ -295,7 +308,9 @@ int iex_gemm(int dtype, int trans_b, int M, int N, int K, const void* A, const v
  * of trans_b) = 256 x 256 tiles with K split over two workgroups per tile; the first of the two to
  * finish leaves its fp32 partial sums in the workspace (M * N * 4 bytes rounded up to whole tiles, plus
  * two words per tile; 256-byte aligned), the other adds them to its own and stores the tile; the result
- * does not depend on which was first.  The exchange goes through the L2 of the XCD that both workgroups
+ * does not depend on which was first.  The second workgroup's wait is bounded; if it ever gave up, the tile is left
+ * unwritten and its "written" word (the second half of the words behind the partial sums) reads -1 after the launch
+ * instead of 1: stale sums are never added.  The exchange goes through the L2 of the XCD that both workgroups
  * run on (workgroup ids b and b + 8: ids are dealt round-robin to the 8 XCDs in the mode this library is
  * built for, one partition spanning the whole GPU).  K >= 64, plain store.  Code 12 fails without the workspace;
  * every other code ignores it and runs exactly as iex_gemm.  iex_gemm_workspace_bytes returns 0 where

@@ -19,10 +19,12 @@ SPMM_ACCUMULATE = 0x2
 SPMM_RELU = 0x4
 SPMM_TABLES_READY = 0x8
 SPMM_LISTS_READY = 0x10
+SPMM_ANY_COLUMN_ORDER = 0x20
 SDDMM_SUM_OVER_BATCH = 0x1
 SDDMM_ACCUMULATE = 0x2
 SDDMM_TABLES_READY = 0x4
 SDDMM_LISTS_READY = 0x8
+SDDMM_ANY_COLUMN_ORDER = 0x10
 CSR_BAD_OFFSETS, CSR_COLUMN_OUT_OF_RANGE, CSR_NOT_ASCENDING = 0x1, 0x2, 0x4
 
 _c = ctypes

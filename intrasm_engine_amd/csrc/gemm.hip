@@ -1,6 +1,6 @@
 // Host side of the dense companion GEMM: kernel wrapper, tile-shape choice, XCD-aware
 // tile order, argument checks and the C entry point.  Device code: gemm_device.cuh.
-#include "gemm_dma_device.cuh"
+#include "gemm_pp_device.cuh"
 
 namespace iex {
 namespace {
@@ -68,6 +68,37 @@ int launch_dma(GemmParams p, int batch, hipStream_t stream) {
   }
   note_kernel("gemm_dma_kernel<%s, %s, %d, %d, %d, %d, %d> (%d x %d tiles, %d waves)", BF16 ? "bf16" : "f16", TRANS_B ? "B(N,K)" : "B(K,N)", WM, WN,
               BK, STAGES, WCN, BM, BN, 2 * WCN);
+  hipLaunchKernelGGL(kern, dim3(per_xcd * kXcds, batch), dim3(WCN * 128), lds, stream, p);
+  return check_hip(hipGetLastError(), "gemm launch");
+}
+
+// Eight wavefronts in two groups that alternate between reading / loading and multiplying (gemm_pp_device.cuh).
+template <bool BF16, bool TRANS_B, int WM, int WN, int WCN>
+__global__ __launch_bounds__(WCN * 128, 1) void gemm_pp_kernel(GemmParams p) {
+  extern __shared__ __align__(16) unsigned char smem[];
+  int tile_m, tile_n;
+  if (!xcd_tile(blockIdx.x, p.tiles_m, p.tiles_n, tile_m, tile_n)) return;  // uniform per block
+  gemm_tile_pp<BF16, TRANS_B, WM, WN, WCN>(p, tile_m, tile_n, blockIdx.y, smem);
+}
+
+template <bool BF16, bool TRANS_B, int WM, int WN, int WCN>
+int launch_pp(GemmParams p, int batch, hipStream_t stream) {
+  constexpr int BM = 2 * WM * 32, BN = WCN * WN * 32;
+  p.tiles_m = ceil_div(p.M, BM);
+  p.tiles_n = ceil_div(p.N, BN);
+  const int total = p.tiles_m * p.tiles_n;
+  const int per_xcd = (total + kXcds - 1) / kXcds;
+  constexpr int lds = gemm_pp_lds_bytes<BF16, TRANS_B, WM, WN, WCN>();
+  auto kern = gemm_pp_kernel<BF16, TRANS_B, WM, WN, WCN>;
+  static thread_local bool raised = false;  // per instantiation
+  if (!raised) {
+    if (int rc = check_hip(hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, lds),
+                           "hipFuncSetAttribute(LDS size)"))
+      return rc;
+    raised = true;
+  }
+  note_kernel("gemm_pp_kernel<%s, %s, %d, %d, %d> (%d x %d tiles, two groups of 4 waves in alternating phases)", BF16 ? "bf16" : "f16",
+              TRANS_B ? "B(N,K)" : "B(K,N)", WM, WN, WCN, BM, BN);
   hipLaunchKernelGGL(kern, dim3(per_xcd * kXcds, batch), dim3(WCN * 128), lds, stream, p);
   return check_hip(hipGetLastError(), "gemm launch");
 }
@@ -153,6 +184,7 @@ int launch_shape(const GemmParams& p, int batch, int force, hipStream_t stream, 
   if (force == 9) return launch_dma<BF16, TRANS_B, 1, 1, 64, 4, 4>(p, batch, stream);
   if (force == 10) return launch_dma<BF16, TRANS_B, 2, 2, 32, 4, 4>(p, batch, stream);
   if (force == 11) return launch_dma<BF16, TRANS_B, 2, 2, 64, 3, 4>(p, batch, stream);
+  if (force == 13) return launch_pp<BF16, TRANS_B, 4, 2, 4>(p, batch, stream);
   // Default: operands straight from global memory into LDS (gemm_dma_device.cuh).  The larger the
   // tile of a wave, the fewer LDS bytes each MFMA needs, and LDS time is what the main loop runs
   // against; the smaller the tile, the more workgroups there are to fill 256 CUs, and a tile wider
@@ -177,7 +209,10 @@ int launch_shape(const GemmParams& p, int batch, int force, hipStream_t stream, 
       return (double)ceil_div(tiles, slots) * slots * bm * bn / rate;
     };
     const double huge = cost(256, 256, 256, 1200.0), wide = cost(128, 256, 256, 930.0), small = cost(128, 128, 512, 750.0);
-    if (huge <= wide && huge <= small) return launch_dma<BF16, TRANS_B, 4, 4, 32, 4>(p, batch, stream);
+    // (256 x 256 by two groups of four waves in alternating phases, same-process comparison with the four-wave tile on
+    // warmed-up clocks: 8192^3 1250 / 1230, 4096 x 8192 x 4096 1109 / 1076, 11008 x 8192 x 4096 1151 / 1109,
+    // 4096^3 1054 / 954; bit-equal results)
+    if (huge <= wide && huge <= small) return launch_pp<BF16, TRANS_B, 4, 2, 4>(p, batch, stream);
     if (wide <= small) return launch_dma<BF16, TRANS_B, 2, 2, 32, 4, 4>(p, batch, stream);
     return launch_dma<BF16, TRANS_B, 2, 2, 32, 4>(p, batch, stream);
   }
@@ -201,7 +236,8 @@ int launch_shape(const GemmParams& p, int batch, int force, hipStream_t stream, 
 // 1 = 128x128 tiles, 2 = 128x256, 3 = 256x256, 4 = 128x128 with K steps of 64.  Operands loaded
 // straight into LDS: 5 = 128x128, 6 = 128x256, 7 = 256x256, 8 = 128x128, 9 = 64x128 by eight waves with K steps of 64,
 // 10 = 128x256 by eight waves, 11 = the same with K steps of 64, 12 = 256x256 with K split over two workgroups per tile
-// (iex_gemm_ws only; never chosen).  0 = choose (one of 5..10).
+// (iex_gemm_ws only; never chosen), 13 = 256x256 by eight waves in two groups that alternate between loading and
+// multiplying.  0 = choose (one of 5, 8, 9, 10, 13).
 extern "C" int iex_gemm(int dtype, int trans_b_and_shape, int M, int N, int K, const void* A, const void* B, void* C, int batch,
                         long long stride_a, long long stride_b, long long stride_c, void* stream) {
   iex::trail_reset();

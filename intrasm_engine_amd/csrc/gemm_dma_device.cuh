@@ -29,8 +29,11 @@
 
 namespace iex {
 
+#ifndef IEX_DMA_MOD
+#define IEX_DMA_MOD ""
+#endif
 __device__ __forceinline__ void lds_dma16(const void* g, unsigned lds_base_uniform) {
-  asm volatile("s_mov_b32 m0, %1\n\tglobal_load_lds_dwordx4 %0, off" ::"v"(g), "s"(lds_base_uniform) : "memory", "m0");
+  asm volatile("s_mov_b32 m0, %1\n\tglobal_load_lds_dwordx4 %0, off" IEX_DMA_MOD ::"v"(g), "s"(lds_base_uniform) : "memory", "m0");
 }
 // (for the loop-ablation benchmark: the address arithmetic of a direct load without the load)
 __device__ __forceinline__ void lds_dma16_address_only(const void* g, unsigned lds_base_uniform) {
@@ -295,18 +298,28 @@ __device__ __forceinline__ void gemm_tile_dma(const GemmParams& p, int tile_m, i
             *reinterpret_cast<f32x4*>(mine + ((i * WN + j) * 4 + q) * 256) = v;
             if (q == 3) __builtin_amdgcn_sched_barrier(0);
           }
-      // The two workgroups of a tile run on one XCD (the launcher's numbering), whose L2 both see: once my stores
-      // have left the CU (the workgroup-scope fence waits for that) the flag may go up.  Device-scope fences here
-      // would write back and invalidate that L2 under every workgroup still multiplying (measured: 2.5 x slower).
+      // The two workgroups of a tile run on one XCD (the launcher's numbering; one partition spanning the whole GPU,
+      // ids dealt round-robin to the XCDs), whose L2 both see.  Every wavefront waits until L2 has acknowledged its own
+      // stores (vmcnt counts stores until then), the barrier collects all of them, and only then the flag goes up.
+      // Device-scope fences here would write back and invalidate that L2 under every workgroup still multiplying
+      // (measured: 2.5 x slower).
+      wait_vmcnt<0>();
       __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
       __syncthreads();
       if (tid == 0) __hip_atomic_store(&written[tile_id], 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
       return;
     }
-    if (tid == 0)   // (bounded: about a tenth of a second, far beyond any epilogue; a kernel must end whatever happens)
-      for (int spins = 0; spins < (1 << 20) && __hip_atomic_load(&written[tile_id], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == 0; ++spins)
+    // (bounded: about a tenth of a second, far beyond any epilogue; a kernel must end whatever happens.  A wait that gives
+    // up says so in the tile's flag word -- the host-visible error mark -- and the tile is not stored: never stale sums.)
+    if (tid == 0) {
+      int seen = 0;
+      for (int spins = 0; spins < (1 << 20) && (seen = __hip_atomic_load(&written[tile_id], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)) == 0; ++spins)
         __builtin_amdgcn_s_sleep(4);
+      if (seen == 0) __hip_atomic_store(&written[tile_id], -1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      *reinterpret_cast<volatile int*>(smem + 4) = seen;   // (the word after the ticket's: slow threads may still be reading that one)
+    }
     __syncthreads();
+    if (*reinterpret_cast<volatile int*>(smem + 4) == 0) return;   // (uniform) the partner never published: leave the tile unwritten, flag = -1
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");   // (this CU has never read these lines: they come from L2)
     partial = mine;   // added where the sums are rounded and stored (adding them here would need all 256 sums in VGPRs at once)
   }

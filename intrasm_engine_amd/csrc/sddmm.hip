@@ -278,7 +278,8 @@ int launch_sddmm_dense(int dtype, const SddmmParams& p, void* ws, hipStream_t st
   for (int z = 0; z < p.batch; ++z) {
     const uint16_t* lhs = static_cast<const uint16_t*>(p.lhs) + (size_t)z * p.m * p.k;
     const uint16_t* rhs = static_cast<const uint16_t*>(p.rhs) + (size_t)z * p.n * p.k;
-    if (int rc = iex_gemm(dtype, 1, p.m, p.n, p.k, lhs, rhs, ws, 1, 0, 0, 0, stream)) return rc;
+    // (the dispatcher, not the public entry point: that one starts a new trail of kernel names)
+    if (int rc = gemm_dispatch(dtype, 1, p.m, p.n, p.k, lhs, rhs, ws, 1, 0, 0, 0, stream, nullptr, 0, 0)) return rc;
     note_kernel("sample_dense_kernel");
     hipLaunchKernelGGL(sample_dense_kernel, dim3(ceil_div(p.m, 4)), dim3(256), 0, stream, p.m, p.n, p.row_offsets, p.cols,
                        static_cast<const uint16_t*>(ws), static_cast<uint16_t*>(p.out) + (size_t)z * p.nnz);
@@ -363,7 +364,8 @@ int sddmm_workspace_kind(int dtype, int flags, int m, int k, int n, int nonzeros
   void* const some_aligned = reinterpret_cast<void*>(size_t(256));
   SddmmParams p{m, k, n, nonzeros, batch, nullptr, nullptr, nullptr, some_aligned, some_aligned, nullptr,
                 (flags & IEX_SDDMM_SUM_OVER_BATCH) != 0, (flags & IEX_SDDMM_ACCUMULATE) != 0};
-  if (variant != 7 && sddmm_mfma_fits(dtype, p) && (variant == 3 || sddmm_mfma_wins(p))) return 3;
+  const bool any_order = (flags & IEX_SDDMM_ANY_COLUMN_ORDER) != 0;
+  if (variant != 7 && sddmm_mfma_fits(dtype, p) && (variant == 3 || (!any_order && sddmm_mfma_wins(p)))) return 3;
   if (variant == 3 || !sddmm_dense_fits(dtype, p)) return 0;
   return (variant == 7 || sddmm_dense_wins(p)) ? 7 : 0;
 }
@@ -375,7 +377,8 @@ size_t sddmm_workspace_bytes(int dtype, int flags, int m, int k, int n, int nonz
   void* const some_aligned = reinterpret_cast<void*>(size_t(256));
   SddmmParams p{m, k, n, nonzeros, batch, nullptr, nullptr, nullptr, some_aligned, some_aligned, nullptr,
                 (flags & IEX_SDDMM_SUM_OVER_BATCH) != 0, (flags & IEX_SDDMM_ACCUMULATE) != 0};
-  if (variant != 7 && sddmm_mfma_fits(dtype, p) && (variant == 3 || sddmm_mfma_wins(p))) return sddmm_mfma_bytes(p);
+  const bool any_order = (flags & IEX_SDDMM_ANY_COLUMN_ORDER) != 0;
+  if (variant != 7 && sddmm_mfma_fits(dtype, p) && (variant == 3 || (!any_order && sddmm_mfma_wins(p)))) return sddmm_mfma_bytes(p);
   if (variant == 3) return 0;
   if (!sddmm_dense_fits(dtype, p)) return 0;
   if (variant == 0 && !sddmm_dense_wins(p)) return 0;
@@ -401,7 +404,8 @@ int sddmm_dispatch(int dtype, int flags, int m, int k, int n, int nonzeros, cons
   if (wpr != 1 && wpr != 4) wpr = ((double)nonzeros / m >= 64.0) ? 4 : 1;
   hipStream_t s = static_cast<hipStream_t>(stream);
   const int variant = (flags >> 16) & 0xf;  // 0 = choose, 1 = gather kernel, 3 = score tiles on the matrix cores, 7 = dense product then sampling
-  if (variant == 0 || variant == 3) {
+  const bool any_order = (flags & IEX_SDDMM_ANY_COLUMN_ORDER) != 0;   // (the tables of variant 3 assume ascending, distinct columns)
+  if ((variant == 0 && !any_order) || variant == 3) {
     const bool fits = sddmm_mfma_fits(dtype, p);
     const bool room = workspace && aligned(workspace, 16) && workspace_bytes >= sddmm_mfma_bytes(p);
     if (variant == 3) {
@@ -458,7 +462,7 @@ int iex_sddmm_workspace_kind(int dtype, int flags, int m, int k, int n, int nonz
 int iex_CudaSddmm2(int m, int k, int n, int nonzeros, const int* row_indices, const int* row_offsets,
                    const int* column_indices, const float* lhs_matrix, const float* rhs_matrix,
                    float* output_values, void* stream, int batch_size) {
-  return iex::sddmm_dispatch(IEX_F32, IEX_SDDMM_SUM_OVER_BATCH, m, k, n, nonzeros, row_indices,
+  return iex::sddmm_dispatch(IEX_F32, IEX_SDDMM_SUM_OVER_BATCH | IEX_SDDMM_ANY_COLUMN_ORDER, m, k, n, nonzeros, row_indices,
                              row_offsets, column_indices, lhs_matrix, rhs_matrix, output_values, stream,
                              batch_size, nullptr, 0);
 }

@@ -357,7 +357,7 @@ template <typename T>
 KsplitPlan ksplit_plan(const SpmmParams& p, int batch, int force_slices, int force_waves) {
   KsplitPlan pl;
   constexpr int kMax = 16 / (int)sizeof(T);
-  if (!(p.nnz > 0 && p.n >= kMax && p.n % kMax == 0 && p.k <= 262144 && aligned(p.dense, 16) && aligned(p.out, 16))) return pl;
+  if (!(p.nnz > 0 && p.k > 0 && p.n >= kMax && p.n % kMax == 0 && p.k <= 262144 && aligned(p.dense, 16) && aligned(p.out, 16))) return pl;
   int vec = kMax;
   while (vec > kMax / 4 && kWave * (vec / 2) >= p.n) vec >>= 1;   // the narrowest tile that holds n
   pl.vec = vec;
@@ -424,6 +424,7 @@ struct Choice {
   int lpg = 0;      // lanes per nonzero of the row kernel: 8, 16, 32 or 64 (0 = choose)
   void* ws = nullptr;   // caller's workspace for the dense form of A (variant 7), may be null
   size_t ws_bytes = 0;
+  bool any_order = false;   // columns of a row in any order, possibly repeated: families 1 and 8 only
 };
 
 // The LDS-staged kernel needs a full-width tile (64 lanes x VEC, VEC the full or half 128-bit
@@ -592,8 +593,14 @@ int launch_dense_path(const SpmmParams& p, int batch, const Choice& ch, hipStrea
 }
 
 template <typename T, typename IT>
-int launch_typed(const SpmmParams& p, int batch, const Choice& ch, hipStream_t stream) {
+int launch_typed(const SpmmParams& p, int batch, const Choice& given, hipStream_t stream) {
   constexpr int kMax = 16 / (int)sizeof(T);
+  Choice ch = given;
+  // Columns in any order: the few-columns kernel where it applies (it takes nonzeros as they come), else the row kernel.
+  if (ch.any_order && ch.variant == 0) {
+    if (smallk_wanted<T>(p, batch)) return launch_smallk<T, IT>(p, batch, stream);
+    ch.variant = 1;
+  }
   // A with few columns and rows that gather, wide output: the tile of the dense operand in LDS, rows
   // streamed (spmm_smallk_device.cuh; smallk_wanted has the measurements).  16-bit products that are
   // dense enough go to the dense-form path first (time model above).
@@ -706,6 +713,7 @@ int spmm_dispatch(int dtype, int itype, int flags, int m, int k, int n, int nonz
   ch.lpg = ((flags >> 28) & 0x7) ? (4 << ((flags >> 28) & 0x7)) : 0;
   ch.ws = workspace;
   ch.ws_bytes = workspace ? workspace_bytes : 0;
+  ch.any_order = (flags & IEX_SPMM_ANY_COLUMN_ORDER) != 0;
   SpmmParams p{m, k, n, nonzeros, row_indices, values, row_offsets, column_indices, dense, bias, out,
                (flags & IEX_SPMM_PER_BATCH_VALUES) != 0, (flags & IEX_SPMM_ACCUMULATE) != 0,
                (flags & IEX_SPMM_RELU) != 0};
@@ -717,7 +725,7 @@ int spmm_dispatch(int dtype, int itype, int flags, int m, int k, int n, int nonz
     ch.wpr = spmm_pick_wpr(m, nonzeros, dtype == IEX_F32 ? 4 : 2, n, batch);   // (bits 8..15 meant the dense-block threshold)
   }
   const int blocks_ready = ((flags & IEX_SPMM_TABLES_READY) ? 1 : 0) | ((flags & IEX_SPMM_LISTS_READY) ? 2 : 0);
-  if (ch.variant == 0 && ch.ws && aligned(ch.ws, 16) && spmm_blocks_fits(dtype, itype, p) && spmm_blocks_wins(p, batch) &&
+  if (ch.variant == 0 && !ch.any_order && ch.ws && aligned(ch.ws, 16) && spmm_blocks_fits(dtype, itype, p) && spmm_blocks_wins(p, batch) &&
       ch.ws_bytes >= spmm_blocks_bytes(p))
     return launch_spmm_blocks(dtype, p, batch, ch.ws, 0, blocks_ready, s);
   if (ch.variant == 10) {
@@ -742,6 +750,7 @@ static size_t workspace_plan(int dtype, int itype, int flags, int m, int k, int 
   *kind = 0;
   if (m <= 0 || k <= 0 || n <= 0 || nonzeros <= 0 || batch <= 0) return 0;
   const int variant = (flags >> 16) & 0xf;
+  if (variant == 0 && (flags & IEX_SPMM_ANY_COLUMN_ORDER)) return 0;   // families 1 and 8 use no workspace
   void* const some_aligned = reinterpret_cast<void*>(size_t(256));
   if (dtype == IEX_F32 && itype == IEX_I32) {
     SpmmParams p{m, k, n, nonzeros, nullptr, nullptr, nullptr, nullptr, some_aligned, nullptr, some_aligned, 0, 0, 0};
@@ -820,6 +829,8 @@ int iex_spmm_static(int dtype, int itype, int flags, int m, int k, int n, int no
                     const void* column_indices, const void* dense, const float* bias, void* out,
                     void* stream, int batch) {
   using namespace iex;
+  // every call shares the array with whatever ran before it: nothing in it counts as "still there"
+  flags &= ~(IEX_SPMM_TABLES_READY | IEX_SPMM_LISTS_READY);
   const size_t need = spmm_workspace_bytes(dtype, itype, flags, m, k, n, nonzeros, batch);
   if (need == 0)  // a call that would not touch a workspace runs as iex_spmm_ex does (a forced family 7 fails there)
     return spmm_dispatch(dtype, itype, flags, m, k, n, nonzeros, row_indices, values, row_offsets, column_indices, dense,
@@ -862,7 +873,7 @@ int iex_spmm_workspace_kind(int dtype, int itype, int flags, int m, int k, int n
 int iex_CudaSpmm2(int m, int k, int n, int nonzeros, const int* row_indices, const float* values,
                   const int* row_offsets, const int* column_indices, const float* dense_matrix,
                   float* output_matrix, void* stream, int batch_size) {
-  return iex::spmm_dispatch(IEX_F32, IEX_I32, IEX_SPMM_PER_BATCH_VALUES | IEX_SPMM_ACCUMULATE, m, k, n,
+  return iex::spmm_dispatch(IEX_F32, IEX_I32, IEX_SPMM_PER_BATCH_VALUES | IEX_SPMM_ACCUMULATE | IEX_SPMM_ANY_COLUMN_ORDER, m, k, n,
                             nonzeros, row_indices, values, row_offsets, column_indices, dense_matrix,
                             nullptr, output_matrix, stream, batch_size, nullptr, 0);
 }
@@ -870,14 +881,14 @@ int iex_CudaSpmm2(int m, int k, int n, int nonzeros, const int* row_indices, con
 int iex_CudaSpmm3(int m, int k, int n, int nonzeros, const int* row_indices, const float* values,
                   const int* row_offsets, const int* column_indices, const float* dense_matrix,
                   float* output_matrix, void* stream, int batch_size) {
-  return iex::spmm_dispatch(IEX_F32, IEX_I32, 0, m, k, n, nonzeros, row_indices, values, row_offsets,
+  return iex::spmm_dispatch(IEX_F32, IEX_I32, IEX_SPMM_ANY_COLUMN_ORDER, m, k, n, nonzeros, row_indices, values, row_offsets,
                             column_indices, dense_matrix, nullptr, output_matrix, stream, batch_size, nullptr, 0);
 }
 
 int iex_CudaSpmm5(int m, int k, int n, int nonzeros, const int* row_indices, const uint16_t* values,
                   const int* row_offsets, const int16_t* column_indices, const uint16_t* dense_matrix,
                   uint16_t* output_matrix, void* stream, int batch_size) {
-  return iex::spmm_dispatch(IEX_F16, IEX_I16, 0, m, k, n, nonzeros, row_indices, values, row_offsets,
+  return iex::spmm_dispatch(IEX_F16, IEX_I16, IEX_SPMM_ANY_COLUMN_ORDER, m, k, n, nonzeros, row_indices, values, row_offsets,
                             column_indices, dense_matrix, nullptr, output_matrix, stream, batch_size, nullptr, 0);
 }
 

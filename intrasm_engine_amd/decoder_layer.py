@@ -25,6 +25,7 @@ import math
 import torch
 
 from . import interleaving as IL
+from .pytorch import ops as _pyops
 from .pytorch.cpp_extensions.cuda_graph_constructor import TorchCUDAGraphConstructor
 
 ops = torch.ops.iex_ops
@@ -44,6 +45,9 @@ class SparseDecoderLayer:
                             torch.from_numpy(csr.values).to(device).half(),
                             torch.from_numpy(csr.row_offsets).to(device),
                             torch.from_numpy(csr.column_indices).to(device).to(idt), csr.m)
+            # (looked at once, here: the layer's schedules run under capture, where a pattern nobody has looked at
+            # keeps to the kernels that take columns in any order)
+            _pyops.prepare_pattern(self.w[name][2], self.w[name][3], csr.k)
 
     # ---- building blocks ---------------------------------------------------------------
     def proj(self, name: str, x: torch.Tensor) -> torch.Tensor:

@@ -155,7 +155,7 @@ class MySpMM(MyAutogradFunc):
                   stream_beg, params):
         grad3 = grad.contiguous().unsqueeze(0)
         grad_dense = grad_sparse = None
-        ci32 = column_indices if column_indices.dtype == torch.int32 else column_indices.to(torch.int32)
+        ci32 = column_indices if column_indices.dtype == torch.int32 else _ops.carry_pattern_note(column_indices, column_indices.to(torch.int32))
         if needs_input_grad[2]:
             # lhs = grad (m, tokens), rhs = b (k, tokens): rhs rows are indexed by the CSR column
             with maybe_captured(backward_constructor, constructor_enabled, stream_beg):

@@ -22,6 +22,7 @@ from __future__ import annotations
 
 import contextlib
 import threading
+import weakref
 
 import torch
 
@@ -40,7 +41,7 @@ def kernel_params(*, spmm: dict | None = None, sddmm: dict | None = None, gemm: 
     """Kernel choices for the operators called inside the block (this thread only), for tuning:
     ``spmm`` = any of force_variant / force_rpw / force_nt / force_lpg / force_wpr (the tuning
     bits of ``iex_spmm_ex``), ``sddmm`` = force_wpr / force_variant, ``gemm`` = tile (the shape code of
-    ``iex_gemm``: 5 = 128x128, 6 = 128x256, 7 = 256x256 tiles, 8 = 128x128 and 9 = 64x128 by eight waves with K steps of 64, 10 = 128x256 by eight waves, 12 = 256x256 with K split over two workgroups per tile; 1..4 = the
+    ``iex_gemm``: 5 = 128x128, 6 = 128x256, 7 = 256x256 tiles, 8 = 128x128 and 9 = 64x128 by eight waves with K steps of 64, 10 = 128x256 by eight waves, 12 = 256x256 with K split over two workgroups per tile, 13 = 256x256 by eight waves in alternating phases; 1..4 = the
     register-staged kernels).
     Without a block, or for a key left out, the library chooses; a category left out (None) keeps
     what an enclosing block set for it.  A kernel family that cannot
@@ -61,6 +62,14 @@ def kernel_params(*, spmm: dict | None = None, sddmm: dict | None = None, gemm: 
         yield
     finally:
         _TUNING.spmm, _TUNING.sddmm, _TUNING.gemm = before["spmm"], before["sddmm"], before["gemm"]
+
+
+def _version(t) -> int:
+    """In-place-change counter of a tensor; tensors created under ``torch.inference_mode()`` keep none (reading it
+    raises) and cannot be changed in place either, so 0 serves."""
+    if t.is_inference():
+        return 0
+    return t._version
 
 
 def _chk(cond: bool, msg: str = "") -> None:
@@ -93,6 +102,63 @@ def _check_index_dtypes(row_indices, row_offsets, column_indices, allow_i16=Fals
     _chk(row_offsets.dtype == torch.int32, "row_offsets must be int32")
     ok = (torch.int32, torch.int16) if allow_i16 else (torch.int32,)
     _chk(column_indices.dtype in ok, "column_indices must be " + " or ".join(str(d) for d in ok))
+
+
+def mark_canonical(row_offsets, column_indices, k):
+    """Record that ``(row_offsets, column_indices)`` is canonical CSR with ``k`` columns (what ``dense_to_sparse`` and
+    ``transpose_info`` build), so that the operators need not look: see :func:`_csr_status`."""
+    column_indices.__dict__["_iex_csr"] = (weakref.ref(row_offsets), _version(row_offsets), _version(column_indices), int(k), 0)
+    return column_indices
+
+
+def _csr_status(row_offsets, column_indices, k):
+    """Status bits of ``iex_csr_check`` for a pattern, or None when they are not known and cannot be found out now
+    (a stream capture is running: the check ends in a synchronising read).
+
+    The reference's kernels take the columns of a row in any order, and repeated (Sputnik: sputnik_spmm.cu.inc:229-243,
+    sputnik_sddmm.cu.inc:137); most kernel families here are faster because they do not.  So every operator looks at a
+    pattern the first time it sees it -- one small launch and one read of four bytes -- and remembers the answer on
+    the ``column_indices`` tensor object, together with the ``row_offsets`` object it belongs to and both version
+    counters: a pattern costs one check, in-place changes and other pairings cost another."""
+    note = column_indices.__dict__.get("_iex_csr")
+    if note is not None and note[0]() is row_offsets and note[1:4] == (_version(row_offsets), _version(column_indices), int(k)):
+        return note[4]
+    if torch.cuda.is_current_stream_capturing():
+        return None
+    status = csr_check(row_offsets, column_indices, k)
+    column_indices.__dict__["_iex_csr"] = (weakref.ref(row_offsets), _version(row_offsets), _version(column_indices), int(k), status)
+    return status
+
+
+def prepare_pattern(row_offsets, column_indices, k):
+    """Look at a pattern now (see :func:`_csr_status`) so that later calls -- under stream capture too, where nothing can
+    be looked at -- take every kernel family for canonical CSR.  Returns the status bits; raises for offsets or columns
+    that point outside the arrays.  Set-up code for patterns that do not come from ``dense_to_sparse``."""
+    status = _csr_status(row_offsets, column_indices, k)
+    _chk(status is not None, "prepare_pattern: cannot look at a pattern while the current stream is being captured")
+    _chk(not (status & (_lib.CSR_BAD_OFFSETS | _lib.CSR_COLUMN_OUT_OF_RANGE)),
+         f"row_offsets must ascend from 0 to the number of nonzeros and every column index must lie in [0, {int(k)})")
+    return status
+
+
+def carry_pattern_note(column_indices, copy):
+    """``copy`` holds the same column indices as ``column_indices`` (another integer type, a clone): what is known about
+    the one holds for the other."""
+    note = column_indices.__dict__.get("_iex_csr")
+    if note is not None and note[2] == _version(column_indices):
+        copy.__dict__["_iex_csr"] = note[:2] + (_version(copy),) + note[3:]
+    return copy
+
+
+def _any_order(row_offsets, column_indices, k, what):
+    """True when the call must keep to the kernels that take columns in any order: the pattern is known to need it, or
+    nothing is known about it.  Offsets or columns that point outside the arrays are refused: no kernel may follow them."""
+    status = _csr_status(row_offsets, column_indices, k)
+    if status is None:
+        return True
+    _chk(not (status & (_lib.CSR_BAD_OFFSETS | _lib.CSR_COLUMN_OUT_OF_RANGE)),
+         f"{what}: row_offsets must ascend from 0 to the number of nonzeros and every column index must lie in [0, {int(k)})")
+    return bool(status & _lib.CSR_NOT_ASCENDING)
 
 
 def _spmm(b, row_indices, values, row_offsets, column_indices, m, *, per_batch_values,
@@ -141,7 +207,8 @@ def _spmm(b, row_indices, values, row_offsets, column_indices, m, *, per_batch_v
     if bias is not None:
         _chk(bias.dtype == torch.float32 and bias.is_contiguous() and bias.numel() == m
              and bias.device == b.device, "bias must be a contiguous fp32 tensor with m entries")
-    flags = (_lib.SPMM_PER_BATCH_VALUES if per_batch_values else 0) | \
+    any_order = nonzeros > 0 and not force_variant and _any_order(row_offsets, column_indices, k, "spmm")
+    flags = (_lib.SPMM_PER_BATCH_VALUES if per_batch_values else 0) | (_lib.SPMM_ANY_COLUMN_ORDER if any_order else 0) | \
             (_lib.SPMM_ACCUMULATE if accumulate else 0) | (_lib.SPMM_RELU if relu else 0) | \
             ((int(force_wpr) & 0xff) << 8) | ((int(force_variant) & 0xf) << 16) | ((int(force_rpw) & 0xf) << 20) | \
             ((int(force_nt) & 0xf) << 24) | ({0: 0, 8: 1, 16: 2, 32: 3, 64: 4}[int(force_lpg)] << 28)
@@ -158,7 +225,7 @@ def _spmm(b, row_indices, values, row_offsets, column_indices, m, *, per_batch_v
         if plan is not None and ws_bytes and lib.iex_spmm_workspace_kind(*shape) == 10:
             # the tables of the dense-blocks kernel depend on the pattern only and are those of the SDDMM for masks
             # with structure: a plan shared with that operator's calls on the pattern serves both
-            key = (row_offsets.data_ptr(), column_indices.data_ptr(), row_offsets._version, column_indices._version,
+            key = (row_offsets.data_ptr(), column_indices.data_ptr(), _version(row_offsets), _version(column_indices),
                    m, k, nonzeros)
             if plan._ready(key, ws_bytes, b.device, (row_offsets, column_indices)):
                 flags |= _lib.SPMM_TABLES_READY
@@ -257,7 +324,8 @@ def _sddmm(a, b, row_indices, row_offsets, column_indices, *, sum_over_batch, dt
     else:
         _chk(tuple(out.shape) == shape and out.dtype == a.dtype and out.is_contiguous()
              and out.device == a.device, "out has the wrong shape, dtype, layout or device")
-    flags = (_lib.SDDMM_SUM_OVER_BATCH if sum_over_batch else 0) | \
+    any_order = nonzeros > 0 and not force_variant and _any_order(row_offsets, column_indices, n, "sddmm")
+    flags = (_lib.SDDMM_SUM_OVER_BATCH if sum_over_batch else 0) | (_lib.SDDMM_ANY_COLUMN_ORDER if any_order else 0) | \
             (_lib.SDDMM_ACCUMULATE if accumulate else 0) | ((int(force_wpr) & 0xff) << 8) | \
             ((int(force_variant) & 0xf) << 16)
     lib = _lib.load()
@@ -269,7 +337,7 @@ def _sddmm(a, b, row_indices, row_offsets, column_indices, *, sum_over_batch, dt
         # cores and pick the nonzeros (16-bit, long k): from torch's allocator, on the current stream
         ws_bytes = 0 if no_workspace else lib.iex_sddmm_workspace_bytes(_DT[a.dtype], flags, m, k, n, nonzeros, batch)
         if plan is not None and ws_bytes and lib.iex_sddmm_workspace_kind(_DT[a.dtype], flags, m, k, n, nonzeros, batch) == 3:
-            key = (row_offsets.data_ptr(), column_indices.data_ptr(), row_offsets._version, column_indices._version,
+            key = (row_offsets.data_ptr(), column_indices.data_ptr(), _version(row_offsets), _version(column_indices),
                    m, n, nonzeros)
             code = (flags >> 8) & 0xff if ((flags >> 16) & 0xf) == 3 else 0     # (what counts as a dense block: the lists depend on it)
             if plan._ready(key, ws_bytes, a.device, (row_offsets, column_indices)):
@@ -435,6 +503,8 @@ def fused_spmm_gemm(b, row_indices, values, row_offsets, column_indices, m, ga, 
     _chk((gb.shape[-1] if trans_b else gb.shape[-2]) == K, "inner dimensions of the GEMM differ")
     gbatch = ga.shape[0] if ga.dim() == 3 else 1
     _chk(ga.dim() == 2 or gb.shape[0] == gbatch, "batch sizes of the GEMM operands differ")
+    _chk(column_indices.size(0) == 0 or not _any_order(row_offsets, column_indices, k, "fused_spmm_gemm"),
+         "fused_spmm_gemm needs canonical CSR (columns of a row ascending and distinct) that has been seen outside a capture")
     out = torch.empty((1, m, n), dtype=b.dtype, device=b.device)
     c = torch.empty((gbatch, M, N) if ga.dim() == 3 else (M, N), dtype=ga.dtype, device=b.device)
     with torch.cuda.device(b.device):

@@ -33,6 +33,9 @@ def dense_to_sparse(matrix: torch.Tensor, device=None):
     torch.cumsum(counts, 0, out=row_offsets[1:])
     column_indices = mask.nonzero()[:, 1].to(torch.int32).contiguous()
     row_offsets = row_offsets.to(torch.int32)
+    if column_indices.is_cuda:
+        from .ops import mark_canonical
+        mark_canonical(row_offsets, column_indices, matrix.shape[1])   # (by construction: the operators need not look)
     return values, row_swizzle(row_offsets), row_offsets, column_indices
 
 
@@ -60,6 +63,9 @@ def transpose_info(m: int, k: int, row_offsets: torch.Tensor, column_indices: to
     row_offsets_t = torch.zeros(k + 1, dtype=torch.int64, device=dev)
     torch.cumsum(counts, 0, out=row_offsets_t[1:])
     row_offsets_t = row_offsets_t.to(torch.int32)
+    if column_indices_t.is_cuda:
+        from .ops import mark_canonical
+        mark_canonical(row_offsets_t, column_indices_t, m)   # (sorted by (column, row): ascending and distinct by construction, given distinct columns per row)
     return row_swizzle(row_offsets_t), row_offsets_t, column_indices_t, perm
 
 
@@ -76,4 +82,5 @@ def to_int16_indices(column_indices: torch.Tensor, k: int) -> torch.Tensor:
     layout, sputnik_kernels.cpp:179-181); needs k <= 32768."""
     if k > 32768:
         raise ValueError("int16 column indices need k <= 32768")
-    return column_indices.to(torch.int16)
+    from .ops import carry_pattern_note
+    return carry_pattern_note(column_indices, column_indices.to(torch.int16))

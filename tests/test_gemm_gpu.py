@@ -38,7 +38,7 @@ def test_gemm_ragged_n_with_transposed_b(oracle, dev, shape):
         ops.gemm_mfma(torch.zeros(8, 8, device=dev).half(), torch.zeros(8, shape[1] | 1, device=dev).half(), False)
 
 
-@pytest.mark.parametrize("shape_code", [1, 2, 3, 4, 5, 6, 7, 8, 9, 10, 11])
+@pytest.mark.parametrize("shape_code", [1, 2, 3, 4, 5, 6, 7, 8, 9, 10, 11, 13])
 @pytest.mark.parametrize("trans_b", [False, True])
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
 @pytest.mark.parametrize("mnk", [(300, 520, 200), (129, 136, 8), (260, 264, 1000)])

@@ -115,10 +115,12 @@ def main():
     mats = {s: W.config2_matrix(s) for s in W.C2_SPARSITIES}
     dens = {n: W.config2_dense(n) for n in W.C2_NS}
 
-    def csr_dev(csr, vdtype=torch.float32, idtype=torch.int32):
+    def csr_dev(csr, vdtype=torch.float32, idtype=torch.int32, tables=False):
         t = (torch.from_numpy(csr.row_indices).to(dev), torch.from_numpy(csr.values).to(dev).to(vdtype),
              torch.from_numpy(csr.row_offsets).to(dev), torch.from_numpy(csr.column_indices).to(dev).to(idtype))
-        pyops.prepare_pattern(t[2], t[3], csr.k)   # looked at once, outside any capture: canonical CSR gets every kernel family
+        # looked at once, outside any capture (the timing loops capture their launches): canonical CSR gets every kernel
+        # family; an attention mask with structure also gets the tables of its kernels made here (tables=True), a weight not
+        pyops.prepare_pattern(t[2], t[3], csr.k, tables=tables)
         return t
 
     mats32 = {s: csr_dev(m) for s, m in mats.items()}
@@ -301,6 +303,10 @@ def main():
                       "GBps": round(by / us / 1e3, 1), "cold_GBps": round(by / cold / 1e3, 1),
                       "hbm_frac": round(by / us / 1e3 / HBM_PEAK_GBPS, 4), "GFLOPs": round(fl / us / 1e3, 1),
                       "valu_frac": round(fl / us / 1e6 / VALU_PEAK_TFLOPS_FP32, 4),
+                      "gather_TBps": round(mats[s].nnz * n * 4 / us / 1e6, 2),
+                      "bound": ("vector ALU (fp32 MFMAs run on it, and so does the expansion of the sparse operand)" if "mfma_f32" in kernel else
+                                "L2 -> CU path (every nonzero gathers n * 4 bytes of the dense operand out of L2: gather_TBps, against about 26 TB/s that this path has delivered at best)"
+                                if mats[s].nnz * n * 4 / us / 1e6 >= 15.0 else "launch and ramp-up (the kernel is a few microseconds long)"),
                       "kernel": kernel, "bytes": by})
         log(f"[bench] fp32 s={s} n={n}: {us:.2f} us warm, {cold:.2f} us cold  {by / us / 1e3:.0f} GB/s  {fl / us / 1e3:.0f} GFLOP/s  {kernel}")
 
@@ -531,9 +537,22 @@ def run_extras(torch, ops, dev, W, IL, mats, dens, csr_dev, time_cell, time_cold
     us = time_cell(lambda: ops.sddmm_sputnik_atomic_upd_weight(l1, r1, ri, ro, ci))
     by = W.sddmm_bytes(a1.m, 64, a1.k, a1.nnz, 1, 4, True)
     out["sddmm_c1_fp32"] = {"us": round(us, 2), "GBps": round(by / us / 1e3, 1), "hbm_frac": round(by / us / 1e3 / HBM_PEAK_GBPS, 4),
-                            "GFLOPs": round(W.sddmm_flops(a1.nnz, 64) / us / 1e3, 1)}
+                            "GFLOPs": round(W.sddmm_flops(a1.nnz, 64) / us / 1e3, 1),
+                            "kernel": kernel_of(lambda: ops.sddmm_sputnik_atomic_upd_weight(l1, r1, ri, ro, ci)),
+                            "bound": "launch (1.4 MB of operands: the kernel is a few microseconds of ramp-up and drain)"}
+    # config 1's SpMM: A 1024 x 1024 at 90 %, B 1024 x 256, fp32
+    v1 = torch.from_numpy(a1.values).to(dev)
+    b1 = torch.from_numpy(W.config1()[1]).to(dev)
+    us = time_cell(lambda: ops.spmm_sputnik_reuse_weight(b1, ri, v1, ro, ci, a1.m))
+    by = W.spmm_bytes(a1.m, a1.k, b1.shape[2], a1.nnz, 1, 4, 4)
+    fl = W.spmm_flops(a1.nnz, b1.shape[2])
+    out["spmm_c1_fp32"] = {"us": round(us, 2), "cold_us": round(time_cold(lambda: ops.spmm_sputnik_reuse_weight(b1, ri, v1, ro, ci, a1.m)), 2),
+                           "GBps": round(by / us / 1e3, 1), "hbm_frac": round(by / us / 1e3 / HBM_PEAK_GBPS, 4),
+                           "GFLOPs": round(fl / us / 1e3, 1), "valu_frac": round(fl / us / 1e6 / VALU_PEAK_TFLOPS_FP32, 4),
+                           "kernel": kernel_of(lambda: ops.spmm_sputnik_reuse_weight(b1, ri, v1, ro, ci, a1.m)),
+                           "bound": "launch (2.9 MB of operands, 0.4 us at either roof)"}
     pat, q, k, v = W.config3()
-    ri3, _, ro3, ci3 = csr_dev(pat)
+    ri3, _, ro3, ci3 = csr_dev(pat, tables=True)
     qt, kt, vt = (torch.from_numpy(x).to(dev).half() for x in (q, k, v))
     us = time_cell(lambda: ops.sddmm_sputnik_half(qt, kt, ri3, ro3, ci3), repeats=10)
     by = W.sddmm_bytes(pat.m, 64, pat.k, pat.nnz, 16, 2, False)
@@ -564,7 +583,7 @@ def run_extras(torch, ops, dev, W, IL, mats, dens, csr_dev, time_cell, time_cold
         masks_[f"equal_rows_random_columns_{d_:.2f}"] = W.CSR(4096, 4096, np_.ones(ci_.shape[0], np_.float32), W.swizzle_from_offsets(ro_), ro_, ci_)
     rows_m = []
     for label_, c_ in masks_.items():
-        rim, _, rom, cim = csr_dev(c_)
+        rim, _, rom, cim = csr_dev(c_, tables=True)
         f_ = lambda: ops.sddmm_sputnik_half(qt, kt, rim, rom, cim)
         us_op = time_cell(f_, repeats=5, samples=3)
         with pyops_k.kernel_params(sddmm={"force_variant": 1}):
@@ -578,7 +597,7 @@ def run_extras(torch, ops, dev, W, IL, mats, dens, csr_dev, time_cell, time_cold
     rows_p = []
     v16_ = torch.randn(16, 4096, 64, device=dev, generator=torch.Generator(dev).manual_seed(5)).half()
     for label_, c_ in masks_.items():
-        rim, _, rom, cim = csr_dev(c_)
+        rim, _, rom, cim = csr_dev(c_, tables=True)
         pr_ = (torch.rand(16, c_.nnz, device=dev, generator=torch.Generator(dev).manual_seed(6)) / 280).half()
         f_ = lambda: ops.spmm_sputnik_batched_values(v16_, rim, pr_, rom, cim, 4096)
         us_op = time_cell(f_, repeats=5, samples=3)
@@ -683,7 +702,7 @@ def run_extras(torch, ops, dev, W, IL, mats, dens, csr_dev, time_cell, time_cold
                      torch.randn(4096, 4096, device=dev, generator=gen).bfloat16() if i else torch.from_numpy(ga).to(dev).bfloat16(),
                      torch.randn(4096, 2048, device=dev, generator=gen).bfloat16() if i else torch.from_numpy(gb).to(dev).bfloat16()))
     for t in sets:
-        pyops.prepare_pattern(t[2], t[3], w.k)
+        pyops.prepare_pattern(t[2], t[3], w.k, tables=False)
     kw4 = dict(per_batch_values=False, accumulate=False, dtypes=(torch.float16,), allow_i16=True)
 
     def spmm_list(**extra):
@@ -693,12 +712,14 @@ def run_extras(torch, ops, dev, W, IL, mats, dens, csr_dev, time_cell, time_cold
     gemm_execs = [(lambda t=t: ops.gemm_mfma(t[5], t[6], False)) for t in sets]
     fused_execs = [(lambda t=t: ops.fused_spmm_gemm(t[4], t[0], t[1], t[2], t[3], w.m, t[5], t[6], False, 0)) for t in sets]
     fused_g_execs = [(lambda t=t: ops.fused_spmm_gemm(t[4], t[0], t[1], t[2], t[3], w.m, t[5], t[6], False, 64)) for t in sets]
+    fused_s_execs = [(lambda t=t: ops.fused_spmm_gemm(t[4], t[0], t[1], t[2], t[3], w.m, t[5], t[6], False, -1)) for t in sets]
     t_spmm = IL.run_non_interleaving(spmm_execs) / reps
     t_gemm = IL.run_non_interleaving(gemm_execs) / reps
     t_serial = IL.run_non_interleaving(spmm_execs, gemm_execs) / reps
     t_graph = IL.run_interleaving(spmm_execs, gemm_execs) / reps
     t_fused = IL.run_non_interleaving(fused_execs) / reps
     t_fused_g = IL.run_non_interleaving(fused_g_execs) / reps
+    t_fused_s = IL.run_non_interleaving(fused_s_execs) / reps
     # the same pair with the SpMM forced onto the gather (row) kernel: vector ALU + L2 beside the matrix cores,
     # the resource split the reference's co-run experiment is about
     gather_execs = spmm_list(force_variant=1)
@@ -716,7 +737,8 @@ def run_extras(torch, ops, dev, W, IL, mats, dens, csr_dev, time_cell, time_cold
     out["config4"] = {
         "spmm_ms": round(t_spmm, 4), "spmm_GBps": round(by_s / t_spmm / 1e6, 1), "spmm_GFLOPs": round(fl_s / t_spmm / 1e6, 1),
         "spmm_hbm_frac": round(by_s / t_spmm / 1e6 / HBM_PEAK_GBPS, 4),
-        "spmm_valu_frac": round(fl_s / t_spmm / 1e9 / VALU_PEAK_TFLOPS_FP32, 4),
+        "spmm_bound": "MFMA (the operator's path multiplies the dense form of the sparse operand on the matrix cores)",
+        "spmm_mfma_frac_dense_equivalent": round(2.0 * w.m * w.k * 2048 / t_spmm / 1e9 / MFMA_PEAK_TFLOPS_16BIT, 4),
         "spmm_kernels": k_spmm, "gemm_kernels": k_gemm, "fused_kernels": k_fused,
         "spmm_cold_ms": round(cold_spmm, 4), "gemm_cold_ms": round(cold_gemm, 4),
         "gemm_ms": round(t_gemm, 4), "gemm_TFLOPs": round(IL.gemm_tflops(4096, 2048, 4096, t_gemm), 1),
@@ -724,6 +746,9 @@ def run_extras(torch, ops, dev, W, IL, mats, dens, csr_dev, time_cell, time_cold
         "serialized_sum_ms": round(t_spmm + t_gemm, 4), "serialized_one_stream_ms": round(t_serial, 4),
         "two_branch_graph_ms": round(t_graph, 4), "fused_launch_ms": round(t_fused, 4),
         "fused_launch_gemm_in_groups_of_64_ms": round(t_fused_g, 4),
+        "fused_launch_spmm_tiles_first_ms": round(t_fused_s, 4),
+        "fused_spmm_tiles_first_pct_of_serialized_matrix_core_kernel": round(100 * t_fused_s / (t_mc + t_gemm), 1),
+        "gemm_bound": "MFMA",
         "graph_makespan_pct_of_serialized": round(100 * t_graph / (t_spmm + t_gemm), 1),
         "fused_makespan_pct_of_serialized": round(100 * t_fused / (t_spmm + t_gemm), 1),
         "spmm_matrix_core_kernel_ms": round(t_mc, 4), "two_branch_graph_matrix_core_kernel_ms": round(t_graph_mc, 4),
@@ -735,7 +760,7 @@ def run_extras(torch, ops, dev, W, IL, mats, dens, csr_dev, time_cell, time_cold
         "repeats_per_graph": reps, "operand_sets": f"{reps} distinct (own copies of the CSR arrays, values, activation and GEMM operands per repetition)",
     }
     log(f"[bench] config 4: spmm {t_spmm:.3f} ms, gemm {t_gemm:.3f} ms, graph {t_graph:.3f} ms, fused {t_fused:.3f} ms")
-    del w, x, ga, gb, riw, vw, row, ciw, sets, spmm_execs, gemm_execs, fused_execs, fused_g_execs, gather_execs, mc_execs
+    del w, x, ga, gb, riw, vw, row, ciw, sets, spmm_execs, gemm_execs, fused_execs, fused_g_execs, fused_s_execs, gather_execs, mc_execs
     reps = 4
 
     # ---- the dense GEMM alone on larger shapes (bf16, B as (K, N)): how far the matrix cores are used
@@ -782,18 +807,20 @@ def run_extras(torch, ops, dev, W, IL, mats, dens, csr_dev, time_cell, time_cold
     t_ser_halves = time_capture(lambda: IL.capture_serialized([lambda: (layer.forward(xa, seqs // 2), layer.forward(xb, seqs // 2))]))
     t_ms = time_capture(lambda: layer.capture_multistream(xa, xb, seqs // 2))
     t_fu = time_capture(lambda: layer.capture_fused(xa, xb, seqs // 2, 0))
+    t_fu_lpt = time_capture(lambda: layer.capture_fused(xa, xb, seqs // 2, None))
     spmm_flops5 = sum(2 * weights[n_].nnz * seqs * L for n_ in weights)
     attn_flops5 = 2 * 2 * seqs * heads * L * L * (hidden // heads)
     out["config5"] = {
         "shape": "hidden 4096, 32 heads, MLP 11008, 16 x 512 tokens, fp16; q/k/v/o 2:4, gate/up/down 80% unstructured",
         "elementwise_ops_included": "softmax(QK^T/sqrt(d)), SiLU(gate)*up, two residual adds (PyTorch kernels); no RoPE / norm / mask",
         "serialized_ms": round(t_ser, 3), "serialized_two_halves_ms": round(t_ser_halves, 3),
-        "multistream_graph_ms": round(t_ms, 3), "fused_ms": round(t_fu, 3),
+        "multistream_graph_ms": round(t_ms, 3), "fused_ms": round(t_fu, 3), "fused_longer_tiles_first_ms": round(t_fu_lpt, 3),
         "multistream_pct_of_serialized": round(100 * t_ms / t_ser, 1), "fused_pct_of_serialized": round(100 * t_fu / t_ser, 1),
+        "fused_longer_tiles_first_pct_of_serialized": round(100 * t_fu_lpt / t_ser, 1),
         "spmm_GFLOP": round(spmm_flops5 / 1e9, 1), "attention_GFLOP": round(attn_flops5 / 1e9, 1),
         "layer_TFLOPs_serialized": round((spmm_flops5 + attn_flops5) / t_ser / 1e9, 1),
     }
-    log(f"[bench] config 5: serialized {t_ser:.2f} ms, two-stream graph {t_ms:.2f} ms, fused {t_fu:.2f} ms")
+    log(f"[bench] config 5: serialized {t_ser:.2f} ms, two-stream graph {t_ms:.2f} ms, fused {t_fu:.2f} ms (GEMM tiles first), {t_fu_lpt:.2f} ms (longer tiles first)")
     del layer
 
     # ---- the SpMM kernel families side by side on three projections of that layer (n = 8192 tokens, fp16,

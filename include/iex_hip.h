@@ -65,6 +65,23 @@ int iex_device_ok(void);
 int iex_csr_check(int itype, int m, int k, int nonzeros, const int* row_offsets, const void* column_indices,
                   int* status, void* stream);
 
+/* Row lengths of a pattern on a coarse scale, for iex_spmm_sched: adds to histogram[j] (device memory, 16 ints that the
+ * caller has set to 0; the launch is asynchronous on `stream`) the number of rows with more than 64 << j nonzeros,
+ * j = 0 .. 15.  A function of row_offsets alone; a caller reads it back once per pattern, as set-up.
+ * No counterpart in the reference (its launchers know the mean row length only: nonzeros / m). */
+int iex_csr_row_histogram(int m, const int* row_offsets, int* histogram, void* stream);
+
+/* How much of a pattern sits in dense blocks: adds to *dense_nonzeros (device memory, an int that the caller has set
+ * to 0; asynchronous on `stream`) the number of nonzeros that lie in 128 x 128 blocks (rows and columns counted from
+ * 0 in steps of 128) holding at least dense_min of them.  The kernels for patterns with structure (SDDMM variant 3,
+ * SpMM family 10) put such blocks on the matrix cores and count a block as dense from 1536 nonzeros; they pay off when
+ * about half of the nonzeros or more sit in such blocks (bands, windows, block diagonals), whatever the overall
+ * density -- which is all that the 0 = choose rule of those entry points can see.  A caller reads the figure back
+ * once per pattern, as set-up, and forces the variant.  k <= 65536; the pattern must pass iex_csr_check's offset test.
+ * No counterpart in the reference. */
+int iex_csr_dense_share(int itype, int m, int k, const int* row_offsets, const void* column_indices, int dense_min,
+                        int* dense_nonzeros, void* stream);
+
 /* dst[0:nbytes] = src[0:nbytes] with a plain 128-bit-per-lane streaming kernel (nbytes and both
  * pointers multiples of 16).  Measurement aid with no counterpart in the reference: hardware
  * traffic counters are scaled by what they read for this copy of known size. */
@@ -98,12 +115,8 @@ int iex_copy_bytes(void* dst, const void* src, size_t nbytes, void* stream);
  * form of A in the caller's workspace, then the dense GEMM (iex_spmm_ws only), 8 = A with at most
  * 128 columns and an output at least one tile (64 128-bit vectors) wide: the dense operand's tile
  * in LDS, rows streamed in natural order (bit-equal to family 1 with one wavefront per row; fails
- * on other shapes), 9 = fp32 with int32 indices only, on request only: a slice of the dense operand resident in
- * LDS (direct-to-LDS loads, double-buffered stages), k split over workgroups, fp32 partial sums added by a second
- * kernel in slice order (deterministic); needs n a multiple of 4, 16-byte aligned dense operands, k <= 262144 and,
- * for more than one slice, iex_spmm_ws with the workspace iex_spmm_workspace_bytes reports (bits 20..23: slices,
- * 0 = choose; bits 24..27 = 2: workgroups of 16 wavefronts and 128 rows instead of 8 and 64); fails on other
- * shapes, 10 = sparse operands with structure (attention probabilities: bands, blocks, windows) times a dense
+ * on other shapes), 9 = unused,
+ * 10 = sparse operands with structure (attention probabilities: bands, blocks, windows) times a dense
  * operand of 64, 128, ... columns (served 64 at a time): per 128 rows, the dense 128 x 128 blocks of A are laid out in LDS and
  * multiplied on the matrix cores, the nonzeros elsewhere are gathered row by row (fp16 / bf16, int32 indices,
  * n a multiple of 64 up to 1024, k <= 65536, plain store without bias or ReLU, values shared or per batch entry;
@@ -114,7 +127,8 @@ int iex_copy_bytes(void* dst, const void* src, size_t nbytes, void* stream);
  * IEX_SPMM_TABLES_READY / IEX_SPMM_LISTS_READY; bits 8..15 set the number of nonzeros from which a block counts
  * as dense: 0 = built in (1536), 1 = every block, 255 = none, else 64 * value); fails on other shapes.
  * 0 = choose.
- * Families 2-6, 9 and 10 rely on strictly ascending column indices inside a row (canonical CSR, what
+ * 11 = the row kernel with wavefronts per row by the row's own length (iex_spmm_sched only: see there).
+ * Families 2-6 and 10 rely on strictly ascending column indices inside a row (canonical CSR, what
  * dense_to_sparse produces); family 1 accepts any order and duplicates -- force it for such
  * input.  Families 3-6 and 10 multiply explicit zeros with the dense operand, so a non-finite entry
  * in a row of `dense` that no nonzero references still reaches the output (0 * inf = NaN).
@@ -161,7 +175,25 @@ int iex_spmm_ws(int dtype, int itype, int flags, int m, int k, int n, int nonzer
                 void* out, void* stream, int batch, void* workspace, size_t workspace_bytes);
 size_t iex_spmm_workspace_bytes(int dtype, int itype, int flags, int m, int k, int n,
                                 int nonzeros, int batch);
-/* What that workspace would hold: 0 = nothing (not used), 7 = the dense form of A, 9 = the partial sums of family 9,
+/* iex_spmm_ws for a caller that knows the pattern's row lengths: `row_histogram` is HOST memory, the 16 counts of
+ * iex_csr_row_histogram for row_offsets (NULL: exactly iex_spmm_ws).  Where the call runs on the row kernel (family 1)
+ * with full 128-bit vectors and would split rows over wavefronts, the split then follows each row's own length
+ * instead of the mean (the reference's remedy for uneven rows is the swizzle alone, sputnik_spmm.cu.inc:109-114):
+ * row_indices lists the rows by decreasing length, so the rows that get 16, 8, 4, 2 wavefronts and 1 are five
+ * consecutive ranges of it, a workgroup of 16 wavefronts serves 1, 2, 4, 8 or 16 rows of one range, and the partial
+ * sums of a row meet in LDS in a fixed order (no atomics: same bits from call to call).  The histogram and the
+ * order of row_indices settle how many wavefronts a row HAS; into how many parts its sum is cut follows from the
+ * row's own length, and a row with fewer wavefronts than parts lets them take the parts in turns.  So every row is
+ * summed completely, and to the same bits, whatever the histogram and whatever the order of row_indices: a wrong
+ * histogram or another order costs time only.  IEX_SPMM_FORCE_VARIANT(11) asks for this kernel and fails without a histogram
+ * (bits 20..23 then force the chunks of 64 nonzeros a wavefront may get: 1 + log2, 0 = choose).
+ * No counterpart in the reference. */
+int iex_spmm_sched(int dtype, int itype, int flags, int m, int k, int n, int nonzeros,
+                   const int* row_indices, const void* values, const int* row_offsets,
+                   const void* column_indices, const void* dense, const float* bias,
+                   void* out, void* stream, int batch, void* workspace, size_t workspace_bytes,
+                   const int* row_histogram);
+/* What that workspace would hold: 0 = nothing (not used), 7 = the dense form of A,
  * 10 = the tables and lists of family 10 (functions of the pattern only: a caller that keeps the workspace for a
  * pattern may say so with IEX_SPMM_TABLES_READY / IEX_SPMM_LISTS_READY on later calls). */
 int iex_spmm_workspace_kind(int dtype, int itype, int flags, int m, int k, int n, int nonzeros, int batch);
@@ -270,6 +302,18 @@ size_t iex_sddmm_workspace_bytes(int dtype, int flags, int m, int k, int n, int 
  * and the index arrays only: see IEX_SDDMM_TABLES_READY), 7 = the dense product. */
 int iex_sddmm_workspace_kind(int dtype, int flags, int m, int k, int n, int nonzeros, int batch);
 
+/* The tables and lists that SDDMM variant 3 and SpMM family 10 derive from a pattern (m rows, n columns: the SpMM's k),
+ * written into the caller's workspace by their two setup kernels, with the built-in threshold for dense blocks: for a
+ * caller that prepares a pattern once, waits for the stream, and then passes the workspace with both READY flags
+ * (IEX_SDDMM_TABLES_READY | IEX_SDDMM_LISTS_READY, IEX_SPMM_TABLES_READY | IEX_SPMM_LISTS_READY) to every call on the
+ * pattern -- the workspace is only read from then on, so calls on different streams may share it.
+ * iex_pattern_tables_bytes: the size (what iex_sddmm_workspace_bytes reports for variant 3 and
+ * iex_spmm_workspace_bytes for family 10 on the pattern), 0 where those kernels do not apply (n > 65536).
+ * int32 column indices, strictly ascending inside a row.  No counterpart in the reference. */
+size_t iex_pattern_tables_bytes(int m, int n, int nonzeros);
+int iex_pattern_tables(int m, int n, int nonzeros, const int* row_offsets, const int* column_indices, void* workspace,
+                       size_t workspace_bytes, void* stream);
+
 /* Drop-in for CudaSddmm2 (csrc/extensions.h:31; sddmm_sputnik_atomic_upd_weight,
  * sputnik_kernels.cpp:182-184): fp32, output (nnz) = sum over the batch, written
  * (not accumulated), so the caller need not zero it. */
@@ -327,8 +371,9 @@ size_t iex_gemm_workspace_bytes(int dtype, int trans_b, int M, int N, int K, int
  * (as iex_gemm: gemm_batch entries, element strides stride_*) and row blocks of the fp16 CSR
  * SpMM (as iex_spmm_ex with dtype IEX_F16, batch 1, no flags).  interleave == 0: the GEMM
  * workgroups come first; interleave == g > 0: they are spread through the grid in groups of
- * g, each group followed by an even share of the SpMM blocks (any g >= 1 is valid; a negative
- * value is refused).  Both results are identical to the separate launches.  No counterpart in the reference
+ * g, each group followed by an even share of the SpMM blocks (any g >= 1 is valid); interleave < 0: the SpMM
+ * workgroups come first (the longer jobs first: the GEMM tiles then fill the CUs that the SpMM's last round leaves
+ * idle).  Both results are identical to the separate launches.  No counterpart in the reference
  * (the name survives only as the unused HORIZONTAL_GRAINED flag, tests/test_interleaving.py:441). */
 int iex_fused_spmm_gemm(int spmm_itype, int m, int k, int n, int nonzeros,
                         const int* row_indices, const void* values, const int* row_offsets,
@@ -339,7 +384,7 @@ int iex_fused_spmm_gemm(int spmm_itype, int m, int k, int n, int nonzeros,
 /* The workgroup-id -> role map of that launch, evaluated on the host: for a grid of gemm_blocks +
  * spmm_blocks workgroups and group size `interleave`, workgroup `id` runs GEMM tile *index
  * (*is_gemm = 1) or SpMM block *index (*is_gemm = 0).  Every tile and every block is the role of
- * exactly one id for any counts and any interleave >= 0; the device code calls the same function.
+ * exactly one id for any counts and any interleave; the device code calls the same function.
  * No launch, no GPU needed.  No counterpart in the reference. */
 int iex_fused_role(int gemm_blocks, int spmm_blocks, int interleave, int id, int* is_gemm, int* index);
 

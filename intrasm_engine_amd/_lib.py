@@ -40,6 +40,9 @@ SIGNATURES = {
     "iex_copy_bytes": (_i, [_vp, _vp, _c.c_size_t, _vp]),
     "iex_spmm_ex": (_i, [_i, _i, _i, _i, _i, _i, _i, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i]),
     "iex_spmm_ws": (_i, [_i, _i, _i, _i, _i, _i, _i, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _vp, _c.c_size_t]),
+    "iex_spmm_sched": (_i, [_i, _i, _i, _i, _i, _i, _i, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _vp, _c.c_size_t, _c.POINTER(_i)]),
+    "iex_csr_row_histogram": (_i, [_i, _vp, _vp, _vp]),
+    "iex_csr_dense_share": (_i, [_i, _i, _i, _vp, _vp, _i, _vp, _vp]),
     "iex_spmm_workspace_bytes": (_c.c_size_t, [_i, _i, _i, _i, _i, _i, _i, _i]),
     "iex_spmm_workspace_kind": (_i, [_i, _i, _i, _i, _i, _i, _i, _i]),
     "iex_spmm_static": (_i, [_i, _i, _i, _i, _i, _i, _i, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i]),
@@ -52,6 +55,8 @@ SIGNATURES = {
     "iex_sddmm_ws": (_i, [_i, _i, _i, _i, _i, _i, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _vp, _c.c_size_t]),
     "iex_sddmm_workspace_bytes": (_c.c_size_t, [_i, _i, _i, _i, _i, _i, _i]),
     "iex_sddmm_workspace_kind": (_i, [_i, _i, _i, _i, _i, _i, _i]),
+    "iex_pattern_tables_bytes": (_c.c_size_t, [_i, _i, _i]),
+    "iex_pattern_tables": (_i, [_i, _i, _i, _vp, _vp, _vp, _c.c_size_t, _vp]),
     "iex_CudaSddmm2": (_i, [_i, _i, _i, _i, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i]),
     "iex_csr_softmax": (_i, [_i, _i, _i, _vp, _vp, _vp, _f, _vp, _i]),
     "iex_gemm": (_i, [_i, _i, _i, _i, _i, _vp, _vp, _vp, _i, _ll, _ll, _ll, _vp]),

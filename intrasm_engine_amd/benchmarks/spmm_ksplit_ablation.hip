@@ -1,4 +1,4 @@
-// Ablation of the k-split SpMM kernel (spmm_ksplit_device.cuh, family 9) on the shape of the 4096 x 4096 fp32
+// Ablation of the k-split SpMM kernel (spmm_ksplit_device.cuh beside this file; it was family 9 of the library until it was measured and taken out) on the shape of the 4096 x 4096 fp32
 // sweep, n = 256: the kernel as shipped, and instrumented builds of the same template that leave out one
 // ingredient each (the DBG switches of spmm_ksplit_block; results of those builds are wrong on purpose, every
 // address they use stays in bounds).  Prints microseconds per launch (HIP events, 20 launches) of the main kernel
@@ -7,7 +7,7 @@
 //   hipcc --offload-arch=gfx950 -O3 -std=c++17 -Xclang -target-feature -Xclang -packed-fp32-ops \
 //         intrasm_engine_amd/benchmarks/spmm_ksplit_ablation.hip -o spmm_ksplit_ablation && ./spmm_ksplit_ablation [densities ...]
 //   IEX_ABLATION_SHORT=1: three launches of the shipped kernel only (8 and 16 wavefronts), for rocprofv3 --pmc.
-#include "../csrc/spmm_ksplit_device.cuh"
+#include "spmm_ksplit_device.cuh"
 
 #include <algorithm>
 #include <cstdio>

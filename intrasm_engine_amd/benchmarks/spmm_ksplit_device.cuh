@@ -28,8 +28,8 @@
 // Requirements (checked by the host): canonical CSR (strictly ascending columns inside a row), row bytes of the
 // dense operand and both dense pointers multiples of 16, n at least one 128-bit vector, k <= 262144.
 #pragma once
-#include "gemm_dma_device.cuh"
-#include "spmm_device.cuh"
+#include "../csrc/gemm_dma_device.cuh"
+#include "../csrc/spmm_device.cuh"
 
 namespace iex {
 

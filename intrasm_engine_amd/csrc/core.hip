@@ -71,9 +71,67 @@ __global__ __launch_bounds__(256) void csr_check_kernel(int m, int k, int nnz, c
   }
   if (bad) atomicOr(status, bad);
 }
+
+// histogram[j] += rows with more than 64 << j nonzeros, j = 0 .. 15 (counts: integer additions commute, so the result
+// does not depend on the order of the atomics); a thread per row, a workgroup adds up in LDS first.
+__global__ __launch_bounds__(256) void csr_row_histogram_kernel(int m, const int* __restrict__ row_offsets, int* histogram) {
+  __shared__ int local[16];
+  if (threadIdx.x < 16) local[threadIdx.x] = 0;
+  __syncthreads();
+  const int r = blockIdx.x * 256 + threadIdx.x;
+  if (r < m) {
+    const long long len = (long long)row_offsets[r + 1] - row_offsets[r];
+    for (int j = 0; j < 16 && len > (64ll << j); ++j) atomicAdd(&local[j], 1);
+  }
+  __syncthreads();
+  if (threadIdx.x < 16 && local[threadIdx.x]) atomicAdd(&histogram[threadIdx.x], local[threadIdx.x]);
+}
+
+// *dense_nonzeros += the nonzeros of this block of 128 rows that sit in 128 x 128 blocks holding at least dense_min of
+// them.  One workgroup (4 wavefronts) per 128 rows; the counters of the row block's column blocks live in LDS.
+constexpr int kShareMaxTiles = 512;   // k <= 65536
+template <typename IT>
+__global__ __launch_bounds__(256) void csr_dense_share_kernel(int m, int k, const int* __restrict__ row_offsets, const IT* __restrict__ cols,
+                                                              int dense_min, int* dense_nonzeros) {
+  __shared__ int count[kShareMaxTiles];
+  __shared__ int total;
+  const int tiles = (k + 127) / 128;
+  for (int t = threadIdx.x; t < tiles; t += 256) count[t] = 0;
+  if (threadIdx.x == 0) total = 0;
+  __syncthreads();
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  for (int r = blockIdx.x * 128 + wave; r < min(m, blockIdx.x * 128 + 128); r += 4) {
+    const int s = row_offsets[r], e = row_offsets[r + 1];
+    for (int j = s + lane; j < e; j += 64) {
+      const int c = (int)cols[j];
+      if (c >= 0 && c < k) atomicAdd(&count[c >> 7], 1);
+    }
+  }
+  __syncthreads();
+  int mine = 0;
+  for (int t = threadIdx.x; t < tiles; t += 256) mine += count[t] >= dense_min ? count[t] : 0;
+  if (mine) atomicAdd(&total, mine);
+  __syncthreads();
+  if (threadIdx.x == 0 && total) atomicAdd(dense_nonzeros, total);
+}
 }  // namespace
 
 extern "C" {
+
+int iex_csr_dense_share(int itype, int m, int k, const int* row_offsets, const void* column_indices, int dense_min, int* dense_nonzeros,
+                        void* stream) {
+  IEX_REQUIRE(m >= 0 && k >= 0 && dense_min >= 0, IEX_ERR_BAD_ARGUMENT, "csr_dense_share: negative argument");
+  IEX_REQUIRE(dense_nonzeros && (m == 0 || (row_offsets && column_indices)), IEX_ERR_BAD_ARGUMENT, "csr_dense_share: null pointer argument");
+  IEX_REQUIRE(itype == IEX_I32 || itype == IEX_I16, IEX_ERR_UNSUPPORTED, "csr_dense_share: column indices must be int32 or int16");
+  IEX_REQUIRE(k <= 128 * kShareMaxTiles, IEX_ERR_TOO_LARGE, "csr_dense_share: more than %d columns", 128 * kShareMaxTiles);
+  if (m == 0 || k == 0) return 0;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  if (itype == IEX_I32)
+    hipLaunchKernelGGL(csr_dense_share_kernel<int>, dim3((m + 127) / 128), dim3(256), 0, s, m, k, row_offsets, static_cast<const int*>(column_indices), dense_min, dense_nonzeros);
+  else
+    hipLaunchKernelGGL(csr_dense_share_kernel<short>, dim3((m + 127) / 128), dim3(256), 0, s, m, k, row_offsets, static_cast<const short*>(column_indices), dense_min, dense_nonzeros);
+  return iex::check_hip(hipGetLastError(), "csr_dense_share launch");
+}
 
 int iex_csr_check(int itype, int m, int k, int nonzeros, const int* row_offsets, const void* column_indices, int* status, void* stream) {
   IEX_REQUIRE(m >= 0 && k >= 0 && nonzeros >= 0, IEX_ERR_BAD_ARGUMENT, "csr_check: negative dimension");
@@ -86,6 +144,14 @@ int iex_csr_check(int itype, int m, int k, int nonzeros, const int* row_offsets,
   else
     hipLaunchKernelGGL(csr_check_kernel<short>, dim3((m + 3) / 4), dim3(256), 0, s, m, k, nonzeros, row_offsets, static_cast<const short*>(column_indices), status);
   return iex::check_hip(hipGetLastError(), "csr_check launch");
+}
+
+int iex_csr_row_histogram(int m, const int* row_offsets, int* histogram, void* stream) {
+  IEX_REQUIRE(m >= 0, IEX_ERR_BAD_ARGUMENT, "csr_row_histogram: negative dimension");
+  IEX_REQUIRE(histogram && (m == 0 || row_offsets), IEX_ERR_BAD_ARGUMENT, "csr_row_histogram: null pointer argument");
+  if (m == 0) return 0;
+  hipLaunchKernelGGL(csr_row_histogram_kernel, dim3((m + 255) / 256), dim3(256), 0, static_cast<hipStream_t>(stream), m, row_offsets, histogram);
+  return iex::check_hip(hipGetLastError(), "csr_row_histogram launch");
 }
 
 int iex_copy_bytes(void* dst, const void* src, size_t nbytes, void* stream) {

@@ -5,6 +5,8 @@
 //
 // Workgroup roles
 //   interleave == 0 : ids [0, G) run GEMM tiles, ids [G, G+S) run SpMM blocks;
+//   interleave < 0  : ids [0, S) run SpMM blocks, ids [S, S+G) run GEMM tiles: the longer jobs first (a CU takes the
+//                     next id whenever it has room), so the short GEMM tiles fill what the SpMM's last round leaves;
 //   interleave == g : the G GEMM workgroups are spread through the id range in ceil(G/g) groups of g
 //                     consecutive ids, each followed by its even share of the SpMM blocks, so both
 //                     kinds are dispatched side by side from start to end while the tiles of a
@@ -39,13 +41,19 @@ constexpr int kFusedWin = 32;
 // Role of workgroup b: GEMM tile `idx` or SpMM block `idx`.  A bijection between the ids [0, G + S) and
 // the G tiles plus the S blocks for every G >= 0, S >= 0 and group size g >= 0:
 //   g == 0: ids [0, G) are the tiles, [G, G + S) the blocks;
+//   g < 0:  ids [0, S) are the blocks, [S, S + G) the tiles;
 //   g >= 1: Q = ceil(G / g) groups, each "its tiles, then its share of the blocks"; group q holds the
 //           tiles [q g, min(G, (q + 1) g)) and floor(S / Q) blocks, one more in the first S mod Q groups
 //           (the last group, the only one that can be short of tiles, never gets the extra block).
 // Host and device: the host side is exported as iex_fused_role for the CPU test of this mapping.
 __host__ __device__ inline void fused_role_of(int gemm_blocks, int spmm_blocks, int interleave, int b, bool& is_gemm, int& idx) {
   const int G = gemm_blocks, S = spmm_blocks, g = interleave;
-  if (g <= 0 || G == 0) {
+  if (g < 0) {
+    is_gemm = b >= S;
+    idx = is_gemm ? b - S : b;
+    return;
+  }
+  if (g == 0 || G == 0) {
     is_gemm = b < G;
     idx = is_gemm ? b : b - G;
     return;
@@ -207,7 +215,7 @@ int launch_gemm_kind(const FusedParams& p, SpmmShape vec, bool bf16, bool trans_
 
 extern "C" int iex_fused_role(int gemm_blocks, int spmm_blocks, int interleave, int id, int* is_gemm, int* index) {
   using namespace iex;
-  IEX_REQUIRE(gemm_blocks >= 0 && spmm_blocks >= 0 && interleave >= 0 && is_gemm && index, IEX_ERR_BAD_ARGUMENT,
+  IEX_REQUIRE(gemm_blocks >= 0 && spmm_blocks >= 0 && is_gemm && index, IEX_ERR_BAD_ARGUMENT,
               "fused role: negative count or null pointer");
   IEX_REQUIRE(id >= 0 && (long long)id < (long long)gemm_blocks + spmm_blocks, IEX_ERR_BAD_ARGUMENT,
               "fused role: id %d outside the grid of %lld workgroups", id, (long long)gemm_blocks + spmm_blocks);
@@ -227,7 +235,6 @@ extern "C" int iex_fused_spmm_gemm(int spmm_itype, int m, int k, int n, int nonz
   using namespace iex;
   IEX_REQUIRE(m > 0 && k > 0 && n > 0 && nonzeros >= 0, IEX_ERR_BAD_ARGUMENT, "fused: SpMM dimensions must be positive");
   IEX_REQUIRE(M > 0 && N > 0 && K > 0 && gemm_batch > 0, IEX_ERR_BAD_ARGUMENT, "fused: GEMM dimensions must be positive");
-  IEX_REQUIRE(interleave >= 0, IEX_ERR_BAD_ARGUMENT, "fused: interleave must be 0 (GEMM workgroups first) or a group size >= 1 (got %d)", interleave);
   IEX_REQUIRE(stride_a % 8 == 0 && stride_b % 8 == 0, IEX_ERR_UNSUPPORTED, "fused: GEMM batch strides must be multiples of 8");
   IEX_REQUIRE(row_indices && row_offsets && dense && spmm_out && A && B && C, IEX_ERR_BAD_ARGUMENT,
               "fused: null pointer argument");

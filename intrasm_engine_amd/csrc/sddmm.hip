@@ -455,6 +455,27 @@ size_t iex_sddmm_workspace_bytes(int dtype, int flags, int m, int k, int n, int 
   return iex::sddmm_workspace_bytes(dtype, flags, m, k, n, nonzeros, batch);
 }
 
+size_t iex_pattern_tables_bytes(int m, int n, int nonzeros) {
+  using namespace iex;
+  if (m <= 0 || n <= 0 || nonzeros <= 0) return 0;
+  const int tiles = ceil_div(n, kSdBN);
+  if (tiles > kSdMaxTiles || (long long)(tiles + 1) * m >= (1ll << 28)) return 0;
+  return sb_words(m, tiles, nonzeros) * sizeof(int);
+}
+
+int iex_pattern_tables(int m, int n, int nonzeros, const int* row_offsets, const int* column_indices, void* workspace,
+                       size_t workspace_bytes, void* stream) {
+  using namespace iex;
+  const size_t need = iex_pattern_tables_bytes(m, n, nonzeros);
+  IEX_REQUIRE(need > 0, IEX_ERR_UNSUPPORTED, "pattern tables: needs m, n, nonzeros > 0 and n <= %d", kSdMaxTiles * kSdBN);
+  IEX_REQUIRE(row_offsets && column_indices && workspace && aligned(workspace, 16) && workspace_bytes >= need, IEX_ERR_BAD_ARGUMENT,
+              "pattern tables: null pointer, or the workspace is not 16-byte aligned or shorter than %zu bytes", need);
+  trail_reset();
+  const int tiles = ceil_div(n, kSdBN);
+  return sb_setup(sd_tables(workspace, m, tiles), sb_lists(workspace, m, tiles, nonzeros), m, tiles, 0, 0, row_offsets, column_indices,
+                  static_cast<hipStream_t>(stream));
+}
+
 int iex_sddmm_workspace_kind(int dtype, int flags, int m, int k, int n, int nonzeros, int batch) {
   return iex::sddmm_workspace_kind(dtype, flags, m, k, n, nonzeros, batch);
 }

@@ -9,7 +9,6 @@
 #include "spmm_mfma_f32_device.cuh"
 #include "spmm_dense_device.cuh"
 #include "spmm_smallk_device.cuh"
-#include "spmm_ksplit_device.cuh"
 
 namespace iex {
 namespace {
@@ -137,6 +136,64 @@ int launch_wpr(const SpmmParams& p, int batch, int wpr, int nt, hipStream_t stre
     case 8: return launch_one<T, IT, VEC, LPG, 8>(p, batch, stream);
   }
   return fail(IEX_ERR_BAD_ARGUMENT, "spmm: waves-per-row must be 1, 4 or 8 (got %d)", wpr);
+}
+
+// ---- row kernel with wavefronts per row that follow the row's own length ---------------------------------
+template <typename T, typename IT, int VEC, int LPG>
+__global__ __launch_bounds__(kRowsWaves * kWave) void spmm_rows_kernel(SpmmParams p, RowClasses rc) {
+  __shared__ float red[spmm_rows_lds_floats<VEC>()];
+  spmm_rows_block<T, IT, VEC, LPG>(p, rc, blockIdx.x, blockIdx.y, blockIdx.z, red);
+}
+
+// From the histogram of row lengths (hist[j] = rows with more than 64 << j nonzeros, j = 0 .. 15) to the five ranges
+// of row slots.  A wavefront should get at most `rounds` chunks of 64 nonzeros (a power of two, 1 .. 16): a row of c
+// chunks gets the smallest power of two >= c / rounds wavefronts, at most 16.  `rounds` follows the work per
+// wavefront slot when every row is cut that way: with fewer chunks than the chip holds wavefronts (256 CUs x 16) one
+// chunk per wavefront is the shortest critical path; with more, cutting finer only adds partial sums.
+inline RowClasses row_classes(const SpmmParams& p, const int* hist, int tiles, int force_log2_rounds_plus_1, int* rounds_out) {
+  const double chunks = (double)p.nnz / kWave * tiles;
+  int r = 0;   // log2(rounds)
+  while (r < 4 && chunks / (1 << r) > 256.0 * 16) ++r;
+  if (force_log2_rounds_plus_1 > 0) r = std::min(force_log2_rounds_plus_1 - 1, 8);
+  auto rows_over = [&](int log2_chunks) { return log2_chunks > 15 ? 0 : std::min(p.m, std::max(0, hist[log2_chunks])); };
+  RowClasses rc;
+  // class c: 16 >> c wavefronts; a row belongs to class c or an earlier one when it has more than (8 >> c) * rounds chunks
+  rc.first_row[0] = 0;
+  int before = 0;
+  for (int c = 0; c < 4; ++c) {
+    const int upto = std::max(before, rows_over(3 - c + r));   // rows with more than 64 << (3 - c + r) nonzeros
+    rc.first_row[c + 1] = upto;
+    before = upto;
+  }
+  rc.first_row[5] = p.m;
+  rc.first_block[0] = 0;
+  for (int c = 0; c < 5; ++c) rc.first_block[c + 1] = rc.first_block[c] + ceil_div(rc.first_row[c + 1] - rc.first_row[c], 1 << c);
+  rc.log2_rounds = r;
+  *rounds_out = 1 << r;
+  return rc;
+}
+
+template <typename T, typename IT, int VEC, int LPG>
+int launch_rows_one(const SpmmParams& p, int batch, const int* hist, int rounds_code, hipStream_t stream) {
+  const int tiles = ceil_div(p.n, LPG * VEC);
+  int rounds = 1;
+  const RowClasses rc = row_classes(p, hist, tiles * batch, rounds_code, &rounds);
+  note_kernel("spmm_rows_kernel<%s, %s, %d, %d> (rows by 16/8/4/2/1 waves: %d/%d/%d/%d/%d, %d chunks per wave)", type_name<T>(), type_name<IT>(), VEC, LPG,
+              rc.first_row[1], rc.first_row[2] - rc.first_row[1], rc.first_row[3] - rc.first_row[2], rc.first_row[4] - rc.first_row[3],
+              rc.first_row[5] - rc.first_row[4], rounds);
+  hipLaunchKernelGGL((spmm_rows_kernel<T, IT, VEC, LPG>), dim3(rc.first_block[5], tiles, batch), dim3(kRowsWaves * kWave), 0, stream, p, rc);
+  return check_hip(hipGetLastError(), "spmm (rows by length) launch");
+}
+
+template <typename T, typename IT>
+int launch_rows(const SpmmParams& p, int batch, int lpg, const int* hist, int rounds_code, hipStream_t stream) {
+  constexpr int kMax = 16 / (int)sizeof(T);
+  switch (lpg) {
+    case 8: return launch_rows_one<T, IT, kMax, 8>(p, batch, hist, rounds_code, stream);
+    case 16: return launch_rows_one<T, IT, kMax, 16>(p, batch, hist, rounds_code, stream);
+    case 32: return launch_rows_one<T, IT, kMax, 32>(p, batch, hist, rounds_code, stream);
+    default: return launch_rows_one<T, IT, kMax, 64>(p, batch, hist, rounds_code, stream);
+  }
 }
 
 // ---- LDS-staged variant -----------------------------------------------------------------
@@ -327,97 +384,9 @@ inline int launch_mfma_f32(const SpmmParams& p, int batch, int arrangement, int 
   return fail(IEX_ERR_BAD_ARGUMENT, "spmm: arrangement of the fp32 matrix-core variant must be 1, 2, 4, 5 or 6 (got %d)", arrangement);
 }
 
-// ---- slice of the dense operand resident in LDS, k split over workgroups ------------------------------
-template <typename T, typename IT, int VEC, int RPW, int WAVES, int KB>
-__global__ __launch_bounds__(WAVES * kWave, WAVES == 8 ? 2 : 1) void spmm_ksplit_kernel(KsplitParams q) {
-  extern __shared__ __align__(16) unsigned char smem[];
-  spmm_ksplit_block<T, IT, VEC, RPW, WAVES, KB>(q, blockIdx.x / q.slices, blockIdx.x % q.slices, blockIdx.y, blockIdx.z, smem);
-}
-
-struct KsplitPlan {
-  int vec = 0;        // elements per lane: the tile is 64 * vec columns (0 = the shape does not fit)
-  int waves = 8;      // wavefronts per workgroup: 8 (two workgroups per CU) or 16 (one, stages twice as long)
-  int slices = 1;     // k slices
-  int slice_rows = 0; // dense rows per slice
-  size_t partial_bytes = 0;
-};
-
-constexpr int kKsplitRpw = 8;
-
-template <typename T>
-constexpr int ksplit_kb(int vec, int waves) {
-  // 32 KB stages (64 KB with 16 wavefronts), at most 64 dense rows (one window of nonzeros per row and stage)
-  const int rb = kWave * vec * (int)sizeof(T);
-  const int kb = (waves == 16 ? 65536 : 32768) / rb;
-  return kb > 64 ? 64 : kb;
-}
-
-// Tile width, slices and partial-sum bytes for a shape; plan.vec == 0 when the kernel cannot take it.
-template <typename T>
-KsplitPlan ksplit_plan(const SpmmParams& p, int batch, int force_slices, int force_waves) {
-  KsplitPlan pl;
-  constexpr int kMax = 16 / (int)sizeof(T);
-  if (!(p.nnz > 0 && p.k > 0 && p.n >= kMax && p.n % kMax == 0 && p.k <= 262144 && aligned(p.dense, 16) && aligned(p.out, 16))) return pl;
-  int vec = kMax;
-  while (vec > kMax / 4 && kWave * (vec / 2) >= p.n) vec >>= 1;   // the narrowest tile that holds n
-  pl.vec = vec;
-  pl.waves = force_waves == 16 && vec == kMax ? 16 : 8;
-  const int kb = ksplit_kb<T>(vec, pl.waves);
-  const long long row_blocks = ceil_div(p.m, pl.waves * kKsplitRpw);
-  const long long cells = row_blocks * ceil_div(p.n, kWave * vec) * batch;
-  // two workgroups of 8 wavefronts (one of 16) per CU, and the slices a multiple of the 8 XCDs where that is
-  // possible: consecutive workgroup ids go to consecutive XCDs, so each L2 then holds one slice of the operand
-  const long long want = pl.waves == 16 ? 256 : 512;
-  int slices = force_slices > 0 ? force_slices : (int)std::min<long long>(16, std::max<long long>(1, (want + cells - 1) / cells));
-  if (force_slices == 0 && slices > 4 && slices < 8) slices = 8;
-  slices = std::min(slices, ceil_div(p.k, kb));
-  pl.slice_rows = ceil_div(ceil_div(p.k, slices), kb) * kb;
-  pl.slices = ceil_div(p.k, pl.slice_rows);
-  pl.partial_bytes = pl.slices > 1 ? (size_t)pl.slices * batch * p.m * p.n * sizeof(float) : 0;
-  return pl;
-}
-
-template <typename T, typename IT, int VEC, int WAVES>
-int launch_ksplit_one(const SpmmParams& p, int batch, const KsplitPlan& pl, float* partial, hipStream_t stream) {
-  constexpr int KB = ksplit_kb<T>(VEC, WAVES);
-  constexpr int lds = spmm_ksplit_lds_bytes<VEC, T, KB>();
-  KsplitParams q{p, ceil_div(p.m, WAVES * kKsplitRpw), pl.slices, pl.slice_rows, partial};
-  IEX_REQUIRE((long long)q.row_blocks * q.slices < (1ll << 31), IEX_ERR_TOO_LARGE, "spmm (k split): grid too large");
-  auto kernel = spmm_ksplit_kernel<T, IT, VEC, kKsplitRpw, WAVES, KB>;
-  if (lds >= 64 * 1024) {
-    static thread_local bool raised = false;   // per instantiation
-    if (!raised) {
-      if (int rc = check_hip(hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, lds),
-                             "hipFuncSetAttribute(LDS size)"))
-        return rc;
-      raised = true;
-    }
-  }
-  note_kernel("spmm_ksplit_kernel<%s, %s, %d, %d, %d, %d> (%d slices)", type_name<T>(), type_name<IT>(), VEC, kKsplitRpw, WAVES, KB, pl.slices);
-  hipLaunchKernelGGL(kernel, dim3(q.row_blocks * q.slices, ceil_div(p.n, kWave * VEC), batch), dim3(WAVES * kWave), lds, stream, q);
-  if (int rc = check_hip(hipGetLastError(), "spmm (k split) launch")) return rc;
-  if (pl.slices > 1) {
-    const size_t quads = (size_t)batch * p.m * p.n / 4;
-    const int blocks = (int)std::min<size_t>((quads + 255) / 256, 256 * 16);
-    note_kernel("spmm_ksplit_reduce_kernel<%s>", type_name<T>());
-    hipLaunchKernelGGL((spmm_ksplit_reduce_kernel<T>), dim3(blocks), dim3(256), 0, stream, p, partial, pl.slices, batch);
-    return check_hip(hipGetLastError(), "spmm (k split) reduction launch");
-  }
-  return 0;
-}
-
-template <typename T, typename IT>
-int launch_ksplit(const SpmmParams& p, int batch, const KsplitPlan& pl, void* ws, hipStream_t stream) {
-  constexpr int kMax = 16 / (int)sizeof(T);
-  float* partial = static_cast<float*>(ws);
-  if (pl.vec == kMax && pl.waves == 16) return launch_ksplit_one<T, IT, kMax, 16>(p, batch, pl, partial, stream);
-  if (pl.vec == kMax) return launch_ksplit_one<T, IT, kMax, 8>(p, batch, pl, partial, stream);
-  if (pl.vec == kMax / 2) return launch_ksplit_one<T, IT, kMax / 2, 8>(p, batch, pl, partial, stream);
-  return launch_ksplit_one<T, IT, kMax / 4, 8>(p, batch, pl, partial, stream);
-}
-
 struct Choice {
   int wpr = 0;      // wavefronts per row of the row kernel
+  bool wpr_forced = false;
   int variant = 0;  // 0 = choose, 1 = row kernel, 2 = LDS-staged kernel, 3 / 4 = matrix-core kernels (16-bit), 5 = (fp32)
   int rpw = 0;      // rows per wavefront of the LDS-staged kernel (0 = choose)
   int nt = 0;       // adjacent column tiles per wavefront of the row kernel (0 = choose)
@@ -425,6 +394,7 @@ struct Choice {
   void* ws = nullptr;   // caller's workspace for the dense form of A (variant 7), may be null
   size_t ws_bytes = 0;
   bool any_order = false;   // columns of a row in any order, possibly repeated: families 1 and 8 only
+  const int* hist = nullptr;   // host: rows with more than 64 << j nonzeros, j = 0 .. 15 (iex_spmm_sched), may be null
 };
 
 // The LDS-staged kernel needs a full-width tile (64 lanes x VEC, VEC the full or half 128-bit
@@ -466,6 +436,9 @@ bool lds_variant(const SpmmParams& p, int batch, const Choice& ch, int& vec, int
 // k < 65535 for the 8-wave arrangement (packed columns).  Sets kind = 3 (4 waves, 128 x 256
 // tiles; param = lanes per row) or 4 (8 waves, 128 x 512 tiles; param = windows per row);
 // kind 0 = use a gather kernel.
+// nothing about the row kernel's waves per row was asked for
+inline bool flags_wpr_free(const Choice& ch) { return !ch.wpr_forced && (ch.variant == 0 || ch.variant == 1); }
+
 struct MfmaChoice {
   int kind = 0, param = 0;
 };
@@ -613,13 +586,6 @@ int launch_typed(const SpmmParams& p, int batch, const Choice& given, hipStream_
     return launch_smallk<T, IT>(p, batch, stream);
   }
   if constexpr (std::is_same<T, float>::value && std::is_same<IT, int>::value) {
-    if (ch.variant == 9) {
-      const KsplitPlan pl = ksplit_plan<T>(p, batch, ch.rpw, ch.nt == 2 ? 16 : 8);
-      IEX_REQUIRE(pl.vec > 0, IEX_ERR_UNSUPPORTED, "spmm: the k-split kernel needs n a multiple of the 128-bit vector, 16-byte aligned dense operands and k <= 262144");
-      IEX_REQUIRE(pl.partial_bytes == 0 || (ch.ws && aligned(ch.ws, 16) && ch.ws_bytes >= pl.partial_bytes), IEX_ERR_BAD_ARGUMENT,
-                  "spmm: the k-split kernel needs a 16-byte aligned workspace of %zu bytes for its partial sums (iex_spmm_ws)", pl.partial_bytes);
-      return launch_ksplit<T, IT>(p, batch, pl, ch.ws, stream);
-    }
     int windows = 0;
     if (const int arr = mfma_f32_variant<T, IT>(p, batch, ch, windows)) return launch_mfma_f32(p, batch, arr, windows, ch.lpg != 8, stream);  // (lanes-per-group code 8 = no role split, for tuning)
   }
@@ -648,13 +614,26 @@ int launch_typed(const SpmmParams& p, int batch, const Choice& given, hipStream_
     return launch_smallk<T, IT>(p, batch, stream);
   }
   int lvec = 0, rpw = 0;
-  if (lds_variant<T>(p, batch, ch, lvec, rpw)) {
+  if (ch.variant != 11 && lds_variant<T>(p, batch, ch, lvec, rpw)) {
     if (lvec == kMax) return launch_lds_rpw<T, IT, kMax>(p, batch, rpw, stream);
     return launch_lds_rpw<T, IT, kMax / 2>(p, batch, rpw, stream);
   }
   const int wpr = ch.wpr;
   SpmmShape sh = spmm_pick_shape<T>(p.n, p.dense, p.out);
   if (ch.lpg && sh.vec == kMax && ch.lpg <= sh.lpg) sh.lpg = ch.lpg;  // narrower tiles on request
+  // The caller knows the pattern's row lengths: wavefronts per row by the row's own length instead of one number for
+  // the whole matrix.  Measured on MI355X (fp32, 4096 x 4096, geometric row lengths, us, four waves for every row /
+  // this kernel at its best chunks-per-wave): 98 % sparse n = 64 9.0 / 7.6, n = 128 12.5 / 11.2, n = 256 17.2 / 20.0;
+  // 95 % 12.7 / 13.9, 19.7 / 22.3, 36.9 / 39.2; 90 % 19.1 / 22.0, 36.7 / 38.6, 69.4 / 67.0; 80 % 33 / 42, 59 / 73,
+  // 119 / 122.  The row kernel is bound by the gathers' way from L2 into the CUs (20-26 TB/s on every n = 256
+  // cell), not by its longest rows: four waves on every row keep more gathers in flight than a schedule that gives short
+  // rows one wave, and that wins wherever the chip is full.  So this kernel is taken where it is not: fewer chunks
+  // of 64 nonzeros than the chip holds wavefronts, and narrow tiles (several nonzeros per gather instruction).
+  if (ch.variant == 11) IEX_REQUIRE(ch.hist && sh.vec == kMax, IEX_ERR_BAD_ARGUMENT, "spmm: the rows-by-length kernel needs the row-length histogram (iex_spmm_sched) and full 128-bit vectors");
+  const double chunk_count = (double)p.nnz / kWave * ceil_div(p.n, sh.lpg * sh.vec) * batch;
+  if (ch.hist && sh.vec == kMax && ch.nt <= 1 &&
+      (ch.variant == 11 || (flags_wpr_free(ch) && ch.hist[0] > 0 && wpr != 1 && sh.lpg <= 32 && chunk_count <= 8192.0)))
+    return launch_rows<T, IT>(p, batch, sh.lpg, ch.hist, ch.variant == 11 ? ch.rpw : 0, stream);
   // Two tiles per wave double the slice of the dense operand that the waves of an XCD share in
   // its L2 and measured slower (2x at k = 4096, n = 8192): only on request.
   const int nt = ch.nt ? ch.nt : 1;
@@ -690,7 +669,7 @@ int spmm_matrix_core_windows(const SpmmParams& p) {
 int spmm_dispatch(int dtype, int itype, int flags, int m, int k, int n, int nonzeros,
                   const int* row_indices, const void* values, const int* row_offsets,
                   const void* column_indices, const void* dense, const float* bias, void* out,
-                  void* stream, int batch, void* workspace, size_t workspace_bytes) {
+                  void* stream, int batch, void* workspace, size_t workspace_bytes, const int* row_histogram = nullptr) {
   IEX_REQUIRE(m >= 0 && k >= 0 && n >= 0 && nonzeros >= 0 && batch >= 0, IEX_ERR_BAD_ARGUMENT,
               "spmm: negative dimension (m=%d k=%d n=%d nnz=%d batch=%d)", m, k, n, nonzeros, batch);
   trail_reset();
@@ -706,7 +685,9 @@ int spmm_dispatch(int dtype, int itype, int flags, int m, int k, int n, int nonz
               "spmm: int16 column indices need k <= 32768 (k=%d)", k);
   Choice ch;
   ch.wpr = (flags >> 8) & 0xff;
+  ch.wpr_forced = ch.wpr != 0;
   if (ch.wpr == 0) ch.wpr = spmm_pick_wpr(m, nonzeros, dtype == IEX_F32 ? 4 : 2, n, batch);
+  ch.hist = row_histogram;
   ch.variant = (flags >> 16) & 0xf;
   ch.rpw = (flags >> 20) & 0xf;
   ch.nt = (flags >> 24) & 0xf;
@@ -723,6 +704,7 @@ int spmm_dispatch(int dtype, int itype, int flags, int m, int k, int n, int nonz
   if (ch.variant == 10 && nonzeros < 8) {   // (its loads of eight values at a time need eight to exist: the row kernel instead)
     ch.variant = 1;
     ch.wpr = spmm_pick_wpr(m, nonzeros, dtype == IEX_F32 ? 4 : 2, n, batch);   // (bits 8..15 meant the dense-block threshold)
+    ch.wpr_forced = false;
   }
   const int blocks_ready = ((flags & IEX_SPMM_TABLES_READY) ? 1 : 0) | ((flags & IEX_SPMM_LISTS_READY) ? 2 : 0);
   if (ch.variant == 0 && !ch.any_order && ch.ws && aligned(ch.ws, 16) && spmm_blocks_fits(dtype, itype, p) && spmm_blocks_wins(p, batch) &&
@@ -752,13 +734,6 @@ static size_t workspace_plan(int dtype, int itype, int flags, int m, int k, int 
   const int variant = (flags >> 16) & 0xf;
   if (variant == 0 && (flags & IEX_SPMM_ANY_COLUMN_ORDER)) return 0;   // families 1 and 8 use no workspace
   void* const some_aligned = reinterpret_cast<void*>(size_t(256));
-  if (dtype == IEX_F32 && itype == IEX_I32) {
-    SpmmParams p{m, k, n, nonzeros, nullptr, nullptr, nullptr, nullptr, some_aligned, nullptr, some_aligned, 0, 0, 0};
-    if (variant != 9) return 0;
-    const size_t bytes = ksplit_plan<float>(p, batch, (flags >> 20) & 0xf, ((flags >> 24) & 0xf) == 2 ? 16 : 8).partial_bytes;
-    if (bytes) *kind = 9;
-    return bytes;
-  }
   if (!(dtype == IEX_F16 || dtype == IEX_BF16) || !(itype == IEX_I32 || itype == IEX_I16)) return 0;
   if (variant != 0 && variant != 7 && variant != 10) return 0;
   SpmmParams p{m, k, n, nonzeros, nullptr, nullptr, nullptr, nullptr, some_aligned, nullptr, some_aligned,
@@ -860,6 +835,14 @@ int iex_spmm_ws(int dtype, int itype, int flags, int m, int k, int n, int nonzer
                 void* stream, int batch, void* workspace, size_t workspace_bytes) {
   return iex::spmm_dispatch(dtype, itype, flags, m, k, n, nonzeros, row_indices, values, row_offsets,
                             column_indices, dense, bias, out, stream, batch, workspace, workspace_bytes);
+}
+
+int iex_spmm_sched(int dtype, int itype, int flags, int m, int k, int n, int nonzeros,
+                   const int* row_indices, const void* values, const int* row_offsets,
+                   const void* column_indices, const void* dense, const float* bias, void* out,
+                   void* stream, int batch, void* workspace, size_t workspace_bytes, const int* row_histogram) {
+  return iex::spmm_dispatch(dtype, itype, flags, m, k, n, nonzeros, row_indices, values, row_offsets,
+                            column_indices, dense, bias, out, stream, batch, workspace, workspace_bytes, row_histogram);
 }
 
 size_t iex_spmm_workspace_bytes(int dtype, int itype, int flags, int m, int k, int n, int nonzeros, int batch) {

@@ -59,152 +59,120 @@ struct row_slab {
   vec_t<T, VEC> t[NT];
 };
 
-// One workgroup's share: block (bx, by, bz) of the grid
-//   (ceil(m / rows_per_block), ceil(n / (NT*LPG*VEC)), batch).
-// `red` must hold spmm_lds_floats<VEC,WPR,NT>() floats.  Every thread of the workgroup
-// must call this when WPR > 1 (it contains a barrier).
+// One wavefront's share of one row: the sums of the nonzeros in the chunks part, part + wpr, part + 2 wpr ... (64
+// nonzeros each) of CSR row `row`, for the NT column tiles that start at col_ld[] (element offsets inside a dense
+// row; lanes beyond n point at a valid address and their sums are never stored).  Any wpr >= 1 and any part < wpr
+// give a correct partition of the row's nonzeros over the wpr wavefronts that call this for the row.
 // WIN = gathers a wave keeps in flight (rolling window); raise it where few waves fit a CU.
-// NT  = adjacent 64*VEC-column tiles a wave covers (G == 1 only): per nonzero the wave then
-//       reads NT*64*VEC contiguous elements of one dense row, which amortises the broadcast
-//       of (column, value) and keeps very wide dense operands on fewer pages.
-// RAGGED = n is not a multiple of VEC: vectors are moved at element alignment, and the one lane of a
-//       row whose vector would reach past the row's end reads VEC elements ending at the row's end
-//       instead (shifted back by `shift`), sums all of them and stores only the ones it owns.
-template <typename T, typename IT, int VEC, int LPG, int WPR, int WIN = kSpmmUnroll, int NT = 1, bool RAGGED = false>
-__device__ __forceinline__ void spmm_block(const SpmmParams& p, int bx, int by, int bz, float* red) {
-  static_assert(!RAGGED || (NT == 1 && LPG == kWave), "ragged rows: one full-width tile per wave");
-  constexpr int kWavesPerBlock = (WPR > 4) ? WPR : 4;
-  constexpr int kRowsPerBlock = kWavesPerBlock / WPR;
+// RAGGED = vectors at element alignment (n not a multiple of VEC).
+template <typename T, typename IT, int VEC, int LPG, int WIN, int NT, bool RAGGED>
+__device__ __forceinline__ void spmm_row_partial(const SpmmParams& p, int z, int row, int part, int wpr, const int (&col_ld)[NT],
+                                                 float (&acc)[NT][VEC]) {
   constexpr int G = kWave / LPG;
-  constexpr int TW = LPG * VEC;  // columns of one tile
-  static_assert(NT == 1 || G == 1, "several tiles per wave need the whole wave on one nonzero");
   typedef row_slab<T, VEC, NT> Slab;
   const int lane = lane_id();
-  const int wave = uniform(threadIdx.x >> 6);
-  const int z = bz;
-  const int row_slot = bx * kRowsPerBlock + wave / WPR;
-  const int part = wave % WPR;  // which share of the row this wave sums
   const int grp = lane / LPG;   // which nonzero of a step this lane works on (0 when G == 1)
+  const int start = uniform(p.row_offsets[row]);
+  const int end = uniform(p.row_offsets[row + 1]);
+  const T* __restrict__ values =
+      static_cast<const T*>(p.values) + (p.per_batch_values ? (size_t)z * p.nnz : (size_t)0);
+  const IT* __restrict__ cols = static_cast<const IT*>(p.cols);
+  const T* __restrict__ dense = static_cast<const T*>(p.dense) + (size_t)z * p.k * p.n;
 
-  const int col0 = by * (NT * TW) + (lane % LPG) * VEC;  // first tile; tile t starts TW*t further
-  const int shift = (RAGGED && col0 < p.n && col0 + VEC > p.n) ? col0 + VEC - p.n : 0;  // (n >= VEC, checked by the host)
-  int col_ld[NT];                                         // idle lanes gather a valid address, result unused
+  auto load_row = [&](int column) {
+    Slab s;
+    const T* r = dense + (size_t)column * p.n;
 #pragma unroll
-  for (int t = 0; t < NT; ++t) col_ld[t] = (col0 + t * TW < p.n) ? col0 + t * TW - shift : 0;
+    for (int t = 0; t < NT; ++t) s.t[t] = load_vec<T, VEC, !RAGGED>(r + col_ld[t]);
+    return s;
+  };
+  auto fma_row = [&](float a, const Slab& s) {
+#pragma unroll
+    for (int t = 0; t < NT; ++t) fma_vec<T, VEC>(acc[t], a, s.t[t]);
+  };
 
-  float acc[NT][VEC];
-#pragma unroll
-  for (int t = 0; t < NT; ++t)
-#pragma unroll
-    for (int i = 0; i < VEC; ++i) acc[t][i] = 0.f;
-
-  const bool row_live = row_slot < p.m;  // wave-uniform
-  int row = 0;
-  if (row_live) {
-    row = uniform(p.row_indices[row_slot]);
-    const int start = uniform(p.row_offsets[row]);
-    const int end = uniform(p.row_offsets[row + 1]);
-    const T* __restrict__ values =
-        static_cast<const T*>(p.values) + (p.per_batch_values ? (size_t)z * p.nnz : (size_t)0);
-    const IT* __restrict__ cols = static_cast<const IT*>(p.cols);
-    const T* __restrict__ dense = static_cast<const T*>(p.dense) + (size_t)z * p.k * p.n;
-
-    auto load_row = [&](int column) {
-      Slab s;
-      const T* r = dense + (size_t)column * p.n;
-#pragma unroll
-      for (int t = 0; t < NT; ++t) s.t[t] = load_vec<T, VEC, !RAGGED>(r + col_ld[t]);
-      return s;
-    };
-    auto fma_row = [&](float a, const Slab& s) {
-#pragma unroll
-      for (int t = 0; t < NT; ++t) fma_vec<T, VEC>(acc[t], a, s.t[t]);
-    };
-
-    // (value, column) of nonzero base+lane; the next chunk is fetched while the current
-    // one is being processed, so its latency hides behind the gathers.
-    int base = start + part * kWave;
-    float v = 0.f;
-    int c = 0;
-    if (base + lane < end) {
-      v = elem<T>::to_float(values[base + lane]);
-      c = (int)cols[base + lane];
+  // (value, column) of nonzero base+lane; the next chunk is fetched while the current
+  // one is being processed, so its latency hides behind the gathers.
+  int base = start + part * kWave;
+  float v = 0.f;
+  int c = 0;
+  if (base + lane < end) {
+    v = elem<T>::to_float(values[base + lane]);
+    c = (int)cols[base + lane];
+  }
+  while (base < end) {
+    const int next = base + kWave * wpr;
+    float v_next = 0.f;
+    int c_next = 0;
+    if (next + lane < end) {
+      v_next = elem<T>::to_float(values[next + lane]);
+      c_next = (int)cols[next + lane];
     }
-    while (base < end) {
-      const int next = base + kWave * WPR;
-      float v_next = 0.f;
-      int c_next = 0;
-      if (next + lane < end) {
-        v_next = elem<T>::to_float(values[next + lane]);
-        c_next = (int)cols[next + lane];
-      }
-      const int cnt = min(kWave, end - base);  // wave-uniform
-      if constexpr (G == 1) {
-        auto gather = [&](int t) { return load_row(bcast_i(c, t)); };
-        if (cnt == kWave) {
-          // full chunk: rolling window of WIN gathers in flight, refilled after every FMA
-          Slab bv[WIN];
+    const int cnt = min(kWave, end - base);  // wave-uniform
+    if constexpr (G == 1) {
+      auto gather = [&](int t) { return load_row(bcast_i(c, t)); };
+      if (cnt == kWave) {
+        // full chunk: rolling window of WIN gathers in flight, refilled after every FMA
+        Slab bv[WIN];
 #pragma unroll
-          for (int u = 0; u < WIN; ++u) bv[u] = gather(u);
+        for (int u = 0; u < WIN; ++u) bv[u] = gather(u);
 #pragma unroll
-          for (int t = 0; t < kWave; ++t) {
-            fma_row(bcast_f(v, t), bv[t % WIN]);
-            if (t + WIN < kWave) bv[t % WIN] = gather(t + WIN);
-          }
-        } else {
-          int t = 0;
-          for (; t + WIN <= cnt; t += WIN) {
-            Slab bv[WIN];
-#pragma unroll
-            for (int u = 0; u < WIN; ++u) bv[u] = gather(t + u);
-#pragma unroll
-            for (int u = 0; u < WIN; ++u) fma_row(bcast_f(v, t + u), bv[u]);
-          }
-          for (; t < cnt; ++t) fma_row(bcast_f(v, t), gather(t));
+        for (int t = 0; t < kWave; ++t) {
+          fma_row(bcast_f(v, t), bv[t % WIN]);
+          if (t + WIN < kWave) bv[t % WIN] = gather(t + WIN);
         }
       } else {
-        // step s: group g works on nonzero s*G + g of this chunk
-        constexpr int kSteps = kWave / G;
-        constexpr int kWin = kSteps < WIN ? kSteps : WIN;
-        auto fetch = [&](int s, float& vs) {
-          const int src = ((s * G + grp) & (kWave - 1)) << 2;
-          vs = __int_as_float(__builtin_amdgcn_ds_bpermute(src, __float_as_int(v)));
-          return __builtin_amdgcn_ds_bpermute(src, c);
-        };
-        if (cnt == kWave) {
+        int t = 0;
+        for (; t + WIN <= cnt; t += WIN) {
+          Slab bv[WIN];
+#pragma unroll
+          for (int u = 0; u < WIN; ++u) bv[u] = gather(t + u);
+#pragma unroll
+          for (int u = 0; u < WIN; ++u) fma_row(bcast_f(v, t + u), bv[u]);
+        }
+        for (; t < cnt; ++t) fma_row(bcast_f(v, t), gather(t));
+      }
+    } else {
+      // step s: group g works on nonzero s*G + g of this chunk
+      constexpr int kSteps = kWave / G;
+      constexpr int kWin = kSteps < WIN ? kSteps : WIN;
+      auto fetch = [&](int s, float& vs) {
+        const int src = ((s * G + grp) & (kWave - 1)) << 2;
+        vs = __int_as_float(__builtin_amdgcn_ds_bpermute(src, __float_as_int(v)));
+        return __builtin_amdgcn_ds_bpermute(src, c);
+      };
+      if (cnt == kWave) {
+        Slab bv[kWin];
+        float vv[kWin];
+#pragma unroll
+        for (int u = 0; u < kWin; ++u) bv[u] = load_row(fetch(u, vv[u]));
+#pragma unroll
+        for (int s = 0; s < kSteps; ++s) {
+          fma_row(vv[s % kWin], bv[s % kWin]);
+          if (s + kWin < kSteps) bv[s % kWin] = load_row(fetch(s + kWin, vv[s % kWin]));
+        }
+      } else {
+        const int steps = cnt / G;  // full steps: every group has a real nonzero
+        int s = 0;
+        for (; s + kWin <= steps; s += kWin) {
           Slab bv[kWin];
           float vv[kWin];
 #pragma unroll
-          for (int u = 0; u < kWin; ++u) bv[u] = load_row(fetch(u, vv[u]));
+          for (int u = 0; u < kWin; ++u) bv[u] = load_row(fetch(s + u, vv[u]));
 #pragma unroll
-          for (int s = 0; s < kSteps; ++s) {
-            fma_row(vv[s % kWin], bv[s % kWin]);
-            if (s + kWin < kSteps) bv[s % kWin] = load_row(fetch(s + kWin, vv[s % kWin]));
-          }
-        } else {
-          const int steps = cnt / G;  // full steps: every group has a real nonzero
-          int s = 0;
-          for (; s + kWin <= steps; s += kWin) {
-            Slab bv[kWin];
-            float vv[kWin];
-#pragma unroll
-            for (int u = 0; u < kWin; ++u) bv[u] = load_row(fetch(s + u, vv[u]));
-#pragma unroll
-            for (int u = 0; u < kWin; ++u) fma_row(vv[u], bv[u]);
-          }
-          for (; s * G < cnt; ++s) {
-            float vu;
-            const int cu = fetch(s, vu);
-            if (s * G + grp < cnt) fma_row(vu, load_row(cu));
-          }
+          for (int u = 0; u < kWin; ++u) fma_row(vv[u], bv[u]);
+        }
+        for (; s * G < cnt; ++s) {
+          float vu;
+          const int cu = fetch(s, vu);
+          if (s * G + grp < cnt) fma_row(vu, load_row(cu));
         }
       }
-      base = next;
-      v = v_next;
-      c = c_next;
     }
+    base = next;
+    v = v_next;
+    c = c_next;
   }
-
   if constexpr (G > 1) {
     // combine the G groups: afterwards every lane holds the sum for its columns
 #pragma unroll
@@ -213,28 +181,12 @@ __device__ __forceinline__ void spmm_block(const SpmmParams& p, int bx, int by, 
       for (int i = 0; i < VEC; ++i) acc[0][i] += __shfl_xor(acc[0][i], off, kWave);
     }
   }
+}
 
-  if constexpr (WPR > 1) {
-    // Every wave of the block reaches this barrier: a block holds exactly one row when
-    // WPR > 1, so row_live is uniform over the block and idle blocks fall through with
-    // zero partials.
-#pragma unroll
-    for (int t = 0; t < NT; ++t)
-#pragma unroll
-      for (int i = 0; i < VEC; ++i) red[((wave * NT + t) * VEC + i) * kWave + lane] = acc[t][i];
-    __syncthreads();
-    if (part != 0) return;
-#pragma unroll
-    for (int t = 0; t < NT; ++t)
-#pragma unroll
-      for (int i = 0; i < VEC; ++i) {
-        float s = acc[t][i];
-        for (int w = 1; w < WPR; ++w) s += red[(((wave + w) * NT + t) * VEC + i) * kWave + lane];
-        acc[t][i] = s;
-      }
-  }
-
-  if (!row_live || grp != 0) return;
+// Bias, ReLU, accumulation and the store of one row's sums (lanes of group 0 only; col0 = first column of tile 0).
+template <typename T, int VEC, int LPG, int NT, bool RAGGED>
+__device__ __forceinline__ void spmm_store_row(const SpmmParams& p, int z, int row, int col0, int shift, float (&acc)[NT][VEC]) {
+  constexpr int TW = LPG * VEC;
   const float bias = p.bias ? p.bias[row] : 0.f;
 #pragma unroll
   for (int t = 0; t < NT; ++t) {
@@ -263,6 +215,179 @@ __device__ __forceinline__ void spmm_block(const SpmmParams& p, int bx, int by, 
       store_vec<T, VEC, !RAGGED>(out, o);
     }
   }
+}
+
+// One workgroup's share: block (bx, by, bz) of the grid
+//   (ceil(m / rows_per_block), ceil(n / (NT*LPG*VEC)), batch).
+// `red` must hold spmm_lds_floats<VEC,WPR,NT>() floats.  Every thread of the workgroup
+// must call this when WPR > 1 (it contains a barrier).
+// NT  = adjacent 64*VEC-column tiles a wave covers (G == 1 only): per nonzero the wave then
+//       reads NT*64*VEC contiguous elements of one dense row, which amortises the broadcast
+//       of (column, value) and keeps very wide dense operands on fewer pages.
+// RAGGED = n is not a multiple of VEC: vectors are moved at element alignment, and the one lane of a
+//       row whose vector would reach past the row's end reads VEC elements ending at the row's end
+//       instead (shifted back by `shift`), sums all of them and stores only the ones it owns.
+template <typename T, typename IT, int VEC, int LPG, int WPR, int WIN = kSpmmUnroll, int NT = 1, bool RAGGED = false>
+__device__ __forceinline__ void spmm_block(const SpmmParams& p, int bx, int by, int bz, float* red) {
+  static_assert(!RAGGED || (NT == 1 && LPG == kWave), "ragged rows: one full-width tile per wave");
+  constexpr int kWavesPerBlock = (WPR > 4) ? WPR : 4;
+  constexpr int kRowsPerBlock = kWavesPerBlock / WPR;
+  constexpr int G = kWave / LPG;
+  constexpr int TW = LPG * VEC;  // columns of one tile
+  static_assert(NT == 1 || G == 1, "several tiles per wave need the whole wave on one nonzero");
+  const int lane = lane_id();
+  const int wave = uniform(threadIdx.x >> 6);
+  const int z = bz;
+  const int row_slot = bx * kRowsPerBlock + wave / WPR;
+  const int part = wave % WPR;  // which share of the row this wave sums
+  const int grp = lane / LPG;   // which nonzero of a step this lane works on (0 when G == 1)
+
+  const int col0 = by * (NT * TW) + (lane % LPG) * VEC;  // first tile; tile t starts TW*t further
+  const int shift = (RAGGED && col0 < p.n && col0 + VEC > p.n) ? col0 + VEC - p.n : 0;  // (n >= VEC, checked by the host)
+  int col_ld[NT];                                         // idle lanes gather a valid address, result unused
+#pragma unroll
+  for (int t = 0; t < NT; ++t) col_ld[t] = (col0 + t * TW < p.n) ? col0 + t * TW - shift : 0;
+
+  float acc[NT][VEC];
+#pragma unroll
+  for (int t = 0; t < NT; ++t)
+#pragma unroll
+    for (int i = 0; i < VEC; ++i) acc[t][i] = 0.f;
+
+  const bool row_live = row_slot < p.m;  // wave-uniform
+  int row = 0;
+  if (row_live) {
+    row = uniform(p.row_indices[row_slot]);
+    spmm_row_partial<T, IT, VEC, LPG, WIN, NT, RAGGED>(p, z, row, part, WPR, col_ld, acc);
+  }
+
+  if constexpr (WPR > 1) {
+    // Every wave of the block reaches this barrier: a block holds exactly one row when
+    // WPR > 1, so row_live is uniform over the block and idle blocks fall through with
+    // zero partials.
+#pragma unroll
+    for (int t = 0; t < NT; ++t)
+#pragma unroll
+      for (int i = 0; i < VEC; ++i) red[((wave * NT + t) * VEC + i) * kWave + lane] = acc[t][i];
+    __syncthreads();
+    if (part != 0) return;
+#pragma unroll
+    for (int t = 0; t < NT; ++t)
+#pragma unroll
+      for (int i = 0; i < VEC; ++i) {
+        float s = acc[t][i];
+        for (int w = 1; w < WPR; ++w) s += red[(((wave + w) * NT + t) * VEC + i) * kWave + lane];
+        acc[t][i] = s;
+      }
+  }
+
+  if (!row_live || grp != 0) return;
+  spmm_store_row<T, VEC, LPG, NT, RAGGED>(p, z, row, col0, shift, acc);
+}
+
+// ---- wavefronts per row that follow the row's own length ------------------------------------------------
+// The rows come sorted by decreasing length (row_indices), so "rows that deserve 16 wavefronts, then those that deserve
+// 8, 4, 2, 1" are five consecutive ranges of row slots, and a workgroup of 16 wavefronts serves 1, 2, 4, 8 or 16 rows
+// of one range.  Workgroup ids run through the ranges in that order: the longest rows start first.  The ranges come
+// from the host (counted once per pattern) and settle how many wavefronts a row slot HAS.  Into how many parts a row's
+// nonzeros are cut, and so the order of its sum, follows from the row's own length alone: with the ranges the host
+// derives from a true histogram and rows in that order the two agree; with any other ranges or order a row that has
+// fewer wavefronts than parts lets them take its parts in turns, one that has more lets some idle -- time, never a
+// different bit of the result.
+constexpr int kRowsWaves = 16;
+struct RowClasses {
+  int first_row[6];     // class c (16 >> c wavefronts per row) holds row slots first_row[c] .. first_row[c + 1] - 1
+  int first_block[6];   // ... served by workgroups first_block[c] .. first_block[c + 1] - 1
+  int log2_rounds;      // a row of more than 64 << (3 - c + log2_rounds) nonzeros is cut into 16 >> c parts or more
+};
+
+template <int VEC>
+constexpr int spmm_rows_lds_floats() { return kRowsWaves * kWave * VEC; }
+
+template <typename T, typename IT, int VEC, int LPG>
+__device__ __forceinline__ void spmm_rows_block(const SpmmParams& p, const RowClasses& rc, int bx, int by, int bz, float* red) {
+  constexpr int TW = LPG * VEC;
+  const int lane = lane_id();
+  const int wave = uniform(threadIdx.x >> 6);
+  int cls = 0;
+#pragma unroll
+  for (int c = 1; c < 5; ++c) cls += (bx >= rc.first_block[c]) ? 1 : 0;   // (uniform; empty classes share a first block)
+  const int wpr = kRowsWaves >> cls;
+  const int row_slot = rc.first_row[cls] + ((bx - rc.first_block[cls]) << cls) + wave / wpr;
+  const int part = wave % wpr;
+  const int grp = lane / LPG;
+  const int col0 = by * TW + (lane % LPG) * VEC;
+  int col_ld[1] = {col0 < p.n ? col0 : 0};
+  float acc[1][VEC];
+#pragma unroll
+  for (int i = 0; i < VEC; ++i) acc[0][i] = 0.f;
+  const bool row_live = row_slot < rc.first_row[cls + 1];   // wave-uniform
+  int row = 0;
+  int parts = 1;   // of this row, by its own length
+  if (row_live) {
+    row = uniform(p.row_indices[row_slot]);
+    const int len = uniform(p.row_offsets[row + 1] - p.row_offsets[row]);
+    int own = 0;
+#pragma unroll
+    for (int c = 0; c < 4; ++c) own += (len > (kWave << (3 - c + rc.log2_rounds))) ? 0 : 1;
+    parts = kRowsWaves >> own;
+  }
+  if (cls == 4) {   // a wavefront per row: its parts one after the other, no LDS
+    if (!row_live) return;
+    spmm_row_partial<T, IT, VEC, LPG, kSpmmUnroll, 1, false>(p, bz, row, 0, parts, col_ld, acc);
+    for (int q = 1; q < parts; ++q) {
+      float more[1][VEC];
+#pragma unroll
+      for (int i = 0; i < VEC; ++i) more[0][i] = 0.f;
+      spmm_row_partial<T, IT, VEC, LPG, kSpmmUnroll, 1, false>(p, bz, row, q, parts, col_ld, more);
+#pragma unroll
+      for (int i = 0; i < VEC; ++i) acc[0][i] += more[0][i];
+    }
+    if (grp == 0) spmm_store_row<T, VEC, LPG, 1, false>(p, bz, row, col0, 0, acc);
+    return;
+  }
+  // (uniform over the workgroup from here) partial sums of a row meet in LDS and are added in the order of the parts
+  if (!__syncthreads_or(parts > wpr)) {
+    if (row_live && part < parts) spmm_row_partial<T, IT, VEC, LPG, kSpmmUnroll, 1, false>(p, bz, row, part, parts, col_ld, acc);
+#pragma unroll
+    for (int i = 0; i < VEC; ++i) red[(wave * VEC + i) * kWave + lane] = acc[0][i];
+    __syncthreads();
+    if (part != 0) return;
+#pragma unroll
+    for (int i = 0; i < VEC; ++i) {
+      float s = acc[0][i];
+      for (int w = 1; w < parts; ++w) s += red[((wave + w) * VEC + i) * kWave + lane];
+      acc[0][i] = s;
+    }
+  } else {
+    // some row of this workgroup has more parts than wavefronts: all take their parts in turns of wpr
+    float sum[VEC];
+#pragma unroll
+    for (int i = 0; i < VEC; ++i) sum[i] = 0.f;
+    for (int q = 0; q < kRowsWaves; q += wpr) {
+#pragma unroll
+      for (int i = 0; i < VEC; ++i) acc[0][i] = 0.f;
+      if (row_live && q + part < parts) spmm_row_partial<T, IT, VEC, LPG, kSpmmUnroll, 1, false>(p, bz, row, q + part, parts, col_ld, acc);
+#pragma unroll
+      for (int i = 0; i < VEC; ++i) red[(wave * VEC + i) * kWave + lane] = acc[0][i];
+      __syncthreads();
+      if (part == 0 && q < parts) {
+#pragma unroll
+        for (int i = 0; i < VEC; ++i) {
+          float s = q == 0 ? acc[0][i] : sum[i] + acc[0][i];
+          for (int w = 1; w < wpr; ++w)
+            if (q + w < parts) s += red[((wave + w) * VEC + i) * kWave + lane];
+          sum[i] = s;
+        }
+      }
+      __syncthreads();   // (the next turn writes the same slots)
+    }
+    if (part != 0) return;
+#pragma unroll
+    for (int i = 0; i < VEC; ++i) acc[0][i] = sum[i];
+  }
+  if (!row_live || grp != 0) return;
+  spmm_store_row<T, VEC, LPG, 1, false>(p, bz, row, col0, 0, acc);
 }
 
 // Host-side shape choice shared by the stand-alone and the fused launcher.

@@ -47,7 +47,7 @@ class SparseDecoderLayer:
                             torch.from_numpy(csr.column_indices).to(device).to(idt), csr.m)
             # (looked at once, here: the layer's schedules run under capture, where a pattern nobody has looked at
             # keeps to the kernels that take columns in any order)
-            _pyops.prepare_pattern(self.w[name][2], self.w[name][3], csr.k)
+            _pyops.prepare_pattern(self.w[name][2], self.w[name][3], csr.k, tables=False)
 
     # ---- building blocks ---------------------------------------------------------------
     def proj(self, name: str, x: torch.Tensor) -> torch.Tensor:
@@ -97,12 +97,12 @@ class SparseDecoderLayer:
         return self.mlp_block(h)
 
     # ---- fused schedule over two half-batches ----------------------------------------------
-    def _fused(self, name: str, x: torch.Tensor, ga: torch.Tensor, gb: torch.Tensor, trans_b: bool, group: int):
+    def _fused(self, name: str, x: torch.Tensor, ga: torch.Tensor, gb: torch.Tensor, trans_b: bool, group):
         ri, v, ro, ci, m = self.w[name]
         out, c = ops.fused_spmm_gemm(x.unsqueeze(0), ri, v, ro, ci, m, ga, gb, trans_b, group)
         return out[0], c
 
-    def forward_fused(self, xa: torch.Tensor, xb: torch.Tensor, seqs_half: int, group: int = 0):
+    def forward_fused(self, xa: torch.Tensor, xb: torch.Tensor, seqs_half: int, group=None):
         """Halves a and b of the batch; the dense GEMMs of one half ride along with sparse
         projections of the other half."""
         qa, ka, va = self.proj("q", xa), self.proj("k", xa), self.proj("v", xa)
@@ -128,5 +128,5 @@ class SparseDecoderLayer:
     def capture_multistream(self, xa: torch.Tensor, xb: torch.Tensor, seqs_half: int):
         return IL.capture_interleaved([lambda: self.forward(xa, seqs_half)], [lambda: self.forward(xb, seqs_half)])
 
-    def capture_fused(self, xa: torch.Tensor, xb: torch.Tensor, seqs_half: int, group: int = 0):
+    def capture_fused(self, xa: torch.Tensor, xb: torch.Tensor, seqs_half: int, group=None):
         return IL.capture_serialized([lambda: self.forward_fused(xa, xb, seqs_half, group)])

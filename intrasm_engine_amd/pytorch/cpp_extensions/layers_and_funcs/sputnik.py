@@ -54,9 +54,11 @@ SPMM_KERNELS: dict[str, dict] = {
     "mfma32_windows4": {"force_variant": 5, "force_nt": 4, "force_rpw": 4},
     "mfma32_windows8": {"force_variant": 5, "force_nt": 4, "force_rpw": 8},
     "mfma32_rows16": {"force_variant": 5, "force_nt": 6, "force_rpw": 4},
-    # fp32: a slice of the dense operand resident in LDS, k split over workgroups (the operator allocates the partial sums)
-    "ksplit_lds": {"force_variant": 9},
-    "ksplit_lds_16waves": {"force_variant": 9, "force_nt": 2},
+    # the row kernel with 16, 8, 4, 2 or 1 wavefronts per row by the row's own length (the operator hands the pattern's
+    # row-length histogram over); a wavefront gets at most 1, 2 or 4 chunks of 64 nonzeros
+    "rows_by_length": {"force_variant": 11},
+    "rows_by_length_1chunk": {"force_variant": 11, "force_rpw": 1},
+    "rows_by_length_4chunks": {"force_variant": 11, "force_rpw": 3},
 }
 
 
@@ -76,7 +78,8 @@ def spmm_kernel_choices(dtype: torch.dtype, n: int, k: int | None = None, m: int
             names.append("dense_form_gemm")
     if dtype == torch.float32 and n % 4 == 0:
         names += [k for k in SPMM_KERNELS if k.startswith("mfma32_")]
-        names += ["ksplit_lds", "ksplit_lds_16waves"]          # (the backward product has the same n)
+    if n % vec == 0:
+        names += [k for k in SPMM_KERNELS if k.startswith("rows_by_length")]    # (full 128-bit vectors; the backward product has the same n)
     return names
 
 

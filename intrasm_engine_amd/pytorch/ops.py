@@ -21,6 +21,7 @@ Registered operators
 from __future__ import annotations
 
 import contextlib
+import ctypes
 import threading
 import weakref
 
@@ -104,40 +105,139 @@ def _check_index_dtypes(row_indices, row_offsets, column_indices, allow_i16=Fals
     _chk(column_indices.dtype in ok, "column_indices must be " + " or ".join(str(d) for d in ok))
 
 
+# from this share of nonzeros in dense blocks the kernels for patterns with structure are taken (SddmmPlan.analyze's rule)
+_STRUCTURE_SHARE = 0.5
+
+
+def _row_histogram_host(row_offsets):
+    """The 16 counts of ``iex_csr_row_histogram`` as a tuple of ints (one small launch, one synchronising read)."""
+    hist = torch.zeros(16, dtype=torch.int32, device=row_offsets.device)
+    with torch.cuda.device(row_offsets.device):
+        rc = _lib.load().iex_csr_row_histogram(row_offsets.numel() - 1, row_offsets.data_ptr(), hist.data_ptr(),
+                                               _stream_ptr(row_offsets.device))
+    _lib.check(rc, "csr_row_histogram")
+    return tuple(int(x) for x in hist.tolist())
+
+
+def _dense_share_host(row_offsets, column_indices, k, dense_min=1536):
+    """Share of the nonzeros that sit in 128 x 128 blocks holding ``dense_min`` of them or more (``iex_csr_dense_share``;
+    one small launch and a synchronising read), or None where the kernel does not apply (more than 65536 columns)."""
+    nonzeros = column_indices.numel()
+    if nonzeros == 0 or int(k) > 65536:
+        return None
+    count = torch.zeros(1, dtype=torch.int32, device=row_offsets.device)
+    with torch.cuda.device(row_offsets.device):
+        rc = _lib.load().iex_csr_dense_share(1 if column_indices.dtype == torch.int16 else 0, row_offsets.numel() - 1, int(k),
+                                             row_offsets.data_ptr(), column_indices.data_ptr(), int(dense_min), count.data_ptr(),
+                                             _stream_ptr(row_offsets.device))
+    _lib.check(rc, "csr_dense_share")
+    return int(count.item()) / nonzeros
+
+
+def _pattern_tables_host(row_offsets, column_indices, k):
+    """The tables and lists of the kernels for patterns with structure, written once (``iex_pattern_tables``) into a
+    tensor that lives as long as the pattern's note; the stream is waited for, so every later call on any stream finds
+    them complete and only reads them.  None where those kernels do not apply."""
+    m, nonzeros = row_offsets.numel() - 1, column_indices.numel()
+    lib = _lib.load()
+    nbytes = lib.iex_pattern_tables_bytes(m, int(k), nonzeros) if column_indices.dtype == torch.int32 else 0
+    if nbytes == 0:
+        return None
+    ws = torch.empty(nbytes, dtype=torch.uint8, device=row_offsets.device)
+    with torch.cuda.device(row_offsets.device):
+        rc = lib.iex_pattern_tables(m, int(k), nonzeros, row_offsets.data_ptr(), column_indices.data_ptr(), ws.data_ptr(), nbytes,
+                                    _stream_ptr(row_offsets.device))
+        _lib.check(rc, "pattern_tables")
+        torch.cuda.current_stream(row_offsets.device).synchronize()
+    return ws
+
+
+def _set_note(row_offsets, column_indices, k, status, hist, share=None):
+    # (last field: the tables of the kernels for patterns with structure, made by the first call that wants them)
+    column_indices.__dict__["_iex_csr"] = (weakref.ref(row_offsets), _version(row_offsets), _version(column_indices), int(k), status, hist, share,
+                                           None)
+
+
 def mark_canonical(row_offsets, column_indices, k):
     """Record that ``(row_offsets, column_indices)`` is canonical CSR with ``k`` columns (what ``dense_to_sparse`` and
-    ``transpose_info`` build), so that the operators need not look: see :func:`_csr_status`."""
-    column_indices.__dict__["_iex_csr"] = (weakref.ref(row_offsets), _version(row_offsets), _version(column_indices), int(k), 0)
+    ``transpose_info`` build), so that the operators need not look: see :func:`_pattern_note`.  Set-up code: reads the
+    pattern's row-length histogram back (a synchronisation)."""
+    on_device = row_offsets.is_cuda and row_offsets.numel() > 1
+    _set_note(row_offsets, column_indices, k, 0, _row_histogram_host(row_offsets) if on_device else None,
+              _dense_share_host(row_offsets, column_indices, k) if on_device else None)
     return column_indices
 
 
-def _csr_status(row_offsets, column_indices, k):
-    """Status bits of ``iex_csr_check`` for a pattern, or None when they are not known and cannot be found out now
-    (a stream capture is running: the check ends in a synchronising read).
+def _pattern_note(row_offsets, column_indices, k):
+    """``(status, histogram)`` of a pattern: the bits of ``iex_csr_check`` and the 16 counts of ``iex_csr_row_histogram``
+    (rows with more than 64 << j nonzeros), or ``(None, None)`` when they are not known and cannot be found out now
+    (a stream capture is running: looking ends in a synchronising read).
 
     The reference's kernels take the columns of a row in any order, and repeated (Sputnik: sputnik_spmm.cu.inc:229-243,
     sputnik_sddmm.cu.inc:137); most kernel families here are faster because they do not.  So every operator looks at a
-    pattern the first time it sees it -- one small launch and one read of four bytes -- and remembers the answer on
-    the ``column_indices`` tensor object, together with the ``row_offsets`` object it belongs to and both version
-    counters: a pattern costs one check, in-place changes and other pairings cost another."""
+    pattern the first time it sees it -- two small launches and one read -- and remembers the answer on the
+    ``column_indices`` tensor object, together with the ``row_offsets`` object it belongs to and both version
+    counters: a pattern costs one look, in-place changes and other pairings cost another.  The histogram lets the
+    row kernel give every row the number of wavefronts its own length deserves (``iex_spmm_sched``)."""
     note = column_indices.__dict__.get("_iex_csr")
     if note is not None and note[0]() is row_offsets and note[1:4] == (_version(row_offsets), _version(column_indices), int(k)):
-        return note[4]
+        return note[4], note[5]
     if torch.cuda.is_current_stream_capturing():
-        return None
+        return None, None
     status = csr_check(row_offsets, column_indices, k)
-    column_indices.__dict__["_iex_csr"] = (weakref.ref(row_offsets), _version(row_offsets), _version(column_indices), int(k), status)
-    return status
+    sound = not (status & _lib.CSR_BAD_OFFSETS)
+    hist = _row_histogram_host(row_offsets) if sound else None
+    share = _dense_share_host(row_offsets, column_indices, k) if sound and row_offsets.numel() > 1 else None
+    _set_note(row_offsets, column_indices, k, status, hist, share)
+    return status, hist
 
 
-def prepare_pattern(row_offsets, column_indices, k):
+def _csr_status(row_offsets, column_indices, k):
+    return _pattern_note(row_offsets, column_indices, k)[0]
+
+
+def _known_dense_share(row_offsets, column_indices, k):
+    """What an earlier look at the pattern found for the share of nonzeros in dense 128 x 128 blocks, or None."""
+    note = column_indices.__dict__.get("_iex_csr")
+    if note is not None and note[0]() is row_offsets and note[1:4] == (_version(row_offsets), _version(column_indices), int(k)):
+        return note[6]
+    return None
+
+
+def _known_tables(row_offsets, column_indices, k):
+    """The tables of the kernels for patterns with structure for a pattern that is known to be canonical: made by the
+    first call that asks (never under stream capture: making them ends in a wait for the stream) and kept with the
+    pattern's note.  None where nothing is known about the pattern, or the tables cannot be made now."""
+    note = column_indices.__dict__.get("_iex_csr")
+    if note is None or note[0]() is not row_offsets or note[1:4] != (_version(row_offsets), _version(column_indices), int(k)) or note[4] != 0:
+        return None
+    if note[7] is None and not torch.cuda.is_current_stream_capturing():
+        tables = _pattern_tables_host(row_offsets, column_indices, k)
+        if tables is not None:
+            column_indices.__dict__["_iex_csr"] = note[:7] + (tables,)
+        return tables
+    return note[7]
+
+
+def structured_tables(row_offsets, column_indices, k):
+    """:func:`_known_tables` for a pattern whose look found structure (at least ``_STRUCTURE_SHARE`` of its nonzeros in
+    dense blocks), None for any other."""
+    share = _known_dense_share(row_offsets, column_indices, k)
+    return _known_tables(row_offsets, column_indices, k) if share is not None and share >= _STRUCTURE_SHARE else None
+
+
+def prepare_pattern(row_offsets, column_indices, k, tables=True):
     """Look at a pattern now (see :func:`_csr_status`) so that later calls -- under stream capture too, where nothing can
     be looked at -- take every kernel family for canonical CSR.  Returns the status bits; raises for offsets or columns
-    that point outside the arrays.  Set-up code for patterns that do not come from ``dense_to_sparse``."""
+    that point outside the arrays.  Set-up code for patterns that do not come from ``dense_to_sparse``.
+    ``tables``: also make, for a pattern with structure, the tables that the kernels for such patterns work from (an
+    attention mask wants them; a weight matrix, whose products never take those kernels, does not: about 8 bytes a nonzero)."""
     status = _csr_status(row_offsets, column_indices, k)
     _chk(status is not None, "prepare_pattern: cannot look at a pattern while the current stream is being captured")
     _chk(not (status & (_lib.CSR_BAD_OFFSETS | _lib.CSR_COLUMN_OUT_OF_RANGE)),
          f"row_offsets must ascend from 0 to the number of nonzeros and every column index must lie in [0, {int(k)})")
+    if tables and status == 0:
+        structured_tables(row_offsets, column_indices, k)
     return status
 
 
@@ -146,7 +246,8 @@ def carry_pattern_note(column_indices, copy):
     the one holds for the other."""
     note = column_indices.__dict__.get("_iex_csr")
     if note is not None and note[2] == _version(column_indices):
-        copy.__dict__["_iex_csr"] = note[:2] + (_version(copy),) + note[3:]
+        # (the tables were made from int32 indices: a copy of another integer type does not inherit them)
+        copy.__dict__["_iex_csr"] = note[:2] + (_version(copy),) + note[3:7] + (note[7] if copy.dtype == column_indices.dtype else None,)
     return copy
 
 
@@ -208,6 +309,15 @@ def _spmm(b, row_indices, values, row_offsets, column_indices, m, *, per_batch_v
         _chk(bias.dtype == torch.float32 and bias.is_contiguous() and bias.numel() == m
              and bias.device == b.device, "bias must be a contiguous fp32 tensor with m entries")
     any_order = nonzeros > 0 and not force_variant and _any_order(row_offsets, column_indices, k, "spmm")
+    if per_batch_values and not accumulate and not any_order and not force_variant and nonzeros > 0 and b.dtype in (torch.float16, torch.bfloat16):
+        # values per batch entry = attention probabilities: the library's own rule for the dense-blocks kernel sees
+        # the density only; what the first look at the pattern found about its structure decides here
+        share = _known_dense_share(row_offsets, column_indices, k)
+        if share is not None and batch * m * k >= (1 << 25):
+            force_variant = 10 if share >= _STRUCTURE_SHARE else 1
+            if force_variant == 10 and _lib.load().iex_spmm_workspace_kind(
+                    _DT[b.dtype], _IT[column_indices.dtype], _lib.SPMM_PER_BATCH_VALUES | (10 << 16), m, k, n, nonzeros, batch) != 10:
+                force_variant = 0      # (the kernel does not serve this call: another n, int16 indices)
     flags = (_lib.SPMM_PER_BATCH_VALUES if per_batch_values else 0) | (_lib.SPMM_ANY_COLUMN_ORDER if any_order else 0) | \
             (_lib.SPMM_ACCUMULATE if accumulate else 0) | (_lib.SPMM_RELU if relu else 0) | \
             ((int(force_wpr) & 0xff) << 8) | ((int(force_variant) & 0xf) << 16) | ((int(force_rpw) & 0xf) << 20) | \
@@ -235,12 +345,27 @@ def _spmm(b, row_indices, values, row_offsets, column_indices, m, *, per_batch_v
             plan.lists_key = (key, (flags >> 8) & 0xff if ((flags >> 16) & 0xf) == 10 else 0)
             ws = plan.workspace
         else:
-            ws = torch.empty(ws_bytes, dtype=torch.uint8, device=b.device) if ws_bytes else None
-        rc = lib.iex_spmm_ws(
+            tables = _known_tables(row_offsets, column_indices, k) if ws_bytes and lib.iex_spmm_workspace_kind(*shape) == 10 and \
+                (((flags >> 16) & 0xf) != 10 or ((flags >> 8) & 0xff) == 0) else None
+            if tables is not None and tables.numel() >= ws_bytes and tables.device == b.device:
+                # written when the pattern was first looked at, with the built-in threshold, and read-only since
+                ws = tables
+                flags |= _lib.SPMM_TABLES_READY | _lib.SPMM_LISTS_READY
+            else:
+                ws = torch.empty(ws_bytes, dtype=torch.uint8, device=b.device) if ws_bytes else None
+        # what is known about the pattern's row lengths (only what an earlier look left, unless the kernel that needs
+        # it was asked for by name)
+        if ((flags >> 16) & 0xf) == 11 and nonzeros > 0:
+            _pattern_note(row_offsets, column_indices, k)
+        note = column_indices.__dict__.get("_iex_csr")
+        hist = note[5] if nonzeros > 0 and note is not None and note[0]() is row_offsets and \
+            note[1:4] == (_version(row_offsets), _version(column_indices), int(k)) else None
+        rc = lib.iex_spmm_sched(
             _DT[b.dtype], _IT[column_indices.dtype], flags, m, k, n, nonzeros,
             row_indices.data_ptr(), values.data_ptr(), row_offsets.data_ptr(),
             column_indices.data_ptr(), b.data_ptr(), bias.data_ptr() if bias is not None else None,
-            out.data_ptr(), _stream_ptr(b.device), batch, ws.data_ptr() if ws is not None else None, ws_bytes)
+            out.data_ptr(), _stream_ptr(b.device), batch, ws.data_ptr() if ws is not None else None, ws_bytes,
+            (ctypes.c_int * 16)(*hist) if hist is not None else None)
     _lib.check(rc, "spmm")
     return out
 
@@ -325,6 +450,13 @@ def _sddmm(a, b, row_indices, row_offsets, column_indices, *, sum_over_batch, dt
         _chk(tuple(out.shape) == shape and out.dtype == a.dtype and out.is_contiguous()
              and out.device == a.device, "out has the wrong shape, dtype, layout or device")
     any_order = nonzeros > 0 and not force_variant and _any_order(row_offsets, column_indices, n, "sddmm")
+    if not sum_over_batch and not accumulate and not any_order and not force_variant and nonzeros > 0 and a.dtype in (torch.float16, torch.bfloat16):
+        # per-entry SDDMM = attention scores: by the pattern's structure where a look at it has told, not by its density
+        share = _known_dense_share(row_offsets, column_indices, n)
+        if share is not None and batch * m * n >= (1 << 25):
+            force_variant = 3 if share >= _STRUCTURE_SHARE else 1
+            if force_variant == 3 and _lib.load().iex_sddmm_workspace_kind(_DT[a.dtype], 3 << 16, m, k, n, nonzeros, batch) != 3:
+                force_variant = 0      # (the kernel does not serve this call: another k)
     flags = (_lib.SDDMM_SUM_OVER_BATCH if sum_over_batch else 0) | (_lib.SDDMM_ANY_COLUMN_ORDER if any_order else 0) | \
             (_lib.SDDMM_ACCUMULATE if accumulate else 0) | ((int(force_wpr) & 0xff) << 8) | \
             ((int(force_variant) & 0xf) << 16)
@@ -347,7 +479,14 @@ def _sddmm(a, b, row_indices, row_offsets, column_indices, *, sum_over_batch, dt
             plan.lists_key = (key, code)
             ws = plan.workspace
         else:
-            ws = torch.empty(ws_bytes, dtype=torch.uint8, device=a.device) if ws_bytes else None
+            kind3 = ws_bytes and lib.iex_sddmm_workspace_kind(_DT[a.dtype], flags, m, k, n, nonzeros, batch) == 3
+            tables = _known_tables(row_offsets, column_indices, n) if kind3 and (((flags >> 16) & 0xf) != 3 or ((flags >> 8) & 0xff) == 0) else None
+            if tables is not None and tables.numel() >= ws_bytes and tables.device == a.device:
+                # written when the pattern was first looked at, with the built-in threshold, and read-only since
+                ws = tables
+                flags |= _lib.SDDMM_TABLES_READY | _lib.SDDMM_LISTS_READY
+            else:
+                ws = torch.empty(ws_bytes, dtype=torch.uint8, device=a.device) if ws_bytes else None
         rc = lib.iex_sddmm_ws(
             _DT[a.dtype], flags, m, k, n, nonzeros, row_indices.data_ptr(), row_offsets.data_ptr(),
             column_indices.data_ptr(), a.data_ptr(), b.data_ptr(), out.data_ptr(),
@@ -482,9 +621,14 @@ def gemm_mfma(a, b, trans_b=False, out=None):
 
 
 def fused_spmm_gemm(b, row_indices, values, row_offsets, column_indices, m, ga, gb, trans_b=False,
-                    interleave=0):
+                    interleave=None):
     """One launch computing ``(A_csr @ b[0], ga @ gb)``; fp16 SpMM, fp16/bf16 GEMM (2-D, or
-    3-D batched with equal batch sizes)."""
+    3-D batched with equal batch sizes).
+    ``interleave``: the order of the two kinds of workgroup in the grid, as ``iex_fused_spmm_gemm`` takes it (0: GEMM
+    tiles first, g > 0: in groups of g through the grid, < 0: SpMM tiles first).  None: the kind with the longer inner
+    dimension first -- a CU runs one tile at a time, the tiles of both kinds have the same outline and last as long as
+    their inner dimension, and a schedule that starts its long tasks first ends soonest (config 4 on MI355X: SpMM
+    tiles first 0.279 ms, GEMM tiles first 0.344 ms, in groups of 64 0.323 ms, against 0.325 ms for one after the other)."""
     _chk(b.dim() == 3 and b.size(0) == 1, "fused launch takes one batch entry")
     _chk(values.dim() == 1 and values.size(0) == column_indices.size(0))
     _check_csr_common(b, row_indices, row_offsets, column_indices, [("b", b), ("values", values)])
@@ -505,6 +649,8 @@ def fused_spmm_gemm(b, row_indices, values, row_offsets, column_indices, m, ga, 
     _chk(ga.dim() == 2 or gb.shape[0] == gbatch, "batch sizes of the GEMM operands differ")
     _chk(column_indices.size(0) == 0 or not _any_order(row_offsets, column_indices, k, "fused_spmm_gemm"),
          "fused_spmm_gemm needs canonical CSR (columns of a row ascending and distinct) that has been seen outside a capture")
+    if interleave is None:
+        interleave = -1 if k >= K else 0
     out = torch.empty((1, m, n), dtype=b.dtype, device=b.device)
     c = torch.empty((gbatch, M, N) if ga.dim() == 3 else (M, N), dtype=ga.dtype, device=b.device)
     with torch.cuda.device(b.device):
@@ -542,7 +688,7 @@ def register() -> None:
          lambda a, b, trans_b=False: gemm_mfma(a, b, trans_b)),
         ("fused_spmm_gemm",
          "(Tensor b, Tensor row_indices, Tensor values, Tensor row_offsets, Tensor column_indices, int m, "
-         "Tensor ga, Tensor gb, bool trans_b=False, int interleave=0) -> (Tensor, Tensor)",
+         "Tensor ga, Tensor gb, bool trans_b=False, int? interleave=None) -> (Tensor, Tensor)",
          fused_spmm_gemm),
     ]
     for name, schema, fn in table:

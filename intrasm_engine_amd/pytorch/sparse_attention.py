@@ -39,8 +39,11 @@ def sparse_attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, row_indi
     if scale is None:
         scale = 1.0 / math.sqrt(q.shape[2])
     from . import ops as _pyops
-    if plan is None and q.dtype in (torch.float16, torch.bfloat16):
-        plan = _pyops.SddmmPlan()     # for this call only: what the first product derives from the mask serves the second too
+    if plan is None and q.dtype in (torch.float16, torch.bfloat16) and \
+            _pyops.structured_tables(row_offsets, column_indices, tokens) is None:
+        # for this call only: what the first product derives from the mask serves the second too.  (Not needed for a
+        # pattern with structure that the operators have looked at before: its tables are kept with the pattern.)
+        plan = _pyops.SddmmPlan()
     if plan is not None:
         scores = _pyops.sddmm_half_planned(q, k, row_indices, row_offsets, column_indices, plan)
     else:

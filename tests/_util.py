@@ -35,12 +35,18 @@ def assert_close(got, want, scale, rtol, what="", atol=0.0):
     return float((err / np.maximum(np.abs(want), 1e-300))[np.abs(want) > 1e-3 * np.maximum(scale, 1e-300)].max(initial=0.0))
 
 
-def to_dev(csr, dev, vdtype=torch.float32, idtype=torch.int32):
-    """(row_indices, values, row_offsets, column_indices) tensors of a workloads.CSR."""
-    return (torch.from_numpy(csr.row_indices).to(dev),
-            torch.from_numpy(csr.values).to(dev).to(vdtype),
-            torch.from_numpy(csr.row_offsets).to(dev),
-            torch.from_numpy(csr.column_indices).to(dev).to(idtype))
+def to_dev(csr, dev, vdtype=torch.float32, idtype=torch.int32, tables=True):
+    """(row_indices, values, row_offsets, column_indices) tensors of a workloads.CSR.  The pattern is looked at here,
+    once (``ops.prepare_pattern``), as set-up code does: operators that meet it under stream capture then know it
+    (``tables`` = False: without making the tables that a pattern with structure keeps for its kernels)."""
+    t = (torch.from_numpy(csr.row_indices).to(dev),
+         torch.from_numpy(csr.values).to(dev).to(vdtype),
+         torch.from_numpy(csr.row_offsets).to(dev),
+         torch.from_numpy(csr.column_indices).to(dev).to(idtype))
+    if t[3].is_cuda and csr.nnz > 0:
+        from intrasm_engine_amd.pytorch import ops as pyops
+        pyops.prepare_pattern(t[2], t[3], csr.k, tables=tables)
+    return t
 
 
 def rounded(x, dtype):

@@ -18,7 +18,7 @@ def _row_kernel_spmm(x, ri, v, ro, ci, m):
                        allow_i16=True, force_variant=1)
 
 
-@pytest.mark.parametrize("interleave", [0, 1, 4, 7])
+@pytest.mark.parametrize("interleave", [0, 1, 4, 7, -1])
 @pytest.mark.parametrize("gdtype,trans_b", [(torch.bfloat16, False), (torch.float16, True)])
 @pytest.mark.parametrize("n,idtype", [(512, torch.int16), (64, torch.int32), (200, torch.int32)])
 def test_fused_equals_separate_launches(dev, interleave, gdtype, trans_b, n, idtype):
@@ -46,7 +46,7 @@ def test_fused_config4_shape(dev):
     alone = ops.spmm_sputnik_reuse_weight_half(xt, ri, v, ro, ci, w.m)
     assert not torch.equal(alone, _row_kernel_spmm(xt, ri, v, ro, ci, w.m))     # i.e. not the row kernel
     c_alone = ops.gemm_mfma(gat, gbt, False)
-    for interleave in (1, 0, 16, 5, 37):
+    for interleave in (1, 0, 16, 5, 37, -1):
         out, c = ops.fused_spmm_gemm(xt, ri, v, ro, ci, w.m, gat, gbt, False, interleave)
         assert torch.equal(out, alone) and torch.equal(c, c_alone), interleave
     gbt_t = gbt.t().contiguous()

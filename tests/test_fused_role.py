@@ -20,7 +20,7 @@ def test_every_tile_and_block_exactly_once():
     lib = _lib.load()
     for G in list(range(0, 24)) + [59, 64, 100]:
         for S in list(range(0, 12)) + [39, 40, 257]:
-            for g in (0, 1, 2, 3, 4, 5, 7, 8, 11, 16, 64, 1000):
+            for g in (-1, -7, 0, 1, 2, 3, 4, 5, 7, 8, 11, 16, 64, 1000):
                 roles = _roles(lib, G, S, g)
                 assert sorted(i for is_gemm, i in roles if is_gemm) == list(range(G)), (G, S, g)
                 assert sorted(i for is_gemm, i in roles if not is_gemm) == list(range(S)), (G, S, g)
@@ -38,12 +38,14 @@ def test_groups_keep_their_tiles_together_and_spread_the_blocks():
     roles = _roles(_lib.load(), 8, 6, 4)      # two groups of 4 tiles, 3 blocks after each
     assert [r[0] for r in roles] == [1, 1, 1, 1, 0, 0, 0, 1, 1, 1, 1, 0, 0, 0]
     assert _roles(_lib.load(), 3, 2, 0) == [(1, 0), (1, 1), (1, 2), (0, 0), (0, 1)]
+    # a negative group size: the blocks first (the longer jobs), then the tiles
+    assert _roles(_lib.load(), 3, 2, -1) == [(0, 0), (0, 1), (1, 0), (1, 1), (1, 2)]
 
 
 def test_arguments_are_checked():
     from intrasm_engine_amd import _lib
     lib = _lib.load()
     ig, idx = ctypes.c_int(), ctypes.c_int()
-    assert lib.iex_fused_role(4, 4, -1, 0, ctypes.byref(ig), ctypes.byref(idx)) == -1
+    assert lib.iex_fused_role(4, -4, 0, 0, ctypes.byref(ig), ctypes.byref(idx)) == -1
     assert lib.iex_fused_role(4, 4, 2, 8, ctypes.byref(ig), ctypes.byref(idx)) == -1
     assert "outside the grid" in _lib.last_error()

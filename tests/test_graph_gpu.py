@@ -78,6 +78,8 @@ def test_replay_spmm_that_uses_a_workspace(dev):
     ro, ci = W.csr_from_row_lengths(rng, m, k, rng.binomial(k, 0.2, m))
     ri = torch.from_numpy(W.swizzle_from_offsets(ro)).to(dev)
     ro_t, ci_t = torch.from_numpy(ro).to(dev), torch.from_numpy(ci.astype(np.int16)).to(dev)
+    from intrasm_engine_amd.pytorch import ops as pyops
+    pyops.prepare_pattern(ro_t, ci_t, k)     # set-up code looks at a pattern once, outside any capture
     v = torch.randn(ci.shape[0], device=dev).half()
     b = torch.randn(1, k, n, device=dev).half()
     assert _lib.load().iex_spmm_workspace_bytes(_lib.F16, _lib.I16, 0, m, k, n, ci.shape[0], 1) == m * k * 2
@@ -241,17 +243,19 @@ def test_current_stream_is_not_the_default_stream(dev):
     assert cs.stream != torch.cuda.default_stream()
 
 
-@pytest.mark.parametrize("kept_plan", [False, True])
-def test_replay_sparse_attention_with_tables_in_the_captured_workspace(dev, kept_plan):
+@pytest.mark.parametrize("tables_from", ["capture_pool", "plan", "pattern"])
+def test_replay_sparse_attention_with_tables_in_the_captured_workspace(dev, tables_from):
     """The attention block on a mask with structure, captured: the workspace with the tables and lists of the two
-    kernels for such masks comes from the capture's pool (the block's own plan) or is the caller's plan, filled before
-    the capture; the second product inside the capture reuses what the first wrote.  Replays with new q, k, v (and
-    other allocations between them) equal the eager block bit for bit."""
+    kernels for such masks comes from the capture's pool (the block's own plan), or is the caller's plan, filled before
+    the capture, or is kept with the pattern since set-up code looked at it; the second product inside the capture
+    reuses what the first wrote.  Replays with new q, k, v (and other allocations between them) equal the eager block
+    bit for bit."""
+    kept_plan = tables_from == "plan"
     from intrasm_engine_amd import _lib
     from intrasm_engine_amd.pytorch import ops as pyops
     from intrasm_engine_amd.pytorch.sparse_attention import sparse_attention
     pattern, q_np, k_np, _ = W.config3(tokens=2048, heads=8, band=128, extra=8)     # (large and dense enough for the structured kernels to be picked)
-    ri, _, ro, ci = to_dev(pattern, dev)
+    ri, _, ro, ci = to_dev(pattern, dev, tables=tables_from == "pattern")
     heads, tokens, d = q_np.shape
     q, k, v = (torch.randn(heads, tokens, d, device=dev).half() for _ in range(3))
     plan = None

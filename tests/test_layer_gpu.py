@@ -71,7 +71,8 @@ def test_three_variants_agree(dev):
 
     for capture in (lambda: layer.capture_multistream(xa, xb, SEQS // 2),
                     lambda: layer.capture_fused(xa, xb, SEQS // 2, 0),
-                    lambda: layer.capture_fused(xa, xb, SEQS // 2, 8)):
+                    lambda: layer.capture_fused(xa, xb, SEQS // 2, 8),
+                    lambda: layer.capture_fused(xa, xb, SEQS // 2)):
         constructor, keep = capture()
         constructor.instantiate_graph_exec()
         for _ in range(2):

@@ -143,8 +143,9 @@ def test_tables_kept_between_calls_of_one_mask(oracle, dev):
     pattern, q, k, v = W.config3(heads=8)
     ri, _, ro, ci = to_dev(pattern, dev)
     qt, kt, vt = (torch.from_numpy(x).to(dev).half() for x in (q, k, v))
+    # (the operator itself keeps the tables of a pattern it has looked at: no setup kernel in its calls either)
     want = ops.sddmm_sputnik_half(qt, kt, ri, ro, ci)
-    assert "sddmm_tile_ptr_kernel" in _lib.last_kernels()
+    assert _lib.last_kernels().startswith("sddmm_mfma_kernel")
     plan = pyops.SddmmPlan()
     first = pyops.sddmm_half_planned(qt, kt, ri, ro, ci, plan)
     assert "sddmm_tile_ptr_kernel" in _lib.last_kernels() and torch.equal(first, want)
@@ -172,12 +173,15 @@ def test_tables_kept_between_calls_of_one_mask(oracle, dev):
     assert torch.equal(a0, a1) and torch.equal(a0, a2)
 
 
-def test_plan_settles_the_kernel_by_the_masks_structure(dev):
+def test_structure_settles_the_kernel(dev):
     """Two masks of the same density: a band (its nonzeros sit in dense 128 x 128 blocks) and columns at random.  The
-    library's rule (by density) takes the kernel for masks with structure for both; a plan that has looked at the
-    pattern keeps it for the band and takes the gather kernel for the random one.  Same results either way."""
+    library's own rule, asked through the C interface with nothing known about the pattern, goes by density and names
+    the kernel for masks with structure for both.  The operator has looked at the pattern (the share of its nonzeros
+    in dense blocks is part of that look) and takes that kernel for the band and the gather kernel for the random one;
+    so does a plan.  Same results either way, and the band's tables are made once: later calls run no setup kernel."""
     from intrasm_engine_amd import _lib
     from intrasm_engine_amd.pytorch import ops as pyops
+    lib = _lib.load()
     rng = np.random.default_rng(5)
     tokens, heads = 2048, 16
     q = rng.standard_normal((heads, tokens, 64)).astype(np.float32)
@@ -188,14 +192,25 @@ def test_plan_settles_the_kernel_by_the_masks_structure(dev):
     ro, ci = W.csr_from_row_lengths(rng, tokens, tokens, np.full(tokens, per_row))
     rand = W.CSR(tokens, tokens, np.ones(ci.shape[0], np.float32), W.swizzle_from_offsets(ro), ro, ci)
     for csr, variant, kernel in ((band, 3, "sddmm_mfma_kernel"), (rand, 1, "sddmm_kernel")):
+        assert lib.iex_sddmm_workspace_kind(_lib.F16, 0, tokens, 64, tokens, csr.nnz, heads) == 3
         ri, _, ro_t, ci_t = to_dev(csr, dev)
-        auto = ops.sddmm_sputnik_half(qt, kt, ri, ro_t, ci_t)
+        share = pyops._known_dense_share(ro_t, ci_t, tokens)
+        assert (share >= 0.5) == (variant == 3), share
+        forced = pyops._sddmm(qt, kt, ri, ro_t, ci_t, sum_over_batch=False, dtypes=(torch.float16,), force_variant=3)
         assert "sddmm_mfma_kernel" in _lib.last_kernels()
+        auto = ops.sddmm_sputnik_half(qt, kt, ri, ro_t, ci_t)
+        assert kernel in _lib.last_kernels()
+        assert torch.allclose(forced.float(), auto.float(), rtol=1e-2, atol=1e-2 * 8.0 * 0.1)
+        if variant == 3:
+            assert torch.equal(forced, auto)
+            again = ops.sddmm_sputnik_half(qt, kt, ri, ro_t, ci_t)
+            assert _lib.last_kernels().startswith("sddmm_mfma_kernel") and torch.equal(again, auto)
         plan = pyops.SddmmPlan()
         assert plan.analyze(ro_t, ci_t, tokens) == variant, plan.dense_share
+        assert abs(plan.dense_share - share) < 1e-6
         planned = pyops.sddmm_half_planned(qt, kt, ri, ro_t, ci_t, plan)
         assert kernel in _lib.last_kernels()
-        assert torch.allclose(planned.float(), auto.float(), rtol=1e-2, atol=1e-2 * 8.0 * 0.1)
+        assert torch.equal(planned, auto)
         # fp32 operands through the same plan: the planned kernel does not serve them, the call runs all the same
         f32 = pyops.sddmm_half_planned(qt.float(), kt.float(), ri, ro_t, ci_t, plan)
         assert torch.allclose(f32, auto.float(), rtol=1e-2, atol=1e-2 * 8.0 * 0.1)

@@ -206,7 +206,7 @@ def test_tables_kept_between_calls_and_shared_with_the_sddmm(dev):
     scores = pyops.sddmm_half_planned(q, kk, ri, rot, cit, plan)
     assert plan.key is not None
     kw = dict(per_batch_values=True, accumulate=False, dtypes=(torch.float16,), allow_i16=False, force_variant=10)
-    fresh = pyops._spmm(v, ri, scores, rot, cit, m, **kw)
+    fresh = pyops._spmm(v, ri, scores, rot.clone(), cit.clone(), m, **kw)    # (copies: nothing kept with them, the call sets up its own tables)
     assert _lib.last_kernels().split(" + ") == ["sddmm_tile_ptr_kernel", "sb_lists_kernel", "spmm_blocks_kernel<false>"]
     first = pyops._spmm(v, ri, scores, rot, cit, m, plan=plan, **kw)      # tables and lists are the SDDMM's: nothing to write
     assert _lib.last_kernels() == "spmm_blocks_kernel<false>"

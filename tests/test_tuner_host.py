@@ -102,14 +102,14 @@ def test_tune_my_autograd_function_front_end():
 
 def test_search_spaces_of_the_path():
     half = spmm_kernel_choices(torch.float16, 128, 64, 256)
-    assert half[0] == "auto" and "mfma8_windows4" in half and "mfma4_lanes16" in half and half[-1] == "dense_form_gemm"
+    assert half[0] == "auto" and "mfma8_windows4" in half and "mfma4_lanes16" in half and "dense_form_gemm" in half
     assert "dense_form_gemm" not in spmm_kernel_choices(torch.float16, 128)          # shape of the sparse operand unknown
     assert "dense_form_gemm" not in spmm_kernel_choices(torch.float16, 128, 64, 100)  # m % 8 != 0 (k of the backward product)
     assert not any(k.startswith("mfma32") for k in half)
     assert not any(k.startswith("mfma") for k in spmm_kernel_choices(torch.float16, 100))    # n % 8 != 0
     single = spmm_kernel_choices(torch.float32, 64)
-    assert "mfma32_windows4" in single and "ksplit_lds" in single and not any(k.startswith(("mfma4", "mfma8")) for k in single)
-    assert "ksplit_lds" not in half and "ksplit_lds" not in spmm_kernel_choices(torch.float32, 66)
+    assert "mfma32_windows4" in single and "rows_by_length" in single and not any(k.startswith(("mfma4", "mfma8")) for k in single)
+    assert "rows_by_length" in half and "rows_by_length" not in spmm_kernel_choices(torch.float32, 66)
     assert "few_columns" in spmm_kernel_choices(torch.float32, 256, 64, 128) and "few_columns" not in single
     assert set(half) | set(single) | {"few_columns"} == set(SPMM_KERNELS)
     for flags in SPMM_KERNELS.values():                       # every name maps to legal tuning keys

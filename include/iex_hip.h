@@ -183,7 +183,7 @@ size_t iex_spmm_workspace_bytes(int dtype, int itype, int flags, int m, int k, i
  * consecutive ranges of it, a workgroup of 16 wavefronts serves 1, 2, 4, 8 or 16 rows of one range, and the partial
  * sums of a row meet in LDS in a fixed order (no atomics: same bits from call to call).  The histogram and the
  * order of row_indices settle how many wavefronts a row HAS; into how many parts its sum is cut follows from the
- * row's own length, and a row with fewer wavefronts than parts lets them take the parts in turns.  So every row is
+ * row's own length, and a row with fewer wavefronts than parts lets one of them take all the parts.  So every row is
  * summed completely, and to the same bits, whatever the histogram and whatever the order of row_indices: a wrong
  * histogram or another order costs time only.  IEX_SPMM_FORCE_VARIANT(11) asks for this kernel and fails without a histogram
  * (bits 20..23 then force the chunks of 64 nonzeros a wavefront may get: 1 + log2, 0 = choose).

@@ -66,14 +66,13 @@ struct row_slab {
 // WIN = gathers a wave keeps in flight (rolling window); raise it where few waves fit a CU.
 // RAGGED = vectors at element alignment (n not a multiple of VEC).
 template <typename T, typename IT, int VEC, int LPG, int WIN, int NT, bool RAGGED>
-__device__ __forceinline__ void spmm_row_partial(const SpmmParams& p, int z, int row, int part, int wpr, const int (&col_ld)[NT],
-                                                 float (&acc)[NT][VEC]) {
+__device__ __forceinline__ void spmm_range_partial(const SpmmParams& p, int z, int start, int end, int part, int wpr, const int (&col_ld)[NT],
+                                                   float (&acc)[NT][VEC]) {
+  // (the row's nonzeros are start .. end - 1, wave-uniform: for a caller that has read the row's offsets already)
   constexpr int G = kWave / LPG;
   typedef row_slab<T, VEC, NT> Slab;
   const int lane = lane_id();
   const int grp = lane / LPG;   // which nonzero of a step this lane works on (0 when G == 1)
-  const int start = uniform(p.row_offsets[row]);
-  const int end = uniform(p.row_offsets[row + 1]);
   const T* __restrict__ values =
       static_cast<const T*>(p.values) + (p.per_batch_values ? (size_t)z * p.nnz : (size_t)0);
   const IT* __restrict__ cols = static_cast<const IT*>(p.cols);
@@ -181,6 +180,12 @@ __device__ __forceinline__ void spmm_row_partial(const SpmmParams& p, int z, int
       for (int i = 0; i < VEC; ++i) acc[0][i] += __shfl_xor(acc[0][i], off, kWave);
     }
   }
+}
+
+template <typename T, typename IT, int VEC, int LPG, int WIN, int NT, bool RAGGED>
+__device__ __forceinline__ void spmm_row_partial(const SpmmParams& p, int z, int row, int part, int wpr, const int (&col_ld)[NT],
+                                                 float (&acc)[NT][VEC]) {
+  spmm_range_partial<T, IT, VEC, LPG, WIN, NT, RAGGED>(p, z, uniform(p.row_offsets[row]), uniform(p.row_offsets[row + 1]), part, wpr, col_ld, acc);
 }
 
 // Bias, ReLU, accumulation and the store of one row's sums (lanes of group 0 only; col0 = first column of tile 0).
@@ -292,7 +297,7 @@ __device__ __forceinline__ void spmm_block(const SpmmParams& p, int bx, int by, 
 // from the host (counted once per pattern) and settle how many wavefronts a row slot HAS.  Into how many parts a row's
 // nonzeros are cut, and so the order of its sum, follows from the row's own length alone: with the ranges the host
 // derives from a true histogram and rows in that order the two agree; with any other ranges or order a row that has
-// fewer wavefronts than parts lets them take its parts in turns, one that has more lets some idle -- time, never a
+// fewer wavefronts than parts lets one of them take all its parts, one that has more lets some idle -- time, never a
 // different bit of the result.
 constexpr int kRowsWaves = 16;
 struct RowClasses {
@@ -313,7 +318,8 @@ __device__ __forceinline__ void spmm_rows_block(const SpmmParams& p, const RowCl
 #pragma unroll
   for (int c = 1; c < 5; ++c) cls += (bx >= rc.first_block[c]) ? 1 : 0;   // (uniform; empty classes share a first block)
   const int wpr = kRowsWaves >> cls;
-  const int row_slot = rc.first_row[cls] + ((bx - rc.first_block[cls]) << cls) + wave / wpr;
+  const int slot0 = rc.first_row[cls] + ((bx - rc.first_block[cls]) << cls);   // the workgroup's first row slot
+  const int mine = wave / wpr;                                                  // this wavefront's row slot among them
   const int part = wave % wpr;
   const int grp = lane / LPG;
   const int col0 = by * TW + (lane % LPG) * VEC;
@@ -321,70 +327,53 @@ __device__ __forceinline__ void spmm_rows_block(const SpmmParams& p, const RowCl
   float acc[1][VEC];
 #pragma unroll
   for (int i = 0; i < VEC; ++i) acc[0][i] = 0.f;
-  const bool row_live = row_slot < rc.first_row[cls + 1];   // wave-uniform
-  int row = 0;
-  int parts = 1;   // of this row, by its own length
-  if (row_live) {
-    row = uniform(p.row_indices[row_slot]);
-    const int len = uniform(p.row_offsets[row + 1] - p.row_offsets[row]);
+  const bool row_live = slot0 + mine < rc.first_row[cls + 1];   // wave-uniform
+  // (all of this is wave-uniform: scalar loads)
+  auto parts_of = [&](int len) {   // of a row, by its own length
     int own = 0;
 #pragma unroll
     for (int c = 0; c < 4; ++c) own += (len > (kWave << (3 - c + rc.log2_rounds))) ? 0 : 1;
-    parts = kRowsWaves >> own;
+    return kRowsWaves >> own;
+  };
+  int row = 0, start = 0, end = 0, parts = 1;
+  if (row_live) {
+    row = uniform(p.row_indices[slot0 + mine]);
+    start = uniform(p.row_offsets[row]);
+    end = uniform(p.row_offsets[row + 1]);
+    parts = parts_of(end - start);
   }
-  if (cls == 4) {   // a wavefront per row: its parts one after the other, no LDS
-    if (!row_live) return;
-    spmm_row_partial<T, IT, VEC, LPG, kSpmmUnroll, 1, false>(p, bz, row, 0, parts, col_ld, acc);
-    for (int q = 1; q < parts; ++q) {
-      float more[1][VEC];
+  // A row slot with as many wavefronts as its row has parts, or more: a part each (the others idle), and the partial
+  // sums meet in LDS.  With fewer -- only where the ranges or the order of the rows are not what the kernel expects --
+  // the slot's first wavefront takes all parts, one after the other, and adds them in the same order.  Either way a
+  // wavefront decides from its own row alone, and every wavefront of the workgroup reaches the one barrier.
+  if (row_live) {
+    if (parts <= wpr) {
+      if (part < parts) spmm_range_partial<T, IT, VEC, LPG, kSpmmUnroll, 1, false>(p, bz, start, end, part, parts, col_ld, acc);
+    } else if (part == 0) {
+      spmm_range_partial<T, IT, VEC, LPG, kSpmmUnroll, 1, false>(p, bz, start, end, 0, parts, col_ld, acc);
+      for (int q = 1; q < parts; ++q) {
+        float more[1][VEC];
 #pragma unroll
-      for (int i = 0; i < VEC; ++i) more[0][i] = 0.f;
-      spmm_row_partial<T, IT, VEC, LPG, kSpmmUnroll, 1, false>(p, bz, row, q, parts, col_ld, more);
+        for (int i = 0; i < VEC; ++i) more[0][i] = 0.f;
+        spmm_range_partial<T, IT, VEC, LPG, kSpmmUnroll, 1, false>(p, bz, start, end, q, parts, col_ld, more);
 #pragma unroll
-      for (int i = 0; i < VEC; ++i) acc[0][i] += more[0][i];
+        for (int i = 0; i < VEC; ++i) acc[0][i] += more[0][i];
+      }
     }
-    if (grp == 0) spmm_store_row<T, VEC, LPG, 1, false>(p, bz, row, col0, 0, acc);
-    return;
   }
-  // (uniform over the workgroup from here) partial sums of a row meet in LDS and are added in the order of the parts
-  if (!__syncthreads_or(parts > wpr)) {
-    if (row_live && part < parts) spmm_row_partial<T, IT, VEC, LPG, kSpmmUnroll, 1, false>(p, bz, row, part, parts, col_ld, acc);
+  if (cls < 4) {   // (uniform over the workgroup) the parts of a row are added in their order: bit-stable
 #pragma unroll
     for (int i = 0; i < VEC; ++i) red[(wave * VEC + i) * kWave + lane] = acc[0][i];
     __syncthreads();
     if (part != 0) return;
+    if (parts <= wpr) {
 #pragma unroll
-    for (int i = 0; i < VEC; ++i) {
-      float s = acc[0][i];
-      for (int w = 1; w < parts; ++w) s += red[((wave + w) * VEC + i) * kWave + lane];
-      acc[0][i] = s;
-    }
-  } else {
-    // some row of this workgroup has more parts than wavefronts: all take their parts in turns of wpr
-    float sum[VEC];
-#pragma unroll
-    for (int i = 0; i < VEC; ++i) sum[i] = 0.f;
-    for (int q = 0; q < kRowsWaves; q += wpr) {
-#pragma unroll
-      for (int i = 0; i < VEC; ++i) acc[0][i] = 0.f;
-      if (row_live && q + part < parts) spmm_row_partial<T, IT, VEC, LPG, kSpmmUnroll, 1, false>(p, bz, row, q + part, parts, col_ld, acc);
-#pragma unroll
-      for (int i = 0; i < VEC; ++i) red[(wave * VEC + i) * kWave + lane] = acc[0][i];
-      __syncthreads();
-      if (part == 0 && q < parts) {
-#pragma unroll
-        for (int i = 0; i < VEC; ++i) {
-          float s = q == 0 ? acc[0][i] : sum[i] + acc[0][i];
-          for (int w = 1; w < wpr; ++w)
-            if (q + w < parts) s += red[((wave + w) * VEC + i) * kWave + lane];
-          sum[i] = s;
-        }
+      for (int i = 0; i < VEC; ++i) {
+        float s = acc[0][i];
+        for (int w = 1; w < parts; ++w) s += red[((wave + w) * VEC + i) * kWave + lane];
+        acc[0][i] = s;
       }
-      __syncthreads();   // (the next turn writes the same slots)
     }
-    if (part != 0) return;
-#pragma unroll
-    for (int i = 0; i < VEC; ++i) acc[0][i] = sum[i];
   }
   if (!row_live || grp != 0) return;
   spmm_store_row<T, VEC, LPG, 1, false>(p, bz, row, col0, 0, acc);

@@ -105,8 +105,13 @@ def _check_index_dtypes(row_indices, row_offsets, column_indices, allow_i16=Fals
     _chk(column_indices.dtype in ok, "column_indices must be " + " or ".join(str(d) for d in ok))
 
 
-# from this share of nonzeros in dense blocks the kernels for patterns with structure are taken (SddmmPlan.analyze's rule)
+# From this share of nonzeros in dense blocks the kernels for patterns with structure are taken (SddmmPlan.analyze's
+# rule).  A block counts as dense here from 2048 nonzeros (an eighth of 128 x 128): the kernels themselves lay a block
+# out for the matrix cores from 1536, but a mask whose blocks all sit at that mark runs no faster through them than
+# through the gather kernels (16 heads x 4096 x 4096, columns at random, MI355X: 10 % dense 172 against 151 us for the
+# SDDMM, 166 against 147 for the SpMM; 20 % dense 172 against 286 and 164 against 278).
 _STRUCTURE_SHARE = 0.5
+_STRUCTURE_BLOCK_NONZEROS = 2048
 
 
 def _row_histogram_host(row_offsets):
@@ -119,12 +124,13 @@ def _row_histogram_host(row_offsets):
     return tuple(int(x) for x in hist.tolist())
 
 
-def _dense_share_host(row_offsets, column_indices, k, dense_min=1536):
+def _dense_share_host(row_offsets, column_indices, k, dense_min=None):
     """Share of the nonzeros that sit in 128 x 128 blocks holding ``dense_min`` of them or more (``iex_csr_dense_share``;
     one small launch and a synchronising read), or None where the kernel does not apply (more than 65536 columns)."""
     nonzeros = column_indices.numel()
     if nonzeros == 0 or int(k) > 65536:
         return None
+    dense_min = _STRUCTURE_BLOCK_NONZEROS if dense_min is None else dense_min
     count = torch.zeros(1, dtype=torch.int32, device=row_offsets.device)
     with torch.cuda.device(row_offsets.device):
         rc = _lib.load().iex_csr_dense_share(1 if column_indices.dtype == torch.int16 else 0, row_offsets.numel() - 1, int(k),
@@ -389,12 +395,13 @@ class SddmmPlan:
         self._index_tensors = ()
         self.dense_share = None
 
-    def analyze(self, row_offsets, column_indices, n, dense_min=1536):
+    def analyze(self, row_offsets, column_indices, n, dense_min=None):
         """Look at the pattern once (copies the index arrays to the host: a synchronisation, so not under capture and
         not per call) and settle which kernel the plan's calls use: the one for masks with structure when at least
         half of the nonzeros sit in 128 x 128 blocks that hold ``dense_min`` or more of them, else the gather kernel.
         The library's own rule only knows the overall density, which a band and a random mask can share."""
         import numpy as np
+        dense_min = _STRUCTURE_BLOCK_NONZEROS if dense_min is None else dense_min
         ro = row_offsets.detach().cpu().numpy().astype(np.int64)
         ci = column_indices.detach().cpu().numpy().astype(np.int64)
         m = ro.shape[0] - 1
@@ -402,7 +409,7 @@ class SddmmPlan:
         tiles_n = (int(n) + 127) // 128
         counts = np.bincount((rows // 128) * tiles_n + np.minimum(ci // 128, tiles_n - 1), minlength=((m + 127) // 128) * tiles_n)
         self.dense_share = float(counts[counts >= dense_min].sum()) / max(1, ci.shape[0])
-        self.variant = 3 if self.dense_share >= 0.5 else 1
+        self.variant = 3 if self.dense_share >= _STRUCTURE_SHARE else 1
         return self.variant
 
     def _ready(self, key, nbytes, device, index_tensors=()):

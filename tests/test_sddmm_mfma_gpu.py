@@ -216,6 +216,28 @@ def test_structure_settles_the_kernel(dev):
         assert torch.allclose(f32, auto.float(), rtol=1e-2, atol=1e-2 * 8.0 * 0.1)
 
 
+@pytest.mark.parametrize("idtype", [torch.int32, torch.int16])
+def test_dense_share_kernel_counts_like_numpy(dev, idtype):
+    """iex_csr_dense_share against a numpy count, for several thresholds, on a band with scattered entries, a random
+    mask, a ragged shape (m and k no multiples of 128) and an empty pattern."""
+    from intrasm_engine_amd.pytorch import ops as pyops
+    rng = np.random.default_rng(3)
+    band, *_ = W.config3(tokens=1024, heads=1, band=96, extra=6)
+    ro, ci = W.csr_from_row_lengths(rng, 700, 1000, rng.integers(0, 300, 700))
+    ragged = W.CSR(700, 1000, np.ones(ci.shape[0], np.float32), W.swizzle_from_offsets(ro), ro, ci)
+    for csr in (band, ragged):
+        rows = np.repeat(np.arange(csr.m), np.diff(csr.row_offsets))
+        tiles_n = (csr.k + 127) // 128
+        counts = np.bincount((rows // 128) * tiles_n + csr.column_indices // 128, minlength=((csr.m + 127) // 128) * tiles_n)
+        ro_t = torch.from_numpy(csr.row_offsets).to(dev)
+        ci_t = torch.from_numpy(csr.column_indices).to(dev).to(idtype)
+        for dense_min in (1, 1536, 2048, 5000, 16384, 16385):
+            want = counts[counts >= dense_min].sum() / csr.nnz
+            assert abs(pyops._dense_share_host(ro_t, ci_t, csr.k, dense_min) - want) < 1e-9, dense_min
+    empty = torch.zeros(65, dtype=torch.int32, device=dev)
+    assert pyops._dense_share_host(empty, torch.zeros(0, dtype=idtype, device=dev), 64) is None
+
+
 def test_refusals(dev):
     from intrasm_engine_amd import _lib
     rng = np.random.default_rng(1)

@@ -63,6 +63,56 @@ def log(*a):
     print(*a, file=sys.stderr, flush=True)
 
 
+def fused_timeline(dev, csr_dev, log):
+    """Per-workgroup timeline of config 4's fused launch (matrix-core kernel) for the three orders of its two kinds of
+    workgroup: which CU ran what, when each CU went idle, and how much CU time the tail leaves unused."""
+    import collections
+    import torch
+    from intrasm_engine_amd import _lib, workloads as W
+    lib = _lib.load()
+    ops = torch.ops.iex_ops
+    w, x, ga, gb = W.config4()
+    riw, vw, row, ciw = csr_dev(w, torch.float16, torch.int16)
+    xt = torch.from_numpy(x).to(dev).half()
+    gat, gbt = torch.from_numpy(ga).to(dev).bfloat16(), torch.from_numpy(gb).to(dev).bfloat16()
+    buf = torch.zeros(4 * 4096, dtype=torch.int64, device=dev)
+    for label, order in (("GEMM tiles first (interleave 0)", 0), ("in groups of 64", 64), ("SpMM tiles first (interleave -1)", -1)):
+        for _ in range(3):
+            ops.fused_spmm_gemm(xt, riw, vw, row, ciw, w.m, gat, gbt, False, order)
+        torch.cuda.synchronize()
+        _lib.check(lib.iex_fused_timeline(buf.data_ptr()), "fused_timeline")
+        try:
+            buf.zero_()
+            ops.fused_spmm_gemm(xt, riw, vw, row, ciw, w.m, gat, gbt, False, order)
+            torch.cuda.synchronize()
+        finally:
+            lib.iex_fused_timeline(None)
+        trail = _lib.last_kernels()
+        t = buf.cpu().numpy().reshape(-1, 4)
+        t = t[t[:, 1] != 0]
+        t0 = t[:, 0].min()
+        began, ended = (t[:, 0] - t0) / 100.0, (t[:, 1] - t0) / 100.0       # microseconds (100 MHz clock)
+        is_gemm = (t[:, 3] >> 32) != 0
+        place = ((t[:, 2] >> 16) << 8) | ((t[:, 2] >> 8) & 0xff)             # (XCD, shader engine / array / CU)
+        per_cu = collections.defaultdict(list)
+        for i in np.argsort(began):
+            per_cu[int(place[i])].append((float(began[i]), float(ended[i]), bool(is_gemm[i])))
+        makespan = float(ended.max())
+        busy = float((ended - began).sum())
+        shapes = collections.Counter("".join("G" if g else "S" for _, _, g in v) for v in per_cu.values())
+        idle_at = np.array(sorted(v[-1][1] for v in per_cu.values()))
+        overlap = sum(1 for v in per_cu.values() for a, b in zip(v, v[1:]) if b[0] < a[1] - 0.5)
+        log(f"== {label}: {trail}")
+        log(f"   {len(t)} workgroups on {len(per_cu)} CUs; SpMM tile {np.median((ended - began)[~is_gemm]):.1f} us (median; "
+            f"{(ended - began)[~is_gemm].min():.1f}-{(ended - began)[~is_gemm].max():.1f}), GEMM tile {np.median((ended - began)[is_gemm]):.1f} us "
+            f"({(ended - began)[is_gemm].min():.1f}-{(ended - began)[is_gemm].max():.1f}); two workgroups on one CU at a time: {overlap} cases")
+        log(f"   makespan {makespan:.1f} us; CU time used {busy:.0f} of {makespan * len(per_cu):.0f} CU-us = {100 * busy / (makespan * len(per_cu)):.1f} %; "
+            f"bound by the work {busy / len(per_cu):.1f} us")
+        log("   what a CU ran, in order (S = SpMM tile, G = GEMM tile): " + ", ".join(f"{k} x {v}" for k, v in sorted(shapes.items(), key=lambda kv: -kv[1])))
+        log("   CUs idle from (us): " + ", ".join(f"{q} %: {idle_at[min(len(idle_at) - 1, int(q / 100 * len(idle_at)))]:.0f}" for q in (0, 10, 25, 50, 75, 90)) +
+            f", last {idle_at[-1]:.0f}")
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -83,6 +133,9 @@ def main():
     ap.add_argument("--sddmm-probe", action="store_true",
                     help="config 3's SDDMM (fp16, 16 heads), 3 launches of what the operator picks and 3 of the gather kernel "
                          "(for rocprofv3 --kernel-trace / --pmc)")
+    ap.add_argument("--fused-timeline", action="store_true",
+                    help="config 4's fused launch in its three workgroup orders with the per-workgroup timeline switched on "
+                         "(iex_fused_timeline): prints, per order, what each CU ran and when it went idle")
     ap.add_argument("--overlap-probe", action="store_true",
                     help="for `rocprofv3 --kernel-trace`: 3 replays of config 4's two-branch graph, and exit")
     ap.add_argument("--summarize-pmc", nargs=3, metavar=("FETCH_CSV", "WRITE_CSV", "CELLS_JSON"),
@@ -220,6 +273,10 @@ def main():
                 ops.spmm_sputnik_batched_values(vt_, ri_, probs_, ro_, ci_, pat_.m)
         log("[spmm-probe] row kernel:", _lib.last_kernels())
         torch.cuda.synchronize()
+        return
+
+    if args.fused_timeline:
+        fused_timeline(dev, csr_dev, log)
         return
 
     if args.overlap_probe:

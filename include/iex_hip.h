@@ -387,6 +387,14 @@ int iex_fused_spmm_gemm(int spmm_itype, int m, int k, int n, int nonzeros,
  * exactly one id for any counts and any interleave; the device code calls the same function.
  * No launch, no GPU needed.  No counterpart in the reference. */
 int iex_fused_role(int gemm_blocks, int spmm_blocks, int interleave, int id, int* is_gemm, int* index);
+/* Diagnostic: where and when every workgroup of a fused launch ran.  After iex_fused_timeline(buffer) the calls of
+ * iex_fused_spmm_gemm that this thread makes and that run on the matrix-core kernel write, per workgroup id, four
+ * 64-bit words into `buffer` (device memory, 32 bytes x workgroups of the launch, the caller's): the constant-rate
+ * clock (100 MHz) when the workgroup began and when its last wavefront ended, the place ((XCD << 16) | the low 16 bits
+ * of the hardware id word: compute unit, shader array and shader engine in bits 8..15), and (1 << 32 for a GEMM tile) |
+ * the tile or block index.  Costs a workgroup barrier and four stores per workgroup; results are unchanged.
+ * iex_fused_timeline(NULL) switches it off.  No counterpart in the reference. */
+int iex_fused_timeline(void* buffer);
 
 /* ------------------------------------------------------------ graph builder ---- */
 /* Opaque builder of ONE hipGraph from per-stream captures; mirrors

@@ -65,6 +65,7 @@ SIGNATURES = {
     "iex_fused_spmm_gemm": (_i, [_i, _i, _i, _i, _i, _vp, _vp, _vp, _vp, _vp, _vp,
                                  _i, _i, _i, _i, _i, _vp, _vp, _vp, _i, _ll, _ll, _ll, _i, _vp]),
     "iex_fused_role": (_i, [_i, _i, _i, _i, _c.POINTER(_i), _c.POINTER(_i)]),
+    "iex_fused_timeline": (_i, [_vp]),
     "iex_graph_create": (_vp, []),
     "iex_graph_wrap": (_vp, [_vp]),
     "iex_graph_destroy": (None, [_vp]),

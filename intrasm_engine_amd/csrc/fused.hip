@@ -31,7 +31,18 @@ struct FusedParams {
   GemmParams g;
   SpmmParams s;
   int gemm_batch, gemm_blocks, spmm_blocks, spmm_by, interleave;
+  unsigned long long* timeline;   // diagnostic (iex_fused_timeline): 4 words per workgroup, or null
 };
+
+// Where and when a workgroup ran, for the diagnostic timeline: constant-rate clock (100 MHz), the XCD and the
+// hardware id word (compute unit, shader array, shader engine in bits 8..15).
+__device__ __forceinline__ unsigned long long fused_clock() { return wall_clock64(); }
+__device__ __forceinline__ unsigned fused_where() {
+  unsigned hw, xcc;
+  asm volatile("s_getreg_b32 %0, hwreg(HW_REG_HW_ID)" : "=s"(hw));
+  asm volatile("s_getreg_b32 %0, hwreg(HW_REG_XCC_ID)" : "=s"(xcc));
+  return ((xcc & 0xf) << 16) | (hw & 0xffff);
+}
 
 constexpr int kFusedWM = 2, kFusedWN = 2;
 // The GEMM role's registers and LDS leave two waves per SIMD; the SpMM role makes up for the
@@ -97,6 +108,7 @@ __global__ __launch_bounds__(kMfma2Threads, 2) void fused_mc_kernel(FusedParams 
   bool is_gemm;
   int idx;
   fused_role(p, blockIdx.x, is_gemm, idx);
+  const unsigned long long began = p.timeline ? fused_clock() : 0ull;
   if (is_gemm) {
     const int per_batch = p.g.tiles_m * p.g.tiles_n;
     const int z = idx / per_batch, t = idx % per_batch;
@@ -104,6 +116,16 @@ __global__ __launch_bounds__(kMfma2Threads, 2) void fused_mc_kernel(FusedParams 
   } else {
     // p.spmm_by = row tiles here: consecutive ids walk the row blocks of one column panel
     spmm_mfma2_block<false, IT, W, 128>(p.s, idx % p.spmm_by, idx / p.spmm_by, 0, smem);
+  }
+  if (p.timeline) {   // (uniform over the grid; the tile routines return to here in every wavefront)
+    __syncthreads();
+    if (threadIdx.x == 0) {
+      unsigned long long* t = p.timeline + 4ull * blockIdx.x;
+      t[0] = began;
+      t[1] = fused_clock();
+      t[2] = fused_where();
+      t[3] = (is_gemm ? 1ull << 32 : 0ull) | (unsigned)idx;
+    }
   }
 }
 
@@ -227,6 +249,13 @@ extern "C" int iex_fused_role(int gemm_blocks, int spmm_blocks, int interleave, 
   return 0;
 }
 
+// The buffer that the next matrix-core fused launches of this thread write their timeline to (null: none).
+static thread_local unsigned long long* g_fused_timeline = nullptr;
+extern "C" int iex_fused_timeline(void* buffer) {
+  g_fused_timeline = static_cast<unsigned long long*>(buffer);
+  return 0;
+}
+
 extern "C" int iex_fused_spmm_gemm(int spmm_itype, int m, int k, int n, int nonzeros, const int* row_indices,
                                    const void* values, const int* row_offsets, const void* column_indices,
                                    const void* dense, void* spmm_out, int gemm_dtype, int trans_b, int M, int N, int K,
@@ -253,8 +282,10 @@ extern "C" int iex_fused_spmm_gemm(int spmm_itype, int m, int k, int n, int nonz
   p.gemm_batch = gemm_batch;
   p.s = SpmmParams{m, k, n, nonzeros, row_indices, values, row_offsets, column_indices, dense, nullptr, spmm_out, 0, 0, 0};
   p.interleave = interleave;
+  p.timeline = nullptr;
   hipStream_t s = static_cast<hipStream_t>(stream);
-  if (const int windows = spmm_matrix_core_windows(p.s)) {  // what the stand-alone SpMM of this shape runs on
+  if (const int windows = spmm_matrix_core_windows(p.s)) {
+    p.timeline = g_fused_timeline;  // what the stand-alone SpMM of this shape runs on
     if (spmm_itype == IEX_I16) return launch_mc_kind<short>(p, windows, gemm_dtype == IEX_BF16, trans_b != 0, s);
     return launch_mc_kind<int>(p, windows, gemm_dtype == IEX_BF16, trans_b != 0, s);
   }

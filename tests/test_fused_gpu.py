@@ -54,6 +54,40 @@ def test_fused_config4_shape(dev):
     assert torch.equal(out, alone) and torch.equal(c, ops.gemm_mfma(gat, gbt_t, True))
 
 
+def test_fused_timeline_records_every_workgroup_and_changes_no_result(dev):
+    """The diagnostic timeline (iex_fused_timeline): one record per workgroup (both clocks set, end after begin, every
+    GEMM tile and every SpMM tile exactly once), the outputs are those of a launch without it, and it is off again after
+    iex_fused_timeline(NULL)."""
+    from intrasm_engine_amd import _lib
+    lib = _lib.load()
+    w, x, ga, gb = W.config4()
+    ri, v, ro, ci = to_dev(w, dev, torch.float16, torch.int16)
+    xt = torch.from_numpy(x).to(dev).half()
+    gat, gbt = torch.from_numpy(ga).to(dev).bfloat16(), torch.from_numpy(gb).to(dev).bfloat16()
+    out0, c0 = ops.fused_spmm_gemm(xt, ri, v, ro, ci, w.m, gat, gbt, False, -1)
+    groups = 344 + 256                                   # 128 x 512 SpMM tiles of 11008 x 2048, 128 x 256 GEMM tiles of 4096 x 2048
+    buf = torch.zeros(4 * (groups + 8), dtype=torch.int64, device=dev)
+    assert lib.iex_fused_timeline(buf.data_ptr()) == 0
+    try:
+        out1, c1 = ops.fused_spmm_gemm(xt, ri, v, ro, ci, w.m, gat, gbt, False, -1)
+        torch.cuda.synchronize()
+    finally:
+        assert lib.iex_fused_timeline(None) == 0
+    assert torch.equal(out0, out1) and torch.equal(c0, c1)
+    t = buf.cpu().numpy().reshape(-1, 4)
+    assert (t[groups:] == 0).all()
+    t = t[:groups]
+    assert (t[:, 0] > 0).all() and (t[:, 1] > t[:, 0]).all()
+    is_gemm, index = (t[:, 3] >> 32) != 0, t[:, 3] & 0xffffffff
+    assert not is_gemm[:344].any() and is_gemm[344:].all()           # SpMM tiles first
+    assert sorted(index[~is_gemm]) == list(range(344)) and sorted(index[is_gemm]) == list(range(256))
+    assert 1 < len(set(int(p) >> 8 for p in t[:, 2])) <= 256         # (XCD and CU: bits 8 and up of the place word)
+    buf.zero_()
+    out2, _ = ops.fused_spmm_gemm(xt, ri, v, ro, ci, w.m, gat, gbt, False, -1)
+    torch.cuda.synchronize()
+    assert torch.equal(out2, out0) and not buf.any()
+
+
 def test_fused_matrix_core_batched_gemm(dev):
     """Matrix-core fused launch with a batched, ragged GEMM (the attention products of the
     decoder layer ride along like this) and int32 column indices."""

@@ -1,11 +1,11 @@
 // Ablation of the main loop of the direct-load GEMM (gemm_dma_device.cuh) on bf16 products with B as (K, N): the kernel
-// as shipped, and instrumented builds of the same template that leave out one ingredient each (the DBG switches of
-// gemm_tile_dma; results of those builds are wrong on purpose, every address they use stays in bounds).  Prints
+// as shipped, and instrumented builds of a copy of its tile routine that leave out one ingredient each (the DBG switches of
+// gemm_tile_dma_ablation, gemm_loop_ablation_device.cuh; results of those builds are wrong on purpose, every address they use stays in bounds).  Prints
 // TFLOP/s from HIP events over 10 launches, for 256 x 256 tiles by four waves and 128 x 256 tiles by eight.
 //
 //   hipcc --offload-arch=gfx950 -O3 -std=c++17 -Xclang -target-feature -Xclang -packed-fp32-ops \
 //         intrasm_engine_amd/benchmarks/gemm_loop_ablation.hip -o gemm_loop_ablation && ./gemm_loop_ablation
-#include "../csrc/gemm_dma_device.cuh"
+#include "gemm_loop_ablation_device.cuh"
 
 #include <cstdio>
 #include <cstdlib>
@@ -23,7 +23,7 @@ __global__ __launch_bounds__(WCN * 128, 1) void ablation_kernel(GemmParams p) {
   extern __shared__ __align__(16) unsigned char smem[];
   int tile_m, tile_n;
   if (!xcd_tile(blockIdx.x, p.tiles_m, p.tiles_n, tile_m, tile_n)) return;
-  gemm_tile_dma<true, false, WM, WN, WCN, 32, 4, false, DBG>(p, tile_m, tile_n, blockIdx.y, smem);
+  gemm_tile_dma_ablation<true, false, WM, WN, WCN, 32, 4, false, DBG>(p, tile_m, tile_n, blockIdx.y, smem);
 }
 
 template <int WM, int WN, int WCN, int DBG>

@@ -36,6 +36,14 @@
 
 namespace iex {
 
+// The direct load of the library, with a cache modifier when the program is built with -DIEX_DMA_MOD='" sc0"' and the like.
+#ifndef IEX_DMA_MOD
+#define IEX_DMA_MOD ""
+#endif
+__device__ __forceinline__ void lds_dma16_mod(const void* g, unsigned lds_base_uniform) {
+  asm volatile("s_mov_b32 m0, %1\n\tglobal_load_lds_dwordx4 %0, off" IEX_DMA_MOD ::"v"(g), "s"(lds_base_uniform) : "memory", "m0");
+}
+
 // GMODE: which wavefronts form group 1: 0 = wavefronts 4..7 (the second wavefront of every SIMD when a
 // workgroup's wavefronts are dealt round-robin to the four SIMDs), 1 = odd wavefronts, 2 = no second group
 // (every wavefront in phase: the control experiment).
@@ -107,19 +115,19 @@ __device__ __forceinline__ void gemm_tile_ppx(const GemmParams& p, int tile_m, i
     const int k0 = (DBG & 128) ? 0 : min(kt, KT - 1) * BK;  // past the end: the last tile again, into a stage nobody reads
     if constexpr ((DBG & 128) != 0) {
       const unsigned base = lds0 + stage * STAGE_BYTES + (q < A_INSTR ? 0 : A_BYTES) + wave * (A_INSTR * 1024);
-      lds_dma16(a_row[q % A_INSTR] + a_k8[q % A_INSTR], __builtin_amdgcn_readfirstlane(base + (q % A_INSTR) * 1024));
+      lds_dma16_mod(a_row[q % A_INSTR] + a_k8[q % A_INSTR], __builtin_amdgcn_readfirstlane(base + (q % A_INSTR) * 1024));
       return;
     }
     if (q < A_INSTR) {
       const unsigned base = lds0 + stage * STAGE_BYTES + wave * (A_INSTR * 1024);
-      lds_dma16(a_row[q] + min(k0 + a_k8[q], last_k8), __builtin_amdgcn_readfirstlane(base + q * 1024));
+      lds_dma16_mod(a_row[q] + min(k0 + a_k8[q], last_k8), __builtin_amdgcn_readfirstlane(base + q * 1024));
     } else {
       const int qb = q - A_INSTR;
       const unsigned bbase = lds0 + stage * STAGE_BYTES + A_BYTES + wave * (B_INSTR * 1024);
       if constexpr (TRANS_B)
-        lds_dma16(b_row[qb] + min(k0 + b_k8[qb], last_k8), __builtin_amdgcn_readfirstlane(bbase + qb * 1024));
+        lds_dma16_mod(b_row[qb] + min(k0 + b_k8[qb], last_k8), __builtin_amdgcn_readfirstlane(bbase + qb * 1024));
       else
-        lds_dma16(b_row[qb] + (size_t)min(k0 + b_k8[qb], p.K - 1) * p.N, __builtin_amdgcn_readfirstlane(bbase + qb * 1024));
+        lds_dma16_mod(b_row[qb] + (size_t)min(k0 + b_k8[qb], p.K - 1) * p.N, __builtin_amdgcn_readfirstlane(bbase + qb * 1024));
     }
   };
   // entries at k >= K of the last tile must be zero: clamped addresses delivered copies of real data

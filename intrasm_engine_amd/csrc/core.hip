@@ -88,28 +88,43 @@ __global__ __launch_bounds__(256) void csr_row_histogram_kernel(int m, const int
 }
 
 // *dense_nonzeros += the nonzeros of this block of 128 rows that sit in 128 x 128 blocks holding at least dense_min of
-// them.  One workgroup (4 wavefronts) per 128 rows; the counters of the row block's column blocks live in LDS.
+// them.  One workgroup (16 wavefronts) per 128 rows; the counters of the row block's column blocks live in LDS.  A
+// wavefront takes 64 nonzeros of a row at a time; neighbours that fall into the same column block (all of them, in
+// runs, when the columns ascend) are counted by the first lane of their run, so a run costs one LDS atomic, not one
+// per nonzero.  Any column order gives the same counts.
 constexpr int kShareMaxTiles = 512;   // k <= 65536
+constexpr int kShareThreads = 1024;
 template <typename IT>
-__global__ __launch_bounds__(256) void csr_dense_share_kernel(int m, int k, const int* __restrict__ row_offsets, const IT* __restrict__ cols,
-                                                              int dense_min, int* dense_nonzeros) {
+__global__ __launch_bounds__(kShareThreads) void csr_dense_share_kernel(int m, int k, const int* __restrict__ row_offsets, const IT* __restrict__ cols,
+                                                                        int dense_min, int* dense_nonzeros) {
   __shared__ int count[kShareMaxTiles];
   __shared__ int total;
   const int tiles = (k + 127) / 128;
-  for (int t = threadIdx.x; t < tiles; t += 256) count[t] = 0;
+  for (int t = threadIdx.x; t < tiles; t += kShareThreads) count[t] = 0;
   if (threadIdx.x == 0) total = 0;
   __syncthreads();
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  for (int r = blockIdx.x * 128 + wave; r < min(m, blockIdx.x * 128 + 128); r += 4) {
+  for (int r = blockIdx.x * 128 + wave; r < min(m, blockIdx.x * 128 + 128); r += kShareThreads / 64) {
     const int s = row_offsets[r], e = row_offsets[r + 1];
-    for (int j = s + lane; j < e; j += 64) {
-      const int c = (int)cols[j];
-      if (c >= 0 && c < k) atomicAdd(&count[c >> 7], 1);
+    for (int base = s; base < e; base += 64) {
+      const int j = base + lane;
+      int t = -1;   // (no nonzero here, or a column outside the matrix: counted nowhere)
+      if (j < e) {
+        const int c = (int)cols[j];
+        if (c >= 0 && c < k) t = c >> 7;
+      }
+      const int before = __shfl_up(t, 1, 64);
+      const unsigned long long heads = __ballot(lane == 0 || t != before);
+      if ((heads >> lane) & 1ull) {
+        const unsigned long long later = lane == 63 ? 0ull : heads >> (lane + 1);
+        const int run = later ? __builtin_ctzll(later) + 1 : 64 - lane;
+        if (t >= 0) atomicAdd(&count[t], run);
+      }
     }
   }
   __syncthreads();
   int mine = 0;
-  for (int t = threadIdx.x; t < tiles; t += 256) mine += count[t] >= dense_min ? count[t] : 0;
+  for (int t = threadIdx.x; t < tiles; t += kShareThreads) mine += count[t] >= dense_min ? count[t] : 0;
   if (mine) atomicAdd(&total, mine);
   __syncthreads();
   if (threadIdx.x == 0 && total) atomicAdd(dense_nonzeros, total);
@@ -127,9 +142,9 @@ int iex_csr_dense_share(int itype, int m, int k, const int* row_offsets, const v
   if (m == 0 || k == 0) return 0;
   hipStream_t s = static_cast<hipStream_t>(stream);
   if (itype == IEX_I32)
-    hipLaunchKernelGGL(csr_dense_share_kernel<int>, dim3((m + 127) / 128), dim3(256), 0, s, m, k, row_offsets, static_cast<const int*>(column_indices), dense_min, dense_nonzeros);
+    hipLaunchKernelGGL(csr_dense_share_kernel<int>, dim3((m + 127) / 128), dim3(kShareThreads), 0, s, m, k, row_offsets, static_cast<const int*>(column_indices), dense_min, dense_nonzeros);
   else
-    hipLaunchKernelGGL(csr_dense_share_kernel<short>, dim3((m + 127) / 128), dim3(256), 0, s, m, k, row_offsets, static_cast<const short*>(column_indices), dense_min, dense_nonzeros);
+    hipLaunchKernelGGL(csr_dense_share_kernel<short>, dim3((m + 127) / 128), dim3(kShareThreads), 0, s, m, k, row_offsets, static_cast<const short*>(column_indices), dense_min, dense_nonzeros);
   return iex::check_hip(hipGetLastError(), "csr_dense_share launch");
 }
 

@@ -29,15 +29,8 @@
 
 namespace iex {
 
-#ifndef IEX_DMA_MOD
-#define IEX_DMA_MOD ""
-#endif
 __device__ __forceinline__ void lds_dma16(const void* g, unsigned lds_base_uniform) {
-  asm volatile("s_mov_b32 m0, %1\n\tglobal_load_lds_dwordx4 %0, off" IEX_DMA_MOD ::"v"(g), "s"(lds_base_uniform) : "memory", "m0");
-}
-// (for the loop-ablation benchmark: the address arithmetic of a direct load without the load)
-__device__ __forceinline__ void lds_dma16_address_only(const void* g, unsigned lds_base_uniform) {
-  asm volatile("s_mov_b32 m0, %1\n\t; no load of %0" ::"v"(g), "s"(lds_base_uniform) : "memory", "m0");
+  asm volatile("s_mov_b32 m0, %1\n\tglobal_load_lds_dwordx4 %0, off" ::"v"(g), "s"(lds_base_uniform) : "memory", "m0");
 }
 
 template <int N>
@@ -73,10 +66,7 @@ __device__ __forceinline__ bool xcd_tile(int block, int tiles_m, int tiles_n, in
   return true;
 }
 
-// DBG (for the loop-ablation benchmark, benchmarks/gemm_loop_ablation.hip; results are wrong on purpose): 1 = no direct
-// loads after the prologue (the stages keep the first tiles' data), 2 = no barrier per K step, 4 = no fragment reads from LDS (the MFMAs multiply what the first read left),
-// 8 = the address arithmetic of the direct loads without the loads.
-template <bool BF16, bool TRANS_B, int WM, int WN, int WCN, int BK, int STAGES, bool SPLIT = false, int DBG = 0>
+template <bool BF16, bool TRANS_B, int WM, int WN, int WCN, int BK, int STAGES, bool SPLIT = false>
 __device__ __forceinline__ void gemm_tile_dma(const GemmParams& p, int tile_m, int tile_n, int z, unsigned char* smem) {
   constexpr int BM = 2 * WM * 32, BN = WCN * WN * 32, WAVES = 2 * WCN;
   constexpr int CPR = BK / 8;          // 16-byte chunks per K-contiguous row
@@ -140,14 +130,14 @@ __device__ __forceinline__ void gemm_tile_dma(const GemmParams& p, int tile_m, i
     const int k0 = min(kt, KT - 1) * BK;  // past the end: the last tile again, into a stage nobody reads
     if (q < A_INSTR) {
       const unsigned base = lds0 + stage * STAGE_BYTES + wave * (A_INSTR * 1024);
-      (DBG & 8 ? lds_dma16_address_only : lds_dma16)(a_row[q] + min(k0 + a_k8[q], last_k8), __builtin_amdgcn_readfirstlane(base + q * 1024));
+      lds_dma16(a_row[q] + min(k0 + a_k8[q], last_k8), __builtin_amdgcn_readfirstlane(base + q * 1024));
     } else {
       const int qb = q - A_INSTR;
       const unsigned bbase = lds0 + stage * STAGE_BYTES + A_BYTES + wave * (B_INSTR * 1024);
       if constexpr (TRANS_B)
-        (DBG & 8 ? lds_dma16_address_only : lds_dma16)(b_row[qb] + min(k0 + b_k8[qb], last_k8), __builtin_amdgcn_readfirstlane(bbase + qb * 1024));
+        lds_dma16(b_row[qb] + min(k0 + b_k8[qb], last_k8), __builtin_amdgcn_readfirstlane(bbase + qb * 1024));
       else
-        (DBG & 8 ? lds_dma16_address_only : lds_dma16)(b_row[qb] + (size_t)min(k0 + b_k8[qb], p.K - 1) * p.N, __builtin_amdgcn_readfirstlane(bbase + qb * 1024));
+        lds_dma16(b_row[qb] + (size_t)min(k0 + b_k8[qb], p.K - 1) * p.N, __builtin_amdgcn_readfirstlane(bbase + qb * 1024));
     }
   };
   auto issue = [&](int kt, int stage) {
@@ -201,12 +191,7 @@ __device__ __forceinline__ void gemm_tile_dma(const GemmParams& p, int tile_m, i
   }
 
   u32x4 fa[2][WM], fb[2][WN];  // operand fragments of two consecutive sub-steps
-  bool have_frags[2] = {false, false};
   auto read_frags = [&](const unsigned char* st, int ks, int buf) {
-    if constexpr ((DBG & 4) != 0) {   // (each register set once, then never again)
-      if (have_frags[buf]) return;
-      have_frags[buf] = true;
-    }
 #pragma unroll
     for (int i = 0; i < WM; ++i) fa[buf][i] = *reinterpret_cast<const u32x4*>(st + a_off[ks] + i * 32 * RB);
 #pragma unroll
@@ -253,7 +238,7 @@ __device__ __forceinline__ void gemm_tile_dma(const GemmParams& p, int tile_m, i
       } else {
         wait_vmcnt<(STAGES - 3) * LOADS>();  // my loads of tile kt + 1 have landed
         if (tail && kt + 2 == KT) zero_tail(kt + 1, (kt + 1) % STAGES);
-        if constexpr ((DBG & 2) == 0) __syncthreads();
+        __syncthreads();
         read_frags(smem + ((kt + 1) % STAGES) * STAGE_BYTES, 0, cur ^ 1);  // (past the last tile: read, never used)
         __builtin_amdgcn_sched_barrier(0);
         const int next = kt + STAGES - 1;
@@ -265,7 +250,7 @@ __device__ __forceinline__ void gemm_tile_dma(const GemmParams& p, int tile_m, i
             const int m = i * WN + j;
 #pragma unroll
             for (int q = m * LOADS / NM; q < (m + 1) * LOADS / NM; ++q)
-              if constexpr ((DBG & 1) == 0) issue_one(next, next % STAGES, q);
+              issue_one(next, next % STAGES, q);
           }
       }
     }

@@ -77,6 +77,11 @@ def test_static_scratch_serves_the_kernel_for_patterns_with_structure_between_ot
     again = _call(lib, lib.iex_spmm_static, dev, band, x, torch.int32, flags=flags)
     assert _lib.last_kernels().split(" + ") == ["sddmm_tile_ptr_kernel", "sb_lists_kernel", "spmm_blocks_kernel<false>"]
     assert torch.equal(first, want) and torch.equal(again, want)
+    # a caller cannot vouch for what another call left in the shared array: the READY flags are ignored here
+    _call(lib, lib.iex_spmm_static, dev, other, torch.randn(1, 1024, 1024, device=dev).half(), torch.int16)
+    vouched = _call(lib, lib.iex_spmm_static, dev, band, x, torch.int32, flags=flags | _lib.SPMM_TABLES_READY | _lib.SPMM_LISTS_READY)
+    assert _lib.last_kernels().split(" + ") == ["sddmm_tile_ptr_kernel", "sb_lists_kernel", "spmm_blocks_kernel<false>"]
+    assert torch.equal(vouched, want)
 
 
 def test_static_scratch_without_workspace_use_runs_as_the_plain_entry_point(dev):

@@ -81,9 +81,20 @@ int main(int argc, char** argv) {
   constexpr int L = gemm_dma_lds_bytes<4, 2, 4, 32, 4>();
   for (int round = 0; round < 2; ++round) {
   int id = 0;
+  // (builds that leave nothing out must give the bits of the 4-wave tile: RUNC compares the output with line 0's)
+  static std::vector<unsigned short> ref_c;
+  auto mismatches = [&]() {
+    std::vector<unsigned short> c((size_t)M * N);
+    hipMemcpy(c.data(), C, c.size() * 2, hipMemcpyDeviceToHost);
+    if (ref_c.empty()) { ref_c = c; return 0ll; }
+    long long bad = 0;
+    for (size_t i = 0; i < c.size(); ++i) bad += c[i] != ref_c[i];
+    return bad;
+  };
+#define RUNC(name, expr) do { if (only < 0 || only == id) { hipMemset(C, 0xff, (size_t)M * N * 2); double t = (expr); printf("  [%2d] %-44s %7.0f   mismatches %lld\n", id, name, t, mismatches()); fflush(stdout);} ++id; } while (0)
 #define RUN(name, expr) do { if (only < 0 || only == id) { double t = (expr); printf("  [%2d] %-44s %7.0f\n", id, name, t); fflush(stdout);} ++id; } while (0)
-  RUN("shipped 256x256 / 4 waves", timeit(ref_kernel<false, 4, 4, 2, 32, 4>, p, 256, 256, 256, gemm_dma_lds_bytes<4, 4, 2, 32, 4>()));
-  RUN("ping-pong 256x256", timeit(ppx_kernel<false, 4, 2, 4, 32, 4, 0, 0>, p, 256, 256, 512, L));
+  RUNC("shipped 256x256 / 4 waves", timeit(ref_kernel<false, 4, 4, 2, 32, 4>, p, 256, 256, 256, gemm_dma_lds_bytes<4, 4, 2, 32, 4>()));
+  RUNC("ping-pong 256x256", timeit(ppx_kernel<false, 4, 2, 4, 32, 4, 0, 0>, p, 256, 256, 512, L));
   RUN("pp: no direct loads in loop", timeit(ppx_kernel<false, 4, 2, 4, 32, 4, 0, 1>, p, 256, 256, 512, L));
   RUN("pp: fragments read once", timeit(ppx_kernel<false, 4, 2, 4, 32, 4, 0, 2>, p, 256, 256, 512, L));
   RUN("pp: neither (MFMA + barriers)", timeit(ppx_kernel<false, 4, 2, 4, 32, 4, 0, 3>, p, 256, 256, 512, L));
@@ -97,7 +108,10 @@ int main(int argc, char** argv) {
   RUN("pp: 3 stages", timeit(ppx_kernel<false, 4, 2, 4, 32, 3, 0, 0>, p, 256, 256, 512, gemm_dma_lds_bytes<4, 2, 4, 32, 3>()));
   RUN("pp: 3 stages, no waits", timeit(ppx_kernel<false, 4, 2, 4, 32, 3, 0, 64>, p, 256, 256, 512, gemm_dma_lds_bytes<4, 2, 4, 32, 3>()));
   RUN("pp: all loads from one L1-resident 16 KB", timeit(ppx_kernel<false, 4, 2, 4, 32, 4, 0, 128>, p, 256, 256, 512, L));
-  RUN("pp, A in 64-k stages (3) + B 32-k (4)", timeit(pp_kernel<false, 4, 2, 4>, p, 256, 256, 512, gemm_pp_lds_bytes<true, false, 4, 2, 4>()));
+  RUNC("pp: B through registers, A direct", timeit(ppx_kernel<false, 4, 2, 4, 32, 4, 0, 256>, p, 256, 256, 512, L));
+  RUNC("pp: A through registers, B direct", timeit(ppx_kernel<false, 4, 2, 4, 32, 4, 0, 512>, p, 256, 256, 512, L));
+  RUNC("pp: A and B through registers", timeit(ppx_kernel<false, 4, 2, 4, 32, 4, 0, 768>, p, 256, 256, 512, L));
+  RUNC("pp, A in 64-k stages (3) + B 32-k (4)", timeit(pp_kernel<false, 4, 2, 4>, p, 256, 256, 512, gemm_pp_lds_bytes<true, false, 4, 2, 4>()));
   }
   return 0;
 }

@@ -173,10 +173,27 @@ __device__ __forceinline__ void gemm_tile_ppx(const GemmParams& p, int tile_m, i
   }
 
   u32x4 fa[2][WM], fb[2][WN];  // the operand fragments of one phase (two sub-steps of 16)
+  // DBG & 256 / & 512: B / A of a later tile comes through registers (a plain load in one memory phase, written to LDS
+  // at the start of the wavefront's next memory phase, to the bytes the direct load would have filled) - K a multiple of BK only
+  u32x4 areg[A_INSTR], breg[B_INSTR];
+  int reg_stage = -1;
   // memory phase h of tile kt
   bool have = false;
   auto mem_phase = [&](int kt, int h) {
     const unsigned char* st = smem + (kt % STAGES) * STAGE_BYTES;
+    if constexpr ((DBG & (256 | 512)) != 0) {
+      if (reg_stage >= 0) {
+        unsigned char* dst = smem + reg_stage * STAGE_BYTES;
+        if constexpr ((DBG & 512) != 0) {
+#pragma unroll
+          for (int q = 0; q < A_INSTR; ++q) *reinterpret_cast<u32x4*>(dst + ((wave * A_INSTR + q) * 64 + lane) * 16) = areg[q];
+        }
+        if constexpr ((DBG & 256) != 0) {
+#pragma unroll
+          for (int q = 0; q < B_INSTR; ++q) *reinterpret_cast<u32x4*>(dst + A_BYTES + ((wave * B_INSTR + q) * 64 + lane) * 16) = breg[q];
+        }
+      }
+    }
     const bool skip = (DBG & 2) && have;
     have = true;
 #pragma unroll
@@ -205,8 +222,19 @@ __device__ __forceinline__ void gemm_tile_ppx(const GemmParams& p, int tile_m, i
       if constexpr ((DBG & 1) != 0) continue;
       if ((DBG & 16) && q < A_INSTR) continue;
       if ((DBG & 32) && q >= A_INSTR) continue;
+      if ((DBG & 512) && q < A_INSTR) {
+        areg[q] = *reinterpret_cast<const u32x4*>(a_row[q] + min(min(next, KT - 1) * BK + a_k8[q], last_k8));
+        continue;
+      }
+      if ((DBG & 256) && q >= A_INSTR) {
+        const int qb = q - A_INSTR;
+        if constexpr (TRANS_B) breg[qb] = *reinterpret_cast<const u32x4*>(b_row[qb] + min(min(next, KT - 1) * BK + b_k8[qb], last_k8));
+        else breg[qb] = *reinterpret_cast<const u32x4*>(b_row[qb] + (size_t)min(min(next, KT - 1) * BK + b_k8[qb], p.K - 1) * p.N);
+        continue;
+      }
       issue_one(next, next % STAGES, q);
     }
+    if constexpr ((DBG & (256 | 512)) != 0) reg_stage = next % STAGES;
   };
   auto compute_phase = [&]() {
     __builtin_amdgcn_s_setprio(1);

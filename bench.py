@@ -306,10 +306,10 @@ def main():
 
     # --------------------------------------------------------------- the timed step
     # One step = the 15 launches of the sweep in one hipGraph.  The launches are independent, so the graph holds them on
-    # two parallel branches (cells dealt longest first, by nnz * n, to the branch with less work): the gap between two
-    # kernels of one branch (2-4 us) and the tails of the short launches are then covered by the other branch.  Three and
-    # four branches measured slower than two (710 / 735 against 671 us where one branch takes 715).  The same graph on
-    # one branch is timed beside it (config.one_branch_sweep_us).
+    # two parallel branches (cells in order of nnz * n, dealt alternately, so the two launches that run side by side are
+    # of similar length): the gap between two kernels of one branch (2-4 us) and the tails of the short launches are then
+    # covered by the other branch.  Three and four branches measured slower than two (710 / 735 against 653-672 us where
+    # one branch takes 716).  The same graph on one branch is timed beside it (config.one_branch_sweep_us).
     def time_sweep(lists):
         constructor, keep = IL.capture_serialized(lists[0]) if len(lists) == 1 else IL.capture_interleaved(*lists)
         constructor.instantiate_graph_exec()
@@ -329,11 +329,8 @@ def main():
         del keep
         return ms, wall
 
-    branches, load = [[], []], [0, 0]
-    for s, n in sorted(cells, key=lambda c: -mats[c[0]].nnz * c[1]):
-        i = load.index(min(load))
-        branches[i].append((s, n))
-        load[i] += mats[s].nnz * n
+    by_cost = sorted(cells, key=lambda c: -mats[c[0]].nnz * c[1])
+    branches = [by_cost[0::2], by_cost[1::2]]      # (neighbours in cost run side by side: 653 us where longest-first dealing gave 672)
     ms_one_branch, _ = time_sweep([[spmm32(s, n) for s, n in cells]])
     ms_per_step, wall_ms = time_sweep([[spmm32(s, n) for s, n in b] for b in branches])
     value = sweep_bytes / 1e9 / (ms_per_step * 1e-3)

@@ -35,6 +35,7 @@ sys.path.insert(0, ROOT)
 HBM_PEAK_GBPS = 8000.0           # MI355X HBM3E
 MFMA_PEAK_TFLOPS_16BIT = 2500.0  # dense bf16 / fp16
 VALU_PEAK_TFLOPS_FP32 = 78.6     # vector fp32 FMA without packed math (the build disables v_pk_*_f32)
+MFMA_PEAK_TFLOPS_FP32 = 157.3    # dense fp32 MFMA
 CELL_REPEATS = 20                # launches of one cell inside its timing graph
 TRAFFIC_PROFILE = os.path.join(ROOT, "profiles", "spmm_fp32_config2_hbm_traffic_pmc.txt")
 COLD_SCRATCH_BYTES = 512 << 20   # written between cold-cache samples (> the 256 MB last-level cache)
@@ -180,9 +181,20 @@ def main():
     dens32 = {n: torch.from_numpy(b).to(dev) for n, b in dens.items()}
     cells = [(s, n) for s in W.C2_SPARSITIES for n in W.C2_NS]
 
-    def spmm32(s, n):
+    def spmm32_alone(s, n):
+        """The launch of a cell as the library chooses it when it knows of no neighbour."""
         ri, v, ro, ci = mats32[s]
         return lambda: ops.spmm_sputnik_reuse_weight(dens32[n], ri, v, ro, ci, mats[s].m)
+
+    def spmm32(s, n):
+        """The launch of a cell as it runs in the timed step: told that it shares the chip with a gather-bound launch
+        (IEX_SPMM_BESIDE_GATHER_KERNEL; the timed graph has two parallel branches)."""
+        alone = spmm32_alone(s, n)
+
+        def call():
+            with pyops.kernel_params(spmm={"beside_gather_kernel": True}):
+                return alone()
+        return call
 
     def cell_bytes(s, n, sv=4, si=4):
         c = mats[s]
@@ -306,10 +318,10 @@ def main():
 
     # --------------------------------------------------------------- the timed step
     # One step = the 15 launches of the sweep in one hipGraph.  The launches are independent, so the graph holds them on
-    # two parallel branches (cells in order of nnz * n, dealt alternately, so the two launches that run side by side are
-    # of similar length): the gap between two kernels of one branch (2-4 us) and the tails of the short launches are then
-    # covered by the other branch.  Three and four branches measured slower than two (710 / 735 against 653-672 us where
-    # one branch takes 716).  The same graph on one branch is timed beside it (config.one_branch_sweep_us).
+    # two parallel branches: the gap between two kernels of one branch (2-4 us) and the tails of the short launches are
+    # covered by the other branch, and kernels bound by different units overlap.  Three and four branches measured slower
+    # than two (710 / 735 against 653-672 us where one branch takes 716).  The same launches on one branch, and on two
+    # branches without the neighbour hint, are timed beside it (config.one_branch_sweep_us, config.two_branches_...).
     def time_sweep(lists):
         constructor, keep = IL.capture_serialized(lists[0]) if len(lists) == 1 else IL.capture_interleaved(*lists)
         constructor.instantiate_graph_exec()
@@ -330,11 +342,24 @@ def main():
         return ms, wall
 
     by_cost = sorted(cells, key=lambda c: -mats[c[0]].nnz * c[1])
-    branches = [by_cost[0::2], by_cost[1::2]]      # (neighbours in cost run side by side: 653 us where longest-first dealing gave 672)
-    ms_one_branch, _ = time_sweep([[spmm32(s, n) for s, n in cells]])
+    ms_one_branch, _ = time_sweep([[spmm32_alone(s, n) for s, n in cells]])
+    # two branches, every launch as the library would choose it alone: neighbours in cost side by side
+    plain_branches = [by_cost[0::2], by_cost[1::2]]
+    ms_two_plain, _ = time_sweep([[spmm32_alone(s, n) for s, n in b] for b in plain_branches])
+    # two branches, and the launches are told that they have a neighbour (IEX_SPMM_BESIDE_GATHER_KERNEL): where the
+    # fp32 matrix-core kernel and the row kernel are close the library then takes the matrix cores, which leaves the
+    # L2 -> CU path to the other branch.  The cells that run on the matrix cores go to one branch, the gather-bound
+    # ones to the other, both longest first: kernels of different units side by side, the reference's co-run premise.
+    hinted_kernel = {c: kernel_of(spmm32(*c)) for c in cells}
+    on_matrix_cores = [c for c in by_cost if "mfma" in hinted_kernel[c]]
+    branches = [on_matrix_cores, [c for c in by_cost if c not in on_matrix_cores]]
+    if not branches[0] or not branches[1]:
+        branches = plain_branches
+    ms_same_serialized, _ = time_sweep([[spmm32(s, n) for s, n in cells]])     # the timed graph's kernels, one after the other
     ms_per_step, wall_ms = time_sweep([[spmm32(s, n) for s, n in b] for b in branches])
     value = sweep_bytes / 1e9 / (ms_per_step * 1e-3)
-    log(f"[bench] {ms_per_step * 1e3:.1f} us per sweep on two branches, {ms_one_branch * 1e3:.1f} us on one "
+    log(f"[bench] {ms_per_step * 1e3:.1f} us per sweep on two branches ({len(branches[0])} cells on the matrix cores beside {len(branches[1])} "
+        f"gather-bound ones), {ms_two_plain * 1e3:.1f} us on two branches with every kernel as chosen alone, {ms_one_branch * 1e3:.1f} us on one "
         f"(host wall {wall_ms / args.steps * 1e3:.1f} us) -> {value:.1f} GB/s")
 
     # ------------------------------------------- per-cell launch durations (HIP events)
@@ -378,6 +403,10 @@ def main():
                                 "L2 -> CU path (every nonzero gathers n * 4 bytes of the dense operand out of L2: gather_TBps, against about 26 TB/s that this path has delivered at best)"
                                 if mats[s].nnz * n * 4 / us / 1e6 >= 15.0 else "launch and ramp-up (the kernel is a few microseconds long)"),
                       "kernel": kernel, "bytes": by})
+        alone_kernel = kernel_of(spmm32_alone(s, n))
+        if alone_kernel != kernel:      # (the library's choice for this cell without a neighbour, and how long that takes alone)
+            table[-1]["kernel_chosen_without_neighbour"] = alone_kernel
+            table[-1]["us_of_that_kernel_alone"] = round(time_cell(spmm32_alone(s, n)), 2)
         log(f"[bench] fp32 s={s} n={n}: {us:.2f} us warm, {cold:.2f} us cold  {by / us / 1e3:.0f} GB/s  {fl / us / 1e3:.0f} GFLOP/s  {kernel}")
 
     by_kernel = {}
@@ -389,21 +418,46 @@ def main():
     measured, measured_commit = read_traffic_profile()
     usable = [measured.get((r["sparsity"], r["n"])) for r in dom_rows]
     traffic_ok = all(u is not None and u[0] == dom_name for u in usable)
-    roofline = {"bound": "hbm", "achieved": round(dom_bytes / dom_us / 1e3, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
-                "frac": round(dom_bytes / dom_us / 1e3 / HBM_PEAK_GBPS, 4),
-                "traffic": round(statistics.mean(u[1] for u in usable)) if traffic_ok else None,
-                "traffic_source": (f"profiles/{os.path.basename(TRAFFIC_PROFILE)}, measured at commit {measured_commit} on the same "
-                                   "kernel instantiation (name compared with what the library reports now)") if traffic_ok else
-                                  "none: the committed counter summary was taken on another kernel than the one the library launches now",
-                "kernel": dom_name, "kernel_name_from": "iex_last_kernels() after an eager call of each cell",
-                "avg_launch_us": round(dom_us, 2),
-                "algorithmic_bytes_per_launch": int(dom_bytes),
-                "cells": [[r["sparsity"], r["n"]] for r in dom_rows],
-                "gather_bytes_per_launch": int(statistics.mean(r["nnz"] * r["n"] * 4 for r in dom_rows)),
-                "gather_TBps": round(statistics.mean(r["nnz"] * r["n"] * 4 for r in dom_rows) / dom_us / 1e6, 2),
-                "note": "every nonzero gathers n*4 bytes of the dense operand from L2 (gather_bytes_per_launch); the "
-                        "kernel is bound by that L2->CU bandwidth (gather_TBps), not by HBM, so frac stays small; "
-                        "traffic = HBM-side bytes per launch from rocprofv3 --pmc FETCH_SIZE + WRITE_SIZE"}
+    traffic = round(statistics.mean(u[1] for u in usable)) if traffic_ok else None
+    traffic_source = (f"profiles/{os.path.basename(TRAFFIC_PROFILE)}, measured at commit {measured_commit} on the same "
+                      "kernel instantiation (name compared with what the library reports now)") if traffic_ok else \
+        "none: the committed counter summary was taken on another kernel than the one the library launches now"
+    common = {"traffic": traffic, "traffic_source": traffic_source, "kernel": dom_name,
+              "kernel_name_from": "iex_last_kernels() after an eager call of each cell, as it runs in the timed graph",
+              "avg_launch_us": round(dom_us, 2), "algorithmic_bytes_per_launch": int(dom_bytes),
+              "cells": [[r["sparsity"], r["n"]] for r in dom_rows],
+              "share_of_the_sweeps_kernel_time": round(sum(r["us"] for r in dom_rows) / sum(r["us"] for r in table), 3)}
+    if "mfma_f32" in dom_name:
+        # the fp32 matrix-core kernel: bound by the matrix / vector ALUs (fp32 MFMAs execute on the vector ALUs), counted
+        # on algorithmic flops (2 * nnz * n); it also multiplies the zeros of the tiles it expands
+        dom_flops = statistics.mean(W.spmm_flops(r["nnz"], r["n"]) for r in dom_rows)
+        dense_flops = statistics.mean(2.0 * mats[r["sparsity"]].m * mats[r["sparsity"]].k * r["n"] for r in dom_rows)
+        roofline = {"bound": "mfma", "achieved": round(dom_flops / dom_us / 1e6, 2), "peak": MFMA_PEAK_TFLOPS_FP32, "unit": "TFLOP/s",
+                    "frac": round(dom_flops / dom_us / 1e6 / MFMA_PEAK_TFLOPS_FP32, 4), **common,
+                    "algorithmic_flops_per_launch": int(dom_flops),
+                    "dense_equivalent_TFLOPs": round(dense_flops / dom_us / 1e6, 1),
+                    "dense_equivalent_frac": round(dense_flops / dom_us / 1e6 / MFMA_PEAK_TFLOPS_FP32, 4),
+                    "hbm_frac": round(dom_bytes / dom_us / 1e3 / HBM_PEAK_GBPS, 4),
+                    "note": "fp32 matrix-core SpMM (v_mfma_f32_32x32x2_f32): achieved = 2 * nnz * n per launch / launch duration "
+                            "against the fp32 MFMA peak; the kernel multiplies whole 32 x 128 tiles of the expanded sparse operand "
+                            "(dense_equivalent_*), and fp32 MFMAs share the vector ALUs with that expansion; traffic = HBM-side bytes "
+                            "per launch from rocprofv3 --pmc FETCH_SIZE + WRITE_SIZE"}
+    else:
+        roofline = {"bound": "hbm", "achieved": round(dom_bytes / dom_us / 1e3, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+                    "frac": round(dom_bytes / dom_us / 1e3 / HBM_PEAK_GBPS, 4), **common,
+                    "gather_bytes_per_launch": int(statistics.mean(r["nnz"] * r["n"] * 4 for r in dom_rows)),
+                    "gather_TBps": round(statistics.mean(r["nnz"] * r["n"] * 4 for r in dom_rows) / dom_us / 1e6, 2),
+                    "note": "every nonzero gathers n*4 bytes of the dense operand from L2 (gather_bytes_per_launch); the "
+                            "kernel is bound by that L2->CU bandwidth (gather_TBps), not by HBM, so frac stays small; "
+                            "traffic = HBM-side bytes per launch from rocprofv3 --pmc FETCH_SIZE + WRITE_SIZE"}
+    # the gather-bound kernel with the largest share, for the record, when the dominant one is the matrix-core kernel
+    gather_rows = max(((k, v) for k, v in by_kernel.items() if "mfma" not in k), key=lambda kv: sum(r["us"] for r in kv[1]), default=None)
+    if gather_rows is not None and gather_rows[0] != dom_name:
+        g_us = statistics.mean(r["us"] for r in gather_rows[1])
+        g_by = statistics.mean(r["bytes"] for r in gather_rows[1])
+        roofline["largest_gather_kernel"] = {"kernel": gather_rows[0], "cells": [[r["sparsity"], r["n"]] for r in gather_rows[1]],
+                                             "avg_launch_us": round(g_us, 2), "hbm_frac": round(g_by / g_us / 1e3 / HBM_PEAK_GBPS, 4),
+                                             "gather_TBps": round(statistics.mean(r["nnz"] * r["n"] * 4 for r in gather_rows[1]) / g_us / 1e6, 2)}
 
     cold_sweep_us = sum(r["cold_us"] for r in table)
     result = {
@@ -412,11 +466,16 @@ def main():
         "ms_per_step": round(ms_per_step, 5), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "f32", "data": "synthetic",
         "config": {"workload": "config 2: fp32 CSR SpMM sweep, A 4096x4096 at {70,80,90,95,98}% sparsity (geometric "
-                               "row lengths), B 4096x{64,128,256}; one step = the 15 launches in one hipGraph (two parallel branches)",
+                               "row lengths), B 4096x{64,128,256}; one step = the 15 launches in one hipGraph on two parallel branches (matrix-core cells beside gather-bound cells)",
                    "value_is": "algorithmic bytes of the sweep / time per sweep",
                    "pct_hbm_peak": round(100 * value / HBM_PEAK_GBPS, 2), "cache": "warm (operands stay in L2 / MALL between steps)",
                    "graph": "two parallel branches: " + " | ".join(", ".join(f"{s}/{n}" for s, n in b) for b in branches),
                    "one_branch_sweep_us": round(ms_one_branch * 1e3, 1),
+                   "two_branches_every_kernel_as_chosen_alone_us": round(ms_two_plain * 1e3, 1),
+                   "same_kernels_on_one_branch_us": round(ms_same_serialized * 1e3, 1),
+                   "corun_makespan_pct_of_the_same_kernels_serialized": round(100 * ms_per_step / ms_same_serialized, 1),
+                   "corun_makespan_pct_of_the_sweep_as_chosen_alone_serialized": round(100 * ms_per_step / ms_one_branch, 1),
+                   "kernels_in_the_timed_graph": {f"{s}/{n}": hinted_kernel[(s, n)].split(" (")[0] for s, n in cells},
                    "cold_cache_sweep_us": round(cold_sweep_us, 1),
                    "cold_cache_GBps": round(sweep_bytes / cold_sweep_us / 1e3, 1),
                    "cold_cache_protocol": "per cell: 512 MB written, then one eager launch between two events; sum of the 15 medians of 7"},

@@ -105,6 +105,14 @@ int iex_copy_bytes(void* dst, const void* src, size_t nbytes, void* stream);
  * The drop-ins iex_CudaSpmm2 / 3 / 5 below always set it: they know nothing about where their arrays come from.
  * Ignored when bits 16..19 force a family.                                                             */
 #define IEX_SPMM_ANY_COLUMN_ORDER 0x20
+/* The launch will share the chip with a launch that is bound by gathers from L2 (the row kernel on a parallel branch
+ * of a graph or on another stream).  Where the fp32 matrix-core kernel (family 5) and the row kernel are close for this
+ * product (fp32, int32 indices, density from 19.5 %, n a multiple of 4 from 128 up; alone the matrix-core kernel is 5-7 %
+ * slower there and the library would not take it) the call then runs on the matrix cores and leaves the L2 -> CU path to
+ * its neighbour: the config-2 sweep on two branches 654 -> 600 us on MI355X.  The reference pairs kernels of different
+ * units by hand (tests/test_interleaving.py:434-476); this is the same choice, made by the callee.  Ignored when bits
+ * 16..19 force a family, with IEX_SPMM_ANY_COLUMN_ORDER, and for every other element type.                      */
+#define IEX_SPMM_BESIDE_GATHER_KERNEL 0x40
 /* bits 8..15: force waves-per-row (1, 4 or 8); 0 = choose from nnz/m.  For tuning.    */
 #define IEX_SPMM_FORCE_WPR(w) (((w) & 0xff) << 8)
 /* bits 16..19: force the kernel family: 1 = row kernel gathering from L2, 2 = LDS-staged

@@ -19,6 +19,7 @@ SPMM_ACCUMULATE = 0x2
 SPMM_RELU = 0x4
 SPMM_TABLES_READY = 0x8
 SPMM_LISTS_READY = 0x10
+SPMM_BESIDE_GATHER_KERNEL = 0x40
 SPMM_ANY_COLUMN_ORDER = 0x20
 SDDMM_SUM_OVER_BATCH = 0x1
 SDDMM_ACCUMULATE = 0x2

@@ -395,6 +395,7 @@ struct Choice {
   size_t ws_bytes = 0;
   bool any_order = false;   // columns of a row in any order, possibly repeated: families 1 and 8 only
   const int* hist = nullptr;   // host: rows with more than 64 << j nonzeros, j = 0 .. 15 (iex_spmm_sched), may be null
+  bool beside_gather = false;  // the launch shares the chip with a gather-bound one (IEX_SPMM_BESIDE_GATHER_KERNEL)
 };
 
 // The LDS-staged kernel needs a full-width tile (64 lanes x VEC, VEC the full or half 128-bit
@@ -503,6 +504,10 @@ int mfma_f32_variant(const SpmmParams& p, int batch, const Choice& ch, int& wind
   // for small outputs stay on request: at 30 % and n = 128 they only tie (0.096 vs 0.100 ms).
   const double fill = (double)p.n / ((double)ceil_div(p.n, 128) * 128);  // share of the computed columns that exist
   if (density >= 0.27 && arrangement == 4 && fill >= 0.75) return arrangement;
+  // Beside a kernel that is bound by gathers the tie at 20 % goes to the matrix cores, also with the 16-row tiles of
+  // n = 128: alone 124 against 118 us (4096 x 4096 at 20 %, n = 256) and 90 against 84 us (30 %, n = 128), but the
+  // neighbour then has the L2 -> CU path to itself (the 15 cells of that sweep on two branches of a graph: 654 -> 600 us).
+  if (ch.beside_gather && density >= 0.195 && p.n >= 128 && fill >= 0.75) return arrangement;
   return 0;
 }
 
@@ -695,6 +700,7 @@ int spmm_dispatch(int dtype, int itype, int flags, int m, int k, int n, int nonz
   ch.ws = workspace;
   ch.ws_bytes = workspace ? workspace_bytes : 0;
   ch.any_order = (flags & IEX_SPMM_ANY_COLUMN_ORDER) != 0;
+  ch.beside_gather = (flags & IEX_SPMM_BESIDE_GATHER_KERNEL) != 0 && !ch.any_order;
   SpmmParams p{m, k, n, nonzeros, row_indices, values, row_offsets, column_indices, dense, bias, out,
                (flags & IEX_SPMM_PER_BATCH_VALUES) != 0, (flags & IEX_SPMM_ACCUMULATE) != 0,
                (flags & IEX_SPMM_RELU) != 0};

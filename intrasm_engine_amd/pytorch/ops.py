@@ -41,7 +41,8 @@ _SPMM_KEYS = ("force_wpr", "force_variant", "force_rpw", "force_nt", "force_lpg"
 def kernel_params(*, spmm: dict | None = None, sddmm: dict | None = None, gemm: dict | None = None):
     """Kernel choices for the operators called inside the block (this thread only), for tuning:
     ``spmm`` = any of force_variant / force_rpw / force_nt / force_lpg / force_wpr (the tuning
-    bits of ``iex_spmm_ex``), ``sddmm`` = force_wpr / force_variant, ``gemm`` = tile (the shape code of
+    bits of ``iex_spmm_ex``) and beside_gather_kernel (true: the calls will share the chip with a gather-bound launch,
+    ``IEX_SPMM_BESIDE_GATHER_KERNEL``), ``sddmm`` = force_wpr / force_variant, ``gemm`` = tile (the shape code of
     ``iex_gemm``: 5 = 128x128, 6 = 128x256, 7 = 256x256 tiles, 8 = 128x128 and 9 = 64x128 by eight waves with K steps of 64, 10 = 128x256 by eight waves, 12 = 256x256 with K split over two workgroups per tile, 13 = 256x256 by eight waves in alternating phases; 1..4 = the
     register-staged kernels).
     Without a block, or for a key left out, the library chooses; a category left out (None) keeps
@@ -49,7 +50,7 @@ def kernel_params(*, spmm: dict | None = None, sddmm: dict | None = None, gemm: 
     take the operands at hand (a matrix-core family for an n that is not a multiple of 8, say)
     falls back to a gather kernel, as the C entry points document: results stay correct, the
     timing is then that of the fallback."""
-    for name, given, known in (("spmm", spmm, _SPMM_KEYS), ("sddmm", sddmm, ("force_wpr", "force_variant")), ("gemm", gemm, ("tile",))):
+    for name, given, known in (("spmm", spmm, _SPMM_KEYS + ("beside_gather_kernel",)), ("sddmm", sddmm, ("force_wpr", "force_variant")), ("gemm", gemm, ("tile",))):
         unknown = set(given or {}) - set(known)
         if unknown:
             raise TypeError(f"unknown {name} kernel parameters: {sorted(unknown)}")
@@ -274,6 +275,7 @@ def _spmm(b, row_indices, values, row_offsets, column_indices, m, *, per_batch_v
     tuned = getattr(_TUNING, "spmm", None)
     if tuned and not (force_wpr or force_variant or force_rpw or force_nt or force_lpg):
         force_wpr, force_variant, force_rpw, force_nt, force_lpg = (tuned.get(key, 0) for key in _SPMM_KEYS)
+    beside_gather = bool(tuned and tuned.get("beside_gather_kernel"))
     if plan is not None and plan.variant and not force_variant:
         # settled by SddmmPlan.analyze(): the dense-blocks kernel for masks with structure (it still has to fit dtype and
         # shape: checked below), else the row kernel
@@ -325,6 +327,7 @@ def _spmm(b, row_indices, values, row_offsets, column_indices, m, *, per_batch_v
                     _DT[b.dtype], _IT[column_indices.dtype], _lib.SPMM_PER_BATCH_VALUES | (10 << 16), m, k, n, nonzeros, batch) != 10:
                 force_variant = 0      # (the kernel does not serve this call: another n, int16 indices)
     flags = (_lib.SPMM_PER_BATCH_VALUES if per_batch_values else 0) | (_lib.SPMM_ANY_COLUMN_ORDER if any_order else 0) | \
+            (_lib.SPMM_BESIDE_GATHER_KERNEL if beside_gather else 0) | \
             (_lib.SPMM_ACCUMULATE if accumulate else 0) | (_lib.SPMM_RELU if relu else 0) | \
             ((int(force_wpr) & 0xff) << 8) | ((int(force_variant) & 0xf) << 16) | ((int(force_rpw) & 0xf) << 20) | \
             ((int(force_nt) & 0xf) << 24) | ({0: 0, 8: 1, 16: 2, 32: 3, 64: 4}[int(force_lpg)] << 28)

@@ -59,6 +59,9 @@ SPMM_KERNELS: dict[str, dict] = {
     "rows_by_length": {"force_variant": 11},
     "rows_by_length_1chunk": {"force_variant": 11, "force_rpw": 1},
     "rows_by_length_4chunks": {"force_variant": 11, "force_rpw": 3},
+    # the library's choice for a launch that shares the chip with a gather-bound launch (a parallel branch of a graph):
+    # fp32 products that are a tie between the row kernel and the matrix cores then take the matrix cores
+    "auto_beside_gather_kernel": {"beside_gather_kernel": True},
 }
 
 
@@ -77,7 +80,7 @@ def spmm_kernel_choices(dtype: torch.dtype, n: int, k: int | None = None, m: int
         if k is not None and m is not None and k % 8 == 0 and m % 8 == 0:
             names.append("dense_form_gemm")
     if dtype == torch.float32 and n % 4 == 0:
-        names += [k for k in SPMM_KERNELS if k.startswith("mfma32_")]
+        names += [k for k in SPMM_KERNELS if k.startswith("mfma32_")] + ["auto_beside_gather_kernel"]
     if n % vec == 0:
         names += [k for k in SPMM_KERNELS if k.startswith("rows_by_length")]    # (full 128-bit vectors; the backward product has the same n)
     return names

@@ -165,11 +165,14 @@ def _set_note(row_offsets, column_indices, k, status, hist, share=None):
                                            None)
 
 
-def mark_canonical(row_offsets, column_indices, k):
+def mark_canonical(row_offsets, column_indices, k, measure=True):
     """Record that ``(row_offsets, column_indices)`` is canonical CSR with ``k`` columns (what ``dense_to_sparse`` and
     ``transpose_info`` build), so that the operators need not look: see :func:`_pattern_note`.  Set-up code: reads the
-    pattern's row-length histogram back (a synchronisation)."""
-    on_device = row_offsets.is_cuda and row_offsets.numel() > 1
+    pattern's row-length histogram and the share of its nonzeros in dense blocks back (two small kernels, two
+    synchronising reads).  ``measure=False`` skips that -- no kernel, no synchronisation, allowed under stream capture:
+    for patterns that change from call to call (a mask made on the device every step) and are canonical by
+    construction; the library's rules then go by the shape and the density alone."""
+    on_device = measure and row_offsets.is_cuda and row_offsets.numel() > 1
     _set_note(row_offsets, column_indices, k, 0, _row_histogram_host(row_offsets) if on_device else None,
               _dense_share_host(row_offsets, column_indices, k) if on_device else None)
     return column_indices

@@ -192,6 +192,36 @@ def test_an_unseen_pattern_under_capture_keeps_to_the_any_order_kernels(oracle, 
     assert_close(keep[0].cpu().numpy(), want, scale, 1e-5, "captured, unseen shuffled pattern")
 
 
+def test_a_pattern_made_under_capture_can_be_vouched_for(oracle, dev):
+    """A mask that changes from step to step is made on the device inside the captured region; nobody can look at it
+    there.  A caller whose construction guarantees canonical CSR says so with mark_canonical(..., measure=False), which
+    launches nothing and reads nothing back: the call then takes the kernel families for canonical CSR (here: the fp32
+    matrix cores, which the any-order path never takes)."""
+    from intrasm_engine_amd import _lib, interleaving as IL
+    from intrasm_engine_amd.pytorch import ops as pyops
+    c = W.config2_matrix(0.70)
+    rng = np.random.default_rng(10)
+    b_np = rng.standard_normal((1, c.k, 256)).astype(np.float32)
+    bt = torch.from_numpy(b_np).to(dev)
+    ri, v, ro, src = (torch.from_numpy(x).to(dev) for x in (c.row_indices, c.values, c.row_offsets, c.column_indices))
+    trail = []
+
+    def step():
+        ci = src.clone()                                    # (stands for: the mask of this step, computed on the device)
+        pyops.mark_canonical(ro, ci, c.k, measure=False)
+        out = ops.spmm_sputnik_reuse_weight(bt, ri, v, ro, ci, c.m)
+        trail.append(_lib.last_kernels())
+        return out
+    constructor, keep = IL.capture_serialized([step])
+    constructor.instantiate_graph_exec()
+    constructor.execute_graph()
+    constructor.synchronize()
+    constructor.destroy_graph_exec()
+    assert "spmm_mfma_f32_kernel" in trail[0], trail
+    want, scale = _spmm_want(oracle, c, b_np, torch.float32)
+    assert_close(keep[0].cpu().numpy(), want, scale, 1e-5, "captured, pattern vouched for")
+
+
 def test_sparse_attention_under_inference_mode(dev):
     """Tensors made under torch.inference_mode() keep no version counter; the plan's key must not ask for one."""
     from intrasm_engine_amd.pytorch.sparse_attention import sparse_attention

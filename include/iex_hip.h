@@ -77,10 +77,11 @@ int iex_csr_row_histogram(int m, const int* row_offsets, int* histogram, void* s
  * SpMM family 10) put such blocks on the matrix cores and count a block as dense from 1536 nonzeros; they pay off when
  * about half of the nonzeros or more sit in such blocks (bands, windows, block diagonals), whatever the overall
  * density -- which is all that the 0 = choose rule of those entry points can see.  A caller reads the figure back
- * once per pattern, as set-up, and forces the variant.  k <= 65536; the pattern must pass iex_csr_check's offset test.
- * No counterpart in the reference. */
-int iex_csr_dense_share(int itype, int m, int k, const int* row_offsets, const void* column_indices, int dense_min,
-                        int* dense_nonzeros, void* stream);
+ * once per pattern, as set-up, and forces the variant.  k <= 65536.  Offsets that point outside the arrays are cut to
+ * [0, nonzeros] and columns outside [0, k) are counted nowhere, so the kernel may be launched together with
+ * iex_csr_check and the two results read back at once.  No counterpart in the reference. */
+int iex_csr_dense_share(int itype, int m, int k, int nonzeros, const int* row_offsets, const void* column_indices,
+                        int dense_min, int* dense_nonzeros, void* stream);
 
 /* dst[0:nbytes] = src[0:nbytes] with a plain 128-bit-per-lane streaming kernel (nbytes and both
  * pointers multiples of 16).  Measurement aid with no counterpart in the reference: hardware

@@ -95,7 +95,7 @@ __global__ __launch_bounds__(256) void csr_row_histogram_kernel(int m, const int
 constexpr int kShareMaxTiles = 512;   // k <= 65536
 constexpr int kShareThreads = 1024;
 template <typename IT>
-__global__ __launch_bounds__(kShareThreads) void csr_dense_share_kernel(int m, int k, const int* __restrict__ row_offsets, const IT* __restrict__ cols,
+__global__ __launch_bounds__(kShareThreads) void csr_dense_share_kernel(int m, int k, int nnz, const int* __restrict__ row_offsets, const IT* __restrict__ cols,
                                                                         int dense_min, int* dense_nonzeros) {
   __shared__ int count[kShareMaxTiles];
   __shared__ int total;
@@ -105,7 +105,8 @@ __global__ __launch_bounds__(kShareThreads) void csr_dense_share_kernel(int m, i
   __syncthreads();
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   for (int r = blockIdx.x * 128 + wave; r < min(m, blockIdx.x * 128 + 128); r += kShareThreads / 64) {
-    const int s = row_offsets[r], e = row_offsets[r + 1];
+    // (offsets that point outside the arrays are cut to them: the kernel may run before anybody has checked the pattern)
+    const int s = min(max(row_offsets[r], 0), nnz), e = min(max(row_offsets[r + 1], s), nnz);
     for (int base = s; base < e; base += 64) {
       const int j = base + lane;
       int t = -1;   // (no nonzero here, or a column outside the matrix: counted nowhere)
@@ -133,18 +134,18 @@ __global__ __launch_bounds__(kShareThreads) void csr_dense_share_kernel(int m, i
 
 extern "C" {
 
-int iex_csr_dense_share(int itype, int m, int k, const int* row_offsets, const void* column_indices, int dense_min, int* dense_nonzeros,
-                        void* stream) {
-  IEX_REQUIRE(m >= 0 && k >= 0 && dense_min >= 0, IEX_ERR_BAD_ARGUMENT, "csr_dense_share: negative argument");
+int iex_csr_dense_share(int itype, int m, int k, int nonzeros, const int* row_offsets, const void* column_indices, int dense_min,
+                        int* dense_nonzeros, void* stream) {
+  IEX_REQUIRE(m >= 0 && k >= 0 && nonzeros >= 0 && dense_min >= 0, IEX_ERR_BAD_ARGUMENT, "csr_dense_share: negative argument");
   IEX_REQUIRE(dense_nonzeros && (m == 0 || (row_offsets && column_indices)), IEX_ERR_BAD_ARGUMENT, "csr_dense_share: null pointer argument");
   IEX_REQUIRE(itype == IEX_I32 || itype == IEX_I16, IEX_ERR_UNSUPPORTED, "csr_dense_share: column indices must be int32 or int16");
   IEX_REQUIRE(k <= 128 * kShareMaxTiles, IEX_ERR_TOO_LARGE, "csr_dense_share: more than %d columns", 128 * kShareMaxTiles);
-  if (m == 0 || k == 0) return 0;
+  if (m == 0 || k == 0 || nonzeros == 0) return 0;
   hipStream_t s = static_cast<hipStream_t>(stream);
   if (itype == IEX_I32)
-    hipLaunchKernelGGL(csr_dense_share_kernel<int>, dim3((m + 127) / 128), dim3(kShareThreads), 0, s, m, k, row_offsets, static_cast<const int*>(column_indices), dense_min, dense_nonzeros);
+    hipLaunchKernelGGL(csr_dense_share_kernel<int>, dim3((m + 127) / 128), dim3(kShareThreads), 0, s, m, k, nonzeros, row_offsets, static_cast<const int*>(column_indices), dense_min, dense_nonzeros);
   else
-    hipLaunchKernelGGL(csr_dense_share_kernel<short>, dim3((m + 127) / 128), dim3(kShareThreads), 0, s, m, k, row_offsets, static_cast<const short*>(column_indices), dense_min, dense_nonzeros);
+    hipLaunchKernelGGL(csr_dense_share_kernel<short>, dim3((m + 127) / 128), dim3(kShareThreads), 0, s, m, k, nonzeros, row_offsets, static_cast<const short*>(column_indices), dense_min, dense_nonzeros);
   return iex::check_hip(hipGetLastError(), "csr_dense_share launch");
 }
 

@@ -134,7 +134,7 @@ def _dense_share_host(row_offsets, column_indices, k, dense_min=None):
     dense_min = _STRUCTURE_BLOCK_NONZEROS if dense_min is None else dense_min
     count = torch.zeros(1, dtype=torch.int32, device=row_offsets.device)
     with torch.cuda.device(row_offsets.device):
-        rc = _lib.load().iex_csr_dense_share(1 if column_indices.dtype == torch.int16 else 0, row_offsets.numel() - 1, int(k),
+        rc = _lib.load().iex_csr_dense_share(1 if column_indices.dtype == torch.int16 else 0, row_offsets.numel() - 1, int(k), nonzeros,
                                              row_offsets.data_ptr(), column_indices.data_ptr(), int(dense_min), count.data_ptr(),
                                              _stream_ptr(row_offsets.device))
     _lib.check(rc, "csr_dense_share")
@@ -172,9 +172,10 @@ def mark_canonical(row_offsets, column_indices, k, measure=True):
     synchronising reads).  ``measure=False`` skips that -- no kernel, no synchronisation, allowed under stream capture:
     for patterns that change from call to call (a mask made on the device every step) and are canonical by
     construction; the library's rules then go by the shape and the density alone."""
-    on_device = measure and row_offsets.is_cuda and row_offsets.numel() > 1
-    _set_note(row_offsets, column_indices, k, 0, _row_histogram_host(row_offsets) if on_device else None,
-              _dense_share_host(row_offsets, column_indices, k) if on_device else None)
+    hist = share = None
+    if measure and row_offsets.is_cuda and row_offsets.numel() > 1:
+        _, hist, share = _look(row_offsets, column_indices, k)      # (the check runs along: one launch more, no read more)
+    _set_note(row_offsets, column_indices, k, 0, hist, share)
     return column_indices
 
 
@@ -194,12 +195,40 @@ def _pattern_note(row_offsets, column_indices, k):
         return note[4], note[5]
     if torch.cuda.is_current_stream_capturing():
         return None, None
-    status = csr_check(row_offsets, column_indices, k)
-    sound = not (status & _lib.CSR_BAD_OFFSETS)
-    hist = _row_histogram_host(row_offsets) if sound else None
-    share = _dense_share_host(row_offsets, column_indices, k) if sound and row_offsets.numel() > 1 else None
+    status, hist, share = _look(row_offsets, column_indices, k)
     _set_note(row_offsets, column_indices, k, status, hist, share)
     return status, hist
+
+
+def _look(row_offsets, column_indices, k):
+    """One look at a pattern: ``iex_csr_check``, ``iex_csr_row_histogram`` and ``iex_csr_dense_share`` launched one after
+    the other into one small buffer and read back at once (one synchronisation).  Histogram and share are None for a
+    pattern whose offsets are unsound (the kernels cut such offsets to the arrays, so launching them is safe)."""
+    for name, t in (("row_offsets", row_offsets), ("column_indices", column_indices)):
+        _chk(t.is_cuda, f"{name} must be a CUDA tensor")
+        _chk(t.is_contiguous(), f"{name} must be a contiguous tensor")
+    _chk(row_offsets.dtype == torch.int32, "row_offsets must be int32")
+    _chk(column_indices.dtype in (torch.int32, torch.int16), "column_indices must be int32 or int16")
+    _chk(row_offsets.device == column_indices.device, "row_offsets should be in the same device as column_indices")
+    _chk(row_offsets.numel() >= 1, "row_offsets must have m + 1 entries")
+    m, nonzeros = row_offsets.numel() - 1, column_indices.numel()
+    itype = 1 if column_indices.dtype == torch.int16 else 0
+    buf = torch.zeros(18, dtype=torch.int32, device=row_offsets.device)      # status | 16 counts | nonzeros in dense blocks
+    lib = _lib.load()
+    with_share = nonzeros > 0 and int(k) <= 65536 and m > 0
+    with torch.cuda.device(row_offsets.device):
+        stream = _stream_ptr(row_offsets.device)
+        _lib.check(lib.iex_csr_check(itype, m, int(k), nonzeros, row_offsets.data_ptr(), column_indices.data_ptr(), buf.data_ptr(), stream), "csr_check")
+        if m > 0:
+            _lib.check(lib.iex_csr_row_histogram(m, row_offsets.data_ptr(), buf.data_ptr() + 4, stream), "csr_row_histogram")
+        if with_share:
+            _lib.check(lib.iex_csr_dense_share(itype, m, int(k), nonzeros, row_offsets.data_ptr(), column_indices.data_ptr(),
+                                               _STRUCTURE_BLOCK_NONZEROS, buf.data_ptr() + 68, stream), "csr_dense_share")
+    got = buf.tolist()
+    status = int(got[0])
+    if status & _lib.CSR_BAD_OFFSETS:
+        return status, None, None
+    return status, tuple(int(x) for x in got[1:17]), (got[17] / nonzeros if with_share else None)
 
 
 def _csr_status(row_offsets, column_indices, k):

@@ -648,17 +648,25 @@ def run_extras(torch, ops, dev, W, IL, mats, dens, csr_dev, time_cell, time_cold
     out = {}
     # ---- fp16 sweep (int16 column indices, the reference's half layout)
     rows = []
+    calls16 = {}
     for s in W.C2_SPARSITIES:
         c = mats[s]
         ri, v, ro, ci = csr_dev(c, torch.float16, torch.int16)
         for n in W.C2_NS:
             b = torch.from_numpy(dens[n]).to(dev).half()
+            calls16[(s, n)] = (lambda b=b, ri=ri, v=v, ro=ro, ci=ci, m=c.m: ops.spmm_sputnik_reuse_weight_half(b, ri, v, ro, ci, m))
             us = time_cell(lambda: ops.spmm_sputnik_reuse_weight_half(b, ri, v, ro, ci, c.m))
             by = W.spmm_bytes(c.m, c.k, n, c.nnz, 1, 2, 2)
             fl = W.spmm_flops(c.nnz, n)
             rows.append({"sparsity": s, "n": n, "us": round(us, 2), "GBps": round(by / us / 1e3, 1),
                          "hbm_frac": round(by / us / 1e3 / HBM_PEAK_GBPS, 4), "GFLOPs": round(fl / us / 1e3, 1)})
     out["cells_fp16_i16"] = rows
+    # the same 15 launches as one graph: on one branch, and on two (cells in order of nnz * n dealt alternately)
+    order16 = sorted(calls16, key=lambda c: -mats[c[0]].nnz * c[1])
+    out["sweep_fp16_i16"] = {
+        "one_branch_us": round(IL.run_non_interleaving([calls16[c] for c in calls16]) * 1e3, 1),
+        "two_branches_us": round(IL.run_interleaving([calls16[c] for c in order16[0::2]], [calls16[c] for c in order16[1::2]]) * 1e3, 1),
+        "sum_of_cells_us": round(sum(r["us"] for r in rows), 1)}
     log("[bench] fp16 sweep done")
 
     # ---- SDDMM: config 1 (fp32, batch-summed) and config 3 (fp16, 16 heads, per-head output)

@@ -52,6 +52,30 @@ __global__ __launch_bounds__(WAVES * 64, 1) void k(const unsigned char* __restri
   __syncthreads();
   if (iters < 0) out[tid] = *reinterpret_cast<unsigned*>(smem + tid * 4);
 }
+// The other way to feed A: every wavefront loads its operand fragments straight into registers in the MFMA layout (lane
+// = row lane & 31 of a 32-row fragment, 16 bytes = 8 k values at k offset (lane >> 5) * 8), four fragments of 32 rows and
+// two 16-k sub-steps per K step of 32, as a 128 x 64 register tile needs.  The four wavefronts that share a row panel
+// (wn = 0 .. 3) load the same bytes.  Plain loads, results folded into a checksum so that they are not dropped.
+__global__ __launch_bounds__(512, 1) void frag_kernel(const unsigned char* __restrict__ ga, unsigned* out, int iters, long long S, int wrap) {
+  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+  const int local = blockIdx.x / 8, xcd = blockIdx.x % 8;
+  const unsigned char* A = ga + ((size_t)xcd * 4 + local / 8) * (256 * S);   // a panel of 256 rows, shared by 8 CUs of the XCD
+  const int wm = wave / 4;                                                    // rows 128 wm .. + 127
+  uint4 sum = {0u, 0u, 0u, 0u};
+  int k = 0;
+  for (int it = 0; it < iters; ++it) {
+#pragma unroll
+    for (int s = 0; s < 2; ++s)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const uint4 v = *reinterpret_cast<const uint4*>(A + (size_t)(wm * 128 + i * 32 + (lane & 31)) * S + k + s * 32 + (lane >> 5) * 16);
+        sum.x ^= v.x; sum.y += v.y; sum.z ^= v.z; sum.w += v.w;
+      }
+    k += 64; if (k >= wrap) k = 0;
+  }
+  if ((sum.x ^ sum.y ^ sum.z ^ sum.w) == 0x12345678u) out[tid] = sum.x;   // (never true for the fill pattern: keeps the loads)
+}
+
 int main() {
   unsigned char *ga, *gb; unsigned* out;
   const size_t abytes = (size_t)768 << 20, bbytes = (size_t)1536 << 20;
@@ -75,6 +99,20 @@ int main() {
     printf("%-58s stride %6lld: %7.3f ms  %5.1f B/clk/CU (2.4 GHz)\n", name, p.S, ms, bytes / (ms * 1e-3 * 2.4e9)); fflush(stdout);
     if (hipGetLastError() != hipSuccess) { printf("error\n"); exit(1); }
   };
+  for (long long S : {16384ll, 8192ll, 22016ll}) {
+    if ((size_t)32 * 256 * S > abytes) continue;
+    hipEvent_t a, b; hipEventCreate(&a); hipEventCreate(&b);
+    hipLaunchKernelGGL(frag_kernel, dim3(256), dim3(512), 0, 0, ga, out, 300, S, 2048);
+    hipEventRecord(a);
+    hipLaunchKernelGGL(frag_kernel, dim3(256), dim3(512), 0, 0, ga, out, iters, S, 2048);
+    hipEventRecord(b); hipEventSynchronize(b);
+    float ms; hipEventElapsedTime(&ms, a, b);
+    // per K step of 32 and CU: 8 wavefronts x 4 fragments x 2 sub-steps x 1 KB = 64 KB into registers (16 KB distinct)
+    printf("%-58s stride %6lld: %7.3f ms  %5.1f B/clk/CU into registers (2.4 GHz), %5.0f clk per K step of 32\n",
+           "A fragments straight into registers (128 x 64 tiles)", S, ms, (double)iters * 65536.0 / (ms * 1e-3 * 2.4e9), ms * 1e-3 * 2.4e9 / iters);
+    fflush(stdout);
+    if (hipGetLastError() != hipSuccess) { printf("error\n"); return 1; }
+  }
   for (long long S : {16384ll, 16384ll + 128, 16384ll + 512, 8192ll, 22016ll}) {
     run("A 64 B/row (16 rows per instruction)", Pat{64, 2048, 0, 256, S, 0, 0, 0});
     run("A 128 B/row (8 rows per instruction)", Pat{128, 2048, 0, 256, S, 0, 0, 0});

@@ -111,6 +111,7 @@ int main(int argc, char** argv) {
   RUNC("pp: B through registers, A direct", timeit(ppx_kernel<false, 4, 2, 4, 32, 4, 0, 256>, p, 256, 256, 512, L));
   RUNC("pp: A through registers, B direct", timeit(ppx_kernel<false, 4, 2, 4, 32, 4, 0, 512>, p, 256, 256, 512, L));
   RUNC("pp: A and B through registers", timeit(ppx_kernel<false, 4, 2, 4, 32, 4, 0, 768>, p, 256, 256, 512, L));
+  RUNC("pp: K steps of 64, two stages of 64 KB", timeit(ppx_kernel<false, 4, 2, 4, 64, 2, 0, 0>, p, 256, 256, 512, gemm_dma_lds_bytes<4, 2, 4, 64, 2>()));
   RUNC("pp, A in 64-k stages (3) + B 32-k (4)", timeit(pp_kernel<false, 4, 2, 4>, p, 256, 256, 512, gemm_pp_lds_bytes<true, false, 4, 2, 4>()));
   }
   return 0;

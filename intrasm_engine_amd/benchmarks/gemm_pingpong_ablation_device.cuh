@@ -66,7 +66,7 @@ __device__ __forceinline__ void gemm_tile_ppx(const GemmParams& p, int tile_m, i
                 "every wavefront fetches whole kilobytes of A and of B");
   static_assert(LOADS % PPT == 0, "the loads of a tile are spread evenly over its phases");
   static_assert(TRANS_B || (CPRB >= 16 && CPRB <= 64), "(K,N) layout: 128 <= BN <= 512");
-  static_assert(STAGES >= 3 && (STAGES - 1) * LOADS < 64, "stages in flight must fit the load counter");
+  static_assert(STAGES >= 2 && (STAGES - 1) * LOADS < 64, "stages in flight must fit the load counter");
   typedef unsigned short u16;
   typedef __attribute__((address_space(3))) unsigned char lds_u8;
 

@@ -6,8 +6,13 @@
 A *step* is one pass of the hot path over the configuration the metric is quoted on:
 the fp32 CSR SpMM sweep of config 2 (4096x4096 sparse A at 70/80/90/95/98 % sparsity with
 geometric row lengths, times a dense 4096 x {64,128,256} B) = 15 SpMM launches, captured
-once into a hipGraph through the graph builder and replayed.  All operands are resident
-in HBM before the timed region; CSR construction is set-up work and is not timed.
+once into a hipGraph through the graph builder and replayed.  The launches are independent
+of each other and the graph holds them on two parallel branches: each launch is told that
+it has a neighbour, the cells that then run on the fp32 matrix cores form one branch and the
+gather-bound cells the other.  The same launches on one branch, and on two branches with
+every kernel as the library chooses it alone, are timed beside the step and reported in
+``config``.  All operands are resident in HBM before the timed region; CSR construction is
+set-up work and is not timed.
 
 One JSON line is printed.  ``value`` = algorithmic GB of one sweep / seconds per sweep.
 ``roofline`` describes the SpMM kernel instantiation that takes the most time in the

@@ -107,19 +107,28 @@ __global__ __launch_bounds__(kShareThreads) void csr_dense_share_kernel(int m, i
   for (int r = blockIdx.x * 128 + wave; r < min(m, blockIdx.x * 128 + 128); r += kShareThreads / 64) {
     // (offsets that point outside the arrays are cut to them: the kernel may run before anybody has checked the pattern)
     const int s = min(max(row_offsets[r], 0), nnz), e = min(max(row_offsets[r + 1], s), nnz);
-    for (int base = s; base < e; base += 64) {
-      const int j = base + lane;
-      int t = -1;   // (no nonzero here, or a column outside the matrix: counted nowhere)
-      if (j < e) {
-        const int c = (int)cols[j];
-        if (c >= 0 && c < k) t = c >> 7;
+    for (int base = s; base < e; base += 256) {   // four loads in flight per lane, then counted 64 nonzeros at a time
+      int t4[4];
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        const int j = base + u * 64 + lane;
+        t4[u] = -1;   // (no nonzero here, or a column outside the matrix: counted nowhere)
+        if (j < e) {
+          const int c = (int)cols[j];
+          if (c >= 0 && c < k) t4[u] = c >> 7;
+        }
       }
-      const int before = __shfl_up(t, 1, 64);
-      const unsigned long long heads = __ballot(lane == 0 || t != before);
-      if ((heads >> lane) & 1ull) {
-        const unsigned long long later = lane == 63 ? 0ull : heads >> (lane + 1);
-        const int run = later ? __builtin_ctzll(later) + 1 : 64 - lane;
-        if (t >= 0) atomicAdd(&count[t], run);
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        if (base + u * 64 >= e) break;   // (uniform)
+        const int t = t4[u];
+        const int before = __shfl_up(t, 1, 64);
+        const unsigned long long heads = __ballot(lane == 0 || t != before);
+        if ((heads >> lane) & 1ull) {
+          const unsigned long long later = lane == 63 ? 0ull : heads >> (lane + 1);
+          const int run = later ? __builtin_ctzll(later) + 1 : 64 - lane;
+          if (t >= 0) atomicAdd(&count[t], run);
+        }
       }
     }
   }

@@ -114,14 +114,14 @@ __global__ void fill_zero_kernel(int* p, int n) {
   if (i < n) p[i] = 0;
 }
 
-template <bool BF16, bool TRANS_B>
-__global__ __launch_bounds__(256, 1) void gemm_dma_splitk_kernel(GemmParams p) {
+template <bool BF16, bool TRANS_B, int WM, int WN, int WCN, int BK, int STAGES>
+__global__ __launch_bounds__(WCN * 128, 1) void gemm_dma_splitk_kernel(GemmParams p) {
   extern __shared__ __align__(16) unsigned char smem[];
   const int b = blockIdx.x;
   const int part = (b >> 3) & 1, slot = (b >> 4) * kXcds + (b & 7);
   int tile_m, tile_n;
   if (!xcd_tile(slot, p.tiles_m, p.tiles_n, tile_m, tile_n)) return;  // uniform per block
-  const int first = ((p.K + 31) / 32 / 2) * 32;   // K entries of the first half: whole steps
+  const int first = ((p.K + BK - 1) / BK / 2) * BK;   // K entries of the first half: whole steps
   GemmParams q = p;
   q.ldk = p.K;
   if (part == 0) {
@@ -131,24 +131,27 @@ __global__ __launch_bounds__(256, 1) void gemm_dma_splitk_kernel(GemmParams p) {
     q.A = static_cast<const unsigned short*>(p.A) + first;
     q.B = static_cast<const unsigned short*>(p.B) + (TRANS_B ? (size_t)first : (size_t)first * p.N);
   }
-  gemm_tile_dma<BF16, TRANS_B, 4, 4, 2, 32, 4, true>(q, tile_m, tile_n, blockIdx.y, smem);
+  gemm_tile_dma<BF16, TRANS_B, WM, WN, WCN, BK, STAGES, true>(q, tile_m, tile_n, blockIdx.y, smem);
 }
 
-inline size_t gemm_splitk_bytes(int M, int N, int batch) {
-  const size_t tiles = (size_t)ceil_div(M, 256) * ceil_div(N, 256) * batch;
-  return tiles * 256 * 256 * sizeof(float) + ((tiles * 2 * sizeof(int) + 255) / 256) * 256;
+// Workspace of a K split: the partial sums of one half per tile (fp32), then two words per tile (ticket, "written").
+inline size_t gemm_splitk_bytes(int M, int N, int batch, int bm, int bn) {
+  const size_t tiles = (size_t)ceil_div(M, bm) * ceil_div(N, bn) * batch;
+  return tiles * bm * bn * sizeof(float) + ((tiles * 2 * sizeof(int) + 255) / 256) * 256;
 }
 
-template <bool BF16, bool TRANS_B>
-int launch_dma_splitk(GemmParams p, int batch, void* ws, hipStream_t stream) {
-  p.tiles_m = ceil_div(p.M, 256);
-  p.tiles_n = ceil_div(p.N, 256);
+// flags_are_zero: the caller has zeroed the tile words on this stream already (they sit behind the partial sums).
+template <bool BF16, bool TRANS_B, int WM, int WN, int WCN, int BK, int STAGES>
+int launch_dma_splitk(GemmParams p, int batch, void* ws, bool flags_are_zero, hipStream_t stream) {
+  constexpr int BM = 2 * WM * 32, BN = WCN * WN * 32;
+  p.tiles_m = ceil_div(p.M, BM);
+  p.tiles_n = ceil_div(p.N, BN);
   const int total = p.tiles_m * p.tiles_n;
   const int per_xcd = (total + kXcds - 1) / kXcds;
   p.split_ws = static_cast<float*>(ws);
-  p.split_flags = reinterpret_cast<int*>(static_cast<unsigned char*>(ws) + (size_t)total * batch * 256 * 256 * sizeof(float));
-  constexpr int lds = gemm_dma_lds_bytes<4, 4, 2, 32, 4>();
-  auto kern = gemm_dma_splitk_kernel<BF16, TRANS_B>;
+  p.split_flags = reinterpret_cast<int*>(static_cast<unsigned char*>(ws) + (size_t)total * batch * BM * BN * sizeof(float));
+  constexpr int lds = gemm_dma_lds_bytes<WM, WN, WCN, BK, STAGES>();
+  auto kern = gemm_dma_splitk_kernel<BF16, TRANS_B, WM, WN, WCN, BK, STAGES>;
   static thread_local bool raised = false;  // per instantiation
   if (!raised) {
     if (int rc = check_hip(hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, lds),
@@ -156,22 +159,37 @@ int launch_dma_splitk(GemmParams p, int batch, void* ws, hipStream_t stream) {
       return rc;
     raised = true;
   }
-  const int flags = 2 * total * batch;
-  note_kernel("fill_zero_kernel");
-  hipLaunchKernelGGL(fill_zero_kernel, dim3(ceil_div(flags, 256)), dim3(256), 0, stream, p.split_flags, flags);
-  note_kernel("gemm_dma_splitk_kernel<%s, %s> (256 x 256 tiles, K in two halves)", BF16 ? "bf16" : "f16", TRANS_B ? "B(N,K)" : "B(K,N)");
-  hipLaunchKernelGGL(kern, dim3(per_xcd * kXcds * 2, batch), dim3(256), lds, stream, p);
+  if (!flags_are_zero) {
+    const int flags = 2 * total * batch;
+    note_kernel("fill_zero_kernel");
+    hipLaunchKernelGGL(fill_zero_kernel, dim3(ceil_div(flags, 256)), dim3(256), 0, stream, p.split_flags, flags);
+  }
+  note_kernel("gemm_dma_splitk_kernel<%s, %s> (%d x %d tiles, K in two halves)", BF16 ? "bf16" : "f16", TRANS_B ? "B(N,K)" : "B(K,N)", BM, BN);
+  hipLaunchKernelGGL(kern, dim3(per_xcd * kXcds * 2, batch), dim3(WCN * 128), lds, stream, p);
   return check_hip(hipGetLastError(), "gemm (split K) launch");
 }
 
+// Few 64 x 128 tiles and a long K: the K loop in two halves on twice the CUs.  Measured on MI355X (fp16, us, 64 x 128
+// tiles unsplit / split, the split with a launch that zeroes the tile words): 4096 x 64 x 4096 24.0 / 20.5, 4096 x 128 x
+// 4096 23.7 / 20.2, 2048 x 256 x 4096 23.5 / 19.8, 1000 x 200 x 4104 23.6 / 18.4, 512 x 512 x 8192 43.2 / 28.8 (64 tiles or
+// fewer); 4096 x 256 x 11008 57.2 / 45.6, but 4096 x 256 x 4096 24.9 / 24.6, 4 x (1024 x 256 x 4096) 25.5 / 24.5, 4096 x
+// 256 x 2048 13.6 / 17.2, 8192 x 128 x 2048 14.8 / 18.5 (128 tiles: only a very long K pays for the exchange).
+inline bool auto_split_wanted(int M, int N, int K, int batch) {
+  if ((long long)ceil_div(M, 128) * ceil_div(N, 128) * batch > 256) return false;
+  const long long half_tiles = (long long)ceil_div(M, 64) * ceil_div(N, 128) * batch;
+  return (half_tiles <= 64 && K >= 4096) || (half_tiles <= 128 && K >= 8192);
+}
+
 template <bool BF16, bool TRANS_B>
-int launch_shape(const GemmParams& p, int batch, int force, hipStream_t stream, void* ws, size_t ws_bytes) {
-  const bool ws_fits = ws && aligned(ws, 256) && ws_bytes >= gemm_splitk_bytes(p.M, p.N, batch);
-  if (force == 12) {
-    IEX_REQUIRE(p.K >= 64, IEX_ERR_UNSUPPORTED, "gemm: the K-split kernel needs K >= 64 (K=%d)", p.K);
-    IEX_REQUIRE(ws_fits && !p.accumulate, IEX_ERR_BAD_ARGUMENT, "gemm: the K-split kernel needs a 256-byte aligned workspace of %zu bytes (iex_gemm_ws) and a plain store",
-                gemm_splitk_bytes(p.M, p.N, batch));
-    return launch_dma_splitk<BF16, TRANS_B>(p, batch, ws, stream);
+int launch_shape(const GemmParams& p, int batch, int force, hipStream_t stream, void* ws, size_t ws_bytes, bool flags_are_zero) {
+  auto ws_fits = [&](int bm, int bn) { return ws && aligned(ws, 256) && ws_bytes >= gemm_splitk_bytes(p.M, p.N, batch, bm, bn); };
+  if (force == 12 || force == 14) {
+    const int bm = force == 12 ? 256 : 64, bn = force == 12 ? 256 : 128;
+    IEX_REQUIRE(p.K >= (force == 12 ? 64 : 128), IEX_ERR_UNSUPPORTED, "gemm: the K-split kernels need two K steps (K >= %d; K=%d)", force == 12 ? 64 : 128, p.K);
+    IEX_REQUIRE(ws_fits(bm, bn) && !p.accumulate, IEX_ERR_BAD_ARGUMENT, "gemm: the K-split kernels need a 256-byte aligned workspace of %zu bytes (iex_gemm_ws) and a plain store",
+                gemm_splitk_bytes(p.M, p.N, batch, bm, bn));
+    if (force == 12) return launch_dma_splitk<BF16, TRANS_B, 4, 4, 2, 32, 4>(p, batch, ws, flags_are_zero, stream);
+    return launch_dma_splitk<BF16, TRANS_B, 1, 1, 4, 64, 4>(p, batch, ws, flags_are_zero, stream);
   }
   if (force == 1) return launch<BF16, TRANS_B, 2, 2>(p, batch, stream);
   if (force == 2) return launch<BF16, TRANS_B, 2, 4>(p, batch, stream);
@@ -224,6 +242,9 @@ int launch_shape(const GemmParams& p, int batch, int force, hipStream_t stream, 
   // Half as tall (64 x 128) where even that leaves at most one tile per CU: twice the CUs at work
   // (4096 x 256 x 4096: 35 -> 27.5 us, 4096 x 512 x 4096: 35 -> 30, 1024 x 2048 x 1024: 13.9 -> 12.4).
   const long long half_tiles = (long long)ceil_div(p.M, 64) * ceil_div(p.N, 128) * batch;
+  // ... and with room for the partial sums, K in two halves where that still leaves at most one workgroup per CU
+  if (auto_split_wanted(p.M, p.N, p.K, batch) && ws_fits(64, 128) && !p.accumulate)
+    return launch_dma_splitk<BF16, TRANS_B, 1, 1, 4, 64, 4>(p, batch, ws, flags_are_zero, stream);
   if (half_tiles <= 256 && p.K >= 512) return launch_dma<BF16, TRANS_B, 1, 1, 64, 4, 4>(p, batch, stream);
   if (p.K >= 2048) return launch_dma<BF16, TRANS_B, 2, 1, 64, 4, 4>(p, batch, stream);
   return launch_dma<BF16, TRANS_B, 2, 2, 32, 4>(p, batch, stream);
@@ -237,7 +258,8 @@ int launch_shape(const GemmParams& p, int batch, int force, hipStream_t stream, 
 // straight into LDS: 5 = 128x128, 6 = 128x256, 7 = 256x256, 8 = 128x128, 9 = 64x128 by eight waves with K steps of 64,
 // 10 = 128x256 by eight waves, 11 = the same with K steps of 64, 12 = 256x256 with K split over two workgroups per tile
 // (iex_gemm_ws only; never chosen), 13 = 256x256 by eight waves in two groups that alternate between loading and
-// multiplying.  0 = choose (one of 5, 8, 9, 10, 13).
+// multiplying, 14 = 64x128 by eight waves with K split over two workgroups per tile (iex_gemm_ws only).
+// 0 = choose (one of 5, 8, 9, 10, 13, and 14 where iex_gemm_workspace_bytes asked for room and got it).
 extern "C" int iex_gemm(int dtype, int trans_b_and_shape, int M, int N, int K, const void* A, const void* B, void* C, int batch,
                         long long stride_a, long long stride_b, long long stride_c, void* stream) {
   iex::trail_reset();
@@ -254,13 +276,24 @@ extern "C" int iex_gemm_ws(int dtype, int trans_b_and_shape, int M, int N, int K
 extern "C" size_t iex_gemm_workspace_bytes(int dtype, int trans_b_and_shape, int M, int N, int K, int batch) {
   if (M <= 0 || N <= 0 || K <= 0 || batch <= 0 || (dtype != IEX_F16 && dtype != IEX_BF16)) return 0;
   const int force = (trans_b_and_shape >> 4) & 0xf;
-  if (force == 12) return iex::gemm_splitk_bytes(M, N, batch);
-  return 0;
+  if (force == 12) return iex::gemm_splitk_bytes(M, N, batch, 256, 256);
+  if (force == 14) return iex::gemm_splitk_bytes(M, N, batch, 64, 128);
+  return force == 0 ? iex::gemm_auto_split_bytes(M, N, K, batch) : 0;
+}
+
+size_t iex::gemm_auto_split_bytes(int M, int N, int K, int batch) {
+  return auto_split_wanted(M, N, K, batch) ? gemm_splitk_bytes(M, N, batch, 64, 128) : 0;
+}
+
+void iex::gemm_auto_split_flags(int M, int N, int batch, size_t* offset_bytes, int* words) {
+  const size_t tiles = (size_t)ceil_div(M, 64) * ceil_div(N, 128) * batch;
+  *offset_bytes = tiles * 64 * 128 * sizeof(float);
+  *words = (int)(2 * tiles);
 }
 
 int iex::gemm_dispatch(int dtype, int trans_b_and_shape, int M, int N, int K, const void* A, const void* B, void* C, int batch,
                        long long stride_a, long long stride_b, long long stride_c, void* stream, const float* row_bias, int relu,
-                       int accumulate, void* workspace, size_t workspace_bytes) {
+                       int accumulate, void* workspace, size_t workspace_bytes, bool workspace_flags_are_zero) {
   const int trans_b = trans_b_and_shape & 1, force = (trans_b_and_shape >> 4) & 0xf;
   IEX_REQUIRE(M >= 0 && N >= 0 && K >= 0 && batch >= 0, IEX_ERR_BAD_ARGUMENT, "gemm: negative dimension");
   if (M == 0 || N == 0 || batch == 0) return 0;
@@ -277,8 +310,8 @@ int iex::gemm_dispatch(int dtype, int trans_b_and_shape, int M, int N, int K, co
   p.stream_out = (double)M * N * batch * 2 >= 128e6;
   hipStream_t s = static_cast<hipStream_t>(stream);
   const bool bf = dtype == IEX_BF16;
-  if (bf && trans_b) return launch_shape<true, true>(p, batch, force, s, workspace, workspace_bytes);
-  if (bf && !trans_b) return launch_shape<true, false>(p, batch, force, s, workspace, workspace_bytes);
-  if (!bf && trans_b) return launch_shape<false, true>(p, batch, force, s, workspace, workspace_bytes);
-  return launch_shape<false, false>(p, batch, force, s, workspace, workspace_bytes);
+  if (bf && trans_b) return launch_shape<true, true>(p, batch, force, s, workspace, workspace_bytes, workspace_flags_are_zero);
+  if (bf && !trans_b) return launch_shape<true, false>(p, batch, force, s, workspace, workspace_bytes, workspace_flags_are_zero);
+  if (!bf && trans_b) return launch_shape<false, true>(p, batch, force, s, workspace, workspace_bytes, workspace_flags_are_zero);
+  return launch_shape<false, false>(p, batch, force, s, workspace, workspace_bytes, workspace_flags_are_zero);
 }

@@ -47,7 +47,12 @@ struct GemmParams {
 // iex_gemm with the epilogue options above (gemm.hip).
 int gemm_dispatch(int dtype, int trans_b_and_shape, int M, int N, int K, const void* A, const void* B, void* C, int batch,
                   long long stride_a, long long stride_b, long long stride_c, void* stream, const float* row_bias, int relu,
-                  int accumulate, void* workspace = nullptr, size_t workspace_bytes = 0);
+                  int accumulate, void* workspace = nullptr, size_t workspace_bytes = 0, bool workspace_flags_are_zero = false);
+// Bytes of workspace with which gemm_dispatch, left to choose, splits K over two workgroups per tile (0: this shape is
+// not split), and where in such a workspace the words sit that must be zero at launch (gemm_dispatch zeroes them with a
+// launch of its own unless the caller says it has: workspace_flags_are_zero).
+size_t gemm_auto_split_bytes(int M, int N, int K, int batch);
+void gemm_auto_split_flags(int M, int N, int batch, size_t* offset_bytes, int* words);
 
 typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));

@@ -558,16 +558,28 @@ inline bool dense_path_wins(const SpmmParams& p, int batch, int matrix_core_kind
   return 1.15 * dense_form < other;
 }
 
+// Behind the dense form (rounded up to 256 bytes) the workspace may hold what the GEMM wants for splitting K over two
+// workgroups per tile (few tiles, long k: gemm_auto_split_bytes); the words it wants zero are zeroed by the kernel
+// that writes the dense form.
+inline size_t dense_path_split_offset(const SpmmParams& p) { return (dense_path_bytes(p) + 255) & ~size_t(255); }
+inline size_t dense_path_split_bytes(const SpmmParams& p, int batch) { return p.accumulate ? 0 : gemm_auto_split_bytes(p.m, p.n, p.k, batch); }
+
 template <typename T, typename IT>
 int launch_dense_path(const SpmmParams& p, int batch, const Choice& ch, hipStream_t stream) {
+  const size_t split = dense_path_split_bytes(p, batch), offset = dense_path_split_offset(p);
+  const bool with_split = split > 0 && aligned(ch.ws, 256) && ch.ws_bytes >= offset + split;
+  unsigned char* split_ws = with_split ? static_cast<unsigned char*>(ch.ws) + offset : nullptr;
+  size_t flags_at = 0;
+  int flag_words = 0;
+  if (with_split) gemm_auto_split_flags(p.m, p.n, batch, &flags_at, &flag_words);
   note_kernel("csr_to_dense_kernel<%s>", type_name<IT>());
   hipLaunchKernelGGL((csr_to_dense_kernel<IT>), dim3(ceil_div(p.m, kDenseWaves)), dim3(kDenseThreads), 0, stream, p.m, p.k,
                      p.row_offsets, static_cast<const IT*>(p.cols), static_cast<const uint16_t*>(p.values),
-                     static_cast<uint16_t*>(ch.ws));
+                     static_cast<uint16_t*>(ch.ws), with_split ? reinterpret_cast<int*>(split_ws + flags_at) : nullptr, flag_words);
   if (int rc = check_hip(hipGetLastError(), "spmm dense-form launch")) return rc;
   const int dtype = std::is_same<T, __half>::value ? IEX_F16 : IEX_BF16;
   return gemm_dispatch(dtype, 0, p.m, p.n, p.k, ch.ws, p.dense, p.out, batch, 0, (long long)p.k * p.n, (long long)p.m * p.n, stream,
-                       p.bias, p.relu, p.accumulate);
+                       p.bias, p.relu, p.accumulate, split_ws, with_split ? split : 0, with_split);
 }
 
 template <typename T, typename IT>
@@ -758,7 +770,8 @@ static size_t workspace_plan(int dtype, int itype, int flags, int m, int k, int 
     if (!dense_path_wins(p, batch, few ? 0 : mfma_variant<__half>(p, batch, ch).kind, few)) return 0;
   }
   *kind = 7;
-  return dense_path_bytes(p);
+  const size_t split = dense_path_split_bytes(p, batch);
+  return split ? dense_path_split_offset(p) + split : dense_path_bytes(p);
 }
 
 size_t spmm_workspace_bytes(int dtype, int itype, int flags, int m, int k, int n, int nonzeros, int batch) {

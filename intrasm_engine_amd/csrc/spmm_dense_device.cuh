@@ -24,8 +24,12 @@ template <typename IT>
 __global__ __launch_bounds__(kDenseThreads) void csr_to_dense_kernel(int m, int k, const int* __restrict__ row_offsets,
                                                                      const IT* __restrict__ cols,
                                                                      const uint16_t* __restrict__ values,
-                                                                     uint16_t* __restrict__ out) {
+                                                                     uint16_t* __restrict__ out, int* __restrict__ zero_words,
+                                                                     int n_zero_words) {
   __shared__ __align__(16) uint16_t smem[kDenseWaves][kDenseSeg];
+  // (words that the kernel after this one wants zero at its launch, a few hundred at most: cheaper here than a launch)
+  if (blockIdx.x == 0)
+    for (int i = threadIdx.x; i < n_zero_words; i += kDenseThreads) zero_words[i] = 0;
   const int lane = lane_id();
   const int wave = uniform(threadIdx.x >> 6);
   const int row = blockIdx.x * kDenseWaves + wave;

@@ -144,18 +144,23 @@ def test_argument_checks(dev):
 @pytest.mark.parametrize("trans_b", [False, True])
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
 @pytest.mark.parametrize("mnk,batch", [((300, 520, 200), 1), ((260, 264, 1000), 3), ((512, 256, 64), 2), ((129, 136, 2048), 1)])
-def test_k_split_over_two_workgroups(oracle, dev, trans_b, dtype, mnk, batch):
-    """256 x 256 tiles with K split over two workgroups per tile (partial sums meet in a workspace, the second
-    workgroup to arrive adds and stores), on request: ragged m, n, a K whose halves are 96 + 104, 512 + 488 (a partial
-    last step), 32 + 32; batches; against the oracle, twice with the same bits, and on integer operands exactly equal
-    to the unsplit kernel."""
+@pytest.mark.parametrize("split,whole", [(12, 7), (14, 9)])
+def test_k_split_over_two_workgroups(oracle, dev, trans_b, dtype, mnk, batch, split, whole):
+    """256 x 256 tiles (code 12) and 64 x 128 tiles (code 14) with K split over two workgroups per tile (partial sums
+    meet in a workspace, the second workgroup to arrive adds and stores), on request: ragged m, n, a K whose halves are
+    96 + 104 (128 + 72 with steps of 64), 512 + 488 (a partial last step), 32 + 32; batches; against the oracle, twice
+    with the same bits, and on integer operands exactly equal to the unsplit kernel of the same tile."""
     from intrasm_engine_amd.pytorch import ops as pyops
     rng = np.random.default_rng(batch)
     M, N, K = mnk
+    if split == 14 and K < 128:
+        with pytest.raises(RuntimeError, match="two K steps"), pyops.kernel_params(gemm={"tile": 14}):
+            ops.gemm_mfma(torch.zeros(M, K, device=dev, dtype=dtype), torch.zeros(K, N, device=dev, dtype=dtype), False)
+        return
     a_np = rng.standard_normal((batch, M, K)).astype(np.float32)
     b_np = rng.standard_normal((batch, N, K) if trans_b else (batch, K, N)).astype(np.float32)
     a, b = torch.from_numpy(a_np).to(dev).to(dtype), torch.from_numpy(b_np).to(dev).to(dtype)
-    with pyops.kernel_params(gemm={"tile": 12}):
+    with pyops.kernel_params(gemm={"tile": split}):
         out = ops.gemm_mfma(a, b, trans_b)
         again = ops.gemm_mfma(a, b, trans_b)
     assert torch.equal(out, again)
@@ -166,11 +171,43 @@ def test_k_split_over_two_workgroups(oracle, dev, trans_b, dtype, mnk, batch):
         assert_close(out[z].float().cpu().numpy(), want, scale, 1e-2, f"split-K gemm {M}x{N}x{K} {dtype} trans_b={trans_b} entry {z}")
     ai = torch.from_numpy(rng.integers(-3, 4, a_np.shape).astype(np.float32)).to(dev).to(dtype)
     bi = torch.from_numpy(rng.integers(-3, 4, b_np.shape).astype(np.float32)).to(dev).to(dtype)
-    with pyops.kernel_params(gemm={"tile": 12}):
-        split = ops.gemm_mfma(ai, bi, trans_b)
-    with pyops.kernel_params(gemm={"tile": 7}):
-        whole = ops.gemm_mfma(ai, bi, trans_b)
-    assert torch.equal(split, whole)
+    with pyops.kernel_params(gemm={"tile": split}):
+        in_halves = ops.gemm_mfma(ai, bi, trans_b)
+    with pyops.kernel_params(gemm={"tile": whole}):
+        at_once = ops.gemm_mfma(ai, bi, trans_b)
+    assert torch.equal(in_halves, at_once)
+
+
+def test_k_split_is_picked_for_few_tiles_and_a_long_k(oracle, dev):
+    """4096 x 128 x 4096 (64 tiles of 64 x 128 on 256 CUs): the operator asks the library how much room the split wants,
+    gets a number, passes the room and the split kernel runs; the entry point without a workspace runs the unsplit tile.
+    Shapes with more tiles or a shorter K ask for nothing.  Twice the same bits; against the oracle on sampled rows."""
+    from intrasm_engine_amd import _lib
+    lib = _lib.load()
+    M, N, K = 4096, 128, 4096
+    assert lib.iex_gemm_workspace_bytes(_lib.F16, 0, M, N, K, 1) == 64 * 64 * 128 * 4 + 512
+    assert lib.iex_gemm_workspace_bytes(_lib.F16, 14 << 4, M, N, K, 1) == 64 * 64 * 128 * 4 + 512
+    assert lib.iex_gemm_workspace_bytes(_lib.F16, 0, M, 256, K, 1) == 0          # 128 tiles, K < 8192
+    assert lib.iex_gemm_workspace_bytes(_lib.F16, 0, M, 256, 11008, 1) != 0      # 128 tiles, a very long K
+    assert lib.iex_gemm_workspace_bytes(_lib.F16, 0, M, N, 2048, 1) == 0
+    assert lib.iex_gemm_workspace_bytes(_lib.F16, 0, M, N, K, 4) == 0            # four times the tiles
+    assert lib.iex_gemm_workspace_bytes(_lib.F16, 9 << 4, M, N, K, 1) == 0       # another kernel on request
+    rng = np.random.default_rng(9)
+    a_np = rng.standard_normal((M, K)).astype(np.float32)
+    b_np = rng.standard_normal((K, N)).astype(np.float32)
+    a, b = torch.from_numpy(a_np).to(dev).half(), torch.from_numpy(b_np).to(dev).half()
+    out = ops.gemm_mfma(a, b, False)
+    assert "gemm_dma_splitk_kernel" in _lib.last_kernels() and "64 x 128" in _lib.last_kernels()
+    assert torch.equal(out, ops.gemm_mfma(a, b, False))
+    rows = np.arange(0, M, 61)
+    a_r, b_r = rounded(a_np[rows], torch.float16), rounded(b_np, torch.float16)
+    scale = np.abs(a_r).astype(np.float64) @ np.abs(b_r).astype(np.float64)
+    assert_close(out[torch.from_numpy(rows).to(dev)].float().cpu().numpy(), oracle.gemm(a_r, b_r), scale, 1e-2, "few tiles, K split")
+    c = torch.empty_like(out)
+    rc = lib.iex_gemm(_lib.F16, 0, M, N, K, a.data_ptr(), b.data_ptr(), c.data_ptr(), 1, 0, 0, 0, torch.cuda.current_stream().cuda_stream)
+    assert rc == 0 and "splitk" not in _lib.last_kernels()
+    torch.cuda.synchronize()
+    assert torch.allclose(c.float(), out.float(), rtol=2e-2, atol=0.5)
 
 
 def test_k_split_on_config4s_product_and_refused_without_workspace(oracle, dev):

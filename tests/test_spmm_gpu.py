@@ -746,6 +746,45 @@ def test_dense_form_path_is_chosen_with_a_workspace_and_only_then(oracle, dev):
     torch.cuda.synchronize()
 
 
+def test_dense_form_path_splits_k_where_the_product_has_few_tiles(oracle, dev):
+    """4096 x 4096 at 70 % sparsity times 4096 x 128 in fp16: the dense form wins, and its product is 64 tiles of 64 x 128
+    with k = 4096, which the GEMM runs with k in two halves when it has room for the partial sums.  The size the
+    library asks for holds that room behind the dense form; the kernel that writes the dense form zeroes the tile words
+    (no launch of its own for that); a workspace of the dense form alone still runs the path, unsplit; both agree with
+    the oracle and every repeat gives the same bits."""
+    from intrasm_engine_amd import _lib
+    from intrasm_engine_amd.pytorch import ops as pyops
+    lib = _lib.load()
+    m = k = 4096
+    n = 128
+    dtype = torch.float16
+    rng = np.random.default_rng(21)
+    csr, b_np, (ri, v, ro_t, ci_t), b = _dense_form_case(rng, m, k, n, 1, dtype, torch.int16, dev, mean_len=0.3 * k)
+    nnz = csr.column_indices.shape[0]
+    need = lib.iex_spmm_workspace_bytes(_lib.F16, _lib.I16, 0, m, k, n, nnz, 1)
+    assert need == m * k * 2 + lib.iex_gemm_workspace_bytes(_lib.F16, 0, m, n, k, 1) and need > m * k * 2
+    assert lib.iex_spmm_workspace_bytes(_lib.F16, _lib.I16, _lib.SPMM_ACCUMULATE, m, k, n, nnz, 1) == m * k * 2   # (the split stores plainly)
+    kw = dict(per_batch_values=False, accumulate=False, dtypes=(dtype,), allow_i16=True)
+    out = pyops._spmm(b, ri, v, ro_t, ci_t, m, **kw)
+    trail = _lib.last_kernels()
+    assert "csr_to_dense_kernel" in trail and "gemm_dma_splitk_kernel" in trail and "fill_zero" not in trail
+    for _ in range(3):
+        assert torch.equal(out, pyops._spmm(b, ri, v, ro_t, ci_t, m, **kw))
+    vals_r, b_r = rounded(csr.values, dtype), rounded(b_np, dtype)
+    want = oracle.spmm(b_r, csr.row_indices, vals_r, csr.row_offsets, csr.column_indices, m)
+    scale = oracle.spmm_abs_scale(b_r, csr.row_indices, vals_r, csr.row_offsets, csr.column_indices, m)
+    assert_close(out.float().cpu().numpy(), want, scale, RTOL[dtype], "dense form, k in two halves")
+    small = torch.empty(m * k * 2, dtype=torch.uint8, device=dev)
+    unsplit = torch.empty_like(out)
+    args = (_lib.F16, _lib.I16, 0, m, k, n, nnz, ri.data_ptr(), v.data_ptr(), ro_t.data_ptr(), ci_t.data_ptr(),
+            b.data_ptr(), None, unsplit.data_ptr(), torch.cuda.current_stream().cuda_stream, 1)
+    assert lib.iex_spmm_ws(*args, small.data_ptr(), m * k * 2) == 0, _lib.last_error()
+    trail = _lib.last_kernels()
+    assert "csr_to_dense_kernel" in trail and "splitk" not in trail
+    torch.cuda.synchronize()
+    assert_close(unsplit.float().cpu().numpy(), want, scale, RTOL[dtype], "dense form, unsplit")
+
+
 def test_csr_check_names_what_a_pattern_lacks(dev):
     """``iex_csr_check``: 0 for what ``dense_to_sparse`` produces; unsorted or duplicated columns (valid for the row
     kernel and for the reference, not for the other families), a column outside the matrix, offsets that do not run

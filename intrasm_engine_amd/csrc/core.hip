@@ -88,12 +88,15 @@ __global__ __launch_bounds__(256) void csr_row_histogram_kernel(int m, const int
 }
 
 // *dense_nonzeros += the nonzeros of this block of 128 rows that sit in 128 x 128 blocks holding at least dense_min of
-// them.  One workgroup (16 wavefronts) per 128 rows; the counters of the row block's column blocks live in LDS.  A
-// wavefront takes 64 nonzeros of a row at a time; neighbours that fall into the same column block (all of them, in
-// runs, when the columns ascend) are counted by the first lane of their run, so a run costs one LDS atomic, not one
-// per nonzero.  Any column order gives the same counts.
+// them.  One workgroup (16 wavefronts) per 128 rows; the counters of the row block's column blocks live in LDS.  Which
+// row a nonzero belongs to does not matter inside a row block, so the block's nonzeros -- one contiguous stretch of the
+// column array -- are dealt to the wavefronts in equal contiguous shares, whatever the row lengths; a wavefront takes
+// 512 of them per step (eight loads in flight, the next step's loads issued before this step's are counted).
+// Neighbours that fall into the same column block (in runs, when the columns ascend) are counted by the first lane of
+// their run, so a run costs one LDS atomic, not one per nonzero.  Any column order gives the same counts.
 constexpr int kShareMaxTiles = 512;   // k <= 65536
 constexpr int kShareThreads = 1024;
+constexpr int kShareLoads = 8;
 template <typename IT>
 __global__ __launch_bounds__(kShareThreads) void csr_dense_share_kernel(int m, int k, int nnz, const int* __restrict__ row_offsets, const IT* __restrict__ cols,
                                                                         int dense_min, int* dense_nonzeros) {
@@ -104,33 +107,41 @@ __global__ __launch_bounds__(kShareThreads) void csr_dense_share_kernel(int m, i
   if (threadIdx.x == 0) total = 0;
   __syncthreads();
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  for (int r = blockIdx.x * 128 + wave; r < min(m, blockIdx.x * 128 + 128); r += kShareThreads / 64) {
-    // (offsets that point outside the arrays are cut to them: the kernel may run before anybody has checked the pattern)
-    const int s = min(max(row_offsets[r], 0), nnz), e = min(max(row_offsets[r + 1], s), nnz);
-    for (int base = s; base < e; base += 256) {   // four loads in flight per lane, then counted 64 nonzeros at a time
-      int t4[4];
+  // (offsets that point outside the arrays are cut to them: the kernel may run before anybody has checked the pattern)
+  const int row0 = (int)blockIdx.x * 128;
+  const int first = min(max(row_offsets[row0], 0), nnz);
+  const int last = min(max(row_offsets[min(m, row0 + 128)], first), nnz);
+  const int share = ((last - first + kShareThreads - 1) / kShareThreads) * 64;   // whole chunks of 64 per wavefront
+  const int begin = min(first + wave * share, last), end = min(begin + share, last);
+  auto fetch = [&](int base, int (&t)[kShareLoads]) {
 #pragma unroll
-      for (int u = 0; u < 4; ++u) {
-        const int j = base + u * 64 + lane;
-        t4[u] = -1;   // (no nonzero here, or a column outside the matrix: counted nowhere)
-        if (j < e) {
-          const int c = (int)cols[j];
-          if (c >= 0 && c < k) t4[u] = c >> 7;
-        }
-      }
-#pragma unroll
-      for (int u = 0; u < 4; ++u) {
-        if (base + u * 64 >= e) break;   // (uniform)
-        const int t = t4[u];
-        const int before = __shfl_up(t, 1, 64);
-        const unsigned long long heads = __ballot(lane == 0 || t != before);
-        if ((heads >> lane) & 1ull) {
-          const unsigned long long later = lane == 63 ? 0ull : heads >> (lane + 1);
-          const int run = later ? __builtin_ctzll(later) + 1 : 64 - lane;
-          if (t >= 0) atomicAdd(&count[t], run);
-        }
+    for (int u = 0; u < kShareLoads; ++u) {
+      const int j = base + u * 64 + lane;
+      t[u] = -1;   // (no nonzero here, or a column outside the matrix: counted nowhere)
+      if (j < end) {
+        const int c = (int)cols[j];
+        if (c >= 0 && c < k) t[u] = c >> 7;
       }
     }
+  };
+  int cur[kShareLoads], next[kShareLoads];
+  if (begin < end) fetch(begin, cur);
+  for (int base = begin; base < end; base += 64 * kShareLoads) {
+    if (base + 64 * kShareLoads < end) fetch(base + 64 * kShareLoads, next);   // (uniform)
+#pragma unroll
+    for (int u = 0; u < kShareLoads; ++u) {
+      if (base + u * 64 >= end) break;   // (uniform)
+      const int t = cur[u];
+      const int before = __shfl_up(t, 1, 64);
+      const unsigned long long heads = __ballot(lane == 0 || t != before);
+      if ((heads >> lane) & 1ull) {
+        const unsigned long long later = lane == 63 ? 0ull : heads >> (lane + 1);
+        const int run = later ? __builtin_ctzll(later) + 1 : 64 - lane;
+        if (t >= 0) atomicAdd(&count[t], run);
+      }
+    }
+#pragma unroll
+    for (int u = 0; u < kShareLoads; ++u) cur[u] = next[u];
   }
   __syncthreads();
   int mine = 0;

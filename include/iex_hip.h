@@ -79,9 +79,16 @@ int iex_csr_row_histogram(int m, const int* row_offsets, int* histogram, void* s
  * density -- which is all that the 0 = choose rule of those entry points can see.  A caller reads the figure back
  * once per pattern, as set-up, and forces the variant.  k <= 65536.  Offsets that point outside the arrays are cut to
  * [0, nonzeros] and columns outside [0, k) are counted nowhere, so the kernel may be launched together with
- * iex_csr_check and the two results read back at once.  No counterpart in the reference. */
+ * iex_csr_check and the two results read back at once.
+ * scratch (device memory, may be NULL): with iex_csr_dense_share_scratch_bytes(m, k) bytes that the caller has set to
+ * 0, a block of 128 rows is counted by several workgroups (a pattern of 4096 rows has 32 such blocks, and one
+ * workgroup per block leaves seven eighths of the chip idle: 8.4 M nonzeros 130 us); without it, or with fewer bytes,
+ * by one.  The call may overwrite the scratch memory until the work it puts on `stream` has run; the counts are the
+ * same either way.  iex_csr_dense_share_scratch_bytes returns 0 where one workgroup per block fills the chip anyway.
+ * No counterpart in the reference. */
 int iex_csr_dense_share(int itype, int m, int k, int nonzeros, const int* row_offsets, const void* column_indices,
-                        int dense_min, int* dense_nonzeros, void* stream);
+                        int dense_min, int* dense_nonzeros, void* scratch, size_t scratch_bytes, void* stream);
+size_t iex_csr_dense_share_scratch_bytes(int m, int k);
 
 /* dst[0:nbytes] = src[0:nbytes] with a plain 128-bit-per-lane streaming kernel (nbytes and both
  * pointers multiples of 16).  Measurement aid with no counterpart in the reference: hardware

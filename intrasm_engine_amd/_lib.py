@@ -43,7 +43,8 @@ SIGNATURES = {
     "iex_spmm_ws": (_i, [_i, _i, _i, _i, _i, _i, _i, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _vp, _c.c_size_t]),
     "iex_spmm_sched": (_i, [_i, _i, _i, _i, _i, _i, _i, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _vp, _c.c_size_t, _c.POINTER(_i)]),
     "iex_csr_row_histogram": (_i, [_i, _vp, _vp, _vp]),
-    "iex_csr_dense_share": (_i, [_i, _i, _i, _i, _vp, _vp, _i, _vp, _vp]),
+    "iex_csr_dense_share": (_i, [_i, _i, _i, _i, _vp, _vp, _i, _vp, _vp, _c.c_size_t, _vp]),
+    "iex_csr_dense_share_scratch_bytes": (_c.c_size_t, [_i, _i]),
     "iex_spmm_workspace_bytes": (_c.c_size_t, [_i, _i, _i, _i, _i, _i, _i, _i]),
     "iex_spmm_workspace_kind": (_i, [_i, _i, _i, _i, _i, _i, _i, _i]),
     "iex_spmm_static": (_i, [_i, _i, _i, _i, _i, _i, _i, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i]),

@@ -88,31 +88,37 @@ __global__ __launch_bounds__(256) void csr_row_histogram_kernel(int m, const int
 }
 
 // *dense_nonzeros += the nonzeros of this block of 128 rows that sit in 128 x 128 blocks holding at least dense_min of
-// them.  One workgroup (16 wavefronts) per 128 rows; the counters of the row block's column blocks live in LDS.  Which
-// row a nonzero belongs to does not matter inside a row block, so the block's nonzeros -- one contiguous stretch of the
-// column array -- are dealt to the wavefronts in equal contiguous shares, whatever the row lengths; a wavefront takes
-// 512 of them per step (eight loads in flight, the next step's loads issued before this step's are counted).
-// Neighbours that fall into the same column block (in runs, when the columns ascend) are counted by the first lane of
-// their run, so a run costs one LDS atomic, not one per nonzero.  Any column order gives the same counts.
+// them.  `parts` workgroups (16 wavefronts each) per 128 rows; the counters of the row block's column blocks live in
+// LDS.  Which row a nonzero belongs to does not matter inside a row block, so the block's nonzeros -- one contiguous
+// stretch of the column array -- are dealt to the workgroups and their wavefronts in equal contiguous shares, whatever
+// the row lengths; a wavefront takes 512 of them per step (eight loads in flight, the next step's loads issued before
+// this step's are counted).  Neighbours that fall into the same column block (in runs, when the columns ascend) are
+// counted by the first lane of their run, so a run costs one LDS atomic, not one per nonzero.  Any column order gives
+// the same counts.  With parts > 1 the workgroups of a row block add their counters into block_counts[row block][tile]
+// (zero at launch) and take a ticket from done[row block] (zero at launch); the one that draws the last ticket finds
+// every sum complete and compares them with dense_min.
 constexpr int kShareMaxTiles = 512;   // k <= 65536
 constexpr int kShareThreads = 1024;
 constexpr int kShareLoads = 8;
+constexpr int kShareMaxParts = 32;
 template <typename IT>
 __global__ __launch_bounds__(kShareThreads) void csr_dense_share_kernel(int m, int k, int nnz, const int* __restrict__ row_offsets, const IT* __restrict__ cols,
-                                                                        int dense_min, int* dense_nonzeros) {
+                                                                        int dense_min, int* dense_nonzeros, int parts, int* block_counts, int* done) {
   __shared__ int count[kShareMaxTiles];
   __shared__ int total;
+  __shared__ int ticket;
   const int tiles = (k + 127) / 128;
   for (int t = threadIdx.x; t < tiles; t += kShareThreads) count[t] = 0;
   if (threadIdx.x == 0) total = 0;
   __syncthreads();
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int row_block = (int)blockIdx.x / parts, part = (int)blockIdx.x % parts;
+  const int row0 = row_block * 128;
   // (offsets that point outside the arrays are cut to them: the kernel may run before anybody has checked the pattern)
-  const int row0 = (int)blockIdx.x * 128;
   const int first = min(max(row_offsets[row0], 0), nnz);
   const int last = min(max(row_offsets[min(m, row0 + 128)], first), nnz);
-  const int share = ((last - first + kShareThreads - 1) / kShareThreads) * 64;   // whole chunks of 64 per wavefront
-  const int begin = min(first + wave * share, last), end = min(begin + share, last);
+  const int share = ((last - first + kShareThreads * parts - 1) / (kShareThreads * parts)) * 64;   // whole chunks of 64 per wavefront
+  const int begin = min(first + (part * (kShareThreads / 64) + wave) * share, last), end = min(begin + share, last);
   auto fetch = [&](int base, int (&t)[kShareLoads]) {
 #pragma unroll
     for (int u = 0; u < kShareLoads; ++u) {
@@ -145,28 +151,66 @@ __global__ __launch_bounds__(kShareThreads) void csr_dense_share_kernel(int m, i
   }
   __syncthreads();
   int mine = 0;
-  for (int t = threadIdx.x; t < tiles; t += kShareThreads) mine += count[t] >= dense_min ? count[t] : 0;
+  if (parts == 1) {
+    for (int t = threadIdx.x; t < tiles; t += kShareThreads) mine += count[t] >= dense_min ? count[t] : 0;
+  } else {
+    int* sums = block_counts + (size_t)row_block * tiles;
+    // Device-scope atomics are carried out where all XCDs see them, and one that returns the old value has been carried
+    // out when that value is back: once every wavefront has waited for its own and the barrier has collected them, the
+    // ticket may be drawn.  (A device-scope fence here instead writes back the L2 of the XCD under everybody else:
+    // measured 150 us for the kernel whatever the pattern.)
+    int seen = 0;
+    for (int t = threadIdx.x; t < tiles; t += kShareThreads)
+      if (count[t]) seen ^= atomicAdd(&sums[t], count[t]);
+    asm volatile("s_waitcnt vmcnt(0)" : "+v"(seen) : : "memory");
+    __syncthreads();
+    if (threadIdx.x == 0) ticket = atomicAdd(&done[row_block], 1);
+    __syncthreads();
+    if (ticket != parts - 1) return;   // (uniform)
+    for (int t = threadIdx.x; t < tiles; t += kShareThreads) {
+      const int sum = __hip_atomic_load(&sums[t], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      mine += sum >= dense_min ? sum : 0;
+    }
+  }
   if (mine) atomicAdd(&total, mine);
   __syncthreads();
   if (threadIdx.x == 0 && total) atomicAdd(dense_nonzeros, total);
+}
+
+// Workgroups per block of 128 rows: enough for two per CU, as far as the scratch memory reaches.
+inline int dense_share_parts(int m, int k, const void* scratch, size_t scratch_bytes) {
+  const int row_blocks = (m + 127) / 128, tiles = (k + 127) / 128;
+  if (!scratch || row_blocks == 0 || scratch_bytes < (size_t)row_blocks * (tiles + 1) * sizeof(int)) return 1;
+  return std::min(kShareMaxParts, std::max(1, 512 / row_blocks));
 }
 }  // namespace
 
 extern "C" {
 
 int iex_csr_dense_share(int itype, int m, int k, int nonzeros, const int* row_offsets, const void* column_indices, int dense_min,
-                        int* dense_nonzeros, void* stream) {
+                        int* dense_nonzeros, void* scratch, size_t scratch_bytes, void* stream) {
   IEX_REQUIRE(m >= 0 && k >= 0 && nonzeros >= 0 && dense_min >= 0, IEX_ERR_BAD_ARGUMENT, "csr_dense_share: negative argument");
   IEX_REQUIRE(dense_nonzeros && (m == 0 || (row_offsets && column_indices)), IEX_ERR_BAD_ARGUMENT, "csr_dense_share: null pointer argument");
   IEX_REQUIRE(itype == IEX_I32 || itype == IEX_I16, IEX_ERR_UNSUPPORTED, "csr_dense_share: column indices must be int32 or int16");
   IEX_REQUIRE(k <= 128 * kShareMaxTiles, IEX_ERR_TOO_LARGE, "csr_dense_share: more than %d columns", 128 * kShareMaxTiles);
+  IEX_REQUIRE(!scratch || iex::aligned(scratch, 4), IEX_ERR_BAD_ARGUMENT, "csr_dense_share: scratch memory must be 4-byte aligned");
   if (m == 0 || k == 0 || nonzeros == 0) return 0;
   hipStream_t s = static_cast<hipStream_t>(stream);
+  const int row_blocks = (m + 127) / 128, tiles = (k + 127) / 128;
+  const int parts = dense_share_parts(m, k, scratch, scratch_bytes);
+  int* block_counts = static_cast<int*>(scratch);
+  int* done = block_counts ? block_counts + (size_t)row_blocks * tiles : nullptr;
   if (itype == IEX_I32)
-    hipLaunchKernelGGL(csr_dense_share_kernel<int>, dim3((m + 127) / 128), dim3(kShareThreads), 0, s, m, k, nonzeros, row_offsets, static_cast<const int*>(column_indices), dense_min, dense_nonzeros);
+    hipLaunchKernelGGL(csr_dense_share_kernel<int>, dim3(row_blocks * parts), dim3(kShareThreads), 0, s, m, k, nonzeros, row_offsets, static_cast<const int*>(column_indices), dense_min, dense_nonzeros, parts, block_counts, done);
   else
-    hipLaunchKernelGGL(csr_dense_share_kernel<short>, dim3((m + 127) / 128), dim3(kShareThreads), 0, s, m, k, nonzeros, row_offsets, static_cast<const short*>(column_indices), dense_min, dense_nonzeros);
+    hipLaunchKernelGGL(csr_dense_share_kernel<short>, dim3(row_blocks * parts), dim3(kShareThreads), 0, s, m, k, nonzeros, row_offsets, static_cast<const short*>(column_indices), dense_min, dense_nonzeros, parts, block_counts, done);
   return iex::check_hip(hipGetLastError(), "csr_dense_share launch");
+}
+
+size_t iex_csr_dense_share_scratch_bytes(int m, int k) {
+  if (m <= 0 || k <= 0) return 0;
+  const size_t row_blocks = ((size_t)m + 127) / 128, tiles = ((size_t)k + 127) / 128;
+  return row_blocks >= 512 ? 0 : row_blocks * (tiles + 1) * sizeof(int);   // (512 row blocks fill the chip by themselves)
 }
 
 int iex_csr_check(int itype, int m, int k, int nonzeros, const int* row_offsets, const void* column_indices, int* status, void* stream) {

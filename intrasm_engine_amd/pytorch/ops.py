@@ -125,6 +125,12 @@ def _row_histogram_host(row_offsets):
     return tuple(int(x) for x in hist.tolist())
 
 
+def _share_scratch(lib, row_offsets, k):
+    """Zeroed memory with which ``iex_csr_dense_share`` counts a block of rows by several workgroups (None: not needed)."""
+    need = lib.iex_csr_dense_share_scratch_bytes(row_offsets.numel() - 1, int(k))
+    return torch.zeros(need, dtype=torch.uint8, device=row_offsets.device) if need else None
+
+
 def _dense_share_host(row_offsets, column_indices, k, dense_min=None):
     """Share of the nonzeros that sit in 128 x 128 blocks holding ``dense_min`` of them or more (``iex_csr_dense_share``;
     one small launch and a synchronising read), or None where the kernel does not apply (more than 65536 columns)."""
@@ -134,9 +140,12 @@ def _dense_share_host(row_offsets, column_indices, k, dense_min=None):
     dense_min = _STRUCTURE_BLOCK_NONZEROS if dense_min is None else dense_min
     count = torch.zeros(1, dtype=torch.int32, device=row_offsets.device)
     with torch.cuda.device(row_offsets.device):
-        rc = _lib.load().iex_csr_dense_share(1 if column_indices.dtype == torch.int16 else 0, row_offsets.numel() - 1, int(k), nonzeros,
-                                             row_offsets.data_ptr(), column_indices.data_ptr(), int(dense_min), count.data_ptr(),
-                                             _stream_ptr(row_offsets.device))
+        lib = _lib.load()
+        scratch = _share_scratch(lib, row_offsets, k)
+        rc = lib.iex_csr_dense_share(1 if column_indices.dtype == torch.int16 else 0, row_offsets.numel() - 1, int(k), nonzeros,
+                                     row_offsets.data_ptr(), column_indices.data_ptr(), int(dense_min), count.data_ptr(),
+                                     scratch.data_ptr() if scratch is not None else None, scratch.numel() if scratch is not None else 0,
+                                     _stream_ptr(row_offsets.device))
     _lib.check(rc, "csr_dense_share")
     return int(count.item()) / nonzeros
 
@@ -222,8 +231,11 @@ def _look(row_offsets, column_indices, k):
         if m > 0:
             _lib.check(lib.iex_csr_row_histogram(m, row_offsets.data_ptr(), buf.data_ptr() + 4, stream), "csr_row_histogram")
         if with_share:
+            scratch = _share_scratch(lib, row_offsets, k)
             _lib.check(lib.iex_csr_dense_share(itype, m, int(k), nonzeros, row_offsets.data_ptr(), column_indices.data_ptr(),
-                                               _STRUCTURE_BLOCK_NONZEROS, buf.data_ptr() + 68, stream), "csr_dense_share")
+                                               _STRUCTURE_BLOCK_NONZEROS, buf.data_ptr() + 68,
+                                               scratch.data_ptr() if scratch is not None else None,
+                                               scratch.numel() if scratch is not None else 0, stream), "csr_dense_share")
     got = buf.tolist()
     status = int(got[0])
     if status & _lib.CSR_BAD_OFFSETS:

@@ -220,7 +220,9 @@ def test_structure_settles_the_kernel(dev):
 def test_dense_share_kernel_counts_like_numpy(dev, idtype):
     """iex_csr_dense_share against a numpy count, for several thresholds, on a band with scattered entries, a random
     mask, a ragged shape (m and k no multiples of 128) and an empty pattern."""
+    from intrasm_engine_amd import _lib
     from intrasm_engine_amd.pytorch import ops as pyops
+    lib = _lib.load()
     rng = np.random.default_rng(3)
     band, *_ = W.config3(tokens=1024, heads=1, band=96, extra=6)
     ro, ci = W.csr_from_row_lengths(rng, 700, 1000, rng.integers(0, 300, 700))
@@ -234,6 +236,17 @@ def test_dense_share_kernel_counts_like_numpy(dev, idtype):
         for dense_min in (1, 1536, 2048, 5000, 16384, 16385):
             want = counts[counts >= dense_min].sum() / csr.nnz
             assert abs(pyops._dense_share_host(ro_t, ci_t, csr.k, dense_min) - want) < 1e-9, dense_min
+            # the entry point itself: one workgroup per block of rows (no scratch memory, or too little), several (zeroed scratch)
+            need = lib.iex_csr_dense_share_scratch_bytes(csr.m, csr.k)
+            assert need == ((csr.m + 127) // 128) * (tiles_n + 1) * 4
+            for scratch in (None, torch.zeros(need - 4, dtype=torch.uint8, device=dev), torch.zeros(need, dtype=torch.uint8, device=dev)):
+                got = torch.zeros(1, dtype=torch.int32, device=dev)
+                rc = lib.iex_csr_dense_share(1 if idtype == torch.int16 else 0, csr.m, csr.k, csr.nnz, ro_t.data_ptr(), ci_t.data_ptr(), dense_min,
+                                             got.data_ptr(), scratch.data_ptr() if scratch is not None else None,
+                                             scratch.numel() if scratch is not None else 0, torch.cuda.current_stream().cuda_stream)
+                assert rc == 0, _lib.last_error()
+                assert int(got.item()) == int(counts[counts >= dense_min].sum()), (dense_min, None if scratch is None else scratch.numel())
+    assert lib.iex_csr_dense_share_scratch_bytes(128 * 512, 4096) == 0   # 512 blocks of rows fill the chip by themselves
     empty = torch.zeros(65, dtype=torch.int32, device=dev)
     assert pyops._dense_share_host(empty, torch.zeros(0, dtype=idtype, device=dev), 64) is None
 

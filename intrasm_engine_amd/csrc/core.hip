@@ -63,10 +63,29 @@ __global__ __launch_bounds__(256) void csr_check_kernel(int m, int k, int nnz, c
   int bad = 0;
   if (s < 0 || e < s || e > nnz || (r == 0 && s != 0) || (r == m - 1 && e != nnz)) bad |= IEX_CSR_BAD_OFFSETS;
   if (!bad) {
-    for (int j = s + lane; j < e; j += 64) {
-      const int c = (int)cols[j];
-      if (c < 0 || c >= k) bad |= IEX_CSR_COLUMN_OUT_OF_RANGE;
-      if (j > s && (int)cols[j - 1] >= c) bad |= IEX_CSR_NOT_ASCENDING;
+    // 256 columns per step (four loads in flight); a column's left neighbour comes from the lane before, the last
+    // lane of the chunk before, or -- across steps -- the carried last column of the step before
+    int carry = 0;
+    for (int base = s; base < e; base += 256) {
+      int c[4];
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        const int j = base + u * 64 + lane;
+        c[u] = j < e ? (int)cols[j] : 0;
+      }
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        if (base + u * 64 >= e) break;   // (uniform)
+        const int j = base + u * 64 + lane;
+        int before = __shfl_up(c[u], 1, 64);
+        const int chunk_before = u == 0 ? carry : __builtin_amdgcn_readlane(c[u > 0 ? u - 1 : 0], 63);
+        if (lane == 0) before = chunk_before;
+        if (j < e) {
+          if (c[u] < 0 || c[u] >= k) bad |= IEX_CSR_COLUMN_OUT_OF_RANGE;
+          if (j > s && before >= c[u]) bad |= IEX_CSR_NOT_ASCENDING;
+        }
+      }
+      carry = __builtin_amdgcn_readlane(c[3], 63);
     }
   }
   if (bad) atomicOr(status, bad);

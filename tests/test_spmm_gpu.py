@@ -785,6 +785,39 @@ def test_dense_form_path_splits_k_where_the_product_has_few_tiles(oracle, dev):
     assert_close(unsplit.float().cpu().numpy(), want, scale, RTOL[dtype], "dense form, unsplit")
 
 
+@pytest.mark.parametrize("idtype", [torch.int32, torch.int16])
+def test_csr_check_finds_one_fault_wherever_it_sits(dev, idtype):
+    """The check kernel reads 256 columns of a row per step, in four chunks of 64 whose left neighbours come from three
+    places (the lane before, the chunk before, the step before): a single swapped pair, a single repeated column and a
+    single column outside the matrix are found at every such seam of a long row, in a row of the middle of the matrix
+    and in the last one, and a clean pattern reads 0."""
+    from intrasm_engine_amd import _lib
+    from intrasm_engine_amd.pytorch import ops as pyops
+    rng = np.random.default_rng(23)
+    m, k = 9, 2000
+    lens = np.array([700, 0, 1, 64, 256, 257, 700, 65, 700])
+    ro, ci = W.csr_from_row_lengths(rng, m, k, lens)
+    rot = torch.from_numpy(ro).to(dev)
+    assert pyops.csr_check(rot, torch.from_numpy(ci).to(dev).to(idtype), k) == 0
+    for r in (0, 6, 8):
+        for at in (1, 63, 64, 65, 127, 128, 255, 256, 257, 319, 320, 511, 512, 513, 699):
+            j = ro[r] + at
+            swapped = ci.copy()
+            swapped[j - 1], swapped[j] = ci[j], ci[j - 1]
+            assert pyops.csr_check(rot, torch.from_numpy(swapped).to(dev).to(idtype), k) == _lib.CSR_NOT_ASCENDING, (r, at)
+            twice = ci.copy()
+            twice[j] = ci[j - 1]
+            assert pyops.csr_check(rot, torch.from_numpy(twice).to(dev).to(idtype), k) == _lib.CSR_NOT_ASCENDING, (r, at)
+            out = ci.copy()
+            out[j] = k
+            assert pyops.csr_check(rot, torch.from_numpy(out).to(dev).to(idtype), k) & _lib.CSR_COLUMN_OUT_OF_RANGE, (r, at)
+    # the first column of a row is compared with nothing: every row starts below the last column of the row before
+    low = ci.copy()
+    for r in (2, 3, 4, 5, 6, 7, 8):
+        low[ro[r]] = 0
+    assert pyops.csr_check(rot, torch.from_numpy(low).to(dev).to(idtype), k) == 0
+
+
 def test_csr_check_names_what_a_pattern_lacks(dev):
     """``iex_csr_check``: 0 for what ``dense_to_sparse`` produces; unsorted or duplicated columns (valid for the row
     kernel and for the reference, not for the other families), a column outside the matrix, offsets that do not run

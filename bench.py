@@ -664,13 +664,19 @@ def run_extras(torch, ops, dev, W, IL, mats, dens, csr_dev, time_cell, time_cold
             by = W.spmm_bytes(c.m, c.k, n, c.nnz, 1, 2, 2)
             fl = W.spmm_flops(c.nnz, n)
             rows.append({"sparsity": s, "n": n, "us": round(us, 2), "GBps": round(by / us / 1e3, 1),
-                         "hbm_frac": round(by / us / 1e3 / HBM_PEAK_GBPS, 4), "GFLOPs": round(fl / us / 1e3, 1)})
+                         "hbm_frac": round(by / us / 1e3 / HBM_PEAK_GBPS, 4), "GFLOPs": round(fl / us / 1e3, 1),
+                         "kernel": kernel_of(calls16[(s, n)])})
     out["cells_fp16_i16"] = rows
-    # the same 15 launches as one graph: on one branch, and on two (cells in order of nnz * n dealt alternately)
+    # the same 15 launches as one graph: on one branch, and on two -- the cells that run on the matrix cores (dense form
+    # + GEMM) on one, the gather-bound ones on the other, as in the timed fp32 step; and dealt alternately by nnz * n
     order16 = sorted(calls16, key=lambda c: -mats[c[0]].nnz * c[1])
+    on_mc = [c for c in order16 if "gemm" in next(r["kernel"] for r in rows if (r["sparsity"], r["n"]) == c)]
+    rest = [c for c in order16 if c not in on_mc]
     out["sweep_fp16_i16"] = {
         "one_branch_us": round(IL.run_non_interleaving([calls16[c] for c in calls16]) * 1e3, 1),
-        "two_branches_us": round(IL.run_interleaving([calls16[c] for c in order16[0::2]], [calls16[c] for c in order16[1::2]]) * 1e3, 1),
+        "two_branches_us": round(IL.run_interleaving([calls16[c] for c in on_mc], [calls16[c] for c in rest]) * 1e3, 1) if on_mc and rest else None,
+        "two_branches_are": f"{len(on_mc)} cells on the matrix cores (dense form + GEMM) | {len(rest)} gather-bound cells",
+        "two_branches_dealt_alternately_us": round(IL.run_interleaving([calls16[c] for c in order16[0::2]], [calls16[c] for c in order16[1::2]]) * 1e3, 1),
         "sum_of_cells_us": round(sum(r["us"] for r in rows), 1)}
     log("[bench] fp16 sweep done")
 

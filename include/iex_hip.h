@@ -181,7 +181,7 @@ int iex_spmm_ex(int dtype, int itype, int flags, int m, int k, int n, int nonzer
  * be distinct).  Needs values shared by the batch and k and n multiples of 8 (bias, ReLU and
  * accumulation ride in the GEMM's epilogue); anything else, and a NULL or short workspace, runs
  * exactly as iex_spmm_ex.  Where the product has few tiles and a long k (iex_gemm_ws) the size asked for includes,
- * behind the dense form rounded up to 256 bytes, the room the GEMM wants for splitting k over two workgroups per
+ * behind the dense form rounded up to 256 bytes, the room the GEMM wants for splitting k over several workgroups per
  * tile; a 16-byte aligned workspace of m * k * 2 bytes still runs the path, without the split.
  * IEX_SPMM_FORCE_VARIANT(7) asks for that path and fails where it cannot run.
  * iex_spmm_workspace_bytes returns the size with which the call described would use the workspace,
@@ -357,7 +357,7 @@ int iex_csr_softmax(int dtype, int m, int nonzeros, const int* row_indices,
  * 8 = 128x128 and 9 = 64x128 by eight waves with K steps of 64 (few tiles, long K), 10 = 128x256 by eight waves
  * (11: with K steps of 64), 12 = 256x256 with K split over two workgroups per tile (iex_gemm_ws only), 13 = 256x256 by
  * eight waves in two groups that take turns: one reads operand fragments and issues loads while the other multiplies,
- * 14 = 64x128 by eight waves with K split over two workgroups per tile (iex_gemm_ws only),
+ * 14 = 64x128 by eight waves with K split over two to eight workgroups per tile (iex_gemm_ws only),
  * all with the operands loaded from global memory straight into LDS (0 = choose picks among 5, 8, 9, 10 and 13, and
  * 14 where iex_gemm_ws got the room iex_gemm_workspace_bytes asks for);
  * 1 = 128x128, 2 = 128x256, 3 = 256x256, 4 = 128x128 with K steps of 64, operands staged through
@@ -368,20 +368,25 @@ int iex_gemm(int dtype, int trans_b, int M, int N, int K, const void* A, const v
              long long stride_c, void* stream);
 
 /* iex_gemm with a workspace in device memory that the call may use (and overwrite) until the work it
- * puts on `stream` has run.  Used by the two kernels that split K over two workgroups per tile: shape code 14
- * (bits 4..7 of trans_b; 64 x 128 tiles), which the library also picks by itself for products with few tiles and a
- * long K (64 tiles or fewer and K >= 4096, 128 or fewer and K >= 8192: half the CUs or more would idle; 4096 x 128 x
- * 4096 23.7 -> 20.2 us, 512 x 512 x 8192 43 -> 29 us), and code 12 (256 x 256 tiles), which runs on request only
- * (measured on the product it was built for, 4096 x 2048 x 4096: slower than what iex_gemm picks by itself).  The
- * first of a tile's two workgroups to finish leaves its fp32 partial sums in the workspace (M * N * 4 bytes rounded
- * up to whole tiles, plus two words per tile; 256-byte aligned), the other adds them to its own and stores the tile;
- * the result does not depend on which was first.  The second workgroup's wait is bounded; if it ever gave up, the tile
- * is left unwritten and its "written" word (the second half of the words behind the partial sums) reads -1 after the
- * launch instead of 1: stale sums are never added.  The exchange goes through the L2 of the XCD that both workgroups
- * run on (workgroup ids b and b + 8: ids are dealt round-robin to the 8 XCDs in the mode this library is
- * built for, one partition spanning the whole GPU).  K >= 128 (code 12: 64), plain store.  Codes 12 and 14 fail without the
- * workspace; code 0 without it (or with one too small) runs exactly as iex_gemm; every other code ignores it.
- * iex_gemm_workspace_bytes returns 0 where the workspace would not be used.  Neither call allocates.
+ * puts on `stream` has run.  Used by the kernels that split K over several workgroups per tile.
+ * Shape code 14 (bits 4..7 of trans_b): 64 x 128 tiles with K in two to eight parts, which the library also picks by
+ * itself for products with few tiles and a long K (64 tiles or fewer, or 128 or fewer and K >= 4096; every part at
+ * least 1024 of K; as many parts as give every CU a workgroup: 4096 x 128 x 4096 23.8 -> 17.1 us in 4 parts, 512 x 512 x
+ * 8192 42.5 -> 17.6 us in 8).  Every workgroup leaves its fp32 partial sums in the workspace and draws a ticket; the one
+ * that draws a tile's last ticket adds the parts up in the order of the parts and stores the tile, so the result does
+ * not depend on which workgroup was last, and nobody waits for anybody.  Workspace: tiles * parts * 64 * 128 * 4 bytes,
+ * then a ticket word per tile; 256-byte aligned.
+ * Shape code 12: 256 x 256 tiles with K in two halves, on request only (measured on the product it was built for, 4096 x
+ * 2048 x 4096: slower than what iex_gemm picks by itself).  The first of a tile's two workgroups to finish leaves its
+ * partial sums in the workspace (M * N * 4 bytes rounded up to whole tiles, plus two words per tile), the other adds
+ * them to its own and stores.  The second workgroup's wait is bounded; if it ever gave up, the tile is left unwritten and
+ * its "written" word (the second half of the words behind the partial sums) reads -1 after the launch instead of 1:
+ * stale sums are never added.
+ * Both exchange through the L2 of the XCD that the workgroups of a tile run on (workgroup ids that differ by multiples
+ * of 8: ids are dealt round-robin to the 8 XCDs in the mode this library is built for, one partition spanning the whole
+ * GPU).  Plain store; a K step for every part.  Codes 12 and 14 fail without the workspace; code 0 without it (or with one
+ * too small) runs exactly as iex_gemm; every other code ignores it.  iex_gemm_workspace_bytes returns 0 where the
+ * workspace would not be used.  Neither call allocates.
  * No counterpart in the reference (its dense companions are library calls). */
 int iex_gemm_ws(int dtype, int trans_b, int M, int N, int K, const void* A, const void* B,
                 void* C, int batch, long long stride_a, long long stride_b,

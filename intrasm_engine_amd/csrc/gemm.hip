@@ -131,7 +131,7 @@ __global__ __launch_bounds__(WCN * 128, 1) void gemm_dma_splitk_kernel(GemmParam
     q.A = static_cast<const unsigned short*>(p.A) + first;
     q.B = static_cast<const unsigned short*>(p.B) + (TRANS_B ? (size_t)first : (size_t)first * p.N);
   }
-  gemm_tile_dma<BF16, TRANS_B, WM, WN, WCN, BK, STAGES, true>(q, tile_m, tile_n, blockIdx.y, smem);
+  gemm_tile_dma<BF16, TRANS_B, WM, WN, WCN, BK, STAGES, 1>(q, tile_m, tile_n, blockIdx.y, smem);
 }
 
 // Workspace of a K split: the partial sums of one half per tile (fp32), then two words per tile (ticket, "written").
@@ -169,27 +169,100 @@ int launch_dma_splitk(GemmParams p, int batch, void* ws, bool flags_are_zero, hi
   return check_hip(hipGetLastError(), "gemm (split K) launch");
 }
 
-// Few 64 x 128 tiles and a long K: the K loop in two halves on twice the CUs.  Measured on MI355X (fp16, us, 64 x 128
-// tiles unsplit / split, the split with a launch that zeroes the tile words): 4096 x 64 x 4096 24.0 / 20.5, 4096 x 128 x
-// 4096 23.7 / 20.2, 2048 x 256 x 4096 23.5 / 19.8, 1000 x 200 x 4104 23.6 / 18.4, 512 x 512 x 8192 43.2 / 28.8 (64 tiles or
-// fewer); 4096 x 256 x 11008 57.2 / 45.6, but 4096 x 256 x 4096 24.9 / 24.6, 4 x (1024 x 256 x 4096) 25.5 / 24.5, 4096 x
-// 256 x 2048 13.6 / 17.2, 8192 x 128 x 2048 14.8 / 18.5 (128 tiles: only a very long K pays for the exchange).
+// ---- K split over several workgroups per tile, every part on one XCD, the last to finish adds up (gemm_dma_device.cuh)
+template <bool BF16, bool TRANS_B, int WM, int WN, int WCN, int BK, int STAGES>
+__global__ __launch_bounds__(WCN * 128, (WCN == 2 && WM * WN <= 8 && gemm_dma_lds_bytes<WM, WN, WCN, BK, STAGES>() <= 80 * 1024 ? 2 : 1)) void gemm_dma_parts_kernel(GemmParams p) {
+  extern __shared__ __align__(16) unsigned char smem[];
+  const int b = blockIdx.x, parts = p.split_parts;
+  const int part = (b >> 3) % parts, slot = ((b >> 3) / parts) * kXcds + (b & 7);
+  int tile_m, tile_n;
+  if (!xcd_tile(slot, p.tiles_m, p.tiles_n, tile_m, tile_n)) return;  // uniform per block
+  const int steps = (p.K + BK - 1) / BK, per = (steps + parts - 1) / parts * BK;   // K entries per part: whole steps
+  const int k0 = part * per;   // (the host has chosen parts so that every part has a step)
+  GemmParams q = p;
+  q.ldk = p.K;
+  q.split_part = part;
+  q.K = min(per, p.K - k0);
+  q.A = static_cast<const unsigned short*>(p.A) + k0;
+  q.B = static_cast<const unsigned short*>(p.B) + (TRANS_B ? (size_t)k0 : (size_t)k0 * p.N);
+  gemm_tile_dma<BF16, TRANS_B, WM, WN, WCN, BK, STAGES, 2>(q, tile_m, tile_n, blockIdx.y, smem);
+}
+
+// Parts per tile: as many as give every CU a workgroup, at most 8, every part at least 1024 of K, none empty.
+inline int split_parts_for(int M, int N, int K, int batch, int bm, int bn, int bk) {
+  const long long tiles = (long long)ceil_div(M, bm) * ceil_div(N, bn) * batch;
+  const int steps = ceil_div(K, bk);
+  int parts = (int)std::min<long long>(8, 256 / std::max<long long>(tiles, 1));
+  parts = std::min(parts, K / 1024);
+  while (parts > 1 && (parts - 1) * ceil_div(steps, parts) >= steps) --parts;
+  return std::max(parts, 1);
+}
+
+// Workspace: per tile `parts` sets of partial sums (fp32), then one ticket word per tile.
+inline size_t gemm_parts_bytes(int M, int N, int batch, int bm, int bn, int parts) {
+  const size_t tiles = (size_t)ceil_div(M, bm) * ceil_div(N, bn) * batch;
+  return tiles * parts * bm * bn * sizeof(float) + ((tiles * sizeof(int) + 255) / 256) * 256;
+}
+
+template <bool BF16, bool TRANS_B, int WM, int WN, int WCN, int BK, int STAGES>
+int launch_dma_parts(GemmParams p, int batch, int parts, void* ws, bool flags_are_zero, hipStream_t stream) {
+  constexpr int BM = 2 * WM * 32, BN = WCN * WN * 32;
+  p.tiles_m = ceil_div(p.M, BM);
+  p.tiles_n = ceil_div(p.N, BN);
+  const int total = p.tiles_m * p.tiles_n;
+  const int per_xcd = (total + kXcds - 1) / kXcds;
+  p.split_parts = parts;
+  p.split_ws = static_cast<float*>(ws);
+  p.split_flags = reinterpret_cast<int*>(static_cast<unsigned char*>(ws) + (size_t)total * batch * parts * BM * BN * sizeof(float));
+  constexpr int lds = gemm_dma_lds_bytes<WM, WN, WCN, BK, STAGES>();
+  auto kern = gemm_dma_parts_kernel<BF16, TRANS_B, WM, WN, WCN, BK, STAGES>;
+  if (lds > 64 * 1024) {
+    static thread_local bool raised = false;  // per instantiation
+    if (!raised) {
+      if (int rc = check_hip(hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, lds),
+                             "hipFuncSetAttribute(LDS size)"))
+        return rc;
+      raised = true;
+    }
+  }
+  if (!flags_are_zero) {
+    note_kernel("fill_zero_kernel");
+    hipLaunchKernelGGL(fill_zero_kernel, dim3(ceil_div(total * batch, 256)), dim3(256), 0, stream, p.split_flags, total * batch);
+  }
+  note_kernel("gemm_dma_parts_kernel<%s, %s> (%d x %d tiles, K in %d parts)", BF16 ? "bf16" : "f16", TRANS_B ? "B(N,K)" : "B(K,N)", BM, BN, parts);
+  hipLaunchKernelGGL(kern, dim3(per_xcd * kXcds * parts, batch), dim3(WCN * 128), lds, stream, p);
+  return check_hip(hipGetLastError(), "gemm (K in parts) launch");
+}
+
+// Few 64 x 128 tiles and a long K: the K loop in parts, on as many CUs as there are.  Measured on MI355X (fp16, us, 64 x
+// 128 tiles unsplit / in parts, the latter with a launch that zeroes the tickets): 4096 x 128 x 4096 23.8 / 17.1 (4 parts),
+// 2048 x 256 x 4096 23.4 / 15.2 (4), 1000 x 200 x 4104 23.6 / 14.1 (8), 512 x 512 x 8192 42.5 / 17.6 (8), 4096 x 256 x 11008
+// 57.1 / 45.6 (2), 4096 x 256 x 4096 24.0 / 21.8 (2), 4 x (1024 x 256 x 4096) 24.9 / 23.1 (2); but 4096 x 256 x 2048 13.5 /
+// 14.4 and 8192 x 128 x 2048 14.1 / 15.2 (128 tiles in 2 parts: K must be long to pay).  128 x 128 tiles by four
+// wavefronts in 4 to 8 parts: 22.7 where 64 x 128 tiles take 16.3.
 inline bool auto_split_wanted(int M, int N, int K, int batch) {
+  if (K <= 256) return false;
   if ((long long)ceil_div(M, 128) * ceil_div(N, 128) * batch > 256) return false;
   const long long half_tiles = (long long)ceil_div(M, 64) * ceil_div(N, 128) * batch;
-  return (half_tiles <= 64 && K >= 4096) || (half_tiles <= 128 && K >= 8192);
+  if (half_tiles > 128 || (half_tiles > 64 && K < 4096)) return false;
+  return split_parts_for(M, N, K, batch, 64, 128, 64) >= 2;
 }
 
 template <bool BF16, bool TRANS_B>
 int launch_shape(const GemmParams& p, int batch, int force, hipStream_t stream, void* ws, size_t ws_bytes, bool flags_are_zero) {
-  auto ws_fits = [&](int bm, int bn) { return ws && aligned(ws, 256) && ws_bytes >= gemm_splitk_bytes(p.M, p.N, batch, bm, bn); };
-  if (force == 12 || force == 14) {
-    const int bm = force == 12 ? 256 : 64, bn = force == 12 ? 256 : 128;
-    IEX_REQUIRE(p.K >= (force == 12 ? 64 : 128), IEX_ERR_UNSUPPORTED, "gemm: the K-split kernels need two K steps (K >= %d; K=%d)", force == 12 ? 64 : 128, p.K);
-    IEX_REQUIRE(ws_fits(bm, bn) && !p.accumulate, IEX_ERR_BAD_ARGUMENT, "gemm: the K-split kernels need a 256-byte aligned workspace of %zu bytes (iex_gemm_ws) and a plain store",
-                gemm_splitk_bytes(p.M, p.N, batch, bm, bn));
-    if (force == 12) return launch_dma_splitk<BF16, TRANS_B, 4, 4, 2, 32, 4>(p, batch, ws, flags_are_zero, stream);
-    return launch_dma_splitk<BF16, TRANS_B, 1, 1, 4, 64, 4>(p, batch, ws, flags_are_zero, stream);
+  if (force == 12) {
+    IEX_REQUIRE(p.K >= 64, IEX_ERR_UNSUPPORTED, "gemm: the K-split kernel needs two K steps (K >= 64; K=%d)", p.K);
+    IEX_REQUIRE(ws && aligned(ws, 256) && ws_bytes >= gemm_splitk_bytes(p.M, p.N, batch, 256, 256) && !p.accumulate, IEX_ERR_BAD_ARGUMENT,
+                "gemm: the K-split kernel needs a 256-byte aligned workspace of %zu bytes (iex_gemm_ws) and a plain store", gemm_splitk_bytes(p.M, p.N, batch, 256, 256));
+    return launch_dma_splitk<BF16, TRANS_B, 4, 4, 2, 32, 4>(p, batch, ws, flags_are_zero, stream);
+  }
+  if (force == 14) {
+    const int parts = std::max(2, split_parts_for(p.M, p.N, p.K, batch, 64, 128, 64)), steps = ceil_div(p.K, 64);
+    IEX_REQUIRE(steps >= parts && (parts - 1) * ceil_div(steps, parts) < steps, IEX_ERR_UNSUPPORTED,
+                "gemm: K in %d parts needs a K step of 64 for every part (K=%d)", parts, p.K);
+    IEX_REQUIRE(ws && aligned(ws, 256) && ws_bytes >= gemm_parts_bytes(p.M, p.N, batch, 64, 128, parts) && !p.accumulate, IEX_ERR_BAD_ARGUMENT,
+                "gemm: K in parts needs a 256-byte aligned workspace of %zu bytes (iex_gemm_ws) and a plain store", gemm_parts_bytes(p.M, p.N, batch, 64, 128, parts));
+    return launch_dma_parts<BF16, TRANS_B, 1, 1, 4, 64, 4>(p, batch, parts, ws, flags_are_zero, stream);
   }
   if (force == 1) return launch<BF16, TRANS_B, 2, 2>(p, batch, stream);
   if (force == 2) return launch<BF16, TRANS_B, 2, 4>(p, batch, stream);
@@ -242,9 +315,12 @@ int launch_shape(const GemmParams& p, int batch, int force, hipStream_t stream, 
   // Half as tall (64 x 128) where even that leaves at most one tile per CU: twice the CUs at work
   // (4096 x 256 x 4096: 35 -> 27.5 us, 4096 x 512 x 4096: 35 -> 30, 1024 x 2048 x 1024: 13.9 -> 12.4).
   const long long half_tiles = (long long)ceil_div(p.M, 64) * ceil_div(p.N, 128) * batch;
-  // ... and with room for the partial sums, K in two halves where that still leaves at most one workgroup per CU
-  if (auto_split_wanted(p.M, p.N, p.K, batch) && ws_fits(64, 128) && !p.accumulate)
-    return launch_dma_splitk<BF16, TRANS_B, 1, 1, 4, 64, 4>(p, batch, ws, flags_are_zero, stream);
+  // ... and with room for the partial sums, K in parts on as many CUs as there are
+  if (auto_split_wanted(p.M, p.N, p.K, batch) && !p.accumulate) {
+    const int parts = split_parts_for(p.M, p.N, p.K, batch, 64, 128, 64);
+    if (ws && aligned(ws, 256) && ws_bytes >= gemm_parts_bytes(p.M, p.N, batch, 64, 128, parts))
+      return launch_dma_parts<BF16, TRANS_B, 1, 1, 4, 64, 4>(p, batch, parts, ws, flags_are_zero, stream);
+  }
   if (half_tiles <= 256 && p.K >= 512) return launch_dma<BF16, TRANS_B, 1, 1, 64, 4, 4>(p, batch, stream);
   if (p.K >= 2048) return launch_dma<BF16, TRANS_B, 2, 1, 64, 4, 4>(p, batch, stream);
   return launch_dma<BF16, TRANS_B, 2, 2, 32, 4>(p, batch, stream);
@@ -258,7 +334,7 @@ int launch_shape(const GemmParams& p, int batch, int force, hipStream_t stream, 
 // straight into LDS: 5 = 128x128, 6 = 128x256, 7 = 256x256, 8 = 128x128, 9 = 64x128 by eight waves with K steps of 64,
 // 10 = 128x256 by eight waves, 11 = the same with K steps of 64, 12 = 256x256 with K split over two workgroups per tile
 // (iex_gemm_ws only; never chosen), 13 = 256x256 by eight waves in two groups that alternate between loading and
-// multiplying, 14 = 64x128 by eight waves with K split over two workgroups per tile (iex_gemm_ws only).
+// multiplying, 14 = 64x128 by eight waves with K split over two to eight workgroups per tile (iex_gemm_ws only).
 // 0 = choose (one of 5, 8, 9, 10, 13, and 14 where iex_gemm_workspace_bytes asked for room and got it).
 extern "C" int iex_gemm(int dtype, int trans_b_and_shape, int M, int N, int K, const void* A, const void* B, void* C, int batch,
                         long long stride_a, long long stride_b, long long stride_c, void* stream) {
@@ -277,18 +353,22 @@ extern "C" size_t iex_gemm_workspace_bytes(int dtype, int trans_b_and_shape, int
   if (M <= 0 || N <= 0 || K <= 0 || batch <= 0 || (dtype != IEX_F16 && dtype != IEX_BF16)) return 0;
   const int force = (trans_b_and_shape >> 4) & 0xf;
   if (force == 12) return iex::gemm_splitk_bytes(M, N, batch, 256, 256);
-  if (force == 14) return iex::gemm_splitk_bytes(M, N, batch, 64, 128);
+  if (force == 14) return iex::gemm_parts_bytes(M, N, batch, 64, 128, 8);
   return force == 0 ? iex::gemm_auto_split_bytes(M, N, K, batch) : 0;
 }
 
 size_t iex::gemm_auto_split_bytes(int M, int N, int K, int batch) {
-  return auto_split_wanted(M, N, K, batch) ? gemm_splitk_bytes(M, N, batch, 64, 128) : 0;
+  return auto_split_wanted(M, N, K, batch) ? gemm_parts_bytes(M, N, batch, 64, 128, split_parts_for(M, N, K, batch, 64, 128, 64)) : 0;
 }
 
-void iex::gemm_auto_split_flags(int M, int N, int batch, size_t* offset_bytes, int* words) {
+int iex::gemm_auto_split_parts(int M, int N, int K, int batch) {
+  return auto_split_wanted(M, N, K, batch) ? split_parts_for(M, N, K, batch, 64, 128, 64) : 1;
+}
+
+void iex::gemm_auto_split_flags(int M, int N, int K, int batch, size_t* offset_bytes, int* words) {
   const size_t tiles = (size_t)ceil_div(M, 64) * ceil_div(N, 128) * batch;
-  *offset_bytes = tiles * 64 * 128 * sizeof(float);
-  *words = (int)(2 * tiles);
+  *offset_bytes = tiles * split_parts_for(M, N, K, batch, 64, 128, 64) * 64 * 128 * sizeof(float);
+  *words = (int)tiles;
 }
 
 int iex::gemm_dispatch(int dtype, int trans_b_and_shape, int M, int N, int K, const void* A, const void* B, void* C, int batch,

@@ -42,6 +42,9 @@ struct GemmParams {
   int ldk = 0;
   float* split_ws = nullptr;
   int* split_flags = nullptr;
+  // K split over split_parts workgroups per tile, every one of which leaves its partial sums in the workspace and draws
+  // a ticket (zero at launch); the one that draws the last adds all parts up in the order of the parts and stores
+  int split_parts = 0, split_part = 0;
 };
 
 // iex_gemm with the epilogue options above (gemm.hip).
@@ -52,7 +55,8 @@ int gemm_dispatch(int dtype, int trans_b_and_shape, int M, int N, int K, const v
 // not split), and where in such a workspace the words sit that must be zero at launch (gemm_dispatch zeroes them with a
 // launch of its own unless the caller says it has: workspace_flags_are_zero).
 size_t gemm_auto_split_bytes(int M, int N, int K, int batch);
-void gemm_auto_split_flags(int M, int N, int batch, size_t* offset_bytes, int* words);
+int gemm_auto_split_parts(int M, int N, int K, int batch);   // parts of K that gemm_dispatch would use with that workspace (1: no split)
+void gemm_auto_split_flags(int M, int N, int K, int batch, size_t* offset_bytes, int* words);
 
 typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));

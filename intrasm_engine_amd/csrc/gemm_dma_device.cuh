@@ -66,7 +66,7 @@ __device__ __forceinline__ bool xcd_tile(int block, int tiles_m, int tiles_n, in
   return true;
 }
 
-template <bool BF16, bool TRANS_B, int WM, int WN, int WCN, int BK, int STAGES, bool SPLIT = false>
+template <bool BF16, bool TRANS_B, int WM, int WN, int WCN, int BK, int STAGES, int SPLIT = 0>
 __device__ __forceinline__ void gemm_tile_dma(const GemmParams& p, int tile_m, int tile_n, int z, unsigned char* smem) {
   constexpr int BM = 2 * WM * 32, BN = WCN * WN * 32, WAVES = 2 * WCN;
   constexpr int CPR = BK / 8;          // 16-byte chunks per K-contiguous row
@@ -258,7 +258,7 @@ __device__ __forceinline__ void gemm_tile_dma(const GemmParams& p, int tile_m, i
   wait_vmcnt<0>();  // the re-fetched last tiles: nothing may still be writing LDS when the workgroup ends
 
   const float* partial = nullptr;
-  if constexpr (SPLIT) {
+  if constexpr (SPLIT == 1) {
     // Two workgroups hold partial sums of this tile (one half of K each).  Whichever finishes first leaves its sums in
     // the workspace and is done; the other adds them to its own and stores the tile (a + b = b + a: the result does
     // not depend on who was first).  The second only ever waits for a workgroup that is past its K loop and waits for
@@ -307,6 +307,53 @@ __device__ __forceinline__ void gemm_tile_dma(const GemmParams& p, int tile_m, i
     if (*reinterpret_cast<volatile int*>(smem + 4) == 0) return;   // (uniform) the partner never published: leave the tile unwritten, flag = -1
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");   // (this CU has never read these lines: they come from L2)
     partial = mine;   // added where the sums are rounded and stored (adding them here would need all 256 sums in VGPRs at once)
+  }
+  if constexpr (SPLIT == 2) {
+    // split_parts workgroups hold partial sums of this tile (a stretch of K each).  Every one leaves its sums in the
+    // workspace, waits until L2 has acknowledged them and draws a ticket; nobody waits for anybody.  The workgroup that
+    // draws the last ticket finds all parts in L2 (the workgroups of a tile run on one XCD: the launcher's numbering),
+    // adds them up in the order of the parts -- its own included, read back, so that the sum does not depend on who was
+    // last -- and stores the tile.
+    constexpr int NMT = WM * WN;
+    const int parts = p.split_parts;
+    const int tile_id = (z * p.tiles_m + tile_m) * p.tiles_n + tile_n;
+    float* all = p.split_ws + (size_t)tile_id * parts * (BM * BN) + (size_t)wave * (NMT * 16 * 64) + lane * 4;
+    float* mine = all + (size_t)p.split_part * (BM * BN);
+#pragma unroll
+    for (int i = 0; i < WM; ++i)
+#pragma unroll
+      for (int j = 0; j < WN; ++j)
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+          const f32x4 v = {acc[i][j][q * 4], acc[i][j][q * 4 + 1], acc[i][j][q * 4 + 2], acc[i][j][q * 4 + 3]};
+          *reinterpret_cast<f32x4*>(mine + ((i * WN + j) * 4 + q) * 256) = v;
+        }
+    wait_vmcnt<0>();   // (vmcnt counts a store until L2 has acknowledged it)
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+    __syncthreads();   // everybody's sums are in L2, and everybody has read its last fragments: the stages are free
+    if (tid == 0) *reinterpret_cast<int*>(smem) = atomicAdd(&p.split_flags[tile_id], 1);
+    __syncthreads();
+    if (*reinterpret_cast<volatile int*>(smem) != parts - 1) return;   // (uniform)
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");   // (this CU has never read the other parts' lines: they come from L2)
+#pragma unroll
+    for (int i = 0; i < WM; ++i)
+#pragma unroll
+      for (int j = 0; j < WN; ++j)
+#pragma unroll
+        for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
+    for (int s = 0; s < parts; ++s) {
+      const float* from = all + (size_t)s * (BM * BN);
+#pragma unroll
+      for (int i = 0; i < WM; ++i)
+#pragma unroll
+        for (int j = 0; j < WN; ++j)
+#pragma unroll
+          for (int q = 0; q < 4; ++q) {
+            const f32x4 v = *reinterpret_cast<const f32x4*>(from + ((i * WN + j) * 4 + q) * 256);
+#pragma unroll
+            for (int e = 0; e < 4; ++e) acc[i][j][q * 4 + e] += v[e];
+          }
+    }
   }
   // the stages are free now: row-contiguous stores through LDS where the shape allows
   static_assert(WAVES * gemm_store_lds_bytes<WN>() <= gemm_dma_lds_bytes<WM, WN, WCN, BK, STAGES>(), "the epilogue fits the stages");

@@ -545,11 +545,14 @@ inline size_t dense_path_bytes(const SpmmParams& p) { return (size_t)p.m * p.k *
 //     per nonzero and tile (same shape at 93 % sparsity: 0.15 ms; 8 x 4096 x 4096, k = 128 at 50 %: 0.58
 //     against 0.17 for the dense form).
 // The dense form has to win by 15 % to be taken.  `few_columns`: the alternative is the few-columns kernel.
-inline bool dense_path_wins(const SpmmParams& p, int batch, int matrix_core_kind, bool few_columns) {
+// split_room: the workspace has room for the GEMM to take k in parts where it would (few tiles, long k: the K loop of a
+// tile then runs on several CUs; 4096^2 at 70-90 %, n = 128 / 256: 40 / 41 -> 27 / 32 us).
+inline bool dense_path_wins(const SpmmParams& p, int batch, int matrix_core_kind, bool few_columns, bool split_room = true) {
   const double cells = (double)p.m * p.k, flops = 2.0 * cells * p.n * batch;
   const double out_bytes = (double)p.m * p.n * batch * 2;
   const double tiles = (double)ceil_div(p.m, 128) * ceil_div(p.n, 128) * batch;
-  const double product = std::max({flops / 1000e12, std::ceil(tiles / 512.0) * (p.k / 32.0) * 0.23e-6, out_bytes / 3e12});
+  const int parts = split_room && !p.accumulate ? gemm_auto_split_parts(p.m, p.n, p.k, batch) : 1;
+  const double product = std::max({flops / 1000e12, std::ceil(tiles / 512.0) * (p.k / 32.0) * 0.23e-6 / parts, out_bytes / 3e12});
   const double dense_form = 8e-6 + cells * 2 / 4e12 + product;
   double other;
   if (few_columns) other = 8e-6 + out_bytes / 4.5e12 + (double)p.nnz * batch * ceil_div(p.n, 512) * 10.0 / (256 * 2.1e9);
@@ -564,14 +567,19 @@ inline bool dense_path_wins(const SpmmParams& p, int batch, int matrix_core_kind
 inline size_t dense_path_split_offset(const SpmmParams& p) { return (dense_path_bytes(p) + 255) & ~size_t(255); }
 inline size_t dense_path_split_bytes(const SpmmParams& p, int batch) { return p.accumulate ? 0 : gemm_auto_split_bytes(p.m, p.n, p.k, batch); }
 
+inline bool dense_path_has_split_room(const SpmmParams& p, int batch, const Choice& ch) {
+  const size_t split = dense_path_split_bytes(p, batch);
+  return split > 0 && ch.ws && aligned(ch.ws, 256) && ch.ws_bytes >= dense_path_split_offset(p) + split;
+}
+
 template <typename T, typename IT>
 int launch_dense_path(const SpmmParams& p, int batch, const Choice& ch, hipStream_t stream) {
   const size_t split = dense_path_split_bytes(p, batch), offset = dense_path_split_offset(p);
-  const bool with_split = split > 0 && aligned(ch.ws, 256) && ch.ws_bytes >= offset + split;
+  const bool with_split = dense_path_has_split_room(p, batch, ch);
   unsigned char* split_ws = with_split ? static_cast<unsigned char*>(ch.ws) + offset : nullptr;
   size_t flags_at = 0;
   int flag_words = 0;
-  if (with_split) gemm_auto_split_flags(p.m, p.n, batch, &flags_at, &flag_words);
+  if (with_split) gemm_auto_split_flags(p.m, p.n, p.k, batch, &flags_at, &flag_words);
   note_kernel("csr_to_dense_kernel<%s>", type_name<IT>());
   hipLaunchKernelGGL((csr_to_dense_kernel<IT>), dim3(p.m), dim3(kDenseThreads), 0, stream, p.m, p.k,
                      p.row_offsets, static_cast<const IT*>(p.cols), static_cast<const uint16_t*>(p.values),
@@ -597,7 +605,7 @@ int launch_typed(const SpmmParams& p, int batch, const Choice& given, hipStream_
   if (ch.variant == 0 && smallk_wanted<T>(p, batch)) {
     if constexpr (sizeof(T) == 2) {
       const bool room = ch.ws && aligned(ch.ws, 16) && ch.ws_bytes >= dense_path_bytes(p);
-      if (room && dense_path_fits(2, p, p.per_batch_values) && dense_path_wins(p, batch, 0, true))
+      if (room && dense_path_fits(2, p, p.per_batch_values) && dense_path_wins(p, batch, 0, true, dense_path_has_split_room(p, batch, ch)))
         return launch_dense_path<T, IT>(p, batch, ch, stream);
     }
     return launch_smallk<T, IT>(p, batch, stream);
@@ -617,7 +625,7 @@ int launch_typed(const SpmmParams& p, int batch, const Choice& given, hipStream_
       IEX_REQUIRE(room, IEX_ERR_BAD_ARGUMENT, "spmm: the dense-form path needs a 16-byte aligned workspace of %zu bytes (iex_spmm_ws)", dense_path_bytes(p));
       return launch_dense_path<T, IT>(p, batch, ch, stream);
     }
-    if (ch.variant == 0 && fits && room && dense_path_wins(p, batch, mc.kind, false)) return launch_dense_path<T, IT>(p, batch, ch, stream);
+    if (ch.variant == 0 && fits && room && dense_path_wins(p, batch, mc.kind, false, dense_path_has_split_room(p, batch, ch))) return launch_dense_path<T, IT>(p, batch, ch, stream);
   }
   // Where the 8-wave kernel would run: the direct-load kernel wins on 2:4 weights (4096 x 4096,
   // n = 8192: 0.37 against 0.40-0.46 ms with five windows), ties at 80 % sparsity (11008 x 4096:

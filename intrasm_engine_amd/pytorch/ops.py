@@ -43,7 +43,7 @@ def kernel_params(*, spmm: dict | None = None, sddmm: dict | None = None, gemm: 
     ``spmm`` = any of force_variant / force_rpw / force_nt / force_lpg / force_wpr (the tuning
     bits of ``iex_spmm_ex``) and beside_gather_kernel (true: the calls will share the chip with a gather-bound launch,
     ``IEX_SPMM_BESIDE_GATHER_KERNEL``), ``sddmm`` = force_wpr / force_variant, ``gemm`` = tile (the shape code of
-    ``iex_gemm``: 5 = 128x128, 6 = 128x256, 7 = 256x256 tiles, 8 = 128x128 and 9 = 64x128 by eight waves with K steps of 64, 10 = 128x256 by eight waves, 12 = 256x256 with K split over two workgroups per tile, 13 = 256x256 by eight waves in alternating phases, 14 = 64x128 with K split over two workgroups per tile; 1..4 = the
+    ``iex_gemm``: 5 = 128x128, 6 = 128x256, 7 = 256x256 tiles, 8 = 128x128 and 9 = 64x128 by eight waves with K steps of 64, 10 = 128x256 by eight waves, 12 = 256x256 with K split over two workgroups per tile, 13 = 256x256 by eight waves in alternating phases, 14 = 64x128 with K split over two to eight workgroups per tile; 1..4 = the
     register-staged kernels).
     Without a block, or for a key left out, the library chooses; a category left out (None) keeps
     what an enclosing block set for it.  A kernel family that cannot

@@ -143,18 +143,19 @@ def test_argument_checks(dev):
 
 @pytest.mark.parametrize("trans_b", [False, True])
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
-@pytest.mark.parametrize("mnk,batch", [((300, 520, 200), 1), ((260, 264, 1000), 3), ((512, 256, 64), 2), ((129, 136, 2048), 1)])
+@pytest.mark.parametrize("mnk,batch", [((300, 520, 200), 1), ((260, 264, 1000), 3), ((512, 256, 64), 2), ((129, 136, 2048), 1), ((70, 136, 8200), 1)])
 @pytest.mark.parametrize("split,whole", [(12, 7), (14, 9)])
 def test_k_split_over_two_workgroups(oracle, dev, trans_b, dtype, mnk, batch, split, whole):
-    """256 x 256 tiles (code 12) and 64 x 128 tiles (code 14) with K split over two workgroups per tile (partial sums
-    meet in a workspace, the second workgroup to arrive adds and stores), on request: ragged m, n, a K whose halves are
-    96 + 104 (128 + 72 with steps of 64), 512 + 488 (a partial last step), 32 + 32; batches; against the oracle, twice
-    with the same bits, and on integer operands exactly equal to the unsplit kernel of the same tile."""
+    """256 x 256 tiles with K in two halves (code 12) and 64 x 128 tiles with K in two to eight parts (code 14: partial
+    sums meet in a workspace, the last workgroup to arrive adds them up in the order of the parts and stores), on
+    request: ragged m, n, a K whose halves are 96 + 104 (128 + 72 with steps of 64), 512 + 488 (a partial last step),
+    32 + 32, a K of 2048 in two parts; batches; against the oracle, twice with the same bits, and on integer operands
+    exactly equal to the unsplit kernel of the same tile."""
     from intrasm_engine_amd.pytorch import ops as pyops
     rng = np.random.default_rng(batch)
     M, N, K = mnk
     if split == 14 and K < 128:
-        with pytest.raises(RuntimeError, match="two K steps"), pyops.kernel_params(gemm={"tile": 14}):
+        with pytest.raises(RuntimeError, match="K step of 64 for every part"), pyops.kernel_params(gemm={"tile": 14}):
             ops.gemm_mfma(torch.zeros(M, K, device=dev, dtype=dtype), torch.zeros(K, N, device=dev, dtype=dtype), False)
         return
     a_np = rng.standard_normal((batch, M, K)).astype(np.float32)
@@ -179,17 +180,18 @@ def test_k_split_over_two_workgroups(oracle, dev, trans_b, dtype, mnk, batch, sp
 
 
 def test_k_split_is_picked_for_few_tiles_and_a_long_k(oracle, dev):
-    """4096 x 128 x 4096 (64 tiles of 64 x 128 on 256 CUs): the operator asks the library how much room the split wants,
+    """4096 x 128 x 4096 (64 tiles of 64 x 128 on 256 CUs: K in four parts): the operator asks the library how much room the split wants,
     gets a number, passes the room and the split kernel runs; the entry point without a workspace runs the unsplit tile.
     Shapes with more tiles or a shorter K ask for nothing.  Twice the same bits; against the oracle on sampled rows."""
     from intrasm_engine_amd import _lib
     lib = _lib.load()
     M, N, K = 4096, 128, 4096
-    assert lib.iex_gemm_workspace_bytes(_lib.F16, 0, M, N, K, 1) == 64 * 64 * 128 * 4 + 512
-    assert lib.iex_gemm_workspace_bytes(_lib.F16, 14 << 4, M, N, K, 1) == 64 * 64 * 128 * 4 + 512
-    assert lib.iex_gemm_workspace_bytes(_lib.F16, 0, M, 256, K, 1) == 0          # 128 tiles, K < 8192
-    assert lib.iex_gemm_workspace_bytes(_lib.F16, 0, M, 256, 11008, 1) != 0      # 128 tiles, a very long K
-    assert lib.iex_gemm_workspace_bytes(_lib.F16, 0, M, N, 2048, 1) == 0
+    assert lib.iex_gemm_workspace_bytes(_lib.F16, 0, M, N, K, 1) == 64 * 4 * 64 * 128 * 4 + 256      # 64 tiles in 4 parts, a ticket per tile
+    assert lib.iex_gemm_workspace_bytes(_lib.F16, 14 << 4, M, N, K, 1) == 64 * 8 * 64 * 128 * 4 + 256  # on request: room for 8 parts
+    assert lib.iex_gemm_workspace_bytes(_lib.F16, 0, M, 256, K, 1) == 128 * 2 * 64 * 128 * 4 + 512    # 128 tiles in 2 parts
+    assert lib.iex_gemm_workspace_bytes(_lib.F16, 0, M, 256, 2048, 1) == 0        # 128 tiles and K < 4096
+    assert lib.iex_gemm_workspace_bytes(_lib.F16, 0, M, N, 2048, 1) == 64 * 2 * 64 * 128 * 4 + 256   # 64 tiles: two parts of 1024
+    assert lib.iex_gemm_workspace_bytes(_lib.F16, 0, M, N, 1024, 1) == 0
     assert lib.iex_gemm_workspace_bytes(_lib.F16, 0, M, N, K, 4) == 0            # four times the tiles
     assert lib.iex_gemm_workspace_bytes(_lib.F16, 9 << 4, M, N, K, 1) == 0       # another kernel on request
     rng = np.random.default_rng(9)
@@ -197,7 +199,7 @@ def test_k_split_is_picked_for_few_tiles_and_a_long_k(oracle, dev):
     b_np = rng.standard_normal((K, N)).astype(np.float32)
     a, b = torch.from_numpy(a_np).to(dev).half(), torch.from_numpy(b_np).to(dev).half()
     out = ops.gemm_mfma(a, b, False)
-    assert "gemm_dma_splitk_kernel" in _lib.last_kernels() and "64 x 128" in _lib.last_kernels()
+    assert "gemm_dma_parts_kernel" in _lib.last_kernels() and "64 x 128 tiles, K in 4 parts" in _lib.last_kernels()
     assert torch.equal(out, ops.gemm_mfma(a, b, False))
     rows = np.arange(0, M, 61)
     a_r, b_r = rounded(a_np[rows], torch.float16), rounded(b_np, torch.float16)
@@ -205,7 +207,7 @@ def test_k_split_is_picked_for_few_tiles_and_a_long_k(oracle, dev):
     assert_close(out[torch.from_numpy(rows).to(dev)].float().cpu().numpy(), oracle.gemm(a_r, b_r), scale, 1e-2, "few tiles, K split")
     c = torch.empty_like(out)
     rc = lib.iex_gemm(_lib.F16, 0, M, N, K, a.data_ptr(), b.data_ptr(), c.data_ptr(), 1, 0, 0, 0, torch.cuda.current_stream().cuda_stream)
-    assert rc == 0 and "splitk" not in _lib.last_kernels()
+    assert rc == 0 and "parts" not in _lib.last_kernels()
     torch.cuda.synchronize()
     assert torch.allclose(c.float(), out.float(), rtol=2e-2, atol=0.5)
 

@@ -748,7 +748,7 @@ def test_dense_form_path_is_chosen_with_a_workspace_and_only_then(oracle, dev):
 
 def test_dense_form_path_splits_k_where_the_product_has_few_tiles(oracle, dev):
     """4096 x 4096 at 70 % sparsity times 4096 x 128 in fp16: the dense form wins, and its product is 64 tiles of 64 x 128
-    with k = 4096, which the GEMM runs with k in two halves when it has room for the partial sums.  The size the
+    with k = 4096, which the GEMM runs with k in four parts when it has room for the partial sums.  The size the
     library asks for holds that room behind the dense form; the kernel that writes the dense form zeroes the tile words
     (no launch of its own for that); a workspace of the dense form alone still runs the path, unsplit; both agree with
     the oracle and every repeat gives the same bits."""
@@ -767,20 +767,20 @@ def test_dense_form_path_splits_k_where_the_product_has_few_tiles(oracle, dev):
     kw = dict(per_batch_values=False, accumulate=False, dtypes=(dtype,), allow_i16=True)
     out = pyops._spmm(b, ri, v, ro_t, ci_t, m, **kw)
     trail = _lib.last_kernels()
-    assert "csr_to_dense_kernel" in trail and "gemm_dma_splitk_kernel" in trail and "fill_zero" not in trail
+    assert "csr_to_dense_kernel" in trail and "gemm_dma_parts_kernel" in trail and "K in 4 parts" in trail and "fill_zero" not in trail
     for _ in range(3):
         assert torch.equal(out, pyops._spmm(b, ri, v, ro_t, ci_t, m, **kw))
     vals_r, b_r = rounded(csr.values, dtype), rounded(b_np, dtype)
     want = oracle.spmm(b_r, csr.row_indices, vals_r, csr.row_offsets, csr.column_indices, m)
     scale = oracle.spmm_abs_scale(b_r, csr.row_indices, vals_r, csr.row_offsets, csr.column_indices, m)
-    assert_close(out.float().cpu().numpy(), want, scale, RTOL[dtype], "dense form, k in two halves")
+    assert_close(out.float().cpu().numpy(), want, scale, RTOL[dtype], "dense form, k in parts")
     small = torch.empty(m * k * 2, dtype=torch.uint8, device=dev)
     unsplit = torch.empty_like(out)
     args = (_lib.F16, _lib.I16, 0, m, k, n, nnz, ri.data_ptr(), v.data_ptr(), ro_t.data_ptr(), ci_t.data_ptr(),
             b.data_ptr(), None, unsplit.data_ptr(), torch.cuda.current_stream().cuda_stream, 1)
     assert lib.iex_spmm_ws(*args, small.data_ptr(), m * k * 2) == 0, _lib.last_error()
     trail = _lib.last_kernels()
-    assert "csr_to_dense_kernel" in trail and "splitk" not in trail
+    assert "csr_to_dense_kernel" in trail and "parts" not in trail
     torch.cuda.synchronize()
     assert_close(unsplit.float().cpu().numpy(), want, scale, RTOL[dtype], "dense form, unsplit")
 

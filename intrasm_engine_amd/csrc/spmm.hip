@@ -581,7 +581,7 @@ int launch_dense_path(const SpmmParams& p, int batch, const Choice& ch, hipStrea
   int flag_words = 0;
   if (with_split) gemm_auto_split_flags(p.m, p.n, p.k, batch, &flags_at, &flag_words);
   note_kernel("csr_to_dense_kernel<%s>", type_name<IT>());
-  hipLaunchKernelGGL((csr_to_dense_kernel<IT>), dim3(p.m), dim3(kDenseThreads), 0, stream, p.m, p.k,
+  hipLaunchKernelGGL((csr_to_dense_kernel<IT>), dim3(ceil_div(p.m, kDenseRows)), dim3(kDenseThreads), 0, stream, p.m, p.k,
                      p.row_offsets, static_cast<const IT*>(p.cols), static_cast<const uint16_t*>(p.values),
                      static_cast<uint16_t*>(ch.ws), with_split ? reinterpret_cast<int*>(split_ws + flags_at) : nullptr, flag_words);
   if (int rc = check_hip(hipGetLastError(), "spmm dense-form launch")) return rc;

@@ -289,7 +289,7 @@ int launch_shape(const GemmParams& p, int batch, int force, hipStream_t stream, 
   if (small_tiles > 256) {
     // More 128 x 128 tiles than CUs: the tile shape that finishes first, counting whole rounds of workgroups (a
     // workgroup of the last round takes as long as any other) at the rate each shape reaches with every CU busy.
-    // TFLOP/s measured: 256 x 256 (one workgroup per CU) 1200; 128 x 256 by eight waves (64 x 64 each, two per
+    // TFLOP/s measured: 256 x 256 (one workgroup per CU, eight waves in two alternating groups) 1250; 128 x 256 by eight waves (64 x 64 each, two per
     // SIMD that cover for each other at the barrier and the waits of every K step; one workgroup per CU) 930,
     // by four waves (64 x 128 each) 790; 128 x 128 (two workgroups per CU) 750.
     //   4096 x 2048 x 4096 (config 4): 627 / 907 / 788 / 750      4096 x 4096 x 4096: 1080 / 985 / 903
@@ -299,10 +299,11 @@ int launch_shape(const GemmParams& p, int batch, int force, hipStream_t stream, 
       const long long tiles = (long long)ceil_div(p.M, bm) * ceil_div(p.N, bn) * batch;
       return (double)ceil_div(tiles, slots) * slots * bm * bn / rate;
     };
-    const double huge = cost(256, 256, 256, 1200.0), wide = cost(128, 256, 256, 930.0), small = cost(128, 128, 512, 750.0);
+    const double huge = cost(256, 256, 256, 1250.0), wide = cost(128, 256, 256, 930.0), small = cost(128, 128, 512, 750.0);
     // (256 x 256 by two groups of four waves in alternating phases, same-process comparison with the four-wave tile on
     // warmed-up clocks: 8192^3 1250 / 1230, 4096 x 8192 x 4096 1109 / 1076, 11008 x 8192 x 4096 1151 / 1109,
-    // 4096^3 1054 / 954; bit-equal results)
+    // 4096^3 1054 / 954; bit-equal results.  11008 x 2048 x 4096, where the two shapes are within 1 % in this count:
+    // 218 us in two rounds of 256 x 256 tiles, 221-230 in three of 128 x 256)
     if (huge <= wide && huge <= small) return launch_pp<BF16, TRANS_B, 4, 2, 4>(p, batch, stream);
     if (wide <= small) return launch_dma<BF16, TRANS_B, 2, 2, 32, 4, 4>(p, batch, stream);
     return launch_dma<BF16, TRANS_B, 2, 2, 32, 4>(p, batch, stream);

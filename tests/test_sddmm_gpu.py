@@ -186,6 +186,32 @@ def test_csr_softmax_pairs_of_16_bit_entries(oracle, dev, dtype, tail):
         assert np.abs(got - want).max() <= (2e-3 if dtype == torch.float16 else 8e-3), batch
 
 
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+def test_csr_softmax_four_rows_of_16_bit_entries_per_wavefront(oracle, dev, dtype):
+    """16-bit tensors whose rows average 512 entries or fewer run four rows per wavefront, 16 lanes per row, as many pairs
+    per lane as the longest of the four needs: row lengths on both sides of every pair count (32 p - 1, 32 p, 32 p + 1 for
+    p = 1 .. 16), in the order of the swizzle and in a shuffled order (rows of very different length in one wavefront, a
+    long row of 900 among them: that wavefront takes its rows one by one), a number of rows that is no multiple of 16, a
+    negative scale and an average above 512 (both: the kernel with a wavefront per row)."""
+    lens = np.array([x for p in range(1, 17) for x in (32 * p - 1, 32 * p, 32 * p + 1)] + [0, 900, 1, 0, 6])
+    ro = np.concatenate([[0], np.cumsum(lens)]).astype(np.int32)
+    rng = np.random.default_rng(5)
+    vals = rng.standard_normal((2, int(ro[-1]))).astype(np.float32) * 4
+    tol = 2e-3 if dtype == torch.float16 else 8e-3
+    for order in (W.swizzle_from_offsets(ro), rng.permutation(len(lens)).astype(np.int32)):
+        for scale in (0.5, -0.5):
+            v = torch.from_numpy(vals).to(dev).to(dtype)
+            ops.csr_softmax_(v, torch.from_numpy(order).to(dev), torch.from_numpy(ro).to(dev), scale)
+            want = oracle.csr_softmax(rounded(vals, dtype).astype(np.float64) * scale, ro)
+            assert np.abs(v.float().cpu().numpy() - want).max() <= tol, scale
+    long_lens = np.array([600, 700, 513, 520])
+    ro2 = np.concatenate([[0], np.cumsum(long_lens)]).astype(np.int32)
+    vals2 = rng.standard_normal((1, int(ro2[-1]))).astype(np.float32)
+    v2 = torch.from_numpy(vals2).to(dev).to(dtype)
+    ops.csr_softmax_(v2, torch.arange(4, dtype=torch.int32, device=dev), torch.from_numpy(ro2).to(dev), 1.0)
+    assert np.abs(v2.float().cpu().numpy() - oracle.csr_softmax(rounded(vals2, dtype).astype(np.float64), ro2)).max() <= tol
+
+
 def test_operator_argument_checks(dev):
     a, _, lhs_np, rhs_np = W.config1()
     ri, _, ro, ci = to_dev(a, dev)

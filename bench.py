@@ -139,6 +139,9 @@ def main():
     ap.add_argument("--sddmm-probe", action="store_true",
                     help="config 3's SDDMM (fp16, 16 heads), 3 launches of what the operator picks and 3 of the gather kernel "
                          "(for rocprofv3 --kernel-trace / --pmc)")
+    ap.add_argument("--softmax-probe", action="store_true",
+                    help="config 3's softmax over CSR rows (fp16, 16 heads): 5 launches with a positive scale (four rows per "
+                         "wavefront) and 5 with a negative one (the kernel with a wavefront per row), for rocprofv3")
     ap.add_argument("--fused-timeline", action="store_true",
                     help="config 4's fused launch in its three workgroup orders with the per-workgroup timeline switched on "
                          "(iex_fused_timeline): prints, per order, what each CU ran and when it went idle")
@@ -273,6 +276,16 @@ def main():
             for _ in range(3):
                 ops.sddmm_sputnik_half(qt_, kt_, ri_, ro_, ci_)
         log("[sddmm-probe] gather kernel:", _lib.last_kernels())
+        torch.cuda.synchronize()
+        return
+
+    if args.softmax_probe:
+        pat_, _, _, _ = W.config3()
+        ri_, _, ro_, _ = csr_dev(pat_)
+        base_ = torch.randn(16, pat_.nnz, device=dev, generator=torch.Generator(dev).manual_seed(5)).half()
+        for scale_ in (0.125, -0.125):
+            for _ in range(5):
+                ops.csr_softmax_(base_.clone(), ri_, ro_, scale_)
         torch.cuda.synchronize()
         return
 
